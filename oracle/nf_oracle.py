@@ -1,0 +1,276 @@
+"""ctypes/numpy binding of the CPU oracle (oracle/nf_oracle.c).
+
+TEST INFRASTRUCTURE ONLY.  Imported by tests/, by the smoke check and by the
+benchmark's cpu_baseline leg; the shipped package never imports it.
+
+All tensors are numpy arrays; fp16 tensors are ``np.float16`` (viewed as uint16
+bit patterns on the C side).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libnf_oracle.so")
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with the Makefile next to this file."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-s", "-C", _HERE] + (["-B"] if force else []))
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _declare(_lib)
+    return _lib
+
+
+_u16p = C.POINTER(C.c_uint16)
+_i32p = C.POINTER(C.c_int32)
+_f32p = C.POINTER(C.c_float)
+_u8p = C.POINTER(C.c_uint8)
+
+
+def _h(a):
+    """fp16 array -> uint16 pointer (None passes NULL)."""
+    if a is None:
+        return None
+    assert a.dtype == np.float16 and a.flags["C_CONTIGUOUS"], (a.dtype, a.flags)
+    return a.ctypes.data_as(_u16p)
+
+
+def _i(a):
+    if a is None:
+        return None
+    assert a.dtype == np.int32 and a.flags["C_CONTIGUOUS"], (a.dtype, a.flags)
+    return a.ctypes.data_as(_i32p)
+
+
+class NfoModel(C.Structure):
+    _fields_ = [
+        ("hidden", C.c_int), ("Hq", C.c_int), ("Hkv", C.c_int), ("d", C.c_int),
+        ("ffn", C.c_int), ("vocab", C.c_int), ("layers", C.c_int), ("page_size", C.c_int),
+        ("eps", C.c_float), ("rope_theta", C.c_float), ("rope_scale", C.c_float),
+        ("smooth_a", C.c_float), ("smooth_b", C.c_float),
+        ("embedding", _u16p), ("lm_head", _u16p), ("model_norm", _u16p),
+        ("w_kqv", C.POINTER(_u16p)), ("w_o", C.POINTER(_u16p)), ("w_gate", C.POINTER(_u16p)),
+        ("w_up", C.POINTER(_u16p)), ("w_down", C.POINTER(_u16p)), ("ln_attn", C.POINTER(_u16p)),
+        ("ln_ffn", C.POINTER(_u16p)), ("kv_data", C.POINTER(_u16p)),
+    ]
+
+
+class NfoBatch(C.Structure):
+    _fields_ = [
+        ("decodePrefillBorder", C.c_int), ("prefillNum", C.c_int), ("prefillTokensNum", C.c_int),
+        ("input_tokens", _i32p), ("input_indptr", _i32p), ("rev_input_indptr", _i32p),
+        ("per_token_offset", _i32p), ("kv_indptr", _i32p), ("kv_indices", _i32p),
+        ("kv_last_page_len", _i32p),
+    ]
+
+
+def _declare(l):
+    l.nfo_half_to_float.restype = C.c_float
+    l.nfo_half_to_float.argtypes = [C.c_uint16]
+    l.nfo_float_to_half.restype = C.c_uint16
+    l.nfo_float_to_half.argtypes = [C.c_float]
+    l.nfo_e4m3_to_float.restype = C.c_float
+    l.nfo_e4m3_to_float.argtypes = [C.c_uint8]
+    l.nfo_gemm_f16.restype = None
+    l.nfo_gemm_f16.argtypes = [_u16p, _u16p, _u16p, _u16p, C.c_int, C.c_int, C.c_int, C.c_float,
+                               C.c_float, C.c_int]
+    l.nfo_dual_swiglu_f16.restype = None
+    l.nfo_dual_swiglu_f16.argtypes = [_u16p, _u16p, _u16p, _u16p, _u16p, _u16p, C.c_int, C.c_int,
+                                      C.c_int]
+    l.nfo_gemm_f8w_f16.restype = None
+    l.nfo_gemm_f8w_f16.argtypes = [_u16p, _u8p, _f32p, _u16p, _u16p, C.c_int, C.c_int, C.c_int,
+                                   C.c_float, C.c_float]
+    l.nfo_rmsnorm_f16.restype = None
+    l.nfo_rmsnorm_f16.argtypes = [_u16p, _u16p, _u16p, C.c_int, C.c_int, C.c_float]
+    l.nfo_embedding_f16.restype = None
+    l.nfo_embedding_f16.argtypes = [_i32p, _u16p, _u16p, C.c_int, C.c_int]
+    l.nfo_keep_token_f16.restype = None
+    l.nfo_keep_token_f16.argtypes = [_u16p, _u16p, _i32p, C.c_int, C.c_int]
+    l.nfo_argmax_f16.restype = None
+    l.nfo_argmax_f16.argtypes = [_u16p, _u16p, _i32p, C.c_int, C.c_int]
+    l.nfo_kv_offset.restype = C.c_int64
+    l.nfo_kv_offset.argtypes = [C.c_int] * 8
+    l.nfo_rope_freq.restype = C.c_float
+    l.nfo_rope_freq.argtypes = [C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float]
+    l.nfo_ref_llama_rope.restype = None
+    l.nfo_ref_llama_rope.argtypes = [_u16p, _f32p, C.c_int, C.c_int, C.c_float, C.c_float]
+    l.nfo_rope_append_f16.restype = None
+    l.nfo_rope_append_f16.argtypes = [_u16p, _u16p, _u16p, _i32p, _i32p, _i32p, _i32p, C.c_int,
+                                      C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float,
+                                      C.c_float, C.c_float, _i32p, _i32p]
+    l.nfo_attention_paged_f16.restype = None
+    l.nfo_attention_paged_f16.argtypes = [_u16p, _u16p, _i32p, _u16p, _i32p, _i32p, _i32p, C.c_int,
+                                          C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    l.nfo_decoder_forward.restype = None
+    l.nfo_decoder_forward.argtypes = [C.POINTER(NfoModel), C.POINTER(NfoBatch), _u16p, _u16p, _u16p,
+                                      _i32p]
+
+
+# ------------------------------------------------------------------ operators
+
+
+def gemm(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False):
+    M, K = A.shape
+    N = B.shape[0] if b_col_major else B.shape[1]
+    assert (B.shape == (N, K)) if b_col_major else (B.shape == (K, N))
+    D = np.empty((M, N), np.float16)
+    lib().nfo_gemm_f16(_h(A), _h(B), _h(Cmat), _h(D), M, N, K, alpha, beta, int(b_col_major))
+    return D
+
+
+def dual_swiglu(A, Bg, Bu, return_parts=False):
+    M, K = A.shape
+    N = Bg.shape[1]
+    assert Bg.shape == (K, N) and Bu.shape == (K, N)
+    out = np.empty((M, N), np.float16)
+    d0 = np.empty((M, N), np.float16) if return_parts else None
+    d1 = np.empty((M, N), np.float16) if return_parts else None
+    lib().nfo_dual_swiglu_f16(_h(A), _h(Bg), _h(Bu), _h(out), _h(d0), _h(d1), M, N, K)
+    return (out, d0, d1) if return_parts else out
+
+
+def gemm_f8w(A, Bq, scale, Cmat=None, alpha=1.0, beta=0.0):
+    M, K = A.shape
+    N = Bq.shape[1]
+    assert Bq.dtype == np.uint8 and Bq.shape == (K, N) and scale.dtype == np.float32
+    D = np.empty((M, N), np.float16)
+    lib().nfo_gemm_f8w_f16(_h(A), Bq.ctypes.data_as(_u8p), scale.ctypes.data_as(_f32p), _h(Cmat),
+                           _h(D), M, N, K, alpha, beta)
+    return D
+
+
+def e4m3_to_float(v: int) -> float:
+    return lib().nfo_e4m3_to_float(v)
+
+
+def rmsnorm(x, w, eps=1e-5):
+    rows, H = x.shape
+    out = np.empty_like(x)
+    lib().nfo_rmsnorm_f16(_h(out), _h(x), _h(w), rows, H, eps)
+    return out
+
+
+def embedding(tokens, table):
+    T = tokens.shape[0]
+    H = table.shape[1]
+    out = np.empty((T, H), np.float16)
+    lib().nfo_embedding_f16(_i(tokens), _h(table), _h(out), T, H)
+    return out
+
+
+def keep_token(x, input_indptr, req_num):
+    H = x.shape[1]
+    out = np.empty((req_num, H), np.float16)
+    lib().nfo_keep_token_f16(_h(x), _h(out), _i(input_indptr), req_num, H)
+    return out
+
+
+def argmax(logits):
+    rows, cols = logits.shape
+    mv = np.empty((rows,), np.float16)
+    arg = np.empty((rows,), np.int32)
+    lib().nfo_argmax_f16(_h(logits), _h(mv), _i(arg), rows, cols)
+    return arg, mv
+
+
+def kv_offset(page, kv, entry, head, feat, page_size, Hkv, d):
+    return lib().nfo_kv_offset(page, kv, entry, head, feat, page_size, Hkv, d)
+
+
+def rope_freq(i, d, rope_scale, rope_theta, smooth_a=0.0, smooth_b=0.0):
+    return lib().nfo_rope_freq(i, d, rope_scale, rope_theta, smooth_a, smooth_b)
+
+
+def ref_llama_rope(x, offset, rope_scale=1.0, rope_theta=1e4):
+    d = x.shape[0]
+    out = np.empty((d,), np.float32)
+    lib().nfo_ref_llama_rope(_h(x), out.ctypes.data_as(_f32p), d, offset, rope_scale, rope_theta)
+    return out
+
+
+def rope_append(kqv, kv_data, kv_indices, kv_indptr, rev_input_indptr, per_token_offset, Hq, Hkv, d,
+                page_size, rope_scale=1.0, rope_theta=1e4, smooth_a=0.0, smooth_b=0.0,
+                return_index=False):
+    """Appends into kv_data IN PLACE; returns q_out (and (page, entry) per token)."""
+    T = kqv.shape[0]
+    assert kqv.shape[1] == (Hq + 2 * Hkv) * d
+    q_out = np.empty((T, Hq * d), np.float16)
+    pg = np.empty((T,), np.int32) if return_index else None
+    en = np.empty((T,), np.int32) if return_index else None
+    lib().nfo_rope_append_f16(_h(kqv), _h(q_out), _h(kv_data), _i(kv_indices), _i(kv_indptr),
+                              _i(rev_input_indptr), _i(per_token_offset), T, Hq, Hkv, d, page_size,
+                              rope_scale, rope_theta, smooth_a, smooth_b, _i(pg), _i(en))
+    return (q_out, pg, en) if return_index else q_out
+
+
+def attention_paged(q, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, Hq, Hkv, d,
+                    page_size, causal, out=None):
+    batch = kv_last_page_len.shape[0]
+    o = np.zeros_like(q) if out is None else out
+    lib().nfo_attention_paged_f16(_h(q), _h(o), _i(qo_indptr), _h(kv_data), _i(kv_indptr),
+                                  _i(kv_indices), _i(kv_last_page_len), batch, Hq, Hkv, d, page_size,
+                                  int(bool(causal)))
+    return o
+
+
+def _ptr_array(arrs):
+    arr = (_u16p * len(arrs))()
+    for i, a in enumerate(arrs):
+        arr[i] = _h(a)
+    return arr
+
+
+def decoder_forward(cfg: dict, weights: dict, kv_data: list, batch: dict, hidden_in=None,
+                    want_hidden=True, want_logits=False, want_sampled=True):
+    """cfg: hidden,Hq,Hkv,d,ffn,vocab,layers,page_size,eps,rope_theta,rope_scale,smooth_a,smooth_b.
+    weights: embedding, lm_head, model_norm and per-layer lists w_kqv,w_o,w_gate,w_up,w_down,
+    ln_attn, ln_ffn.  kv_data: per-layer pools, appended IN PLACE.  batch: the update-data arrays.
+    """
+    m = NfoModel()
+    for k in ("hidden", "Hq", "Hkv", "d", "ffn", "vocab", "layers", "page_size"):
+        setattr(m, k, int(cfg[k]))
+    for k in ("eps", "rope_theta", "rope_scale", "smooth_a", "smooth_b"):
+        setattr(m, k, float(cfg.get(k, {"eps": 1e-5, "rope_theta": 1e4, "rope_scale": 1.0}.get(k, 0.0))))
+    keep = []
+    m.embedding = _h(weights["embedding"])
+    m.lm_head = _h(weights["lm_head"])
+    m.model_norm = _h(weights["model_norm"])
+    for k in ("w_kqv", "w_o", "w_gate", "w_up", "w_down", "ln_attn", "ln_ffn"):
+        pa = _ptr_array(weights[k])
+        keep.append(pa)
+        setattr(m, k, pa)
+    kva = _ptr_array(kv_data)
+    m.kv_data = kva
+    b = NfoBatch()
+    b.decodePrefillBorder = int(batch["decodePrefillBorder"])
+    b.prefillNum = int(batch["prefillNum"])
+    b.prefillTokensNum = int(batch["prefillTokensNum"])
+    for k in ("input_tokens", "input_indptr", "rev_input_indptr", "per_token_offset", "kv_indptr",
+              "kv_indices", "kv_last_page_len"):
+        arr = None if batch.get(k) is None else np.ascontiguousarray(batch[k], dtype=np.int32)
+        keep.append(arr)  # the struct only holds raw pointers
+        setattr(b, k, _i(arr))
+    T = b.decodePrefillBorder + b.prefillTokensNum
+    req = b.decodePrefillBorder + b.prefillNum
+    hidden = np.empty((T, cfg["hidden"]), np.float16) if want_hidden else None
+    logits = np.empty((req, cfg["vocab"]), np.float16) if want_logits else None
+    sampled = np.empty((req,), np.int32) if want_sampled else None
+    lib().nfo_decoder_forward(C.byref(m), C.byref(b), _h(hidden_in), _h(hidden), _h(logits),
+                              _i(sampled))
+    return hidden, logits, sampled

@@ -1,0 +1,493 @@
+"""Pins the CPU oracle (oracle/nf_oracle.c) against what fixes its answers
+independently of its own formulas: float64 closed forms, brute force on tiny
+inputs, invariants, and the known-answer inputs of the reference's own test
+programs.  No GPU needed."""
+import math
+
+import numpy as np
+import pytest
+
+from nanoflow_amd import synth
+
+
+def f64(a):
+    return a.astype(np.float64)
+
+
+def rel_err(got, ref):
+    ref = f64(ref)
+    return np.abs(f64(got) - ref).max() / max(np.abs(ref).max(), 1e-30)
+
+
+# ------------------------------------------------------------------ fp16 helpers
+
+def test_half_roundtrip_all_bit_patterns(oracle):
+    l = oracle.lib()
+    pats = np.arange(65536, dtype=np.uint16)
+    as_f = pats.view(np.float16).astype(np.float32)
+    for p in list(range(0, 65536, 257)) + [0, 1, 0x3ff, 0x400, 0x7bff, 0x7c00, 0x8000, 0xfbff]:
+        v = l.nfo_half_to_float(p)
+        if math.isnan(as_f[p]):
+            assert math.isnan(v)
+        else:
+            assert v == as_f[p]
+            assert l.nfo_float_to_half(v) == p
+
+
+def test_float_to_half_rounding_matches_numpy(oracle):
+    l = oracle.lib()
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([rng.standard_normal(2000).astype(np.float32) * s
+                         for s in (1e-7, 1e-4, 1.0, 100.0, 7e4)])
+    xs = np.concatenate([xs, np.float32([65504, 65519.9, 65520, 1e-8, 5.96e-8, 2.98e-8, 2.9802326e-8])])
+    for x in xs:
+        with np.errstate(over="ignore"):
+            want = np.float32(x).astype(np.float16).view(np.uint16)
+        assert l.nfo_float_to_half(float(x)) == int(want), x
+
+
+# ------------------------------------------------------------------ GEMM
+
+@pytest.mark.parametrize("M,N,K", [(1, 8, 16), (7, 24, 40), (33, 130, 257), (128, 64, 512)])
+def test_gemm_closed_form(oracle, M, N, K):
+    rng = np.random.default_rng(1)
+    A = synth.normal_f16(rng, (M, K))
+    B = synth.normal_f16(rng, (K, N), 0.05)
+    Cm = synth.normal_f16(rng, (M, N))
+    ref = f64(A) @ f64(B)
+    D = oracle.gemm(A, B)
+    assert rel_err(D, ref) < 1e-3
+    D2 = oracle.gemm(A, B, Cm, alpha=0.5, beta=1.0)
+    assert rel_err(D2, 0.5 * ref + f64(Cm)) < 1e-3
+    # transposed-weight storage gives the same product
+    D3 = oracle.gemm(A, np.ascontiguousarray(B.T), b_col_major=True)
+    assert rel_err(D3, ref) < 1e-3
+
+
+def test_gemm_identity_and_operand_order(oracle):
+    # A.I == A exactly; a non-symmetric case fails if operands were transposed/swapped
+    rng = np.random.default_rng(2)
+    A = synth.normal_f16(rng, (5, 16))
+    I = np.eye(16, dtype=np.float16)
+    assert np.array_equal(oracle.gemm(A, I), A)
+    B = np.zeros((16, 8), np.float16)
+    B[3, 5] = 2.0  # picks column 3 of A into output column 5
+    D = oracle.gemm(A, B)
+    want = np.zeros((5, 8), np.float16)
+    want[:, 5] = (A[:, 3].astype(np.float32) * 2).astype(np.float16)
+    assert np.array_equal(D, want)
+
+
+def test_gemm_residual_beta_one_is_single_rounding(oracle):
+    # D = half(acc + C): one rounding, not half(half(acc) + C)
+    A = np.array([[1.0]], np.float16)
+    B = np.array([[2.0 ** -12]], np.float16)          # acc = 2^-12, below half ulp of 1.0 ... kept in fp32
+    Cm = np.array([[1.0 + 2.0 ** -10]], np.float16)
+    D = oracle.gemm(A, B, Cm, beta=1.0)
+    want = np.float16(np.float32(2.0 ** -12) + np.float32(Cm[0, 0]))
+    assert D[0, 0] == want
+
+
+# ------------------------------------------------------------------ dual GEMM (gate/up SwiGLU)
+
+def test_dual_known_answer_from_reference_test_inputs(oracle):
+    """Inputs of pipeline/src/test_dual.cu:13-22: every operand is the 128x128 matrix
+    X[j][k] = half((j+k)/2560); expected values computed here analytically in float64
+    from the rounded inputs (the program itself only prints)."""
+    M = N = K = 128
+    j, k = np.meshgrid(np.arange(M), np.arange(N), indexing="ij")
+    X = ((j + k).astype(np.float32) / 20 / 128).astype(np.float16)
+    out, d0, d1 = oracle.dual_swiglu(X, X, X, return_parts=True)
+    acc = f64(X) @ f64(X)
+    assert rel_err(d0, acc) < 1e-3 and rel_err(d1, acc) < 1e-3
+    g = f64(acc.astype(np.float16))
+    want = g / (1 + np.exp(-g)) * g
+    assert rel_err(out, want) < 1e-3
+    # spot values that a swapped gate/up or a missing SiLU would miss by far more
+    assert abs(float(out[0, 0]) - want[0, 0]) <= 1e-3 * abs(want[0, 0]) + 1e-6
+    assert abs(float(out[127, 127]) - want[127, 127]) <= 1e-3 * abs(want[127, 127])
+
+
+def test_dual_gate_is_first_weight(oracle):
+    rng = np.random.default_rng(3)
+    A = synth.normal_f16(rng, (9, 32))
+    Bg = synth.normal_f16(rng, (32, 16), 0.3)
+    Bu = synth.normal_f16(rng, (32, 16), 0.3)
+    out = oracle.dual_swiglu(A, Bg, Bu)
+    g = f64((f64(A) @ f64(Bg)).astype(np.float16))
+    u = f64((f64(A) @ f64(Bu)).astype(np.float16))
+    assert rel_err(out, g / (1 + np.exp(-g)) * u) < 2e-3
+    swapped = u / (1 + np.exp(-u)) * g
+    assert rel_err(out, swapped) > 5e-2
+
+
+# ------------------------------------------------------------------ fp8 weights
+
+def test_e4m3_decode_table(oracle):
+    # OCP e4m3fn: bias 7, no inf, max 448, subnormal step 2^-9
+    assert oracle.e4m3_to_float(0x00) == 0.0
+    assert oracle.e4m3_to_float(0x01) == 2.0 ** -9
+    assert oracle.e4m3_to_float(0x08) == 2.0 ** -6
+    assert oracle.e4m3_to_float(0x38) == 1.0
+    assert oracle.e4m3_to_float(0x7e) == 448.0
+    assert oracle.e4m3_to_float(0xfe) == -448.0
+    assert math.isnan(oracle.e4m3_to_float(0x7f))
+    import torch
+    t = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    for v in range(256):
+        got = oracle.e4m3_to_float(v)
+        assert (math.isnan(got) and math.isnan(t[v])) or got == t[v]
+
+
+def test_gemm_f8w_is_dequantise_then_gemm(oracle):
+    import torch
+    rng = np.random.default_rng(4)
+    M, N, K = 6, 24, 64
+    A = synth.normal_f16(rng, (M, K))
+    W = rng.standard_normal((K, N)).astype(np.float32) * 0.02
+    scale = (np.abs(W).max(axis=0) / 448.0).astype(np.float32)
+    Wq = torch.from_numpy(W / scale).to(torch.float8_e4m3fn)
+    Bq = Wq.view(torch.uint8).numpy()
+    deq = Wq.to(torch.float32).numpy().astype(np.float64) * scale
+    D = oracle.gemm_f8w(A, Bq, scale)
+    assert rel_err(D, f64(A) @ deq) < 1e-3
+
+
+# ------------------------------------------------------------------ row ops
+
+def test_rmsnorm_closed_form(oracle):
+    rng = np.random.default_rng(5)
+    x = synth.normal_f16(rng, (11, 256), 3.0)
+    w = synth.normal_f16(rng, (256,), 0.02, 1.0)
+    got = oracle.rmsnorm(x, w, 1e-5)
+    xf = f64(x)
+    want = xf / np.sqrt((xf ** 2).mean(axis=1, keepdims=True) + 1e-5) * f64(w)
+    assert rel_err(got, want) < 1e-3
+    # eps matters for a zero row: output must be exactly 0, not NaN
+    z = np.zeros((1, 256), np.float16)
+    assert np.array_equal(oracle.rmsnorm(z, w), z)
+
+
+def test_embedding_keep_token_bruteforce(oracle):
+    rng = np.random.default_rng(6)
+    table = synth.normal_f16(rng, (50, 64))
+    tok = rng.integers(0, 50, size=13, dtype=np.int32)
+    assert np.array_equal(oracle.embedding(tok, table), table[tok])
+    x = synth.normal_f16(rng, (13, 64))
+    indptr = np.array([0, 1, 2, 7, 13], np.int32)
+    assert np.array_equal(oracle.keep_token(x, indptr, 4), x[[0, 1, 6, 12]])
+
+
+def _argmax_literal(row):
+    """Literal python transcription of the 1024-slot scan + halving tree."""
+    NT = 1024
+    sval = [-10000.0] * NT
+    sidx = [0] * NT
+    for i, v in enumerate(row):
+        t = i % NT
+        if float(v) > sval[t]:
+            sval[t] = float(v)
+            sidx[t] = i
+    s = NT // 2
+    while s > 0:
+        for t in range(s):
+            if sval[t] < sval[t + s]:
+                sval[t] = sval[t + s]
+                sidx[t] = sidx[t + s]
+        s //= 2
+    return sidx[0], sval[0]
+
+
+def test_argmax_unique_max_and_ties(oracle):
+    rng = np.random.default_rng(7)
+    x = synth.normal_f16(rng, (6, 3000))
+    arg, mv = oracle.argmax(x)
+    assert np.array_equal(arg, x.astype(np.float32).argmax(axis=1))
+    assert np.array_equal(mv, x.max(axis=1))
+    # ties: equal maxima at several columns -> the reference's scan/tree order decides
+    t = np.full((4, 2500), -1.0, np.float16)
+    t[0, [5, 1029, 6]] = 3.0          # same slot 5 twice (first wins), slot 6
+    t[1, [512, 256, 768]] = 3.0       # bit-reversed priority: 512 (0b1000000000) wins over 256
+    t[2, [1, 2]] = 3.0                # even slot wins the last tree level
+    t[3, :] = -20000.0                # nothing above the -10000 start: index 0
+    arg, mv = oracle.argmax(t)
+    for r in range(4):
+        want_i, want_v = _argmax_literal(t[r])
+        assert arg[r] == want_i, (r, arg[r], want_i)
+        assert float(mv[r]) == np.float16(want_v)
+    assert arg[1] == 512 and arg[2] == 2 and arg[3] == 0
+
+
+# ------------------------------------------------------------------ RoPE + paged append
+
+def test_kv_offset_layout(oracle):
+    # pool[page][kv][entry][head][feat]; V half sits page_size*Hkv*d elements after K
+    P, Hkv, d = 16, 8, 128
+    pool = np.arange(3 * 2 * P * Hkv * d).reshape(3, 2, P, Hkv, d)
+    for idx in [(0, 0, 0, 0, 0), (2, 1, 15, 7, 127), (1, 0, 3, 2, 5), (1, 1, 3, 2, 5)]:
+        assert oracle.kv_offset(*idx, P, Hkv, d) == pool[idx]
+    assert oracle.kv_offset(1, 1, 3, 2, 5, P, Hkv, d) - oracle.kv_offset(1, 0, 3, 2, 5, P, Hkv, d) == P * Hkv * d
+
+
+def _rope_f64(x, pos, theta, d, scale=1.0):
+    i = np.arange(d)
+    inv = (pos / scale) / theta ** (2.0 * (i % (d // 2)) / d)
+    perm = np.where(i < d // 2, -np.roll(f64(x), -d // 2), np.roll(f64(x), d // 2))
+    return np.cos(inv) * f64(x) + np.sin(inv) * perm
+
+
+def test_rope_matches_reference_cpu_rule_and_float64(oracle):
+    rng = np.random.default_rng(8)
+    d = 128
+    for pos in (0, 1, 17, 1023, 1535):
+        x = synth.normal_f16(rng, (d,))
+        ref32 = oracle.ref_llama_rope(x, pos, 1.0, 5e5)
+        want = _rope_f64(x, pos, 5e5, d)
+        assert np.abs(ref32 - want).max() < 2e-3 * np.abs(want).max()
+
+
+def test_rope_append_indices_values_and_invariants(oracle):
+    rng = np.random.default_rng(9)
+    Hq, Hkv, d, P = 8, 2, 128, 16
+    b = synth.make_batch([5, 31, 16, 0], [(0, 20), (37, 9)], vocab=100, page_size=P, seed=1,
+                         extra_pages=3)
+    T = b.tokens
+    kqv = synth.normal_f16(rng, (T, (Hq + 2 * Hkv) * d))
+    pool = np.zeros((b.num_pages, 2, P, Hkv, d), np.float16)
+    q, pg, en = oracle.rope_append(kqv, pool, b.kv_indices, b.kv_indptr, b.rev_input_indptr,
+                                   b.per_token_offset, Hq, Hkv, d, P, 1.0, 5e5, return_index=True)
+    touched = np.zeros((b.num_pages, P), bool)
+    for t in range(T):
+        r, p = b.rev_input_indptr[t], b.per_token_offset[t]
+        page = b.kv_indices[b.kv_indptr[r] + p // P]
+        assert (pg[t], en[t]) == (page, p % P)                      # bit-exact index rule
+        assert not touched[page, p % P]
+        touched[page, p % P] = True
+        row = kqv[t].reshape(Hq + 2 * Hkv, d)
+        assert np.array_equal(pool[page, 1, p % P], row[Hkv:2 * Hkv])  # V copied bit-exact
+        for h in range(Hkv):
+            want = _rope_f64(row[h], p, 5e5, d)
+            assert np.abs(f64(pool[page, 0, p % P, h]) - want).max() < 2e-3 * np.abs(want).max() + 1e-3
+        for h in range(Hq):
+            want = _rope_f64(row[2 * Hkv + h], p, 5e5, d)
+            got = q[t].reshape(Hq, d)[h]
+            assert np.abs(f64(got) - want).max() < 2e-3 * np.abs(want).max() + 1e-3
+            # rotation preserves the norm of each (i, i+d/2) pair
+            n_in = f64(row[2 * Hkv + h][:64]) ** 2 + f64(row[2 * Hkv + h][64:]) ** 2
+            n_out = f64(got[:64]) ** 2 + f64(got[64:]) ** 2
+            assert np.abs(n_in - n_out).max() < 2e-2 * max(n_in.max(), 1.0)
+        if p == 0:  # position 0 is the identity
+            assert np.array_equal(pool[page, 0, 0], row[:Hkv])
+            assert np.array_equal(q[t].reshape(Hq, d), row[2 * Hkv:])
+    # nothing else in the pool was written
+    untouched = np.transpose(pool, (0, 2, 1, 3, 4))[~touched]
+    assert not untouched.any()
+    assert touched.sum() == T
+
+
+def test_rope_llama31_smoothing_matches_wavelength_form(oracle):
+    # Llama-3.1 rule written over wavelengths (the published form) vs the reference's
+    # smooth_a/smooth_b form (pipeline/include/config.h:101-110)
+    factor, low, high, orig, theta, d = 8.0, 1.0, 4.0, 8192, 5e5, 128
+    smooth_a = orig / (2 * math.pi * high - 2 * math.pi * low)
+    smooth_b = -1.0 / (high / low - 1.0)
+    for i in range(d):
+        f = theta ** (-2.0 * (i % (d // 2)) / d)
+        wavelen = 2 * math.pi / f
+        if wavelen < orig / high:
+            want = f
+        elif wavelen > orig / low:
+            want = f / factor
+        else:
+            s = (orig / wavelen - low) / (high - low)
+            want = (1 - s) * f / factor + s * f
+        got = oracle.rope_freq(i, d, factor, theta, smooth_a, smooth_b)
+        assert abs(got - want) <= 2e-5 * want, (i, got, want)
+    # no scaling: plain theta^(-2i/d)
+    assert abs(oracle.rope_freq(3, d, 1.0, theta) - theta ** (-6.0 / d)) < 1e-6
+
+
+# ------------------------------------------------------------------ attention
+
+def _dense_attention_f64(q, k, v, causal, group):
+    # q [qo, Hq, d], k/v [kv, Hkv, d]
+    qo, Hq, d = q.shape
+    kv = k.shape[0]
+    out = np.zeros((qo, Hq, d))
+    for h in range(Hq):
+        s = f64(q[:, h]) @ f64(k[:, h // group]).T / math.sqrt(d)
+        if causal:
+            qi, ki = np.meshgrid(np.arange(qo), np.arange(kv), indexing="ij")
+            s = np.where(ki > kv + qi - qo, -np.inf, s)
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        p /= p.sum(axis=1, keepdims=True)
+        out[:, h] = p @ f64(v[:, h // group])
+    return out
+
+
+def _gather_kv(pool, b, r, P):
+    pages = b.kv_indices[b.kv_indptr[r]:b.kv_indptr[r + 1]]
+    L = b.kv_len[r]
+    k = pool[pages, 0].reshape(-1, *pool.shape[3:])[:L]
+    v = pool[pages, 1].reshape(-1, *pool.shape[3:])[:L]
+    return k, v
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (8, 1), (4, 4)])
+def test_attention_vs_dense_float64(oracle, Hq, Hkv):
+    rng = np.random.default_rng(10)
+    d, P = 128, 16
+    b = synth.make_batch([15, 16, 40], [(0, 20), (21, 13)], vocab=10, page_size=P, seed=2, extra_pages=2)
+    pool = synth.make_kv_pool(b.num_pages, synth.ModelShape(Hq=Hq, Hkv=Hkv), rng)
+    q = synth.normal_f16(rng, (b.tokens, Hq * d))
+    nd = b.decodePrefillBorder
+    o = oracle.attention_paged(q, b.input_indptr[:nd + 1], pool, b.kv_indptr[:nd + 1], b.kv_indices,
+                               b.kv_last_page_len[:nd], Hq, Hkv, d, P, causal=False)
+    o = oracle.attention_paged(q, b.input_indptr[nd:], pool, b.kv_indptr[nd:], b.kv_indices,
+                               b.kv_last_page_len[nd:], Hq, Hkv, d, P, causal=True, out=o)
+    for r in range(b.req_num):
+        k, v = _gather_kv(pool, b, r, P)
+        rows = slice(b.input_indptr[r], b.input_indptr[r + 1])
+        want = _dense_attention_f64(q[rows].reshape(-1, Hq, d), k, v, causal=r >= nd, group=Hq // Hkv)
+        got = f64(o[rows]).reshape(-1, Hq, d)
+        assert np.abs(got - want).max() < 2e-3 * np.abs(want).max() + 1e-3, r
+
+
+def test_attention_invariants(oracle):
+    rng = np.random.default_rng(11)
+    Hq, Hkv, d, P = 8, 2, 128, 16
+    shape = synth.ModelShape(Hq=Hq, Hkv=Hkv)
+    # (1) all keys equal -> uniform softmax -> output = mean of V
+    b = synth.make_batch([36], [], vocab=10, page_size=P, seed=3)
+    pool = synth.make_kv_pool(b.num_pages, shape, rng)
+    pool[:, 0] = pool[0, 0, 0]
+    q = synth.normal_f16(rng, (1, Hq * d))
+    o = oracle.attention_paged(q, b.input_indptr, pool, b.kv_indptr, b.kv_indices, b.kv_last_page_len,
+                               Hq, Hkv, d, P, causal=False)
+    k, v = _gather_kv(pool, b, 0, P)
+    want = np.repeat(f64(v).mean(axis=0), Hq // Hkv, axis=0).reshape(-1)
+    assert np.abs(f64(o[0]) - want).max() < 2e-3
+
+    # (2) one-hot: one key aligned with q and huge -> output = that V row
+    pool2 = synth.make_kv_pool(b.num_pages, shape, rng)
+    pool2[:, 0] = 0
+    pg, en = b.kv_indices[1], 3                       # token 19 of the request
+    qv = np.zeros((1, Hq, d), np.float16)
+    qv[..., 0] = 30.0
+    pool2[pg, 0, en, :, 0] = 30.0
+    o = oracle.attention_paged(qv.reshape(1, -1), b.input_indptr, pool2, b.kv_indptr, b.kv_indices,
+                               b.kv_last_page_len, Hq, Hkv, d, P, causal=False)
+    want = np.repeat(f64(pool2[pg, 1, en]), Hq // Hkv, axis=0).reshape(-1)
+    assert np.abs(f64(o[0]) - want).max() < 2e-3
+
+    # (3) page-table permutation invariance: move pages, same result
+    b3 = synth.make_batch([50, 20], [(0, 33)], vocab=10, page_size=P, seed=4, extra_pages=5)
+    pool3 = synth.make_kv_pool(b3.num_pages, shape, rng)
+    q3 = synth.normal_f16(rng, (b3.tokens, Hq * d))
+    o_a = oracle.attention_paged(q3, b3.input_indptr, pool3, b3.kv_indptr, b3.kv_indices,
+                                 b3.kv_last_page_len, Hq, Hkv, d, P, causal=True)
+    perm = rng.permutation(b3.num_pages)
+    pool3p = np.empty_like(pool3)
+    pool3p[perm] = pool3
+    o_b = oracle.attention_paged(q3, b3.input_indptr, pool3p, b3.kv_indptr,
+                                 perm[b3.kv_indices].astype(np.int32), b3.kv_last_page_len, Hq, Hkv,
+                                 d, P, causal=True)
+    assert np.array_equal(o_a, o_b)
+
+    # (4) decode == prefill with qo_len 1 (causal flag irrelevant for a single last row)
+    b4 = synth.make_batch([29], [], vocab=10, page_size=P, seed=5)
+    pool4 = synth.make_kv_pool(b4.num_pages, shape, rng)
+    q4 = synth.normal_f16(rng, (1, Hq * d))
+    args = (q4, b4.input_indptr, pool4, b4.kv_indptr, b4.kv_indices, b4.kv_last_page_len, Hq, Hkv, d, P)
+    assert np.array_equal(oracle.attention_paged(*args, causal=False),
+                          oracle.attention_paged(*args, causal=True))
+
+
+def test_chunked_prefill_equals_single_prefill(oracle):
+    """A 45-token prompt in chunks 20+25 (second chunk sees the first's KV) gives the
+    same rows as one 45-token causal prefill."""
+    rng = np.random.default_rng(12)
+    Hq, Hkv, d, P = 4, 2, 128, 16
+    shape = synth.ModelShape(Hq=Hq, Hkv=Hkv)
+    full = synth.make_batch([], [(0, 45)], vocab=10, page_size=P, seed=6, permute=False)
+    pool = synth.make_kv_pool(full.num_pages, shape, rng)
+    q = synth.normal_f16(rng, (45, Hq * d))
+    o_full = oracle.attention_paged(q, full.input_indptr, pool, full.kv_indptr, full.kv_indices,
+                                    full.kv_last_page_len, Hq, Hkv, d, P, causal=True)
+    c1 = synth.make_batch([], [(0, 20)], vocab=10, page_size=P, seed=6, permute=False)
+    o1 = oracle.attention_paged(q[:20].copy(), c1.input_indptr, pool, c1.kv_indptr, c1.kv_indices,
+                                c1.kv_last_page_len, Hq, Hkv, d, P, causal=True)
+    c2 = synth.make_batch([], [(20, 25)], vocab=10, page_size=P, seed=6, permute=False)
+    o2 = oracle.attention_paged(q[20:].copy(), c2.input_indptr, pool, c2.kv_indptr, c2.kv_indices,
+                                c2.kv_last_page_len, Hq, Hkv, d, P, causal=True)
+    assert np.array_equal(o_full[:20], o1)
+    assert np.array_equal(o_full[20:], o2)
+
+
+# ------------------------------------------------------------------ whole decoder
+
+def _numpy_decoder_f64(shape, w, pools, b):
+    """Independent float64 forward of the same model (no fp16 rounding between ops)."""
+    d, Hq, Hkv, P = shape.d, shape.Hq, shape.Hkv, shape.page_size
+    x = f64(w["embedding"][b.input_tokens])
+    pools = [f64(p) for p in pools]
+
+    def norm(v, g):
+        return v / np.sqrt((v ** 2).mean(axis=1, keepdims=True) + shape.eps) * f64(g)
+
+    for l in range(shape.layers):
+        kqv = norm(x, w["ln_attn"][l]) @ f64(w["w_kqv"][l])
+        attn = np.zeros((b.tokens, Hq * d))
+        qrot = np.zeros((b.tokens, Hq, d))
+        for t in range(b.tokens):
+            r, p = b.rev_input_indptr[t], b.per_token_offset[t]
+            page = b.kv_indices[b.kv_indptr[r] + p // P]
+            row = kqv[t].reshape(Hq + 2 * Hkv, d)
+            for h in range(Hkv):
+                pools[l][page, 0, p % P, h] = _rope_f64(row[h], p, shape.rope_theta, d)
+                pools[l][page, 1, p % P, h] = row[Hkv + h]
+            for h in range(Hq):
+                qrot[t, h] = _rope_f64(row[2 * Hkv + h], p, shape.rope_theta, d)
+        for r in range(b.req_num):
+            pages = b.kv_indices[b.kv_indptr[r]:b.kv_indptr[r + 1]]
+            L = b.kv_len[r]
+            k = pools[l][pages, 0].reshape(-1, Hkv, d)[:L]
+            v = pools[l][pages, 1].reshape(-1, Hkv, d)[:L]
+            rows = slice(b.input_indptr[r], b.input_indptr[r + 1])
+            attn[rows] = _dense_attention_f64(qrot[rows], k, v, r >= b.decodePrefillBorder,
+                                              Hq // Hkv).reshape(-1, Hq * d)
+        xo = attn @ f64(w["w_o"][l]) + x
+        h = norm(xo, w["ln_ffn"][l])
+        g = h @ f64(w["w_gate"][l])
+        u = h @ f64(w["w_up"][l])
+        x = (g / (1 + np.exp(-g)) * u) @ f64(w["w_down"][l]) + xo
+    last = x[b.input_indptr[1:] - 1]
+    logits = norm(last, w["model_norm"]) @ f64(w["lm_head"])
+    return x, logits
+
+
+def test_decoder_forward_vs_independent_float64_model(oracle):
+    shape = synth.tiny_shape(layers=2, vocab=512, hidden=256, Hq=4, Hkv=2, ffn=384)
+    # larger-than-init weights so the residual stream is not dominated by the embedding
+    w = synth.make_weights(shape, seed=0)
+    for k in ("w_kqv", "w_o", "w_gate", "w_up", "w_down"):
+        w[k] = [(a.astype(np.float32) * 3).astype(np.float16) for a in w[k]]
+    w["embedding"] = (w["embedding"].astype(np.float32) * 30).astype(np.float16)
+    b = synth.make_batch([17, 40, 3], [(0, 21), (16, 10)], vocab=shape.vocab, seed=7, extra_pages=2)
+    rng = np.random.default_rng(1)
+    pools = [synth.make_kv_pool(b.num_pages, shape, rng) for _ in range(shape.layers)]
+    pools_in = [p.copy() for p in pools]
+    hidden, logits, sampled = oracle.decoder_forward(shape.as_dict(), w, pools, b.as_dict(),
+                                                     want_logits=True)
+    ref_x, ref_logits = _numpy_decoder_f64(shape, w, pools_in, b)
+    assert rel_err(hidden, ref_x) < 4e-3
+    assert rel_err(logits, ref_logits) < 6e-3
+    # sampled ids agree wherever the float64 top-1/top-2 gap is clear of fp16 noise
+    top2 = np.sort(ref_logits, axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 1e-2 * np.abs(ref_logits).max()
+    assert clear.sum() >= 1
+    assert np.array_equal(sampled[clear], ref_logits.argmax(axis=1)[clear])
+    # the pools changed only at the appended slots
+    for l in range(shape.layers):
+        diff = (pools[l] != pools_in[l]).any(axis=(1, 3, 4))
+        assert diff.sum() == b.tokens
