@@ -1,0 +1,133 @@
+/*
+ * nanoflow_kernels.h -- C ABI of the MI355X (gfx950) kernel layer.
+ *
+ * One entry point per operator of the reference's single-device nano-batch
+ * pipeline.  Every function takes raw DEVICE pointers, plain sizes and a HIP
+ * stream (as void*; NULL = the default stream), enqueues its kernels on that
+ * stream without synchronising, and returns 0 on success or a negative
+ * NF_ERR_* code (nf_last_error() gives the text).  fp16 tensors are IEEE
+ * binary16 bit patterns (uint16_t).  No function allocates device memory.
+ *
+ * Each declaration cites the reference interface it replaces
+ * (paths relative to the reference checkout).
+ */
+#ifndef NANOFLOW_KERNELS_H
+#define NANOFLOW_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* nf_stream_t; /* hipStream_t */
+
+/* Exported symbols (the library is built with hidden default visibility). */
+#define NF_API __attribute__((visibility("default")))
+
+#define NF_OK 0
+#define NF_ERR_INVALID_ARGUMENT (-1) /* shape/pointer rejected before any launch */
+#define NF_ERR_UNSUPPORTED (-2)      /* valid request this build has no kernel for */
+#define NF_ERR_RUNTIME (-3)          /* HIP runtime reported an error */
+#define NF_ERR_WORKSPACE (-4)        /* caller's workspace is too small */
+
+/* ABI version of this header (bumped on any signature change). */
+NF_API int nf_abi_version(void);
+/* Text of the last error raised on the calling thread ("" if none). */
+NF_API const char* nf_last_error(void);
+
+/* x[t,:] = table[tokens[t],:]; hidden % 8 == 0.
+ * Replaces genEmbedding<<<>>> as launched by GenEmbedding::work
+ * (pipeline/src/small_cuda_operator.cu:9-24, pipeline/include/otherWrapper.cuh:166-171). */
+NF_API int nf_embedding_f16(const int32_t* tokens, const uint16_t* table, uint16_t* out, int n_tokens,
+                     int hidden, nf_stream_t stream);
+
+/* out = half(x * rsqrt(mean(x^2) + eps) * weight), fp32 math; hidden % 8 == 0.
+ * Replaces rms_norm() (pipeline/include/rms_norm.cuh:48-127,210-233) called by
+ * LayerNorm::work (pipeline/include/otherWrapper.cuh:94-102). */
+NF_API int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* weight, int rows, int hidden,
+                   float eps, nf_stream_t stream);
+
+/* D = half(alpha * A.B + beta * C), fp16 operands, fp32 accumulate on MFMA.
+ * A [M,K] row-major; B [K,N] row-major when b_col_major == 0, [N,K] row-major
+ * (K contiguous) when 1; C and D [M,N] row-major; C may alias D or be NULL when
+ * beta == 0.  K % 32 == 0, N % 8 == 0.
+ * Replaces CutlassGEMMWrapper::work / cutlass::gemm::device::Gemm
+ * (pipeline/include/cutlassGemmWrapperImpl.cuh:68-166). */
+NF_API int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
+                int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
+
+/* out = half(silu(float(half(A.Bgate))) * float(half(A.Bup))); A [M,K], Bgate/Bup [K,N],
+ * out [M,N], all row-major.  K % 32 == 0, N % 8 == 0.
+ * Replaces DualWrapper::work / cutlass DualGemm + LeftSiLUAndMul
+ * (pipeline/include/dualWrapper.cuh:95-144,192-194). */
+NF_API int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
+                       int M, int N, int K, nf_stream_t stream);
+
+/* D = half(alpha * scale[n] * A.dequant(Bq) + beta * C) with Bq [K,N] OCP fp8 e4m3
+ * bytes and one fp32 scale per output channel.  No counterpart in the reference
+ * (its GEMM wrappers are half-only, pipeline/include/cutlassGemmWrapperImpl.cuh:24-27);
+ * same operand roles as nf_gemm_f16. */
+NF_API int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* scale, const uint16_t* C,
+                    uint16_t* D, int M, int N, int K, float alpha, float beta, nf_stream_t stream);
+
+/* Per token t of kqv [n_tokens,(Hq+2Hkv)*d] (columns K | V | Q): request
+ * r = rev_input_indptr[t], position p = per_token_offset[t],
+ * page = kv_indices[kv_indptr[r] + p / page_size], entry = p % page_size;
+ * K heads -> rotate-half RoPE at p -> kv_data[page][0][entry]; V heads -> copied to
+ * kv_data[page][1][entry]; Q heads -> RoPE -> q_out[t].  kv_data is one layer's pool
+ * [pages][2][page_size][Hkv][d].  head_dim must be 128.
+ * rope_scale / smooth_a / smooth_b implement the Llama-3.1 frequency rule; pass
+ * 1, 0, 0 for plain RoPE.
+ * Replaces flashinfer::splitRopeAppend (pipeline/include/small_cuda_operator.cuh:21-133)
+ * called by RoPEAppend::work (pipeline/include/otherWrapper.cuh:345-380). */
+NF_API int nf_rope_append_f16(const uint16_t* kqv, uint16_t* q_out, uint16_t* kv_data,
+                       const int32_t* kv_indices, const int32_t* kv_indptr,
+                       const int32_t* rev_input_indptr, const int32_t* per_token_offset,
+                       int n_tokens, int num_qo_heads, int num_kv_heads, int head_dim,
+                       int page_size, float rope_scale, float rope_theta, float smooth_a,
+                       float smooth_b, nf_stream_t stream);
+
+/* Bytes of device workspace nf_attention_paged_f16 needs for this problem size. */
+NF_API size_t nf_attention_workspace_bytes(int batch, int max_qo_rows, int num_qo_heads);
+
+/* Batched attention over a paged KV pool.  For request i in [0,batch): query rows
+ * qo_indptr[i]..qo_indptr[i+1] of q/o (ABSOLUTE row indices into buffers of row
+ * width Hq*d), keys/values = pages kv_indices[kv_indptr[i]..kv_indptr[i+1]) with
+ * kv_last_page_len[i] valid entries in the last page.  causal != 0: row j of a
+ * request with qo_len rows sees keys <= kv_len - qo_len + j.  sm_scale = 1/sqrt(d),
+ * no position encoding inside.  head_dim 128, page_size 16, Hq/Hkv in {1,2,4,8}.
+ * max_qo_rows: an upper bound on the total number of query rows of the batch
+ * (sizes the launch; a bound that is too small is an error the kernel cannot see).
+ * num_blocks > 0 caps the number of workgroups (the reference's sm_blk); 0 = fill
+ * the device.  workspace: nf_attention_workspace_bytes() bytes of device scratch.
+ * Replaces BatchPrefillWithPagedKVCacheWrapper as used by DecodeGemvWrapper::work
+ * (causal=false, pipeline/include/gemvWrapper.cuh:201-228) and PrefillGemvWrapper::work
+ * (causal=true, :322-374), including the planning done by BatchPrefillHandler::BeginForward
+ * (gemv/include/attention/handler.cuh:557-595), which here runs on the device. */
+NF_API int nf_attention_paged_f16(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
+                           const uint16_t* kv_data, const int32_t* kv_indptr,
+                           const int32_t* kv_indices, const int32_t* kv_last_page_len, int batch,
+                           int max_qo_rows, int num_qo_heads, int num_kv_heads, int head_dim,
+                           int page_size, int causal, int num_blocks, void* workspace,
+                           size_t workspace_bytes, nf_stream_t stream);
+
+/* out[r,:] = in[input_indptr[r+1]-1,:] (last token of each request); hidden % 8 == 0.
+ * Replaces copySelectedRows (pipeline/src/small_cuda_operator.cu:217-251) called by
+ * KeepToken::work (pipeline/include/otherWrapper.cuh:521-523). */
+NF_API int nf_keep_token_f16(const uint16_t* in, uint16_t* out, const int32_t* input_indptr, int req_num,
+                      int hidden, nf_stream_t stream);
+
+/* Row argmax over fp16 logits [rows, cols] -> argmax[rows] (and max_vals[rows] when not
+ * NULL), with the tie order of the reference kernel (values <= -10000 never win;
+ * equal maxima: smallest bit-reversed (col mod 1024), then smallest col).
+ * Replaces computeRowMax (pipeline/src/small_cuda_operator.cu:165-214) called by
+ * MaxSampling::work (pipeline/include/otherWrapper.cuh:489-491). */
+NF_API int nf_argmax_f16(const uint16_t* logits, uint16_t* max_vals, int32_t* argmax, int rows, int cols,
+                  nf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NANOFLOW_KERNELS_H */

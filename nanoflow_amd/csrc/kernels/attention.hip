@@ -1,0 +1,373 @@
+// Paged-KV attention for gfx950: decode (one query row per request, HBM-bound) and
+// chunked prefill (causal, many rows) from one kernel template on v_mfma_f32_16x16x32_f16.
+//
+// Formulation per (request, kv head):   S^T = K . Q^T   then   O^T = V^T . P^T
+//   * the MFMA "column" dimension (16 wide) carries query rows: column c of a block is
+//     (token c / GROUP, q head c % GROUP) of the kv head's GQA group, so decode with GROUP 4
+//     uses 4 live columns and a prefill block packs 16 / GROUP tokens;
+//   * S^T comes out of the first MFMA with a lane holding 4 consecutive kv positions of one
+//     column -- exactly the B-operand layout of the second MFMA, so P never leaves registers;
+//   * K rows are loaded straight into A-operand registers (16 bytes per lane per MFMA);
+//   * V^T operands are built from eight 16-byte row loads by an 8x8 half transpose in
+//     registers (32 byte-permutes); the output row order is chosen so that each lane ends with
+//     8 consecutive features per register quad (16-byte stores).
+// Online softmax runs in the exp2 domain with fp32 state per column; masked keys contribute
+// exactly zero (the reference's -5e4 mask underflows to zero in fp32 as well).
+//
+// Decode mode: a workgroup's 4 wavefronts split the request's pages (32 keys per step each)
+// and merge (m, l, O) through LDS.  Prefill mode: each wavefront owns its own query tile.
+// Work items are (tile, kv head) with the head fastest, so concurrently running workgroups
+// stream the same pages.  Tiles are planned on the device from qo_indptr (prefix of tiles per
+// request), no host round trip.
+#include "common.h"
+
+namespace nf {
+
+constexpr int D = 128;      // head_dim
+constexpr int PAGE = 16;    // kv entries per page
+
+__device__ __forceinline__ uint32_t pk_lo(uint32_t x, uint32_t y) {
+  return __builtin_amdgcn_perm(y, x, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t pk_hi(uint32_t x, uint32_t y) {
+  return __builtin_amdgcn_perm(y, x, 0x07060302u);
+}
+
+union H8 {
+  u32x4 u;
+  half8_t h;
+  uint32_t w[4];
+};
+
+// tile_start[i] = number of tiles of requests < i; tile_start[batch] = total.
+__global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restrict__ qo_indptr,
+                                                        int32_t* __restrict__ tile_start, int batch,
+                                                        int wg_tok) {
+  __shared__ int s_sum[256];
+  const int per = (batch + 255) / 256;
+  const int lo = threadIdx.x * per, hi = min(lo + per, batch);
+  int sum = 0;
+  for (int i = lo; i < hi; ++i) {
+    int len = qo_indptr[i + 1] - qo_indptr[i];
+    sum += len > 0 ? (len + wg_tok - 1) / wg_tok : 0;
+  }
+  s_sum[threadIdx.x] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int t = 0; t < 256; ++t) {
+      int v = s_sum[t];
+      s_sum[t] = run;
+      run += v;
+    }
+    tile_start[batch] = run;
+  }
+  __syncthreads();
+  int run = s_sum[threadIdx.x];
+  for (int i = lo; i < hi; ++i) {
+    tile_start[i] = run;
+    int len = qo_indptr[i + 1] - qo_indptr[i];
+    run += len > 0 ? (len + wg_tok - 1) / wg_tok : 0;
+  }
+}
+
+template <int GROUP, int NQB, bool SPLIT>
+__global__ __launch_bounds__(256) void attn_paged_kernel(
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ o, const int32_t* __restrict__ qo_indptr,
+    const uint16_t* __restrict__ kv_data, const int32_t* __restrict__ kv_indptr,
+    const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_last_page_len,
+    const int32_t* __restrict__ tile_start, int batch, int Hq, int Hkv, int causal,
+    float scale_log2) {
+  constexpr int TPB = 16 / GROUP;        // tokens per 16-column block
+  constexpr int WAVE_TOK = NQB * TPB;    // tokens per wavefront tile
+  constexpr int WG_TOK = SPLIT ? WAVE_TOK : 4 * WAVE_TOK;
+  static_assert(!SPLIT || NQB == 1, "split-KV merge is written for one column block");
+
+  __shared__ float s_o[SPLIT ? 4 * 8 * 4 * 64 : 1];
+  __shared__ float s_m[SPLIT ? 4 * 64 : 1];
+  __shared__ float s_l[SPLIT ? 4 * 64 : 1];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c16 = lane & 15, g = lane >> 4;
+  const int total_tiles = tile_start[batch];
+  const size_t page_halves = (size_t)2 * PAGE * Hkv * D;
+  const size_t v_off = (size_t)PAGE * Hkv * D;
+
+  for (long long w = blockIdx.x; w < (long long)total_tiles * Hkv; w += gridDim.x) {
+    const int tile = (int)(w / Hkv), kvh = (int)(w % Hkv);
+    // request = largest i with tile_start[i] <= tile
+    int lo = 0, hi = batch;
+    while (hi - lo > 1) {
+      int mid = (lo + hi) >> 1;
+      if (tile_start[mid] <= tile) lo = mid; else hi = mid;
+    }
+    const int req = lo;
+    const int qo0 = qo_indptr[req];
+    const int qo_len = qo_indptr[req + 1] - qo0;
+    const int pg0 = kv_indptr[req];
+    const int npages = kv_indptr[req + 1] - pg0;
+    const int kv_len = npages > 0 ? (npages - 1) * PAGE + kv_last_page_len[req] : 0;
+    const int tok0 = (tile - tile_start[req]) * WG_TOK + (SPLIT ? 0 : wave * WAVE_TOK);
+    const bool wave_active = tok0 < qo_len;
+
+    float4_t oacc[NQB][8];
+    float m_run[NQB], l_run[NQB];
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+      m_run[nb] = -1e30f;
+      l_run[nb] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) oacc[nb][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    if (wave_active) {
+      // Q operands: column c16 of block nb = (token tok0 + nb*TPB + c16/GROUP, head c16%GROUP)
+      H8 qf[NQB][4];
+      int key_limit[NQB];  // last visible key index for this lane's column
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) {
+        const int tq = tok0 + nb * TPB + c16 / GROUP;
+        const bool live = tq < qo_len;
+        const uint16_t* qp =
+            q + ((size_t)(qo0 + (live ? tq : 0)) * Hq + kvh * GROUP + c16 % GROUP) * D + g * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          qf[nb][j].u = live ? *reinterpret_cast<const u32x4*>(qp + j * 32) : u32x4{0, 0, 0, 0};
+        key_limit[nb] = causal ? kv_len - qo_len + tq : kv_len - 1;
+        if (!live) key_limit[nb] = -1;
+      }
+      const int tok_last = min(tok0 + WAVE_TOK, qo_len) - 1;
+      const int kv_end = causal ? min(kv_len, kv_len - qo_len + tok_last + 1) : kv_len;
+      const int npairs = (kv_end + 31) >> 5;
+
+      for (int pp = SPLIT ? wave : 0; pp < npairs; pp += SPLIT ? 4 : 1) {
+        const int t_base = pp * 32;
+        H8 kf[2][4], vf[2][4];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+          const int pidx = 2 * pp + blk;
+          const bool page_ok = pidx < npages;
+          const int page = kv_indices[pg0 + (page_ok ? pidx : 0)];
+          const uint16_t* kp = kv_data + (size_t)page * page_halves;
+          const uint16_t* krow = kp + ((size_t)c16 * Hkv + kvh) * D + g * 8;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) kf[blk][j].u = *reinterpret_cast<const u32x4*>(krow + j * 32);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int t = t_base + blk * 16 + g * 4 + r;
+            const uint16_t* vrow = kp + v_off + ((size_t)(g * 4 + r) * Hkv + kvh) * D + c16 * 8;
+            // entries past kv_len may hold anything (NaN x 0 = NaN): feed zeros instead
+            vf[blk][r].u = (t < kv_len) ? *reinterpret_cast<const u32x4*>(vrow) : u32x4{0, 0, 0, 0};
+          }
+        }
+        // V^T operands: vt[i] = {V[tok a0..a3][d], V[tok b0..b3][d]} with d = c16*8 + i
+        H8 vt[8];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t a0 = vf[0][0].w[k], a1 = vf[0][1].w[k];
+          const uint32_t a2 = vf[0][2].w[k], a3 = vf[0][3].w[k];
+          const uint32_t b0 = vf[1][0].w[k], b1 = vf[1][1].w[k];
+          const uint32_t b2 = vf[1][2].w[k], b3 = vf[1][3].w[k];
+          vt[2 * k].u = u32x4{pk_lo(a0, a1), pk_lo(a2, a3), pk_lo(b0, b1), pk_lo(b2, b3)};
+          vt[2 * k + 1].u = u32x4{pk_hi(a0, a1), pk_hi(a2, a3), pk_hi(b0, b1), pk_hi(b2, b3)};
+        }
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) {
+          float4_t s[2];
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk) {
+            s[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              s[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[blk][j].h, qf[nb][j].h, s[blk], 0, 0, 0);
+          }
+          // lane holds keys t_base + blk*16 + g*4 + r of column c16
+          float mx = -1e30f;
+          bool ok[2][4];
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int t = t_base + blk * 16 + g * 4 + r;
+              ok[blk][r] = t <= key_limit[nb] && t < kv_len;
+              s[blk][r] *= scale_log2;
+              if (ok[blk][r]) mx = fmaxf(mx, s[blk][r]);
+            }
+          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          const float m_new = fmaxf(m_run[nb], mx);
+          const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+          m_run[nb] = m_new;
+          float psum = 0.f;
+          H8 pf;
+          uint32_t pw[4];
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int rr = 0; rr < 2; ++rr) {
+              float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[blk][2 * rr] - m_new) : 0.f;
+              float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[blk][2 * rr + 1] - m_new) : 0.f;
+              // the reference rounds P to fp16 before P.V and sums the unrounded values
+              psum += p0 + p1;
+              pw[blk * 2 + rr] = f2h_bits(p0) | (f2h_bits(p1) << 16);
+            }
+          pf.u = u32x4{pw[0], pw[1], pw[2], pw[3]};
+          l_run[nb] = l_run[nb] * alpha + psum;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            oacc[nb][i] *= alpha;
+            oacc[nb][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt[i].h, pf.h, oacc[nb][i], 0, 0, 0);
+          }
+        }
+      }
+      // row sums were kept per lane; columns are spread over the 4 lane groups
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) {
+        l_run[nb] += __shfl_xor(l_run[nb], 16, 64);
+        l_run[nb] += __shfl_xor(l_run[nb], 32, 64);
+      }
+    }
+
+    // oacc[nb][i][r] = O[column c16][feature (4g + r)*8 + i]
+    if constexpr (SPLIT) {
+      __syncthreads();  // previous work item's merge reads are done
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s_o[((wave * 8 + i) * 4 + r) * 64 + lane] = oacc[0][i][r];
+      s_m[wave * 64 + lane] = m_run[0];
+      s_l[wave * 64 + lane] = l_run[0];
+      __syncthreads();
+      const int tq = c16 / GROUP;  // tok0 == tile token base in split mode
+      const int tok = (tile - tile_start[req]) * WG_TOK + tq;
+      float M = -1e30f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) M = fmaxf(M, s_m[ww * 64 + lane]);
+      float wgt[4], L = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        wgt[ww] = __builtin_amdgcn_exp2f(s_m[ww * 64 + lane] - M);
+        L += wgt[ww] * s_l[ww * 64 + lane];
+      }
+      const float inv = L > 0.f ? 1.0f / L : 0.f;
+      if (tok < qo_len) {
+        uint16_t* op = o + ((size_t)(qo0 + tok) * Hq + kvh * GROUP + c16 % GROUP) * D;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const int i = 2 * wave + e;
+            float acc = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < 4; ++ww) acc += wgt[ww] * s_o[((ww * 8 + i) * 4 + r) * 64 + lane];
+            v[e] = acc * inv;
+          }
+          *reinterpret_cast<uint32_t*>(op + (4 * g + r) * 8 + 2 * wave) =
+              f2h_bits(v[0]) | (f2h_bits(v[1]) << 16);
+        }
+      }
+    } else {
+      if (wave_active) {
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) {
+          const int tq = tok0 + nb * TPB + c16 / GROUP;
+          if (tq >= qo_len) continue;
+          const float inv = l_run[nb] > 0.f ? 1.0f / l_run[nb] : 0.f;
+          uint16_t* op = o + ((size_t)(qo0 + tq) * Hq + kvh * GROUP + c16 % GROUP) * D;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            uint32_t pwd[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+              pwd[k] = f2h_bits(oacc[nb][2 * k][r] * inv) | (f2h_bits(oacc[nb][2 * k + 1][r] * inv) << 16);
+            *reinterpret_cast<u32x4*>(op + (4 * g + r) * 8) = u32x4{pwd[0], pwd[1], pwd[2], pwd[3]};
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int GROUP>
+static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
+                       const uint16_t* kv_data, const int32_t* kv_indptr, const int32_t* kv_indices,
+                       const int32_t* kv_last_page_len, int32_t* tile_start, int batch,
+                       int max_qo_rows, int Hq, int Hkv, int causal, int num_blocks,
+                       hipStream_t stream) {
+  const float scale_log2 = 1.4426950408889634f / sqrtf((float)D);
+  constexpr int TPB = 16 / GROUP;
+  const bool decode_mode = max_qo_rows <= batch;
+  constexpr int NQB_PREFILL = 4;
+  const int wg_tok = decode_mode ? TPB : 4 * NQB_PREFILL * TPB;
+  attn_plan_kernel<<<1, 256, 0, stream>>>(qo_indptr, tile_start, batch, wg_tok);
+  long long bound = ((long long)batch + max_qo_rows / wg_tok) * Hkv;
+  if (num_blocks > 0 && bound > num_blocks) bound = num_blocks;
+  if (bound > 0x7fffffffLL) bound = 0x7fffffffLL;
+  if (bound < 1) bound = 1;
+  if (decode_mode)
+    attn_paged_kernel<GROUP, 1, true><<<(int)bound, 256, 0, stream>>>(
+        q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, batch, Hq,
+        Hkv, causal, scale_log2);
+  else
+    attn_paged_kernel<GROUP, NQB_PREFILL, false><<<(int)bound, 256, 0, stream>>>(
+        q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, batch, Hq,
+        Hkv, causal, scale_log2);
+  return check_launch("nf_attention_paged_f16");
+}
+
+}  // namespace nf
+
+using namespace nf;
+
+extern "C" {
+
+size_t nf_attention_workspace_bytes(int batch, int max_qo_rows, int num_qo_heads) {
+  (void)max_qo_rows;
+  (void)num_qo_heads;
+  if (batch < 0) batch = 0;
+  return (((size_t)batch + 2) * sizeof(int32_t) + 255) & ~(size_t)255;
+}
+
+int nf_attention_paged_f16(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
+                           const uint16_t* kv_data, const int32_t* kv_indptr,
+                           const int32_t* kv_indices, const int32_t* kv_last_page_len, int batch,
+                           int max_qo_rows, int num_qo_heads, int num_kv_heads, int head_dim,
+                           int page_size, int causal, int num_blocks, void* workspace,
+                           size_t workspace_bytes, nf_stream_t stream) {
+  NF_REQUIRE(head_dim == D && page_size == PAGE,
+             "nf_attention_paged_f16: head_dim=%d page_size=%d, only 128/16 are built", head_dim,
+             page_size);
+  NF_REQUIRE(batch >= 0 && max_qo_rows >= 0 && num_qo_heads > 0 && num_kv_heads > 0 &&
+                 num_qo_heads % num_kv_heads == 0,
+             "nf_attention_paged_f16: bad sizes batch=%d rows=%d Hq=%d Hkv=%d", batch, max_qo_rows,
+             num_qo_heads, num_kv_heads);
+  if (batch == 0 || max_qo_rows == 0) return NF_OK;
+  NF_REQUIRE(q && o && qo_indptr && kv_data && kv_indptr && kv_indices && kv_last_page_len,
+             "nf_attention_paged_f16: null pointer");
+  if (!workspace || workspace_bytes < nf_attention_workspace_bytes(batch, max_qo_rows, num_qo_heads)) {
+    set_error("nf_attention_paged_f16: workspace of %zu bytes, need %zu", workspace_bytes,
+              nf_attention_workspace_bytes(batch, max_qo_rows, num_qo_heads));
+    return NF_ERR_WORKSPACE;
+  }
+  int32_t* tile_start = static_cast<int32_t*>(workspace);
+  hipStream_t s = (hipStream_t)stream;
+  const int group = num_qo_heads / num_kv_heads;
+#define NF_ATTN_CASE(G)                                                                          \
+  case G:                                                                                        \
+    return launch_attn<G>(q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len,     \
+                          tile_start, batch, max_qo_rows, num_qo_heads, num_kv_heads, causal,    \
+                          num_blocks, s)
+  switch (group) {
+    NF_ATTN_CASE(1);
+    NF_ATTN_CASE(2);
+    NF_ATTN_CASE(4);
+    NF_ATTN_CASE(8);
+    default:
+      set_error("nf_attention_paged_f16: GQA group %d not built (1, 2, 4, 8 are)", group);
+      return NF_ERR_UNSUPPORTED;
+  }
+#undef NF_ATTN_CASE
+}
+
+}  // extern "C"

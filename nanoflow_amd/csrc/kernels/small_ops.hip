@@ -1,0 +1,289 @@
+// Row-wise HBM-bound operators of the nano-batch pipeline for gfx950:
+// embedding gather, RMSNorm, last-token gather, greedy sampler, split+RoPE+paged-KV append.
+// All use 16-byte vector accesses on rows that are multiples of 8 halves.
+#include "common.h"
+
+#include <cmath>
+#include <cstring>
+
+namespace nf {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+// ---------------------------------------------------------------- row gathers
+
+// out[r,:] = src[row_of(r),:]; one workgroup per output row.
+template <bool kKeepToken>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const int32_t* __restrict__ idx,
+                                                          const u32x4* __restrict__ src,
+                                                          u32x4* __restrict__ out, int vec_per_row) {
+  const int r = blockIdx.x;
+  const long long srow = kKeepToken ? (long long)idx[r + 1] - 1 : (long long)idx[r];
+  const u32x4* s = src + srow * vec_per_row;
+  u32x4* o = out + (long long)r * vec_per_row;
+  for (int i = threadIdx.x; i < vec_per_row; i += blockDim.x) o[i] = s[i];
+}
+
+// ---------------------------------------------------------------- RMSNorm
+
+// One workgroup per row.  Two passes over the row (second pass hits L1/L2); fp32 math,
+// single rounding on output.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
+                                                      const u32x4* __restrict__ in,
+                                                      const u32x4* __restrict__ w, int vec_per_row,
+                                                      float inv_n, float eps) {
+  __shared__ float s_part[4];
+  const int r = blockIdx.x;
+  const u32x4* x = in + (long long)r * vec_per_row;
+  u32x4* y = out + (long long)r * vec_per_row;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < vec_per_row; i += 256) {
+    u32x4 v = x[i];
+    const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float a = h2f_bits(p[j] & 0xffffu), b = h2f_bits(p[j] >> 16);
+      ss += a * a + b * b;
+    }
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float tot = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+  const float scale = 1.0f / sqrtf(tot * inv_n + eps);
+  for (int i = threadIdx.x; i < vec_per_row; i += 256) {
+    u32x4 v = x[i];
+    u32x4 g = w[i];
+    const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+    const uint32_t q[4] = {g.x, g.y, g.z, g.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float a = h2f_bits(p[j] & 0xffffu) * scale * h2f_bits(q[j] & 0xffffu);
+      float b = h2f_bits(p[j] >> 16) * scale * h2f_bits(q[j] >> 16);
+      o[j] = f2h_bits(a) | (f2h_bits(b) << 16);
+    }
+    y[i] = u32x4{o[0], o[1], o[2], o[3]};
+  }
+}
+
+// ---------------------------------------------------------------- greedy sampler
+
+// Candidate order of the reference sampler: larger value wins; equal values: smaller key,
+// key = bitreverse10(col mod 1024) << 20 | col.  Values <= -10000 (and NaN) never win.
+struct ArgBest {
+  float v;
+  uint32_t key;
+};
+__device__ __forceinline__ bool arg_better(float v, uint32_t key, const ArgBest& b) {
+  return v > b.v || (v == b.v && key < b.key);
+}
+__device__ __forceinline__ uint32_t arg_key(uint32_t col) {
+  return ((__brev(col & 1023u) >> 22) << 20) | col;
+}
+
+__global__ __launch_bounds__(1024) void argmax_kernel(const uint16_t* __restrict__ logits,
+                                                      uint16_t* __restrict__ max_vals,
+                                                      int32_t* __restrict__ arg, int cols) {
+  __shared__ float s_v[16];
+  __shared__ uint32_t s_k[16];
+  const int r = blockIdx.x;
+  const uint16_t* x = logits + (long long)r * cols;
+  ArgBest best{-10000.f, 0u};
+  const int nvec = cols >> 3;
+  const u32x4* xv = reinterpret_cast<const u32x4*>(x);
+  for (int i = threadIdx.x; i < nvec; i += 1024) {
+    u32x4 v = xv[i];
+    const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t c0 = (uint32_t)i * 8u + 2u * j;
+      float a = h2f_bits(p[j] & 0xffffu), b = h2f_bits(p[j] >> 16);
+      uint32_t ka = arg_key(c0), kb = arg_key(c0 + 1);
+      if (a > -10000.f && arg_better(a, ka, best)) best = ArgBest{a, ka};
+      if (b > -10000.f && arg_better(b, kb, best)) best = ArgBest{b, kb};
+    }
+  }
+  for (int c = (nvec << 3) + threadIdx.x; c < cols; c += 1024) {
+    float a = h2f_bits(x[c]);
+    uint32_t ka = arg_key((uint32_t)c);
+    if (a > -10000.f && arg_better(a, ka, best)) best = ArgBest{a, ka};
+  }
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) {
+    float ov = __shfl_xor(best.v, m, 64);
+    uint32_t ok = __shfl_xor(best.key, m, 64);
+    if (arg_better(ov, ok, best)) best = ArgBest{ov, ok};
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_v[threadIdx.x >> 6] = best.v;
+    s_k[threadIdx.x >> 6] = best.key;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    ArgBest b{s_v[0], s_k[0]};
+    for (int i = 1; i < 16; ++i)
+      if (arg_better(s_v[i], s_k[i], b)) b = ArgBest{s_v[i], s_k[i]};
+    arg[r] = (int32_t)(b.key & 0xfffffu);
+    if (max_vals) max_vals[r] = (uint16_t)f2h_bits(b.v);
+  }
+}
+
+// ---------------------------------------------------------------- split + RoPE + paged append
+
+// One workgroup per token.  The 64 rotation angles of the token (one per frequency) are
+// evaluated once into LDS and shared by all heads.  A work item is (head, 8-feature chunk of
+// the first half): it loads the chunk and its rotate-half partner (two 16-byte loads), and
+// writes both rotated chunks.  V heads are copied.
+__global__ __launch_bounds__(256) void rope_append_kernel(
+    const uint16_t* __restrict__ kqv, uint16_t* __restrict__ q_out, uint16_t* __restrict__ kv_data,
+    const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_indptr,
+    const int32_t* __restrict__ rev_input_indptr, const int32_t* __restrict__ per_token_offset,
+    int Hq, int Hkv, int page_size, float rope_rcp_scale, float rope_rcp_theta, float smooth_a,
+    float smooth_b) {
+  constexpr int D = 128;
+  __shared__ float s_cos[D / 2], s_sin[D / 2];
+  const int t = blockIdx.x;
+  const int r = rev_input_indptr[t];
+  const int pos = per_token_offset[t];
+  const int page = kv_indices[kv_indptr[r] + pos / page_size];
+  const int entry = pos % page_size;
+  if (threadIdx.x < D / 2) {
+    float f = powf(rope_rcp_theta, (float)(2 * threadIdx.x) / (float)D);
+    float smooth = f * smooth_a + smooth_b;
+    smooth = fmaxf(0.0f, fminf(1.0f, smooth));
+    f = (1.f - smooth) * (f * rope_rcp_scale) + smooth * f;
+    float ang = (float)pos * f;
+    s_cos[threadIdx.x] = cosf(ang);
+    s_sin[threadIdx.x] = sinf(ang);
+  }
+  __syncthreads();
+  const int heads = Hq + 2 * Hkv;
+  const uint16_t* row = kqv + (long long)t * heads * D;
+  // pool[page][kv][entry][head][feat]
+  uint16_t* kdst = kv_data + ((((long long)page * 2 + 0) * page_size + entry) * Hkv) * D;
+  uint16_t* vdst = kv_data + ((((long long)page * 2 + 1) * page_size + entry) * Hkv) * D;
+  uint16_t* qdst = q_out + (long long)t * Hq * D;
+  for (int item = threadIdx.x; item < heads * 8; item += 256) {
+    const int h = item >> 3, c = item & 7;  // chunk c covers features 8c..8c+7 and 64+8c..
+    const uint16_t* src = row + h * D;
+    u32x4 lo = *reinterpret_cast<const u32x4*>(src + 8 * c);
+    u32x4 hi = *reinterpret_cast<const u32x4*>(src + 64 + 8 * c);
+    uint16_t* dst;
+    if (h < Hkv) {
+      dst = kdst + h * D;
+    } else if (h < 2 * Hkv) {
+      dst = vdst + (h - Hkv) * D;
+      *reinterpret_cast<u32x4*>(dst + 8 * c) = lo;
+      *reinterpret_cast<u32x4*>(dst + 64 + 8 * c) = hi;
+      continue;
+    } else {
+      dst = qdst + (h - 2 * Hkv) * D;
+    }
+    const uint32_t pl[4] = {lo.x, lo.y, lo.z, lo.w};
+    const uint32_t ph[4] = {hi.x, hi.y, hi.z, hi.w};
+    uint32_t ol[4], oh[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t l16[2], h16[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int fi = 8 * c + 2 * j + e;
+        const float cs = s_cos[fi], sn = s_sin[fi];
+        const float a = h2f_bits(e ? pl[j] >> 16 : pl[j] & 0xffffu);
+        const float b = h2f_bits(e ? ph[j] >> 16 : ph[j] & 0xffffu);
+        l16[e] = f2h_bits(a * cs + (-b) * sn);  // i <  d/2: x[i]*cos - x[i+d/2]*sin
+        h16[e] = f2h_bits(b * cs + a * sn);     // i >= d/2: x[i]*cos + x[i-d/2]*sin
+      }
+      ol[j] = l16[0] | (l16[1] << 16);
+      oh[j] = h16[0] | (h16[1] << 16);
+    }
+    *reinterpret_cast<u32x4*>(dst + 8 * c) = u32x4{ol[0], ol[1], ol[2], ol[3]};
+    *reinterpret_cast<u32x4*>(dst + 64 + 8 * c) = u32x4{oh[0], oh[1], oh[2], oh[3]};
+  }
+}
+
+}  // namespace nf
+
+using namespace nf;
+
+extern "C" {
+
+int nf_abi_version(void) { return 1; }
+const char* nf_last_error(void) { return nf::g_err; }
+
+int nf_embedding_f16(const int32_t* tokens, const uint16_t* table, uint16_t* out, int n_tokens,
+                     int hidden, nf_stream_t stream) {
+  NF_REQUIRE(n_tokens >= 0 && hidden > 0 && hidden % 8 == 0,
+             "nf_embedding_f16: hidden=%d must be a positive multiple of 8 (n_tokens=%d)", hidden,
+             n_tokens);
+  if (n_tokens == 0) return NF_OK;
+  NF_REQUIRE(tokens && table && out, "nf_embedding_f16: null pointer");
+  gather_rows_kernel<false><<<n_tokens, 256, 0, (hipStream_t)stream>>>(
+      tokens, reinterpret_cast<const u32x4*>(table), reinterpret_cast<u32x4*>(out), hidden / 8);
+  return check_launch("nf_embedding_f16");
+}
+
+int nf_keep_token_f16(const uint16_t* in, uint16_t* out, const int32_t* input_indptr, int req_num,
+                      int hidden, nf_stream_t stream) {
+  NF_REQUIRE(req_num >= 0 && hidden > 0 && hidden % 8 == 0,
+             "nf_keep_token_f16: hidden=%d must be a positive multiple of 8 (req_num=%d)", hidden,
+             req_num);
+  if (req_num == 0) return NF_OK;
+  NF_REQUIRE(in && out && input_indptr, "nf_keep_token_f16: null pointer");
+  gather_rows_kernel<true><<<req_num, 256, 0, (hipStream_t)stream>>>(
+      input_indptr, reinterpret_cast<const u32x4*>(in), reinterpret_cast<u32x4*>(out), hidden / 8);
+  return check_launch("nf_keep_token_f16");
+}
+
+int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* weight, int rows, int hidden,
+                   float eps, nf_stream_t stream) {
+  NF_REQUIRE(rows >= 0 && hidden > 0 && hidden % 8 == 0,
+             "nf_rmsnorm_f16: hidden=%d must be a positive multiple of 8 (rows=%d)", hidden, rows);
+  if (rows == 0) return NF_OK;
+  NF_REQUIRE(out && in && weight, "nf_rmsnorm_f16: null pointer");
+  rmsnorm_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(
+      reinterpret_cast<u32x4*>(out), reinterpret_cast<const u32x4*>(in),
+      reinterpret_cast<const u32x4*>(weight), hidden / 8, 1.0f / (float)hidden, eps);
+  return check_launch("nf_rmsnorm_f16");
+}
+
+int nf_argmax_f16(const uint16_t* logits, uint16_t* max_vals, int32_t* argmax, int rows, int cols,
+                  nf_stream_t stream) {
+  NF_REQUIRE(rows >= 0 && cols > 0 && cols < (1 << 20) && cols % 8 == 0,
+             "nf_argmax_f16: cols=%d must be a multiple of 8 below 2^20 (rows=%d)", cols, rows);
+  if (rows == 0) return NF_OK;
+  NF_REQUIRE(logits && argmax, "nf_argmax_f16: null pointer");
+  argmax_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(logits, max_vals, argmax, cols);
+  return check_launch("nf_argmax_f16");
+}
+
+int nf_rope_append_f16(const uint16_t* kqv, uint16_t* q_out, uint16_t* kv_data,
+                       const int32_t* kv_indices, const int32_t* kv_indptr,
+                       const int32_t* rev_input_indptr, const int32_t* per_token_offset,
+                       int n_tokens, int num_qo_heads, int num_kv_heads, int head_dim,
+                       int page_size, float rope_scale, float rope_theta, float smooth_a,
+                       float smooth_b, nf_stream_t stream) {
+  NF_REQUIRE(head_dim == 128, "nf_rope_append_f16: head_dim=%d, only 128 is built", head_dim);
+  NF_REQUIRE(n_tokens >= 0 && num_qo_heads > 0 && num_kv_heads > 0 && page_size > 0,
+             "nf_rope_append_f16: bad sizes tokens=%d Hq=%d Hkv=%d page=%d", n_tokens, num_qo_heads,
+             num_kv_heads, page_size);
+  NF_REQUIRE(rope_scale > 0.f && rope_theta > 0.f, "nf_rope_append_f16: rope_scale/theta must be > 0");
+  if (n_tokens == 0) return NF_OK;
+  NF_REQUIRE(kqv && q_out && kv_data && kv_indices && kv_indptr && rev_input_indptr &&
+                 per_token_offset,
+             "nf_rope_append_f16: null pointer");
+  rope_append_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(
+      kqv, q_out, kv_data, kv_indices, kv_indptr, rev_input_indptr, per_token_offset, num_qo_heads,
+      num_kv_heads, page_size, 1.0f / rope_scale, 1.0f / rope_theta, smooth_a, smooth_b);
+  return check_launch("nf_rope_append_f16");
+}
+
+}  // extern "C"

@@ -1,0 +1,192 @@
+"""ctypes binding of the gfx950 kernel library (C ABI: include/nanoflow_kernels.h).
+
+Operands are torch CUDA tensors used purely as device buffers; every call enqueues on
+torch's current stream and returns without synchronising.  There is no CPU or PyTorch
+fallback: if the compiled library is missing or a call is rejected, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
+
+SYMBOLS = [
+    "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16",
+    "nf_dual_swiglu_f16", "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
+    "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
+]
+
+
+class NanoflowKernelError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Loads libnf_kernels.so (built by ``make -C nanoflow_amd/csrc`` / ``__graft_entry__.build``)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise NanoflowKernelError(
+                f"{LIB_PATH} is missing: build it with `make -C nanoflow_amd/csrc` "
+                "(there is no fallback path)")
+        l = C.CDLL(LIB_PATH)
+        vp, i32, f32, sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+        l.nf_abi_version.restype = i32
+        l.nf_last_error.restype = C.c_char_p
+        l.nf_embedding_f16.argtypes = [vp, vp, vp, i32, i32, vp]
+        l.nf_rmsnorm_f16.argtypes = [vp, vp, vp, i32, i32, f32, vp]
+        l.nf_gemm_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
+        l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
+        l.nf_gemm_f8w_f16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp]
+        l.nf_rope_append_f16.argtypes = [vp] * 7 + [i32] * 5 + [f32] * 4 + [vp]
+        l.nf_attention_workspace_bytes.restype = sz
+        l.nf_attention_workspace_bytes.argtypes = [i32, i32, i32]
+        l.nf_attention_paged_f16.argtypes = [vp] * 7 + [i32] * 8 + [vp, sz, vp]
+        l.nf_keep_token_f16.argtypes = [vp, vp, vp, i32, i32, vp]
+        l.nf_argmax_f16.argtypes = [vp, vp, vp, i32, i32, vp]
+        for name in SYMBOLS:
+            if name not in ("nf_last_error", "nf_attention_workspace_bytes"):
+                getattr(l, name).restype = i32
+        _lib = l
+    return _lib
+
+
+def _check(rc: int, what: str):
+    if rc != 0:
+        raise NanoflowKernelError(f"{what} failed ({rc}): {lib().nf_last_error().decode()}")
+
+
+def _p(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensor required"
+    return t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _f16(t):
+    assert t.dtype == torch.float16, t.dtype
+
+
+def _i32(t):
+    assert t.dtype == torch.int32, t.dtype
+
+
+def embedding(tokens, table, out=None):
+    _i32(tokens); _f16(table)
+    T, H = tokens.numel(), table.shape[1]
+    out = torch.empty((T, H), dtype=torch.float16, device=table.device) if out is None else out
+    _check(lib().nf_embedding_f16(_p(tokens), _p(table), _p(out), T, H, _stream()), "nf_embedding_f16")
+    return out
+
+
+def rmsnorm(x, w, eps=1e-5, out=None):
+    _f16(x); _f16(w)
+    rows, H = x.shape
+    out = torch.empty_like(x) if out is None else out
+    _check(lib().nf_rmsnorm_f16(_p(out), _p(x), _p(w), rows, H, eps, _stream()), "nf_rmsnorm_f16")
+    return out
+
+
+def gemm(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None):
+    _f16(A); _f16(B)
+    M, K = A.shape
+    N = B.shape[0] if b_col_major else B.shape[1]
+    assert tuple(B.shape) == ((N, K) if b_col_major else (K, N)), (A.shape, B.shape)
+    if Cmat is not None:
+        _f16(Cmat)
+        assert tuple(Cmat.shape) == (M, N)
+    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
+    _check(lib().nf_gemm_f16(_p(A), _p(B), _p(Cmat), _p(out), M, N, K, alpha, beta,
+                             int(b_col_major), _stream()), "nf_gemm_f16")
+    return out
+
+
+def dual_swiglu(A, Bg, Bu, out=None):
+    _f16(A); _f16(Bg); _f16(Bu)
+    M, K = A.shape
+    N = Bg.shape[1]
+    assert tuple(Bg.shape) == (K, N) and tuple(Bu.shape) == (K, N)
+    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
+    _check(lib().nf_dual_swiglu_f16(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, _stream()),
+           "nf_dual_swiglu_f16")
+    return out
+
+
+def gemm_f8w(A, Bq, scale, Cmat=None, alpha=1.0, beta=0.0, out=None):
+    _f16(A)
+    assert Bq.dtype in (torch.uint8, torch.float8_e4m3fn) and scale.dtype == torch.float32
+    M, K = A.shape
+    N = Bq.shape[1]
+    assert tuple(Bq.shape) == (K, N) and scale.numel() == N
+    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
+    _check(lib().nf_gemm_f8w_f16(_p(A), _p(Bq), _p(scale), _p(Cmat), _p(out), M, N, K, alpha, beta,
+                                 _stream()), "nf_gemm_f8w_f16")
+    return out
+
+
+def rope_append(kqv, kv_data, kv_indices, kv_indptr, rev_input_indptr, per_token_offset, Hq, Hkv,
+                d=128, page_size=16, rope_scale=1.0, rope_theta=1e4, smooth_a=0.0, smooth_b=0.0,
+                q_out=None, n_tokens=None):
+    """Appends K/V into kv_data IN PLACE and returns the rotated Q rows."""
+    _f16(kqv); _f16(kv_data)
+    for t in (kv_indices, kv_indptr, rev_input_indptr, per_token_offset):
+        _i32(t)
+    T = kqv.shape[0] if n_tokens is None else n_tokens
+    assert kqv.shape[1] == (Hq + 2 * Hkv) * d
+    q_out = torch.empty((kqv.shape[0], Hq * d), dtype=torch.float16, device=kqv.device) \
+        if q_out is None else q_out
+    _check(lib().nf_rope_append_f16(_p(kqv), _p(q_out), _p(kv_data), _p(kv_indices), _p(kv_indptr),
+                                    _p(rev_input_indptr), _p(per_token_offset), T, Hq, Hkv, d,
+                                    page_size, rope_scale, rope_theta, smooth_a, smooth_b, _stream()),
+           "nf_rope_append_f16")
+    return q_out
+
+
+def attention_paged(q, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, Hq, Hkv, d=128,
+                    page_size=16, causal=False, out=None, batch=None, max_qo_rows=None,
+                    num_blocks=0, workspace=None):
+    _f16(q); _f16(kv_data)
+    for t in (qo_indptr, kv_indptr, kv_indices, kv_last_page_len):
+        _i32(t)
+    batch = kv_last_page_len.numel() if batch is None else batch
+    max_qo_rows = q.shape[0] if max_qo_rows is None else max_qo_rows
+    out = torch.zeros_like(q) if out is None else out
+    need = lib().nf_attention_workspace_bytes(batch, max_qo_rows, Hq)
+    if workspace is None:
+        workspace = torch.empty((max(need, 1),), dtype=torch.uint8, device=q.device)
+    _check(lib().nf_attention_paged_f16(_p(q), _p(out), _p(qo_indptr), _p(kv_data), _p(kv_indptr),
+                                        _p(kv_indices), _p(kv_last_page_len), batch, max_qo_rows,
+                                        Hq, Hkv, d, page_size, int(bool(causal)), num_blocks,
+                                        _p(workspace), workspace.numel(), _stream()),
+           "nf_attention_paged_f16")
+    return out
+
+
+def keep_token(x, input_indptr, req_num, out=None):
+    _f16(x); _i32(input_indptr)
+    H = x.shape[1]
+    out = torch.empty((req_num, H), dtype=torch.float16, device=x.device) if out is None else out
+    _check(lib().nf_keep_token_f16(_p(x), _p(out), _p(input_indptr), req_num, H, _stream()),
+           "nf_keep_token_f16")
+    return out
+
+
+def argmax(logits, rows=None):
+    _f16(logits)
+    rows = logits.shape[0] if rows is None else rows
+    cols = logits.shape[1]
+    mv = torch.empty((rows,), dtype=torch.float16, device=logits.device)
+    arg = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _check(lib().nf_argmax_f16(_p(logits), _p(mv), _p(arg), rows, cols, _stream()), "nf_argmax_f16")
+    return arg, mv

@@ -1,0 +1,257 @@
+"""Parity of every HIP operator (through the C ABI) with the CPU oracle on the same seeded
+inputs.  Integer/index/copy results are compared bit-exactly; floating-point results within
+2e-3 relative (fp16 storage, fp32 accumulate)."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+from nanoflow_amd import synth  # noqa: E402
+
+RTOL = 2e-3
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def assert_close(got, ref, rtol=RTOL, what=""):
+    """|got-ref| <= rtol*|ref| + rtol*rms(ref) elementwise, and max-norm relative <= rtol."""
+    g = got.astype(np.float64)
+    r = ref.astype(np.float64)
+    assert np.isfinite(g).all(), f"{what}: non-finite output"
+    scale = max(np.sqrt((r ** 2).mean()), 1e-6)
+    err = np.abs(g - r)
+    bad = err > rtol * np.abs(r) + rtol * scale
+    assert not bad.any(), f"{what}: {bad.sum()} of {bad.size} elements off, max err {err.max():.3e} (rms {scale:.3e})"
+    assert err.max() <= rtol * max(np.abs(r).max(), 1e-6) * 2, f"{what}: max-norm error {err.max():.3e}"
+
+
+@pytest.fixture(scope="module")
+def K():
+    from nanoflow_amd import kernels
+    assert torch.cuda.is_available()
+    kernels.lib()
+    return kernels
+
+
+# ---------------------------------------------------------------- copies / sampler (bit-exact)
+
+def test_embedding_and_keep_token_bit_exact(K, oracle):
+    rng = np.random.default_rng(0)
+    table = synth.normal_f16(rng, (1000, 4096))
+    tok = rng.integers(0, 1000, size=77, dtype=np.int32)
+    assert np.array_equal(host(K.embedding(dev(tok), dev(table))), oracle.embedding(tok, table))
+    x = synth.normal_f16(rng, (77, 4096))
+    indptr = np.concatenate([[0], np.sort(rng.choice(np.arange(1, 77), 9, replace=False)), [77]]).astype(np.int32)
+    got = host(K.keep_token(dev(x), dev(indptr), 10))
+    assert np.array_equal(got, oracle.keep_token(x, indptr, 10))
+
+
+def test_embedding_empty_batch(K):
+    table = dev(np.zeros((4, 64), np.float16))
+    out = K.embedding(torch.zeros(0, dtype=torch.int32, device="cuda"), table)
+    assert out.shape == (0, 64)
+
+
+def test_argmax_matches_reference_tie_order(K, oracle):
+    rng = np.random.default_rng(1)
+    x = synth.normal_f16(rng, (9, 128256))
+    x[1, [7, 1031, 100000]] = 9.0            # ties across scanner slots
+    x[2, [512, 256, 768]] = 9.0
+    x[3, :] = -20000.0                       # nothing above the -10000 start
+    x[4, :] = np.float16(-1.5)               # all equal
+    x[5, 128255] = 11.0                      # last column
+    x[6, ::1024] = 8.0                       # same slot, many times
+    want_i, want_v = oracle.argmax(x)
+    got_i, got_v = K.argmax(dev(x))
+    assert np.array_equal(host(got_i), want_i)
+    assert np.array_equal(host(got_v), want_v)
+
+
+# ---------------------------------------------------------------- RMSNorm
+
+@pytest.mark.parametrize("rows,H", [(1, 4096), (64, 4096), (7, 256), (3, 8192)])
+def test_rmsnorm(K, oracle, rows, H):
+    rng = np.random.default_rng(2)
+    x = synth.normal_f16(rng, (rows, H), 2.0)
+    w = synth.normal_f16(rng, (H,), 0.02, 1.0)
+    assert_close(host(K.rmsnorm(dev(x), dev(w), 1e-5)), oracle.rmsnorm(x, w, 1e-5), what="rmsnorm")
+
+
+# ---------------------------------------------------------------- GEMM family
+
+GEMM_SHAPES = [
+    (64, 6144, 4096),     # config-1 QKV (short-M tile)
+    (64, 4096, 14336),    # config-1 down projection, long K
+    (1, 256, 64),         # single row
+    (33, 136, 200),       # ragged M, N, K (K % 8 == 0 only)
+    (130, 384, 256),      # 128-row tiles with an M tail
+    (257, 512, 128),      # M tail of one row
+    (384, 4096, 4096),    # nano-batch O projection
+    (1408, 6144, 512),    # 256x256 tiles with an M tail, XCD-remapped grid
+]
+
+
+@pytest.mark.parametrize("M,N,K_", GEMM_SHAPES)
+def test_gemm_plain_and_residual(K, oracle, M, N, K_):
+    rng = np.random.default_rng(3)
+    A = synth.normal_f16(rng, (M, K_))
+    B = synth.normal_f16(rng, (K_, N), 0.02)
+    Cm = synth.normal_f16(rng, (M, N))
+    assert_close(host(K.gemm(dev(A), dev(B))), oracle.gemm(A, B), what="gemm beta=0")
+    assert_close(host(K.gemm(dev(A), dev(B), dev(Cm), alpha=1.0, beta=1.0)),
+                 oracle.gemm(A, B, Cm, 1.0, 1.0), what="gemm beta=1")
+
+
+def test_gemm_alpha_beta_and_in_place_residual(K, oracle):
+    rng = np.random.default_rng(4)
+    A = synth.normal_f16(rng, (96, 256))
+    B = synth.normal_f16(rng, (256, 264), 0.05)
+    Cm = synth.normal_f16(rng, (96, 264))
+    want = oracle.gemm(A, B, Cm, 0.5, -2.0)
+    d = dev(Cm)
+    K.gemm(dev(A), dev(B), d, alpha=0.5, beta=-2.0, out=d)     # C aliases D
+    assert_close(host(d), want, what="gemm in place")
+
+
+def test_gemm_column_major_weights(K, oracle):
+    rng = np.random.default_rng(5)
+    for (M, N, K_) in [(64, 512, 256), (300, 384, 320)]:
+        A = synth.normal_f16(rng, (M, K_))
+        Bt = synth.normal_f16(rng, (N, K_), 0.05)
+        assert_close(host(K.gemm(dev(A), dev(Bt), b_col_major=True)),
+                     oracle.gemm(A, Bt, b_col_major=True), what="gemm col-major B")
+
+
+def test_gemm_identity_is_exact(K):
+    rng = np.random.default_rng(6)
+    A = synth.normal_f16(rng, (70, 128))
+    I = np.eye(128, dtype=np.float16)
+    assert np.array_equal(host(K.gemm(dev(A), dev(I))), A)
+
+
+@pytest.mark.parametrize("M,N,K_", [(64, 14336, 4096), (5, 136, 72), (200, 512, 256), (640, 2048, 512)])
+def test_dual_swiglu(K, oracle, M, N, K_):
+    rng = np.random.default_rng(7)
+    A = synth.normal_f16(rng, (M, K_))
+    Bg = synth.normal_f16(rng, (K_, N), 0.04)
+    Bu = synth.normal_f16(rng, (K_, N), 0.04)
+    assert_close(host(K.dual_swiglu(dev(A), dev(Bg), dev(Bu))), oracle.dual_swiglu(A, Bg, Bu),
+                 what="dual swiglu")
+
+
+def test_dual_known_answer_inputs(K, oracle):
+    # inputs of the reference's dual-GEMM test program (all operands (j+k)/2560, 128^3)
+    j, k = np.meshgrid(np.arange(128), np.arange(128), indexing="ij")
+    X = ((j + k).astype(np.float32) / 20 / 128).astype(np.float16)
+    assert_close(host(K.dual_swiglu(dev(X), dev(X), dev(X))), oracle.dual_swiglu(X, X, X), what="dual KAT")
+
+
+# ---------------------------------------------------------------- RoPE + paged append
+
+@pytest.mark.parametrize("Hq,Hkv,theta,scale,sa,sb", [
+    (32, 8, 5e5, 1.0, 0.0, 0.0),
+    (8, 2, 1e4, 1.0, 0.0, 0.0),
+    (64, 8, 5e5, 8.0, 8192 / (2 * np.pi * 3), -1.0 / 3),   # Llama-3.1 smoothing
+])
+def test_rope_append(K, oracle, Hq, Hkv, theta, scale, sa, sb):
+    rng = np.random.default_rng(8)
+    d, P = 128, 16
+    b = synth.make_batch(rng.integers(0, 1500, size=20), [(0, 40), (123, 17)], vocab=10, seed=3,
+                         extra_pages=7)
+    kqv = synth.normal_f16(rng, (b.tokens, (Hq + 2 * Hkv) * d))
+    shape = synth.ModelShape(Hq=Hq, Hkv=Hkv)
+    pool0 = synth.make_kv_pool(b.num_pages, shape, rng)
+    pool_ref = pool0.copy()
+    q_ref = oracle.rope_append(kqv, pool_ref, b.kv_indices, b.kv_indptr, b.rev_input_indptr,
+                               b.per_token_offset, Hq, Hkv, d, P, scale, theta, sa, sb)
+    pool_dev = dev(pool0)
+    q_dev = K.rope_append(dev(kqv), pool_dev, dev(b.kv_indices), dev(b.kv_indptr),
+                          dev(b.rev_input_indptr), dev(b.per_token_offset), Hq, Hkv, d, P, scale,
+                          theta, sa, sb)
+    pool_got = host(pool_dev)
+    # index rule bit-exact: exactly the same pool slots changed, V rows bit-identical
+    changed_ref = (pool_ref != pool0).any(axis=(3, 4))
+    changed_got = (pool_got != pool0).any(axis=(3, 4))
+    assert np.array_equal(changed_ref, changed_got)
+    assert np.array_equal(pool_got[:, 1], pool_ref[:, 1])
+    assert_close(pool_got[:, 0], pool_ref[:, 0], what="rope K pages")
+    assert_close(host(q_dev), q_ref, what="rope Q")
+
+
+# ---------------------------------------------------------------- attention
+
+def _attn_case(K, oracle, Hq, Hkv, decode_lens, prefill, seed, num_blocks=0):
+    rng = np.random.default_rng(seed)
+    d, P = 128, 16
+    b = synth.make_batch(decode_lens, prefill, vocab=10, seed=seed, extra_pages=3)
+    shape = synth.ModelShape(Hq=Hq, Hkv=Hkv)
+    pool = synth.make_kv_pool(b.num_pages, shape, rng)
+    # poison the unused tail of every request's last page: results must not depend on it
+    for r in range(b.req_num):
+        last = b.kv_indices[b.kv_indptr[r + 1] - 1]
+        pool[last, :, b.kv_last_page_len[r]:] = np.float16(np.nan)
+    q = synth.normal_f16(rng, (b.tokens, Hq * d))
+    nd = b.decodePrefillBorder
+    ref = np.zeros_like(q)
+    got = torch.zeros(q.shape, dtype=torch.float16, device="cuda")
+    dq, dpool, dind = dev(q), dev(pool), dev(b.kv_indices)
+    if nd:
+        oracle.attention_paged(q, b.input_indptr[:nd + 1], pool, b.kv_indptr[:nd + 1], b.kv_indices,
+                               b.kv_last_page_len[:nd], Hq, Hkv, d, P, causal=False, out=ref)
+        K.attention_paged(dq, dev(b.input_indptr[:nd + 1]), dpool, dev(b.kv_indptr[:nd + 1]), dind,
+                          dev(b.kv_last_page_len[:nd]), Hq, Hkv, causal=False, out=got, batch=nd,
+                          max_qo_rows=nd, num_blocks=num_blocks)
+    if b.prefillNum:
+        oracle.attention_paged(q, b.input_indptr[nd:], pool, b.kv_indptr[nd:], b.kv_indices,
+                               b.kv_last_page_len[nd:], Hq, Hkv, d, P, causal=True, out=ref)
+        K.attention_paged(dq, dev(b.input_indptr[nd:]), dpool, dev(b.kv_indptr[nd:]), dind,
+                          dev(b.kv_last_page_len[nd:]), Hq, Hkv, causal=True, out=got,
+                          batch=b.prefillNum, max_qo_rows=b.tokens, num_blocks=num_blocks)
+    assert_close(host(got), ref, what=f"attention Hq={Hq} Hkv={Hkv}")
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (64, 8), (8, 4), (4, 4)])
+def test_attention_decode(K, oracle, Hq, Hkv):
+    lens = [0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 100, 127, 128, 129, 500, 1023]
+    _attn_case(K, oracle, Hq, Hkv, lens, [], seed=11)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (64, 8), (8, 4), (4, 4)])
+def test_attention_chunked_prefill(K, oracle, Hq, Hkv):
+    _attn_case(K, oracle, Hq, Hkv, [], [(0, 1), (0, 37), (100, 64), (5, 130), (256, 3)], seed=12)
+
+
+def test_attention_mixed_batch_with_capped_workgroups(K, oracle):
+    # persistent-grid path: fewer workgroups than work items
+    _attn_case(K, oracle, 32, 8, list(range(40, 72)), [(64, 200)], seed=13, num_blocks=24)
+
+
+def test_attention_long_context_prefill(K, oracle):
+    _attn_case(K, oracle, 8, 2, [], [(1900, 147)], seed=14)
+
+
+def test_attention_page_permutation_invariance(K):
+    rng = np.random.default_rng(15)
+    Hq, Hkv, d, P = 32, 8, 128, 16
+    shape = synth.ModelShape(Hq=Hq, Hkv=Hkv)
+    b = synth.make_batch([300, 77, 1000], [], vocab=10, seed=15, extra_pages=9)
+    pool = synth.make_kv_pool(b.num_pages, shape, rng)
+    q = synth.normal_f16(rng, (3, Hq * d))
+    perm = rng.permutation(b.num_pages)
+    pool_p = np.empty_like(pool)
+    pool_p[perm] = pool
+    args = (dev(b.input_indptr), )
+    o1 = K.attention_paged(dev(q), dev(b.input_indptr), dev(pool), dev(b.kv_indptr), dev(b.kv_indices),
+                           dev(b.kv_last_page_len), Hq, Hkv, max_qo_rows=3)
+    o2 = K.attention_paged(dev(q), dev(b.input_indptr), dev(pool_p), dev(b.kv_indptr),
+                           dev(perm[b.kv_indices].astype(np.int32)), dev(b.kv_last_page_len), Hq, Hkv,
+                           max_qo_rows=3)
+    assert np.array_equal(host(o1), host(o2))
