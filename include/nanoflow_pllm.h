@@ -1,0 +1,170 @@
+/*
+ * nanoflow_pllm.h -- C ABI of the pipeline control plane (host library libnf_pipeline.so).
+ *
+ * Flat-C mirror of what the reference exports to its Python frontend through the
+ * pybind11 module `pllm_python` (pipeline/src/pybind.cu:189-284) and to C++ callers
+ * through pipeline/include/computeBound.cuh:76-87: one pipeline on one GPU, driven
+ * by init -> config -> (update -> run | run_async .. run_async_wait)* -> finalize.
+ * Structs have the reference's fields in the reference's order
+ * (pipeline/include/vortexData.cuh:7-111) with std::vector / std::string members
+ * replaced by pointer + count.  fp16 data is uint16_t bit patterns.
+ *
+ * Every function returns 0 on success and a negative NF_PLLM_ERR_* code otherwise
+ * (pllm_last_error() gives the text).  As in the reference, a failing GPU runtime
+ * call inside the pipeline terminates the process.
+ */
+#ifndef NANOFLOW_PLLM_H
+#define NANOFLOW_PLLM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NF_PLLM_API __attribute__((visibility("default")))
+
+#define NF_PLLM_OK 0
+#define NF_PLLM_ERR_INVALID_ARGUMENT (-1)
+#define NF_PLLM_ERR_STATE (-2)       /* call out of order (e.g. update before config) */
+#define NF_PLLM_ERR_UNSUPPORTED (-3) /* tensor-parallel pipeline types, more than one rank */
+
+/* Worker::PipelineType (pipeline/include/computeBound.cuh:22-34). */
+enum nf_pipeline_type {
+  NF_PIPE_PLLM = 0,
+  NF_PIPE_NONOVERLAP = 1,
+  NF_PIPE_NANOBATCH = 2,
+  NF_PIPE_PLLMOFFLOAD = 3,
+  NF_PIPE_KQVBIAS = 4,
+  NF_PIPE_NONOVERLAP_KQVBIAS = 5,
+  NF_PIPE_NANOBATCH_KQVBIAS = 6,
+  NF_PIPE_LOCAL = 7,             /* two nano-batches, GEMM and attention streams overlapped */
+  NF_PIPE_NON_OVERLAP_LOCAL = 8, /* sequential baseline */
+  NF_PIPE_NANOBATCH_LOCAL = 9    /* nano-batched, single stream */
+};
+
+/* vortexWeight (vortexData.cuh:7-12) */
+typedef struct nf_vortex_weight {
+  uint16_t* ptr;
+  int N;
+  int K;
+} nf_vortex_weight;
+
+/* vortexLayerWeight (vortexData.cuh:14-25).  Weights are K x N row-major; W_KQV columns are
+ * ordered K | V | Q (pipeline/utils/weightSaver.py:118). */
+typedef struct nf_vortex_layer_weight {
+  nf_vortex_weight W_O1, W_O2, W_U, W_G, W_D, W_KQV, B_KQV, W_LN_Attention, W_LN_FFN, W_ROT;
+} nf_vortex_layer_weight;
+
+/* vortexModelWeight (vortexData.cuh:27-32) */
+typedef struct nf_vortex_model_weight {
+  nf_vortex_weight lm_head;
+  nf_vortex_weight embedding;
+  nf_vortex_weight model_layernorm;
+  const nf_vortex_layer_weight* layer_weight;
+  int num_layers;
+} nf_vortex_model_weight;
+
+/* vortexInitData (vortexData.cuh:35-53).  All pointers are DEVICE memory owned by the caller
+ * for the life of the pipeline. */
+typedef struct nf_vortex_init_data {
+  uint16_t** kv_data; /* host array of num_layers device pools [pages,2,page,Hkv,d] */
+  nf_vortex_model_weight weight;
+  size_t weight_size;
+  uint16_t* tmp_buffer;
+  size_t tmp_buffer_size; /* in halves */
+} nf_vortex_init_data;
+
+/* vortexUpdateData (vortexData.cuh:55-90).  All arrays are HOST memory (pinned or not); they
+ * are staged during pllm_update and may be reused when it returns. */
+typedef struct nf_vortex_update_data {
+  int decodePrefillBorder;
+  int prefillNum;
+  int prefillTokensNum;
+  int keepTokenListLength;
+  int* input_tokens; /* the prefill tokens only; decode tokens come from the last samples */
+  int32_t* input_indptr;
+  int32_t* rev_input_indptr;
+  int32_t* keep_token_list;
+  int32_t* kv_indptr;
+  int32_t* kv_indices;
+  int32_t* kv_last_page_len;
+  int32_t* per_token_offset;
+  int32_t* gemv_batch_size; /* [4] */
+  int32_t* gemv_num_blocks; /* [4] */
+} nf_vortex_update_data;
+
+/* vortexConfigData (vortexData.cuh:104-110) */
+typedef struct nf_vortex_config_data {
+  const char* const* gemm_op_tag;
+  int num_gemm_op_tag;
+  int global_batch_size;
+  int nanobatch_1_size;
+  int kqv1_size;
+  int kqv3_size;
+} nf_vortex_config_data;
+
+NF_PLLM_API const char* pllm_last_error(void);
+
+/* setModelConfig (pybind.cu:154-156 -> updateVortexModelConfig, load_config.cu:11-112). */
+NF_PLLM_API int pllm_set_model_config(const char* json_path);
+/* setRank (pybind.cu:10-13); only nranks == 1 is accepted. */
+NF_PLLM_API int pllm_set_rank(int nranks, int vnranks);
+/* Size of the tmp buffer (in halves) and of one layer's KV pool (in pages) that the current
+ * model configuration asks for (ModelConfig.k_temp_size / max_page_num, config.h:99-100). */
+NF_PLLM_API size_t pllm_tmp_buffer_halves(void);
+NF_PLLM_API size_t pllm_max_page_num(void);
+/* pllm_python.init (pybind.cu:73-98) with weights already on the device
+ * (the C++ init(), computeBound.cu:65-113).  Spawns the worker thread. */
+NF_PLLM_API int pllm_init(const nf_vortex_init_data* input, int pipeline_type);
+/* modelWeightToGPU (vortexData.cu:340-373): uploads a host-resident weight set; the device
+ * copies are written to *device_weight / device_layers[num_layers]. */
+NF_PLLM_API int pllm_model_weight_to_gpu(const nf_vortex_model_weight* host_weight,
+                                         nf_vortex_model_weight* device_weight,
+                                         nf_vortex_layer_weight* device_layers);
+/* pllm_python.config (pybind.cu:106-108). */
+NF_PLLM_API int pllm_config(const nf_vortex_config_data* config);
+/* pllm_python.update (pybind.cu:100-104 -> update(), computeBound.cu:115-161). */
+NF_PLLM_API int pllm_update(const nf_vortex_update_data* update);
+/* run / run_async / run_async_wait (computeBound.cu:27-61). */
+NF_PLLM_API int pllm_run(void);
+NF_PLLM_API int pllm_run_async(void);
+NF_PLLM_API int pllm_run_async_wait(void);
+/* getPipelineOutput (pybind.cu:158-186): non-owning view of the sampled token ids of the
+ * last completed run, valid until the next run_async_wait. */
+NF_PLLM_API int pllm_get_pipeline_output(const int32_t** tokens, int* count);
+/* finalize (computeBound.cu:180-193). */
+NF_PLLM_API int pllm_finalize(void);
+
+/* The decode-token feed that update() applies before uploading (computeBound.cu:121-150),
+ * exposed for host-side tests: out = [prev_output[i] for kept slots i] ++ prefill_tokens;
+ * prev_count == 0 feeds token id 1 to every kept slot.  Returns the count written. */
+NF_PLLM_API int pllm_build_input_tokens(const int32_t* prev_output, int prev_count,
+                                        const int32_t* keep_token_list, int keep_token_list_length,
+                                        const int32_t* prefill_tokens, int prefill_tokens_num,
+                                        int32_t* out);
+
+/* Measurement (no counterpart in the reference, which only logs the iteration time,
+ * pipeline_local.cu:444-463).  With profiling on, every attention launch is bracketed by
+ * events on its own stream.  pllm_get_timings returns the last iteration's time and the
+ * durations accumulated since the last pllm_reset_timings. */
+typedef struct nf_pipeline_timings {
+  double iter_ms;
+  double decode_attn_ms;
+  long decode_attn_launches;
+  double prefill_attn_ms;
+  long prefill_attn_launches;
+} nf_pipeline_timings;
+NF_PLLM_API int pllm_set_profiling(int on);
+NF_PLLM_API int pllm_get_timings(nf_pipeline_timings* out);
+NF_PLLM_API int pllm_reset_timings(void);
+/* Device address of an intermediate of the current pipeline, for parity checks:
+ * name in {"hidden" (residual stream after the last layer, [T, hidden]),
+ *          "logits" ([T, vocab])}. */
+NF_PLLM_API int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NANOFLOW_PLLM_H */

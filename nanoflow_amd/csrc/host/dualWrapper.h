@@ -1,0 +1,57 @@
+// DualWrapper: fused gate/up projection with the SwiGLU epilogue,
+// D2 = silu(A.B0) * (A.B1); the two plain products are not stored (kStoreD0/kStoreD1 are
+// false in the reference).  Interface of pipeline/include/dualWrapper.cuh:47-321; the tile
+// template parameters of the reference type are dropped (tiling is the kernel layer's).
+#pragma once
+#include "nanoflow_kernels.h"
+#include "operatorWrapper.h"
+#include "vortexData.h"
+
+struct DualWrapper : public OperatorWrapper {
+  int M = 0, N = 0, K = 0;
+  pllmTensor<half> pllm_tensor_a, pllm_tensor_b1, pllm_tensor_b2, pllm_tensor_c;
+  pllmTensor<half> pllm_tensor_d0, pllm_tensor_d1, pllm_tensor_d2;
+  bool inited = false;
+
+  void set_shape(int m, int n, int k) {
+    M = m;
+    N = n;
+    K = k;
+    NF_LOG_INFO("name:%s M:%d, N:%d, K:%d", name.c_str(), M, N, K);
+  }
+  void work() override {
+    NF_KERNEL_CHECK(nf_dual_swiglu_f16(pllm_tensor_a.ptr, pllm_tensor_b1.ptr, pllm_tensor_b2.ptr,
+                                       pllm_tensor_d2.ptr, M, N, K, stream));
+  }
+  DualWrapper& setA(pllmTensor<half> a) {
+    assert(a.layout == PllmLayout::ROW_MAJOR && (int)a.dim1 == M && (int)a.dim2 == K);
+    pllm_tensor_a = a;
+    return *this;
+  }
+  DualWrapper& setC(pllmTensor<half> c) {  // bias operand; unused (kUseBias is false)
+    pllm_tensor_c = c;
+    return *this;
+  }
+  DualWrapper& setD(pllmTensor<half> d0, pllmTensor<half> d1, pllmTensor<half> d2) {
+    pllm_tensor_d0 = d0;
+    pllm_tensor_d1 = d1;
+    pllm_tensor_d2 = d2;
+    return *this;
+  }
+  pllmTensor<half> getA() { return pllm_tensor_a; }
+  pllmTensor<half> getD() { return pllm_tensor_d2; }
+  pllmTensor<half> getC() { return pllm_tensor_c; }
+  void init() { inited = true; }
+  // weight1 = gate (goes through SiLU), weight2 = up
+  bool set_weight(vortexWeight& weight1, vortexWeight& weight2) {
+    if (weight1.size() != (size_t)K * N || weight2.size() != (size_t)K * N) {
+      std::fprintf(stderr, "Dual weight size mismatch %zu %zu vs %d x %d\n", weight1.size(),
+                   weight2.size(), K, N);
+      return false;
+    }
+    pllm_tensor_b1 = pllmTensor<half>(weight1.ptr, K, N, PllmLayout::ROW_MAJOR);
+    pllm_tensor_b2 = pllmTensor<half>(weight2.ptr, K, N, PllmLayout::ROW_MAJOR);
+    return true;
+  }
+  double totalCompute() { return 4.0 * (double)M * (double)N * (double)K; }
+};

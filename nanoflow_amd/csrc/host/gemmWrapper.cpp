@@ -1,0 +1,110 @@
+#include "gemmWrapper.h"
+
+#include <cmath>
+#include <cstring>
+#include <sstream>
+#include <vector>
+
+bool parseGemmTag(const std::string& tag, GemmTag& out) {
+  std::vector<std::string> parts;
+  std::stringstream ss(tag);
+  std::string tok;
+  while (std::getline(ss, tok, '_')) parts.push_back(tok);
+  if (parts.size() != 11) return false;
+  int* fields[8] = {&out.cta_m, &out.cta_n, &out.cta_k, &out.warp_m,
+                    &out.warp_n, &out.warp_k, &out.split_k, &out.stages};
+  for (int i = 0; i < 8; ++i) {
+    char* end = nullptr;
+    long v = std::strtol(parts[i].c_str(), &end, 10);
+    if (end == parts[i].c_str() || *end != '\0' || v <= 0) return false;
+    *fields[i] = (int)v;
+  }
+  PllmLayout* layouts[3] = {&out.layout_a, &out.layout_b, &out.layout_out};
+  for (int i = 0; i < 3; ++i) {
+    if (parts[8 + i] == "RowMajor") *layouts[i] = PllmLayout::ROW_MAJOR;
+    else if (parts[8 + i] == "ColumnMajor") *layouts[i] = PllmLayout::COL_MAJOR;
+    else return false;
+  }
+  return true;
+}
+
+BaseGEMMWrapper* generateGEMM(const std::string& tag) {
+  GemmTag t;
+  if (!parseGemmTag(tag, t)) {
+    NF_LOG_ERROR("generateGEMM: malformed tag \"%s\"", tag.c_str());
+    return nullptr;
+  }
+  if (t.layout_a != PllmLayout::ROW_MAJOR || t.layout_out != PllmLayout::ROW_MAJOR) {
+    NF_LOG_ERROR("generateGEMM: tag \"%s\": A and output must be RowMajor in this build", tag.c_str());
+    return nullptr;
+  }
+  return new HipGEMMWrapper(t);
+}
+
+void HipGEMMWrapper::work() {
+  NF_KERNEL_CHECK(nf_gemm_f16(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
+                              pllm_tensor_d.ptr, (int)M, (int)N, (int)K, alpha, beta,
+                              tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, stream));
+}
+
+void HipGEMMWrapper::profile() {
+  hipEvent_t e0, e1;
+  HIP_CHECK(hipEventCreate(&e0));
+  HIP_CHECK(hipEventCreate(&e1));
+  const int iters = 100;
+  work();
+  HIP_CHECK(hipEventRecord(e0, stream));
+  for (int i = 0; i < iters; ++i) work();
+  HIP_CHECK(hipEventRecord(e1, stream));
+  HIP_CHECK(hipEventSynchronize(e1));
+  float ms = 0;
+  HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+  std::printf("%s M=%zu N=%zu K=%zu: %.3f ms, %.1f GFLOP/s\n", name.c_str(), M, N, K, ms / iters,
+              gflops(ms / iters));
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+}
+
+static float half_bits_to_float(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1f, man = h & 0x3ffu, bits;
+  if (exp == 0) {
+    if (man == 0) bits = sign;
+    else {
+      int e = -1;
+      do { man <<= 1; ++e; } while (!(man & 0x400u));
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3ffu) << 13);
+    }
+  } else if (exp == 31) bits = sign | 0x7f800000u | (man << 13);
+  else bits = sign | ((exp + 112) << 23) | (man << 13);
+  float f;
+  std::memcpy(&f, &bits, 4);
+  return f;
+}
+
+// Runs the GEMM once and compares 64 sampled outputs with a host float64 dot product
+// (pass rule of the reference's checkResult: (|d - ref| - 0.01) / |ref| <= 0.1).
+bool HipGEMMWrapper::checkResult() {
+  work();
+  HIP_CHECK(hipStreamSynchronize(stream));
+  const bool bcol = tag.layout_b == PllmLayout::COL_MAJOR;
+  std::vector<uint16_t> arow(K), bcolv(K);
+  bool ok = true;
+  for (int s = 0; s < 64 && ok; ++s) {
+    size_t m = (size_t)(s * 2654435761u) % M, n = (size_t)(s * 40503u + 7) % N;
+    HIP_CHECK(hipMemcpy(arow.data(), pllm_tensor_a.ptr + m * K, K * 2, hipMemcpyDeviceToHost));
+    if (bcol) HIP_CHECK(hipMemcpy(bcolv.data(), pllm_tensor_b.ptr + n * K, K * 2, hipMemcpyDeviceToHost));
+    else HIP_CHECK(hipMemcpy2D(bcolv.data(), 2, pllm_tensor_b.ptr + n, N * 2, 2, K, hipMemcpyDeviceToHost));
+    double ref = 0;
+    for (size_t k = 0; k < K; ++k) ref += (double)half_bits_to_float(arow[k]) * half_bits_to_float(bcolv[k]);
+    ref *= alpha;
+    uint16_t c16 = 0, d16 = 0;
+    if (beta != 0.f) {
+      HIP_CHECK(hipMemcpy(&c16, pllm_tensor_c.ptr + m * N + n, 2, hipMemcpyDeviceToHost));
+      ref += beta * half_bits_to_float(c16);
+    }
+    HIP_CHECK(hipMemcpy(&d16, pllm_tensor_d.ptr + m * N + n, 2, hipMemcpyDeviceToHost));
+    double d = half_bits_to_float(d16);
+    if ((std::fabs(d - ref) - 0.01) / std::max(std::fabs(ref), 1e-6) > 0.1) ok = false;
+  }
+  return ok;
+}

@@ -1,0 +1,127 @@
+// GEMM operator wrappers over the kernel layer's C ABI.
+//   BaseGEMMWrapper  -- same virtual interface as the reference's
+//                       pipeline/include/cutlassGemmWrapperImpl.cuh:23-66;
+//   HipGEMMWrapper   -- D = alpha*A.B + beta*C on the MFMA kernel; takes the place of
+//                       CutlassGEMMWrapper<...> (:68-437).  The tile/stage fields of the tag
+//                       are accepted and recorded, but tiling is chosen by the kernel layer
+//                       from the problem shape; the three layout fields are honoured
+//                       (A and output must be RowMajor, B may be Row- or ColumnMajor);
+//   generateGEMM(tag) -- tag -> wrapper factory (pipeline/include/gemmFactory.cuh).
+#pragma once
+#include <string>
+
+#include "nanoflow_kernels.h"
+#include "operatorWrapper.h"
+#include "vortexData.h"
+
+struct BaseGEMMWrapper : public OperatorWrapper {
+  using ElementInputA = half;
+  using ElementInputB = half;
+  using ElementOutput = half;
+  using ElementAccumulator = float;
+
+  size_t M = 0, N = 0, K = 0;
+  void set_shape(int m, int n, int k) {
+    M = m;
+    N = n;
+    K = k;
+    NF_LOG_INFO("name:%s M:%zu, N:%zu, K:%zu", name.c_str(), M, N, K);
+  }
+  size_t mk() const { return M * K; }
+  size_t kn() const { return K * N; }
+  size_t mn() const { return M * N; }
+
+  virtual void init(ElementAccumulator beta_ = ElementAccumulator(0)) = 0;
+  virtual void profile() = 0;
+  virtual double totalCompute() = 0;
+  virtual float gflops(double runtime_ms) = 0;
+  virtual bool checkResult() = 0;
+  virtual ~BaseGEMMWrapper() = default;
+  virtual void set_weight(ElementInputB* data_b) = 0;
+  virtual bool set_weight(vortexWeight& weight) = 0;
+  virtual BaseGEMMWrapper& setOutput(pllmTensor<ElementOutput> data) = 0;
+  virtual BaseGEMMWrapper& setA(pllmTensor<ElementInputA> data_a) = 0;
+  virtual BaseGEMMWrapper& setB(pllmTensor<ElementInputB> data_b) = 0;
+  virtual BaseGEMMWrapper& setC(pllmTensor<ElementOutput> data_c) = 0;
+  virtual BaseGEMMWrapper& setD(pllmTensor<ElementOutput> data_d) = 0;
+  virtual pllmTensor<ElementInputA> getA() = 0;
+  virtual pllmTensor<ElementOutput> getD() = 0;
+  virtual pllmTensor<ElementInputB> getB() = 0;
+  virtual pllmTensor<ElementOutput> getC() = 0;
+  virtual void set_alpha(float alpha_) = 0;
+  virtual void set_beta(float beta_) = 0;
+};
+
+struct GemmTag {
+  int cta_m = 0, cta_n = 0, cta_k = 0, warp_m = 0, warp_n = 0, warp_k = 0, split_k = 1, stages = 0;
+  PllmLayout layout_a = PllmLayout::ROW_MAJOR, layout_b = PllmLayout::ROW_MAJOR,
+             layout_out = PllmLayout::ROW_MAJOR;
+};
+// Parses the tag grammar; returns false on malformed input.
+bool parseGemmTag(const std::string& tag, GemmTag& out);
+
+struct HipGEMMWrapper : public BaseGEMMWrapper {
+  GemmTag tag;
+  pllmTensor<half> pllm_tensor_a, pllm_tensor_b, pllm_tensor_c, pllm_tensor_d;
+  float alpha = 1.f, beta = 0.f;
+  bool inited = false;
+
+  explicit HipGEMMWrapper(const GemmTag& t) : tag(t) {}
+
+  void work() override;
+
+  HipGEMMWrapper& setOutput(pllmTensor<half> data) override { return setD(data); }
+  HipGEMMWrapper& setA(pllmTensor<half> a) override {
+    assert(a.layout == PllmLayout::ROW_MAJOR && a.dim1 == M && a.dim2 == K);
+    pllm_tensor_a = a;
+    return *this;
+  }
+  HipGEMMWrapper& setB(pllmTensor<half> b) override {
+    pllm_tensor_b = b;
+    return *this;
+  }
+  HipGEMMWrapper& setC(pllmTensor<half> c) override {
+    assert(c.layout == PllmLayout::ROW_MAJOR && c.dim1 == M && c.dim2 == N);
+    pllm_tensor_c = c;
+    return *this;
+  }
+  HipGEMMWrapper& setD(pllmTensor<half> d) override {
+    assert(d.layout == PllmLayout::ROW_MAJOR && d.dim1 == M && d.dim2 == N);
+    pllm_tensor_d = d;
+    return *this;
+  }
+  pllmTensor<half> getA() override { return pllm_tensor_a; }
+  pllmTensor<half> getB() override { return pllm_tensor_b; }
+  pllmTensor<half> getC() override { return pllm_tensor_c; }
+  pllmTensor<half> getD() override { return pllm_tensor_d; }
+
+  // All operands are expected to be set; (re)binds the problem size and beta.
+  void init(float beta_ = 0.f) override {
+    beta = beta_;
+    inited = true;
+  }
+  void set_weight(half* data_b) override {
+    pllm_tensor_b = tag.layout_b == PllmLayout::ROW_MAJOR
+                        ? pllmTensor<half>(data_b, K, N, PllmLayout::ROW_MAJOR)
+                        : pllmTensor<half>(data_b, N, K, PllmLayout::COL_MAJOR);
+  }
+  bool set_weight(vortexWeight& weight) override {
+    if (weight.size() != K * N) {
+      std::fprintf(stderr, "Weight size mismatch  %zu %zu %zu\n", weight.size(), K, N);
+      return false;
+    }
+    set_weight(weight.ptr);
+    return true;
+  }
+  void set_alpha(float a) override { alpha = a; }
+  void set_beta(float b) override { beta = b; }
+
+  double totalCompute() override { return 2.0 * (double)M * (double)N * (double)K; }
+  float gflops(double runtime_ms) override { return float(totalCompute() / 1e9 / (runtime_ms / 1e3)); }
+  void profile() override;      // times 100 launches on the op's stream, logs GFLOP/s
+  bool checkResult() override;  // spot-checks D against a host fp64 dot product
+};
+
+// Unknown or unsupported tags are an error here (nullptr + logged message) rather than the
+// reference's null dereference (pipeline/include/gemmFactory.cuh, pipeline_local.cu:850).
+BaseGEMMWrapper* generateGEMM(const std::string& tag);

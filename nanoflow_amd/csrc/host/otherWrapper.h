@@ -1,0 +1,181 @@
+// Row-wise operators of the pipeline: RMSNorm, embedding gather, split+RoPE+paged-KV append,
+// last-token gather, greedy sampler.  Interfaces of pipeline/include/otherWrapper.cuh:17-540
+// (only the operators the single-device pipelines use).
+#pragma once
+#include "config.h"
+#include "nanoflow_kernels.h"
+#include "operatorWrapper.h"
+#include "vortexData.h"
+
+class OtherWrapper : public OperatorWrapper {};
+
+// input_size / output_size == I_O_Ratio
+template <size_t I_O_Ratio = 1>
+class VectorOpWrapper : public OtherWrapper {
+public:
+  using Element = half;
+  Element* input = nullptr;
+  Element* output = nullptr;
+  pllmTensor<Element> pllm_tensor_input, pllm_tensor_output;
+  size_t input_size = 0, output_size = 0;
+
+  VectorOpWrapper& setInput(pllmTensor<Element> t) {
+    input = t.ptr;
+    input_size = t.size();
+    pllm_tensor_input = t;
+    assert(output_size == 0 || input_size == output_size * I_O_Ratio);
+    return *this;
+  }
+  VectorOpWrapper& setOutput(pllmTensor<Element> t) {
+    output = t.ptr;
+    output_size = t.size();
+    pllm_tensor_output = t;
+    assert(input_size == 0 || input_size == output_size * I_O_Ratio);
+    return *this;
+  }
+  pllmTensor<Element> getOutput() { return pllm_tensor_output; }
+  pllmTensor<Element> getInput() { return pllm_tensor_input; }
+};
+
+// RMSNorm over rows of model_hidden_dim (the reference's class name is LayerNorm).
+class LayerNorm : public VectorOpWrapper<1> {
+public:
+  Element* weight = nullptr;
+  pllmTensor<half> pllm_tensor_weight;
+
+  LayerNorm& setWeight(Element* w) {
+    weight = w;
+    return *this;
+  }
+  bool setWeight(vortexWeight w) {
+    weight = w.ptr;
+    pllm_tensor_weight = pllmTensor<half>(w.ptr, size_t(1), w.size(), PllmLayout::ROW_MAJOR);
+    return true;
+  }
+  void work() override {
+    assert(pllm_tensor_input.dim2 == (size_t)ModelConfig.model_hidden_dim);
+    NF_KERNEL_CHECK(nf_rmsnorm_f16(output, input, weight,
+                                   (int)(input_size / ModelConfig.model_hidden_dim),
+                                   ModelConfig.model_hidden_dim, ModelConfig.rms_norm_eps, stream));
+  }
+};
+
+class GenEmbedding : public OtherWrapper {
+public:
+  half* weight = nullptr;
+  int* tokens = nullptr;
+  half* output = nullptr;
+  pllmTensor<int> pllm_tensor_tokens;
+  pllmTensor<half> pllm_tensor_output, pllm_tensor_weight;
+  int input_size = 0, output_size = 0;
+
+  bool setWeight(vortexWeight w) {
+    weight = w.ptr;
+    pllm_tensor_weight = pllmTensor<half>(w.ptr, w.K, w.N, PllmLayout::ROW_MAJOR);
+    return true;
+  }
+  void setInput(pllmTensor<int> t) {
+    tokens = t.ptr;
+    input_size = (int)t.size();
+    pllm_tensor_tokens = t;
+    if (output_size) assert(input_size * ModelConfig.model_hidden_dim == output_size);
+  }
+  pllmTensor<half> getOutput() { return pllm_tensor_output; }
+  void setOutput(pllmTensor<half> o) {
+    output = o.ptr;
+    output_size = (int)o.size();
+    pllm_tensor_output = o;
+    if (input_size) assert(input_size * ModelConfig.model_hidden_dim == output_size);
+  }
+  void work() override {
+    NF_KERNEL_CHECK(nf_embedding_f16(tokens, weight, output, input_size,
+                                     ModelConfig.model_hidden_dim, stream));
+  }
+};
+
+class RoPEAppend : public OtherWrapper {
+public:
+  pllmTensor<half> kqv_input, q_out;
+  pllmTensor<int32_t> rev_input_indptr, per_token_offset;
+  int dense_batch_size = 0;
+  pllmTensor<half> kv_data;
+  pllmTensor<int32_t> kv_indices, kv_indptr, kv_last_page_len;
+  int* kqv_ready_counter = nullptr;
+
+  void setKVData(half* kv) {
+    kv_data = pllmTensor<half>(kv, size_t(ModelConfig.max_page_num * ModelConfig.frame_page_size * 2),
+                               size_t(ModelConfig.model_head_dim * ModelConfig.model_kv_heads_gpu),
+                               PllmLayout::ROW_MAJOR);
+  }
+  void setKVData(pllmTensor<half> kv) { kv_data = kv; }
+
+  // kqv_input / q_out / rev_input_indptr / per_token_offset are the nano-batch's slices;
+  // the kv_* arrays are the whole iteration's.
+  void update(int dense_batch_size, pllmTensor<half> kqv_input, pllmTensor<half> q_out,
+              pllmTensor<int32_t> rev_input_indptr, pllmTensor<int32_t> per_token_offset,
+              pllmTensor<int32_t> kv_indices, pllmTensor<int32_t> kv_indptr,
+              pllmTensor<int32_t> kv_last_page_len, int* kqv_ready_counter = nullptr) {
+    this->kqv_input = kqv_input;
+    this->q_out = q_out;
+    this->rev_input_indptr = rev_input_indptr;
+    this->per_token_offset = per_token_offset;
+    this->dense_batch_size = dense_batch_size;
+    this->kv_indices = kv_indices;
+    this->kv_indptr = kv_indptr;
+    this->kv_last_page_len = kv_last_page_len;
+    this->kqv_ready_counter = kqv_ready_counter;
+  }
+  void work() override {
+    NF_KERNEL_CHECK(nf_rope_append_f16(
+        kqv_input.ptr, q_out.ptr, kv_data.ptr, kv_indices.ptr, kv_indptr.ptr, rev_input_indptr.ptr,
+        per_token_offset.ptr, dense_batch_size, ModelConfig.model_qo_heads_gpu,
+        ModelConfig.model_kv_heads_gpu, ModelConfig.model_head_dim, ModelConfig.frame_page_size,
+        ModelConfig.factor, ModelConfig.rope_theta, ModelConfig.smooth_a, ModelConfig.smooth_b,
+        stream));
+  }
+};
+
+class MaxSampling : public OtherWrapper {
+public:
+  pllmTensor<half> d_matrix, d_maxVals;
+  pllmTensor<int> d_argMax;
+  int batch_size = 0;
+
+  void init(pllmTensor<half> d_matrix, pllmTensor<half> d_maxVals, pllmTensor<int> d_argMax) {
+    this->d_matrix = d_matrix;
+    this->d_maxVals = d_maxVals;
+    this->d_argMax = d_argMax;
+  }
+  void work() override {
+    NF_KERNEL_CHECK(nf_argmax_f16(d_matrix.ptr, d_maxVals.ptr, d_argMax.ptr, batch_size,
+                                  (int)d_matrix.dim2, stream));
+  }
+  OperatorWrapper& set_batch_size(int b) {
+    batch_size = b;
+    return *this;
+  }
+};
+
+class KeepToken : public OtherWrapper {
+public:
+  int req_num = 0;
+  pllmTensor<half> input, output;
+  int32_t* input_indptr = nullptr;
+
+  void update(int req_num, int32_t* input_indptr) {
+    this->req_num = req_num;
+    this->input_indptr = input_indptr;
+  }
+  void work() override {
+    NF_KERNEL_CHECK(nf_keep_token_f16(input.ptr, output.ptr, input_indptr, req_num,
+                                      (int)input.dim2, stream));
+  }
+  KeepToken& setOutput(pllmTensor<half> o) {
+    output = o;
+    return *this;
+  }
+  KeepToken& setInput(pllmTensor<half> i) {
+    input = i;
+    return *this;
+  }
+};

@@ -1,0 +1,193 @@
+// Pipeline schedules for one GPU.
+//   PipelineBase              config / update / run interface (pipeline/include/pipeline.h:22-51)
+//   LocalPipeline             two nano-batches; dense ops on stream_gemm, attention on
+//                             stream_gemv, cross-stream edges are event waits
+//                             (pipeline/include/pipeline.h:322-403, pipeline/src/pipeline_local.cu)
+//   NonOverlapLocalPipeline   same math on one stream, no nano-batching
+//                             (pipeline/include/pipeline.h:405-465,
+//                              pipeline/src/pipeline_nonoverlap_local.cu)
+// The tensor-parallel pipelines of the reference are outside this build.
+#pragma once
+#include <array>
+#include <memory>
+
+#include "allocManager.h"
+#include "config.h"
+#include "dualWrapper.h"
+#include "eventManager.h"
+#include "gemmWrapper.h"
+#include "gemvWrapper.h"
+#include "otherWrapper.h"
+#include "vortexData.h"
+
+#define SET_NAME_PTR(var) (var)->name = #var;
+#define SET_NAME_REF(var) (var).name = #var;
+#define GEMM_ALIAS(x) BaseGEMMWrapper*& x = gemms[static_cast<int>(GEMM_NAME::x)]
+
+// Accumulated per-iteration timings (filled when profiling is on).
+struct PipelineTimings {
+  double iter_ms = 0;        // last iteration, start of first op to end of sampler
+  double decode_attn_ms = 0; // sum of decode-attention launch durations
+  long decode_attn_launches = 0;
+  double prefill_attn_ms = 0;
+  long prefill_attn_launches = 0;
+  double gemm_ms = 0;        // sum over the timed dense GEMM launches (when enabled)
+  long gemm_launches = 0;
+};
+
+class PipelineBase {
+public:
+  PipelineBase(vortexInitData* input_data, int nrank, int nranks, int vnranks);
+  virtual ~PipelineBase() = default;
+
+protected:
+  vortexInitData* input_data;
+  vortexUpdateData update_data;       // device pointers
+  vortexUpdateData host_update_data;  // same iteration, host (staged) pointers
+  vortexConfigData config_data;
+  int rank;
+  int nranks;
+  int vnranks;
+  AllocationManager<half> tmpBufferM;
+  EventManager ev;
+  std::vector<hipEvent_t>& events = ev.events;
+  bool profiling = false;
+  PipelineTimings timings;
+
+public:
+  virtual vortexOutputData run() = 0;
+  virtual void update(vortexUpdateData* update_data) = 0;
+  virtual void config(vortexConfigData* config_data) = 0;
+  virtual void setName() {}
+  // stream on which update data must be uploaded so that it is ordered before run()
+  virtual hipStream_t uploadStream() = 0;
+  virtual void setProfiling(bool on) { profiling = on; }
+  const PipelineTimings& getTimings() const { return timings; }
+  void resetTimings() { timings = PipelineTimings(); }
+  void setHostUpdate(const vortexUpdateData& h) { host_update_data = h; }
+};
+
+class LocalPipeline : public PipelineBase {
+public:
+  void assignSameStream();
+  enum class GEMM_NAME { O1 = 0, O2, D1, D2, KQV1, KQV2, LOGITS, NUM };
+  static constexpr std::array gemmConfig = {
+      "128_256_64_64_64_64_1_3_RowMajor_RowMajor_RowMajor",  // O1
+      "128_256_64_64_64_64_1_3_RowMajor_RowMajor_RowMajor",  // O2
+      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // D1
+      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // D2
+      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV1
+      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV2
+      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // LOGITS
+  };
+  static constexpr int gemmNum = static_cast<int>(GEMM_NAME::NUM);
+  std::array<BaseGEMMWrapper*, gemmNum> gemms{};
+  GEMM_ALIAS(O1);
+  GEMM_ALIAS(O2);
+  GEMM_ALIAS(D1);
+  GEMM_ALIAS(D2);
+  GEMM_ALIAS(KQV1);
+  GEMM_ALIAS(KQV2);
+  GEMM_ALIAS(LOGITS);
+
+  DualWrapper dual1, dual2;
+  GenEmbedding genEmbedding1, genEmbedding2;
+  DecodeGemvWrapper GEMV1, GEMV2, GEMV3, GEMV4;
+  std::array<DecodeGemvWrapper*, 4> gemvs{&GEMV1, &GEMV2, &GEMV3, &GEMV4};
+  LayerNorm layerNormAttention1, layerNormAttention2;
+  LayerNorm layerNormFFN1, layerNormFFN2;
+  LayerNorm layerNormModel;
+  RoPEAppend roPEAppends[2];
+  PrefillGemvWrapper prefill1, prefill2;
+  MaxSampling maxSampler;
+  KeepToken keepToken;
+
+  pllmTensor<half> gemvQ1, gemvQ2;
+  pllmTensor<half> gemvAggregateOutput1, gemvAggregateOutput2;
+  pllmTensor<half> KQV_output1, KQV_output2;
+  BaseGEMMWrapper* KQV_ptrs[2] = {nullptr, nullptr};
+  vortexOutputData output_data;
+  hipStream_t stream_gemm = nullptr;
+  hipStream_t stream_gemv = nullptr;
+  hipStream_t stream_other = nullptr;
+  int update_token_num = 0;
+  vortexUpdateData prefill1_update;   // device copies patched for a prefill request that
+  vortexUpdateData prefill1_staging;  // straddles the nano-batch border (+ pinned staging)
+  bool nanobatch_only = false;
+
+  LocalPipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks,
+                bool nanobatch_only = false);
+  ~LocalPipeline() override;
+  void ScheduleInit();
+  void GEMMOpInit();
+  void GEMVOpInit();
+  void OtherOpInit();
+  void setWeight(int layer);
+  void setWeight_group_O(int layer);
+  void setWeight_group_LN(int layer);
+  vortexOutputData run() override;
+  void update(vortexUpdateData* update_data) override;
+  void config(vortexConfigData* config_data) override;
+  void GEMVOpUpdate();
+  void setName() override;
+  hipStream_t uploadStream() override { return stream_gemm; }
+  void setProfiling(bool on) override;
+
+private:
+  void init();
+  double totalCompute();
+  void enqueueIteration();
+};
+
+class NonOverlapLocalPipeline : public PipelineBase {
+public:
+  enum class GEMM_NAME { O = 0, D, KQV, LOGITS, NUM };
+  static constexpr std::array gemmConfig = {
+      "128_256_64_64_64_64_1_3_RowMajor_RowMajor_RowMajor",  // O
+      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // D
+      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV
+      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // LOGITS
+  };
+  static constexpr int gemmNum = static_cast<int>(GEMM_NAME::NUM);
+  std::array<BaseGEMMWrapper*, gemmNum> gemms{};
+  GEMM_ALIAS(O);
+  GEMM_ALIAS(D);
+  GEMM_ALIAS(KQV);
+  GEMM_ALIAS(LOGITS);
+
+  DualWrapper dual;
+  GenEmbedding genEmbedding;
+  DecodeGemvWrapper GEMV;
+  LayerNorm layerNormAttention, layerNormFFN, layerNormModel;
+  RoPEAppend roPEAppend;
+  PrefillGemvWrapper prefill;
+  MaxSampling maxSampler;
+  KeepToken keepToken;
+
+  pllmTensor<half> gemvInput, gemvOutput;
+  vortexOutputData output_data;
+  hipStream_t stream_all = nullptr;
+  int update_token_num = 0;
+
+  NonOverlapLocalPipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks);
+  ~NonOverlapLocalPipeline() override;
+  void ScheduleInit();
+  void GEMMOpInit();
+  void GEMVOpInit();
+  void OtherOpInit();
+  void setWeight(int layer);
+  vortexOutputData run() override;
+  void update(vortexUpdateData* update_data) override;
+  void config(vortexConfigData* config_data) override;
+  void GEMVOpUpdate();
+  void setName() override;
+  hipStream_t uploadStream() override { return stream_all; }
+  void setProfiling(bool on) override;
+
+private:
+  double totalCompute();
+};
+
+// Creates a stream restricted to `num_cus` compute units starting at CU `first_cu` of every
+// XCD-interleaved numbering (0 = no restriction, plain stream).
+hipStream_t createPipelineStream(int first_cu, int num_cus);

@@ -1,0 +1,243 @@
+// NonOverlapLocalPipeline: the sequential single-stream schedule (no nano-batching).
+// The plainest statement of the layer math and the baseline the overlapped schedule must
+// agree with.  Operator order follows the reference's
+// pipeline/src/pipeline_nonoverlap_local.cu:25-62, wiring :245-304, update :108-126,327-385.
+#include "pipeline.h"
+
+NonOverlapLocalPipeline::NonOverlapLocalPipeline(vortexInitData* input_data, int nrank, int nranks,
+                                                 int vnranks)
+    : PipelineBase(input_data, nrank, nranks, vnranks) {
+  stream_all = createPipelineStream(0, 0);
+  NF_LOG_INFO("Init pipeline (non-overlap local)");
+}
+
+NonOverlapLocalPipeline::~NonOverlapLocalPipeline() {
+  for (auto g : gemms) delete g;
+  delete[] output_data.sampled_token_array;
+  if (stream_all) (void)hipStreamDestroy(stream_all);
+}
+
+void NonOverlapLocalPipeline::setProfiling(bool on) {
+  profiling = on;
+  const size_t n = on ? (size_t)ModelConfig.run_layer : 0;
+  GEMV.enableProfiling(n);
+  prefill.enableProfiling(n);
+}
+
+vortexOutputData NonOverlapLocalPipeline::run() {
+  setWeight(0);
+  HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_START], stream_all));
+  genEmbedding.run();
+  for (int iter = 0; iter < ModelConfig.run_layer; ++iter) {
+    setWeight(iter % ModelConfig.model_layer);
+    layerNormAttention.run();
+    KQV->run();
+    roPEAppend.run();
+    if (GEMV.batch_size > 0) GEMV.run();
+    if (update_data.prefillNum > 0) prefill.run();
+    O->run();
+    layerNormFFN.run();
+    dual.run();
+    D->run();
+  }
+  keepToken.run();
+  layerNormModel.run();
+  LOGITS->run();
+  maxSampler.run();
+  HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_END], stream_all));
+  HIP_CHECK(hipMemcpyAsync(output_data.sampled_token_array, maxSampler.d_argMax.ptr,
+                           output_data.sampled_tokens * sizeof(int), hipMemcpyDeviceToHost,
+                           stream_all));
+  HIP_CHECK(hipStreamSynchronize(stream_all));
+  float runtime_ms = 0;
+  HIP_CHECK(hipEventElapsedTime(&runtime_ms, events[EventManager::GEMM_TIMING_START],
+                                events[EventManager::GEMM_TIMING_END]));
+  timings.iter_ms = runtime_ms;
+  if (profiling) {
+    GEMV.collectProfile(timings.decode_attn_ms, timings.decode_attn_launches);
+    prefill.collectProfile(timings.prefill_attn_ms, timings.prefill_attn_launches);
+  }
+  NF_LOG_INFO("Total running cost (ms) of one microbatch is %f", runtime_ms);
+  return output_data;
+}
+
+void NonOverlapLocalPipeline::update(vortexUpdateData* update_data_) {
+  this->update_data = *update_data_;
+  const int T = config_data.global_batch_size;
+  genEmbedding.setInput(pllmTensor<int>(update_data.input_tokens, T, 1, PllmLayout::ROW_MAJOR));
+  const int req_num = update_data.decodePrefillBorder + update_data.prefillNum;
+  update_token_num = update_data.decodePrefillBorder + update_data.prefillTokensNum;
+  maxSampler.set_batch_size(req_num / nranks);
+  keepToken.update(req_num, update_data.input_indptr);
+  LOGITS->set_shape(std::min((req_num / nranks + 127) / 128 * 128, T), (int)ModelConfig.vocab_size,
+                    ModelConfig.model_hidden_dim);
+  LOGITS->init();
+  output_data.sampled_tokens = req_num;
+  GEMVOpUpdate();
+}
+
+void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
+  NF_LOG_INFO("Config non-overlap local pipeline");
+  this->config_data = *config_data_;
+  for (int i = 0; i < gemmNum; ++i) {
+    const std::string& tag =
+        i < (int)config_data.gemm_op_tag.size() ? config_data.gemm_op_tag[i] : std::string(gemmConfig[i]);
+    gemms[i] = generateGEMM(tag);
+    if (!gemms[i]) {
+      std::fprintf(stderr, "NonOverlapLocalPipeline::config: cannot build GEMM %d from tag \"%s\"\n", i,
+                   tag.c_str());
+      std::exit(EXIT_FAILURE);
+    }
+  }
+  const int globalbatch = config_data.global_batch_size;
+  if (globalbatch <= 0 || globalbatch > ModelConfig.max_batch_size) {
+    std::fprintf(stderr, "NonOverlapLocalPipeline::config: global batch %d exceeds max batch %d\n",
+                 globalbatch, ModelConfig.max_batch_size);
+    std::exit(EXIT_FAILURE);
+  }
+  O->set_shape(globalbatch, ModelConfig.model_hidden_dim_pergpu, ModelConfig.model_hidden_dim);
+  D->set_shape(globalbatch, ModelConfig.model_hidden_dim, ModelConfig.model_ff_dim_gpu);
+  KQV->set_shape(globalbatch,
+                 (2 * ModelConfig.model_kv_heads_gpu + ModelConfig.model_qo_heads_gpu) *
+                     ModelConfig.model_head_dim,
+                 ModelConfig.model_hidden_dim);
+  LOGITS->set_shape(globalbatch, (int)ModelConfig.vocab_size, ModelConfig.model_hidden_dim);
+  dual.set_shape(globalbatch, ModelConfig.model_ff_dim_gpu, ModelConfig.model_hidden_dim);
+  ScheduleInit();
+  GEMMOpInit();
+  GEMVOpInit();
+  OtherOpInit();
+  setName();
+  output_data = vortexOutputData();
+  output_data.sampled_token_array = new int[globalbatch];
+  output_data.global_batch_size = globalbatch;
+  if (profiling) setProfiling(true);
+}
+
+void NonOverlapLocalPipeline::setName() {
+  SET_NAME_PTR(KQV);
+  SET_NAME_PTR(LOGITS);
+  SET_NAME_PTR(O);
+  SET_NAME_REF(dual);
+  SET_NAME_PTR(D);
+  SET_NAME_REF(genEmbedding);
+  SET_NAME_REF(layerNormAttention);
+  SET_NAME_REF(layerNormFFN);
+  SET_NAME_REF(layerNormModel);
+  SET_NAME_REF(GEMV);
+  SET_NAME_REF(prefill);
+  SET_NAME_REF(roPEAppend);
+  SET_NAME_REF(maxSampler);
+  SET_NAME_REF(keepToken);
+}
+
+void NonOverlapLocalPipeline::setWeight(int layer) {
+  auto& lw = input_data->weight.layer_weight[layer];
+  bool success = true;
+  success &= O->set_weight(lw.W_O1);
+  success &= D->set_weight(lw.W_D);
+  success &= KQV->set_weight(lw.W_KQV);
+  success &= layerNormAttention.setWeight(lw.W_LN_Attention);
+  success &= layerNormFFN.setWeight(lw.W_LN_FFN);
+  success &= dual.set_weight(lw.W_G, lw.W_U);
+  if (!success) NF_LOG_ERROR("Failed to set weight for layer %d", layer);
+  GEMV.setKVData(input_data->kv_data[layer]);
+  prefill.setKVData(input_data->kv_data[layer]);
+  roPEAppend.setKVData(input_data->kv_data[layer]);
+}
+
+void NonOverlapLocalPipeline::ScheduleInit() {
+  const auto ROW = PllmLayout::ROW_MAJOR;
+  const int T = config_data.global_batch_size;
+  const int qdim = ModelConfig.model_head_dim * ModelConfig.model_qo_heads_gpu;
+  gemvOutput = tmpBufferM.allocTensor(T, qdim, ROW);
+  const auto O_output = tmpBufferM.allocTensor((int)O->M, (int)O->N, ROW);
+  O->setA(gemvOutput);
+  O->setD(O_output);
+  const auto LayerNormFFN_output = tmpBufferM.allocTensor(dual.M, dual.K, ROW);
+  layerNormFFN.setInput(O_output).setOutput(LayerNormFFN_output);
+  const auto activation_output = tmpBufferM.allocTensor((int)D->M, (int)D->K, ROW);
+  dual.setA(LayerNormFFN_output);
+  dual.setD(pllmTensor<half>(), pllmTensor<half>(), activation_output);
+  const auto D_output = tmpBufferM.allocTensor((int)D->M, (int)D->N, ROW);
+  D->setA(activation_output);
+  D->setC(O_output);   // residual: output of the attention block
+  D->setOutput(D_output);
+  const auto layerNormAttention_output = tmpBufferM.allocTensor((int)D->M, (int)D->N, ROW);
+  layerNormAttention.setInput(D_output).setOutput(layerNormAttention_output);
+  O->setC(D_output);   // residual stream lives in the D output
+  KQV->setA(layerNormAttention_output).setOutput(tmpBufferM.allocTensor((int)KQV->M, (int)KQV->N, ROW));
+  gemvInput = tmpBufferM.allocTensor(T, qdim, ROW);
+  const auto keepTokenOutput = tmpBufferM.allocTensor(T, (int)D->N, ROW);
+  keepToken.setInput(D_output).setOutput(keepTokenOutput);
+  const auto layerNormModel_output = tmpBufferM.allocTensor(T, (int)D->N, ROW);
+  layerNormModel.setInput(keepTokenOutput).setOutput(layerNormModel_output);
+  const auto LOGITS_output = tmpBufferM.allocTensor(T, (int)LOGITS->N, ROW);
+  LOGITS->setA(layerNormModel_output);
+  LOGITS->setOutput(LOGITS_output);
+  int* sample_output_alloc = (int*)tmpBufferM.alloc((size_t)T * sizeof(int) / sizeof(half));
+  pllmTensor<int> sample_output = {sample_output_alloc, T, 1, ROW};
+  const auto maxSampler_maxVals = tmpBufferM.allocTensor(T, 1, ROW);
+  maxSampler.init(LOGITS_output, maxSampler_maxVals, sample_output);
+  genEmbedding.setOutput(D->getD());
+  NF_LOG_INFO("allocated %zu halfs", tmpBufferM.getAllocation());
+}
+
+void NonOverlapLocalPipeline::GEMMOpInit() {
+  setWeight(0);
+  O->init(1.f);
+  dual.init();
+  D->init(1.f);
+  KQV->init();
+  for (int i = 0; i < gemmNum; ++i) gemms[i]->setStream(stream_all);
+  LOGITS->set_weight(input_data->weight.lm_head);
+  LOGITS->init();
+  dual.setStream(stream_all);
+}
+
+void NonOverlapLocalPipeline::GEMVOpUpdate() {
+  const uint32_t dpb = update_data.decodePrefillBorder;
+  uint32_t arr[] = {dpb, uint32_t(update_data.prefillNum)};
+  std::span<uint32_t, 2> batch_sizes(arr, 2);
+  const size_t total_batch_size = arr[0] + arr[1];
+  const uint32_t T = config_data.global_batch_size;
+  const auto kv_indptr_split = pllmTensor<int32_t>{update_data.kv_indptr, total_batch_size + 1}
+                                   .splitTensor(PllmDimension::ROW, batch_sizes, 1U);
+  const auto kv_last_page_len_split = pllmTensor<int32_t>{update_data.kv_last_page_len, total_batch_size}
+                                          .splitTensor(PllmDimension::ROW, batch_sizes);
+  const auto input_ptr_split = pllmTensor<int32_t>{update_data.input_indptr, total_batch_size + 1}
+                                   .splitTensor(PllmDimension::ROW, batch_sizes, 1U);
+  GEMV.init(dpb, update_data.gemv_num_blocks[0], input_ptr_split[0], kv_indptr_split[0],
+            update_data.kv_indices, kv_last_page_len_split[0], gemvInput, gemvOutput);
+  prefill.init(update_data.prefillNum, 0, input_ptr_split[1], kv_indptr_split[1],
+               update_data.kv_indices, kv_last_page_len_split[1], gemvInput, gemvOutput);
+  roPEAppend.update(update_token_num, KQV->getD(), gemvInput,
+                    pllmTensor<int32_t>(update_data.rev_input_indptr, (size_t)T),
+                    pllmTensor<int32_t>(update_data.per_token_offset, (size_t)T),
+                    pllmTensor<int32_t>(update_data.kv_indices, ModelConfig.max_page_num),
+                    pllmTensor<int32_t>(update_data.kv_indptr, (size_t)T + 1),
+                    pllmTensor<int32_t>(update_data.kv_last_page_len, (size_t)T));
+}
+
+void NonOverlapLocalPipeline::OtherOpInit() {
+  layerNormAttention.setStream(stream_all);
+  layerNormFFN.setStream(stream_all);
+  genEmbedding.setStream(stream_all);
+  layerNormModel.setStream(stream_all);
+  roPEAppend.setStream(stream_all);
+  maxSampler.setStream(stream_all);
+  keepToken.setStream(stream_all);
+  genEmbedding.setWeight(input_data->weight.embedding);
+  layerNormModel.setWeight(input_data->weight.model_layernorm);
+}
+
+void NonOverlapLocalPipeline::GEMVOpInit() {
+  GEMV.setStream(stream_all);
+  prefill.setStream(stream_all);
+}
+
+double NonOverlapLocalPipeline::totalCompute() {
+  double total = 0;
+  for (auto gemm : gemms) total += gemm->totalCompute();
+  return total;
+}

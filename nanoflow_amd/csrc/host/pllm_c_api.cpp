@@ -1,0 +1,330 @@
+// Flat C ABI over the C++ control plane (include/nanoflow_pllm.h).
+#include "nanoflow_pllm.h"
+
+#include <cstdarg>
+#include <cstring>
+
+#include "computeBound.h"
+
+static thread_local char g_err[512] = "";
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  std::vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static int g_nranks = 1, g_vnranks = 1;
+static bool g_config_loaded = false, g_inited = false, g_configured = false, g_updated = false;
+static bool g_running = false;
+static std::vector<vortexInitData> g_init(1);
+static std::vector<vortexOutputData> g_out(1);
+static std::vector<vortexConfigData> g_cfg(1);
+static std::vector<vortexUpdateData> g_upd(1);
+
+static vortexWeight to_cpp(const nf_vortex_weight& w) {
+  vortexWeight r;
+  r.ptr = w.ptr;
+  r.N = w.N;
+  r.K = w.K;
+  return r;
+}
+static nf_vortex_weight to_c(const vortexWeight& w) { return nf_vortex_weight{w.ptr, w.N, w.K}; }
+
+static vortexModelWeight to_cpp(const nf_vortex_model_weight& m) {
+  vortexModelWeight r;
+  r.lm_head = to_cpp(m.lm_head);
+  r.embedding = to_cpp(m.embedding);
+  r.model_layernorm = to_cpp(m.model_layernorm);
+  r.layer_weight.resize(m.num_layers);
+  for (int i = 0; i < m.num_layers; ++i) {
+    const auto& s = m.layer_weight[i];
+    auto& t = r.layer_weight[i];
+    t.W_O1 = to_cpp(s.W_O1); t.W_O2 = to_cpp(s.W_O2); t.W_U = to_cpp(s.W_U); t.W_G = to_cpp(s.W_G);
+    t.W_D = to_cpp(s.W_D); t.W_KQV = to_cpp(s.W_KQV); t.B_KQV = to_cpp(s.B_KQV);
+    t.W_LN_Attention = to_cpp(s.W_LN_Attention); t.W_LN_FFN = to_cpp(s.W_LN_FFN);
+    t.W_ROT = to_cpp(s.W_ROT);
+  }
+  return r;
+}
+
+extern "C" {
+
+const char* pllm_last_error(void) { return g_err; }
+
+int pllm_set_model_config(const char* json_path) {
+  if (!json_path) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_set_model_config: null path");
+  if (g_inited) return fail(NF_PLLM_ERR_STATE, "pllm_set_model_config: pipeline already initialised");
+  if (!updateVortexModelConfig(json_path))
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_set_model_config: cannot load %s", json_path);
+  const auto& c = ModelConfig;
+  if (c.gpu_num != 1)
+    return fail(NF_PLLM_ERR_UNSUPPORTED, "model_configs.gpu_num=%d: this build runs one GPU", c.gpu_num);
+  if (c.model_head_dim != 128 || c.frame_page_size != 16)
+    return fail(NF_PLLM_ERR_UNSUPPORTED, "head_dim=%d page_size=%d: kernels are built for 128 / 16",
+                c.model_head_dim, c.frame_page_size);
+  if (c.model_hidden_dim % 8 || c.model_ff_dim % 8 || c.vocab_size % 8 || c.run_layer < 1 ||
+      c.model_layer < 1)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "hidden/ffn/vocab must be multiples of 8, layers >= 1");
+  g_config_loaded = true;
+  return NF_PLLM_OK;
+}
+
+int pllm_set_rank(int nranks, int vnranks) {
+  if (nranks != 1 || vnranks != 1)
+    return fail(NF_PLLM_ERR_UNSUPPORTED, "pllm_set_rank(%d, %d): this build runs exactly one rank",
+                nranks, vnranks);
+  g_nranks = nranks;
+  g_vnranks = vnranks;
+  return NF_PLLM_OK;
+}
+
+size_t pllm_tmp_buffer_halves(void) { return ModelConfig.k_temp_size; }
+size_t pllm_max_page_num(void) { return ModelConfig.max_page_num; }
+
+int pllm_init(const nf_vortex_init_data* input, int pipeline_type) {
+  if (!g_config_loaded) return fail(NF_PLLM_ERR_STATE, "pllm_init: call pllm_set_model_config first");
+  if (g_inited) return fail(NF_PLLM_ERR_STATE, "pllm_init: already initialised");
+  if (!input || !input->kv_data || !input->tmp_buffer || !input->weight.layer_weight)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_init: null pointer in init data");
+  if (pipeline_type < 0 || pipeline_type > NF_PIPE_NANOBATCH_LOCAL)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_init: unknown pipeline type %d", pipeline_type);
+  auto ty = static_cast<Worker::PipelineType>(pipeline_type);
+  if (!Worker::isSupported(ty))
+    return fail(NF_PLLM_ERR_UNSUPPORTED,
+                "pllm_init: pipeline type %d is a tensor-parallel schedule; LOCAL(7), "
+                "NON_OVERLAP_LOCAL(8) and NANOBATCH_LOCAL(9) are implemented", pipeline_type);
+  if (input->weight.num_layers < ModelConfig.model_layer)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_init: %d layers of weights, model has %d",
+                input->weight.num_layers, ModelConfig.model_layer);
+  vortexInitData d;
+  d.kv_data = new half*[ModelConfig.model_layer];
+  for (int i = 0; i < ModelConfig.model_layer; ++i) {
+    if (!input->kv_data[i]) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_init: kv_data[%d] is null", i);
+    d.kv_data[i] = input->kv_data[i];
+  }
+  d.weight = to_cpp(input->weight);
+  d.weight_size = input->weight_size;
+  d.tmp_buffer = input->tmp_buffer;
+  d.tmp_buffer_size = input->tmp_buffer_size;
+  g_init[0] = d;
+  g_out[0] = vortexOutputData();
+  HIP_CHECK(hipSetDevice(0));
+  TensorManager::getInstance().init(g_nranks, g_vnranks);
+  init(g_nranks, g_vnranks, g_init, g_out, ty);
+  g_inited = true;
+  g_configured = g_updated = g_running = false;
+  return NF_PLLM_OK;
+}
+
+int pllm_model_weight_to_gpu(const nf_vortex_model_weight* host_weight,
+                             nf_vortex_model_weight* device_weight,
+                             nf_vortex_layer_weight* device_layers) {
+  if (!host_weight || !device_weight || !device_layers)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_model_weight_to_gpu: null pointer");
+  vortexModelWeight h = to_cpp(*host_weight);
+  vortexModelWeight d = modelWeightToGPU(h, 0);
+  device_weight->lm_head = to_c(d.lm_head);
+  device_weight->embedding = to_c(d.embedding);
+  device_weight->model_layernorm = to_c(d.model_layernorm);
+  device_weight->num_layers = (int)d.layer_weight.size();
+  device_weight->layer_weight = device_layers;
+  for (size_t i = 0; i < d.layer_weight.size(); ++i) {
+    const auto& s = d.layer_weight[i];
+    device_layers[i] = nf_vortex_layer_weight{to_c(s.W_O1), to_c(s.W_O2), to_c(s.W_U), to_c(s.W_G),
+                                              to_c(s.W_D), to_c(s.W_KQV), to_c(s.B_KQV),
+                                              to_c(s.W_LN_Attention), to_c(s.W_LN_FFN), to_c(s.W_ROT)};
+  }
+  return NF_PLLM_OK;
+}
+
+int pllm_config(const nf_vortex_config_data* c) {
+  if (!g_inited) return fail(NF_PLLM_ERR_STATE, "pllm_config: call pllm_init first");
+  if (g_configured) return fail(NF_PLLM_ERR_STATE, "pllm_config: already configured");
+  if (!c) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: null config");
+  const bool local = Worker::PipeTy != Worker::PipelineType::NON_OVERLAP_LOCAL;
+  if (c->global_batch_size <= 0 || c->global_batch_size > ModelConfig.max_batch_size)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: global_batch_size %d not in (0, %d]",
+                c->global_batch_size, ModelConfig.max_batch_size);
+  if (local && (c->nanobatch_1_size <= 0 || c->nanobatch_1_size >= c->global_batch_size))
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: nanobatch_1_size %d not in (0, %d)",
+                c->nanobatch_1_size, c->global_batch_size);
+  vortexConfigData d;
+  for (int i = 0; i < c->num_gemm_op_tag; ++i) {
+    GemmTag t;
+    if (!c->gemm_op_tag[i] || !parseGemmTag(c->gemm_op_tag[i], t) ||
+        t.layout_a != PllmLayout::ROW_MAJOR || t.layout_out != PllmLayout::ROW_MAJOR)
+      return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: bad GEMM tag %d: \"%s\"", i,
+                  c->gemm_op_tag[i] ? c->gemm_op_tag[i] : "(null)");
+    d.gemm_op_tag.push_back(c->gemm_op_tag[i]);
+  }
+  d.global_batch_size = c->global_batch_size;
+  d.nanobatch_1_size = c->nanobatch_1_size;
+  d.kqv1_size = c->kqv1_size;
+  d.kqv3_size = c->kqv3_size;
+  // tmp buffer must hold the schedule's intermediates (upper bound of the buffer plan)
+  const size_t T = d.global_batch_size, H = ModelConfig.model_hidden_dim;
+  const size_t need = T * ((size_t)ModelConfig.kqv_n + 8 * H + 2 * (size_t)ModelConfig.model_ff_dim +
+                           ModelConfig.vocab_size + 8);
+  if (g_init[0].tmp_buffer_size < need)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: tmp buffer has %zu halves, schedule needs %zu",
+                g_init[0].tmp_buffer_size, need);
+  g_cfg[0] = d;
+  config(g_nranks, g_cfg);
+  g_configured = true;
+  return NF_PLLM_OK;
+}
+
+int pllm_update(const nf_vortex_update_data* u) {
+  if (!g_configured) return fail(NF_PLLM_ERR_STATE, "pllm_update: call pllm_config first");
+  if (g_running) return fail(NF_PLLM_ERR_STATE, "pllm_update: a run is in flight; call pllm_run_async_wait");
+  if (!u || !u->input_indptr || !u->rev_input_indptr || !u->kv_indptr || !u->kv_indices ||
+      !u->kv_last_page_len || !u->per_token_offset || !u->gemv_batch_size || !u->gemv_num_blocks ||
+      (u->prefillTokensNum > 0 && !u->input_tokens) || (u->keepTokenListLength > 0 && !u->keep_token_list))
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: null pointer in update data");
+  const int T = g_cfg[0].global_batch_size;
+  const int req = u->decodePrefillBorder + u->prefillNum;
+  const int tok = u->decodePrefillBorder + u->prefillTokensNum;
+  if (u->decodePrefillBorder < 0 || u->prefillNum < 0 || u->prefillTokensNum < 0 || tok > T || req > T ||
+      tok < 1)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: %d requests / %d tokens do not fit batch %d",
+                req, tok, T);
+  if (u->input_indptr[req] != tok)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: input_indptr[%d]=%d but the batch has %d tokens",
+                req, u->input_indptr[req], tok);
+  if ((size_t)u->kv_indptr[req] > ModelConfig.max_page_num)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: %d pages in use, pool has %zu",
+                u->kv_indptr[req], ModelConfig.max_page_num);
+  const int gsum = u->gemv_batch_size[0] + u->gemv_batch_size[1] + u->gemv_batch_size[2] + u->gemv_batch_size[3];
+  if (gsum != u->decodePrefillBorder)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: gemv_batch_size sums to %d, decode requests %d",
+                gsum, u->decodePrefillBorder);
+  if (Worker::PipeTy != Worker::PipelineType::NON_OVERLAP_LOCAL) {
+    // decode groups 0 and 1 are the decode rows of nano-batch 1, groups 2 and 3 those of
+    // nano-batch 2 (the O projection of nano-batch 1 waits for groups 0/1 only)
+    const int want = std::min(u->decodePrefillBorder, g_cfg[0].nanobatch_1_size);
+    if (u->gemv_batch_size[0] + u->gemv_batch_size[1] != want)
+      return fail(NF_PLLM_ERR_INVALID_ARGUMENT,
+                  "pllm_update: decode groups 0+1 hold %d requests, nano-batch 1 has %d decode rows",
+                  u->gemv_batch_size[0] + u->gemv_batch_size[1], want);
+  }
+  vortexUpdateData d;
+  d.decodePrefillBorder = u->decodePrefillBorder;
+  d.prefillNum = u->prefillNum;
+  d.prefillTokensNum = u->prefillTokensNum;
+  d.keepTokenListLength = u->keepTokenListLength;
+  d.input_tokens = u->input_tokens;
+  d.input_indptr = u->input_indptr;
+  d.rev_input_indptr = u->rev_input_indptr;
+  d.keep_token_list = u->keep_token_list;
+  d.kv_indptr = u->kv_indptr;
+  d.kv_indices = u->kv_indices;
+  d.kv_last_page_len = u->kv_last_page_len;
+  d.per_token_offset = u->per_token_offset;
+  d.gemv_batch_size = u->gemv_batch_size;
+  d.gemv_num_blocks = u->gemv_num_blocks;
+  // kept slots + prefill tokens must add up to the batch rows
+  int kept = 0;
+  for (int i = 0; i < u->keepTokenListLength; ++i) kept += u->keep_token_list[i] == 1;
+  if (kept != u->decodePrefillBorder)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: keep_token_list keeps %d slots, decode rows %d",
+                kept, u->decodePrefillBorder);
+  if (!aggregated_output.empty() && u->keepTokenListLength > (int)aggregated_output.size())
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: keep list of %d over %zu previous outputs",
+                u->keepTokenListLength, aggregated_output.size());
+  g_upd[0] = d;
+  update(g_nranks, g_upd);
+  g_updated = true;
+  return NF_PLLM_OK;
+}
+
+int pllm_run_async(void) {
+  if (!g_updated) return fail(NF_PLLM_ERR_STATE, "pllm_run_async: call pllm_update first");
+  if (g_running) return fail(NF_PLLM_ERR_STATE, "pllm_run_async: a run is already in flight");
+  run_async();
+  g_running = true;
+  return NF_PLLM_OK;
+}
+
+int pllm_run_async_wait(void) {
+  if (!g_running) return fail(NF_PLLM_ERR_STATE, "pllm_run_async_wait: no run in flight");
+  run_async_wait();
+  g_running = false;
+  return NF_PLLM_OK;
+}
+
+int pllm_run(void) {
+  int rc = pllm_run_async();
+  return rc ? rc : pllm_run_async_wait();
+}
+
+int pllm_get_pipeline_output(const int32_t** tokens, int* count) {
+  if (!tokens || !count) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_get_pipeline_output: null pointer");
+  *tokens = aggregated_output.data();
+  *count = (int)aggregated_output.size();
+  return NF_PLLM_OK;
+}
+
+int pllm_finalize(void) {
+  if (g_running) pllm_run_async_wait();
+  if (g_inited) finalize();
+  g_inited = g_configured = g_updated = g_running = false;
+  delete[] g_init[0].kv_data;
+  g_init[0] = vortexInitData();
+  return NF_PLLM_OK;
+}
+
+int pllm_build_input_tokens(const int32_t* prev_output, int prev_count, const int32_t* keep_token_list,
+                            int keep_token_list_length, const int32_t* prefill_tokens,
+                            int prefill_tokens_num, int32_t* out) {
+  if ((keep_token_list_length > 0 && !keep_token_list) || (prefill_tokens_num > 0 && !prefill_tokens) || !out)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_build_input_tokens: null pointer");
+  return buildInputTokens(prev_output, prev_count, keep_token_list, keep_token_list_length, prefill_tokens,
+                          prefill_tokens_num, out);
+}
+
+int pllm_set_profiling(int on) {
+  setPipelineProfiling(on != 0);
+  return NF_PLLM_OK;
+}
+
+int pllm_get_timings(nf_pipeline_timings* out) {
+  PipelineBase* p = currentPipeline();
+  if (!p || !out) return fail(NF_PLLM_ERR_STATE, "pllm_get_timings: no pipeline");
+  const PipelineTimings& t = p->getTimings();
+  out->iter_ms = t.iter_ms;
+  out->decode_attn_ms = t.decode_attn_ms;
+  out->decode_attn_launches = t.decode_attn_launches;
+  out->prefill_attn_ms = t.prefill_attn_ms;
+  out->prefill_attn_launches = t.prefill_attn_launches;
+  return NF_PLLM_OK;
+}
+
+int pllm_reset_timings(void) {
+  PipelineBase* p = currentPipeline();
+  if (!p) return fail(NF_PLLM_ERR_STATE, "pllm_reset_timings: no pipeline");
+  p->resetTimings();
+  return NF_PLLM_OK;
+}
+
+int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols) {
+  PipelineBase* p = currentPipeline();
+  if (!p || !g_configured || !name || !ptr || !rows || !cols)
+    return fail(NF_PLLM_ERR_STATE, "pllm_debug_buffer: no configured pipeline");
+  pllmTensor<half> t;
+  if (auto* lp = dynamic_cast<LocalPipeline*>(p)) {
+    if (!std::strcmp(name, "hidden")) t = lp->keepToken.input;
+    else if (!std::strcmp(name, "logits")) t = lp->maxSampler.d_matrix;
+  } else if (auto* np = dynamic_cast<NonOverlapLocalPipeline*>(p)) {
+    if (!std::strcmp(name, "hidden")) t = np->keepToken.input;
+    else if (!std::strcmp(name, "logits")) t = np->maxSampler.d_matrix;
+  }
+  if (!t.ptr) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_debug_buffer: unknown buffer \"%s\"", name);
+  *ptr = t.ptr;
+  *rows = (int)t.dim1;
+  *cols = (int)t.dim2;
+  return NF_PLLM_OK;
+}
+
+}  // extern "C"

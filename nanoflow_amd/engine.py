@@ -1,0 +1,212 @@
+"""Harness around the pipeline control plane: builds the config file, device-resident
+weights / KV pools / tmp buffer, and turns a synthetic batch into update data.
+
+Plays the part of the reference's Python glue (pipeline/utils/pybindUtil.py:63-112
+``genInitData`` / ``load_pipeline_config`` / ``initUpdateData`` and the set-up half of
+pipeline/utils/serve_8B.py:124-146).  torch is used only to own device memory.
+"""
+from __future__ import annotations
+
+import json
+import os
+import tempfile
+
+import numpy as np
+import torch
+
+from . import pllm_python as P
+from . import synth
+
+# Tags are accepted for interface parity; tiling is chosen by the kernel layer.
+DEFAULT_TAG = "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor"
+
+
+def write_config(path, shape: synth.ModelShape, *, global_batch, nano1, kqv1, kqv3, pipeline_type,
+                 kv_pages, run_layer=None, distinct_layers=None, max_batch=None, n_tags=7):
+    """Writes a pipeline JSON in the reference's schema (pipeline/config_all/llama3-8B/1024.json)."""
+    layers = shape.layers if distinct_layers is None else distinct_layers
+    cfg = {
+        "model": {
+            "hidden_size": shape.hidden, "intermediate_size": shape.ffn,
+            "num_attention_heads": shape.Hq, "num_key_value_heads": shape.Hkv,
+            "num_hidden_layers": layers, "rms_norm_eps": shape.eps, "rope_theta": shape.rope_theta,
+            "rope_scaling": None, "vocab_size": shape.vocab,
+        },
+        "model_configs": {
+            "gpu_num": 1, "run_layer": shape.layers if run_layer is None else run_layer,
+            "allocate_kv_data_batch": (kv_pages + 63) // 64, "frame_page_size": shape.page_size,
+            "max_batch_size": global_batch if max_batch is None else max_batch,
+        },
+        "pipeline_configs": {
+            "gemm_op_tag": [DEFAULT_TAG] * n_tags, "global_batch_size": global_batch,
+            "nanobatch_1_size": nano1, "kqv1_size": kqv1, "kqv3_size": kqv3,
+        },
+        "serve_configs": {"actual_gpu_num": 1, "pipeline_type": pipeline_type.name},
+    }
+    with open(path, "w") as f:
+        json.dump(cfg, f, indent=1)
+    return cfg
+
+
+def _weight(t: torch.Tensor, N: int, K: int) -> P.VortexWeight:
+    assert t.is_cuda and t.dtype == torch.float16 and t.is_contiguous() and t.numel() == N * K
+    w = P.VortexWeight()
+    w.setPtr(t.data_ptr())
+    w.N, w.K = N, K
+    return w
+
+
+class Engine:
+    """One pipeline on cuda:0.  ``weights`` is a dict of numpy fp16 arrays (see
+    synth.make_weights) or None for N(0, 0.02) weights generated on the device."""
+
+    def __init__(self, shape: synth.ModelShape, pipeline_type=P.PipelineType.LOCAL, *, global_batch,
+                 nano1, kqv1=None, kqv3=None, kv_pages, weights=None, kv_pools=None, run_layer=None,
+                 distinct_layers=None, seed=0, profiling=False, kv_fill="randn"):
+        self.shape = shape
+        self.pipeline_type = pipeline_type
+        self.T = global_batch
+        self.nano1 = nano1
+        self.kqv1 = nano1 if kqv1 is None else kqv1
+        self.kqv3 = (global_batch - nano1) if kqv3 is None else kqv3
+        self.layers = shape.layers if distinct_layers is None else distinct_layers
+        self.dev = torch.device("cuda:0")
+        fd, self.cfg_path = tempfile.mkstemp(suffix=".json", prefix="nanoflow_cfg_")
+        os.close(fd)
+        n_tags = 4 if pipeline_type == P.PipelineType.NON_OVERLAP_LOCAL else 7
+        write_config(self.cfg_path, shape, global_batch=global_batch, nano1=nano1, kqv1=self.kqv1,
+                     kqv3=self.kqv3, pipeline_type=pipeline_type, kv_pages=kv_pages,
+                     run_layer=run_layer, distinct_layers=distinct_layers, n_tags=n_tags)
+        P.setRank(1, 1)
+        P.setModelConfig(self.cfg_path)
+        self.max_pages = P.maxPageNum()
+        gen = torch.Generator(device=self.dev).manual_seed(seed)
+        H, V, F, d = shape.hidden, shape.vocab, shape.ffn, shape.d
+        kqv_n = shape.kqv_n
+
+        def mk(key, layer, rows, cols, std=0.02, mean=0.0):
+            if weights is not None:
+                a = weights[key] if layer is None else weights[key][layer]
+                return torch.from_numpy(np.ascontiguousarray(a)).to(self.dev)
+            t = torch.empty((rows, cols), dtype=torch.float16, device=self.dev)
+            t.normal_(mean, std, generator=gen)
+            return t
+
+        self.t = {"embedding": mk("embedding", None, V, H), "lm_head": mk("lm_head", None, H, V),
+                  "model_norm": mk("model_norm", None, 1, H, 0.02, 1.0), "layers": []}
+        mw = P.VortexModelWeight()
+        mw.lm_head = _weight(self.t["lm_head"], H, V)
+        mw.embedding = _weight(self.t["embedding"], V, H)
+        mw.model_layernorm = _weight(self.t["model_norm"], H, 1)
+        for l in range(self.layers):
+            lt = {"w_kqv": mk("w_kqv", l, H, kqv_n), "w_o": mk("w_o", l, shape.Hq * d, H),
+                  "w_gate": mk("w_gate", l, H, F), "w_up": mk("w_up", l, H, F),
+                  "w_down": mk("w_down", l, F, H), "ln_attn": mk("ln_attn", l, 1, H, 0.02, 1.0),
+                  "ln_ffn": mk("ln_ffn", l, 1, H, 0.02, 1.0)}
+            self.t["layers"].append(lt)
+            lw = P.VortexLayerWeight()
+            lw.W_O1 = _weight(lt["w_o"], H, shape.Hq * d)
+            lw.W_O2 = _weight(lt["w_o"], H, shape.Hq * d)
+            lw.W_U = _weight(lt["w_up"], F, H)
+            lw.W_G = _weight(lt["w_gate"], F, H)
+            lw.W_D = _weight(lt["w_down"], H, F)
+            lw.W_KQV = _weight(lt["w_kqv"], kqv_n, H)
+            lw.W_LN_Attention = _weight(lt["ln_attn"], H, 1)
+            lw.W_LN_FFN = _weight(lt["ln_ffn"], H, 1)
+            mw.layer_weight.append(lw)
+        # KV pools [pages, 2, page, Hkv, d] per distinct layer
+        self.kv = []
+        for l in range(self.layers):
+            if kv_pools is not None:
+                pool = torch.zeros((self.max_pages, 2, shape.page_size, shape.Hkv, d),
+                                   dtype=torch.float16, device=self.dev)
+                src = torch.from_numpy(np.ascontiguousarray(kv_pools[l])).to(self.dev)
+                pool[:src.shape[0]] = src
+            else:
+                pool = torch.empty((self.max_pages, 2, shape.page_size, shape.Hkv, d),
+                                   dtype=torch.float16, device=self.dev)
+                if kv_fill == "randn":
+                    pool.normal_(0.0, 1.0, generator=gen)
+                else:
+                    pool.zero_()
+            self.kv.append(pool)
+        self.tmp = torch.empty((P.tmpBufferHalves(),), dtype=torch.float16, device=self.dev)
+        init = P.VortexInitData()
+        init.setKVdata([p.data_ptr() for p in self.kv])
+        init.setWeight(mw, H * H * 3)
+        init.setTmpBuffer(self.tmp.data_ptr(), self.tmp.numel())
+        torch.cuda.synchronize()
+        if profiling:
+            P.setProfiling(True)
+        P.init([init], pipeline_type)
+        cfg = P.VortexConfigData()
+        cfg.setGemmOpTag([DEFAULT_TAG] * n_tags)
+        cfg.globalBatchSize, cfg.nanobatch1Size = global_batch, nano1
+        cfg.kqv1Size, cfg.kqv3Size = self.kqv1, self.kqv3
+        P.config([cfg])
+        self._open = True
+        self._hold = None
+
+    # ------------------------------------------------------------------ per iteration
+    def update(self, b: synth.Batch, keep_token_list=None, num_blocks=(0, 0, 0, 0)):
+        """Stages one iteration.  keep_token_list marks, per slot of the PREVIOUS iteration's
+        output, the requests that decode again (default: all of them, first iteration: the
+        decode rows are fed token id 1 by the control plane)."""
+        nd = b.decodePrefillBorder
+        keep = np.ones(nd, np.int32) if keep_token_list is None else \
+            np.ascontiguousarray(keep_token_list, dtype=np.int32)
+        arrs = {
+            "prefill_tokens": np.ascontiguousarray(b.input_tokens[nd:], dtype=np.int32),
+            "input_indptr": b.input_indptr, "rev": b.rev_input_indptr, "off": b.per_token_offset,
+            "kv_indptr": b.kv_indptr, "kv_indices": b.kv_indices, "kv_last": b.kv_last_page_len,
+            "keep": keep,
+        }
+        arrs = {k: np.ascontiguousarray(v, dtype=np.int32) for k, v in arrs.items()}
+        u = P.VortexUpdateData()
+        u.decodePrefillBorder, u.prefillNum = nd, b.prefillNum
+        u.prefillTokensNum, u.keepTokenListLength = b.prefillTokensNum, len(keep)
+        u.setInputEmbedding(arrs["prefill_tokens"].ctypes.data)
+        u.setInputIndptr(arrs["input_indptr"].ctypes.data)
+        u.setRevInputIndptr(arrs["rev"].ctypes.data)
+        u.setPerTokenOffset(arrs["off"].ctypes.data)
+        u.setKVIndptr(arrs["kv_indptr"].ctypes.data)
+        u.setKVIndices(arrs["kv_indices"].ctypes.data)
+        u.setKVLastPageLen(arrs["kv_last"].ctypes.data)
+        u.setKeepTokenList(arrs["keep"].ctypes.data)
+        u.setGemvBatchSize(synth.gemv_batch_split(nd, self.kqv1, self.nano1, self.kqv3)
+                           if self.pipeline_type != P.PipelineType.NON_OVERLAP_LOCAL else [nd, 0, 0, 0])
+        u.setGemvNumBlocks(list(num_blocks))
+        self._hold = (arrs, u)
+        P.update([u])
+
+    def run(self) -> np.ndarray:
+        P.run()
+        return P.getPipelineOutput()
+
+    def buffer(self, name: str) -> torch.Tensor:
+        """Copy of an intermediate ("hidden" or "logits") as a torch tensor."""
+        ptr, rows, cols = P.debugBuffer(name)
+        out = torch.empty((rows, cols), dtype=torch.float16, device=self.dev)
+        torch.cuda.synchronize()
+        import ctypes as C
+        hip = C.CDLL("libamdhip64.so")
+        rc = hip.hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(ptr), C.c_size_t(rows * cols * 2),
+                           C.c_int(3))  # hipMemcpyDeviceToDevice
+        if rc != 0:
+            raise RuntimeError(f"hipMemcpy failed: {rc}")
+        return out
+
+    def close(self):
+        if self._open:
+            P.finalize()
+            self._open = False
+            try:
+                os.unlink(self.cfg_path)
+            except OSError:
+                pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()

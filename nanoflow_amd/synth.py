@@ -44,10 +44,12 @@ LLAMA3_8B = ModelShape()
 LLAMA3_70B = ModelShape(hidden=8192, Hq=64, Hkv=8, d=128, ffn=28672, vocab=128256, layers=80)
 
 
-def tiny_shape(layers: int = 2, vocab: int = 1024, hidden: int = 256, Hq: int = 8, Hkv: int = 2,
-               ffn: int = 512) -> ModelShape:
-    """Small shape with the real head_dim/page_size, for end-to-end parity checks."""
-    return ModelShape(hidden=hidden, Hq=Hq, Hkv=Hkv, d=128, ffn=ffn, vocab=vocab, layers=layers)
+def tiny_shape(layers: int = 2, vocab: int = 1024, Hq: int = 8, Hkv: int = 2, ffn: int = 512,
+               hidden: int | None = None) -> ModelShape:
+    """Small shape with the real head_dim/page_size, for end-to-end parity checks.  The
+    pipeline derives head_dim as hidden / Hq (as the reference does), so hidden = Hq * 128."""
+    return ModelShape(hidden=Hq * 128 if hidden is None else hidden, Hq=Hq, Hkv=Hkv, d=128, ffn=ffn,
+                      vocab=vocab, layers=layers)
 
 
 def normal_f16(rng: np.random.Generator, shape, std: float = 1.0, mean: float = 0.0) -> np.ndarray:

@@ -467,7 +467,7 @@ def _numpy_decoder_f64(shape, w, pools, b):
 
 
 def test_decoder_forward_vs_independent_float64_model(oracle):
-    shape = synth.tiny_shape(layers=2, vocab=512, hidden=256, Hq=4, Hkv=2, ffn=384)
+    shape = synth.tiny_shape(layers=2, vocab=512, Hq=4, Hkv=2, ffn=384, hidden=256)
     # larger-than-init weights so the residual stream is not dominated by the embedding
     w = synth.make_weights(shape, seed=0)
     for k in ("w_kqv", "w_o", "w_gate", "w_up", "w_down"):
