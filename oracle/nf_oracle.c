@@ -101,6 +101,18 @@ static inline uint16_t f2h(float f) {
 #endif
 }
 
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+/* Threads the parallel loops below will use. */
+NFO_API int nfo_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
 NFO_API float nfo_half_to_float(uint16_t h) { return h2f(h); }
 NFO_API uint16_t nfo_float_to_half(float f) { return f2h(f); }
 

@@ -81,6 +81,7 @@ class NfoBatch(C.Structure):
 
 
 def _declare(l):
+    l.nfo_num_threads.restype = C.c_int
     l.nfo_half_to_float.restype = C.c_float
     l.nfo_half_to_float.argtypes = [C.c_uint16]
     l.nfo_float_to_half.restype = C.c_uint16
@@ -123,6 +124,10 @@ def _declare(l):
 
 
 # ------------------------------------------------------------------ operators
+
+
+def num_threads() -> int:
+    return lib().nfo_num_threads()
 
 
 def gemm(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False):
