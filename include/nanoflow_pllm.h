@@ -145,6 +145,65 @@ NF_PLLM_API int pllm_build_input_tokens(const int32_t* prev_output, int prev_cou
                                         const int32_t* prefill_tokens, int prefill_tokens_num,
                                         int32_t* out);
 
+/* ---- CPU batch formation and the asynchronous serving loop ------------------------------
+ * Replaces the Python scheduler that drives pllm_python in the reference:
+ * DistKVPool / DistKVCache / BatchedDistKVCache (pipeline/utils/kv_cache.py:20-135) and
+ * Scheduler.schedule_req / bench_text_gen (pipeline/utils/serve_8B.py:177-569).  The former
+ * owns request queue, worksets and page tables; pllm_sched_form fills a
+ * nf_vortex_update_data whose arrays stay valid until the next form call. */
+typedef struct nf_batch_former nf_batch_former;
+
+/* Scheduler(memory_pool, ..., decode_length, prefill_length) + init_pipe's batch sizes
+ * (serve_8B.py:104-146); kv_pages = DistKVPool capacity (serve_8B.py:643). */
+NF_PLLM_API nf_batch_former* pllm_sched_create(int kv_pages, int page_size, int global_batch_size,
+                                               int nanobatch_1_size, int kqv1_size, int kqv3_size,
+                                               int average_prefill_length,
+                                               int average_decode_length);
+NF_PLLM_API void pllm_sched_destroy(nf_batch_former* f);
+/* NewRequestQueue.put (pipeline/utils/request_info.py:13-31). */
+NF_PLLM_API int pllm_sched_add_request(nf_batch_former* f, int req_idx, const int32_t* prompt,
+                                       int prompt_len, int output_len, double start_time);
+/* schedule_req (serve_8B.py:212-346). */
+NF_PLLM_API int pllm_sched_schedule(nf_batch_former* f);
+/* bench_text_gen up to initUpdateData (serve_8B.py:356-451). */
+NF_PLLM_API int pllm_sched_form(nf_batch_former* f, nf_vortex_update_data* out);
+/* back-fill of the outputs of the iteration that just completed (serve_8B.py:499-520);
+ * n == 0 when none has. */
+NF_PLLM_API int pllm_sched_harvest(nf_batch_former* f, const int32_t* ids, int n);
+/* predict_output (serve_8B.py:523-569): length-only retirement, keep list, next worksets.
+ * placeholder_zero != 0 is the skip-cycle mode.  *n_retired = requests retired by this call. */
+NF_PLLM_API int pllm_sched_advance(nf_batch_former* f, double now, int placeholder_zero,
+                                   int* n_retired);
+/* counts[0..4] = queued requests, decoding requests, prefilling requests, free pages,
+ * retired requests so far. */
+NF_PLLM_API int pllm_sched_state(nf_batch_former* f, int counts[5]);
+/* Copies the outputs of retired request number `which` (retirement order): returns the number
+ * of tokens written (<= cap), *req_idx its id; negative on error. */
+NF_PLLM_API int pllm_sched_retired_output(nf_batch_former* f, int which, int* req_idx, int32_t* out,
+                                          int cap);
+/* check_future_page_usage (serve_8B.py:177-203): out[0..n) pages in use i iterations ahead;
+ * returns the forecast length (average_prefill + average_decode + 2). */
+NF_PLLM_API int pllm_sched_future_page_usage(nf_batch_former* f, int64_t* out, int cap);
+
+/* What the reference prints to its .stat file (serve_8B.py:755-793) plus the CPU-side split
+ * of a cycle. */
+typedef struct nf_serve_stats {
+  int cycles;
+  int retired;
+  double wall_s;
+  double tokens_per_s; /* retired * (average_prefill + average_decode) / wall_s */
+  double cycle_ms;
+  double form_ms;     /* CPU: schedule + form per cycle (overlaps the GPU run) */
+  double wait_ms;     /* blocked in run_async_wait per cycle */
+  double update_ms;   /* update() per cycle */
+  double gpu_iter_ms; /* device time of an iteration */
+  long long tokens_processed;
+} nf_serve_stats;
+/* The serving loop of serve_8B.py:655-700 over an initialised and configured pipeline:
+ * skip_cycles simulated cycles (scheduler only), then run_cycles executed and timed cycles in
+ * which batch i+1 is formed on the CPU while the GPU runs batch i. */
+NF_PLLM_API int pllm_serve(nf_batch_former* f, int skip_cycles, int run_cycles, nf_serve_stats* stats);
+
 /* Measurement (no counterpart in the reference, which only logs the iteration time,
  * pipeline_local.cu:444-463).  With profiling on, every attention launch is bracketed by
  * events on its own stream.  pllm_get_timings returns the last iteration's time and the

@@ -328,3 +328,148 @@ int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols) {
 }
 
 }  // extern "C"
+
+// ---------------------------------------------------------------- batch former / serve loop
+#include "batchFormer.h"
+
+struct nf_batch_former {
+  BatchFormer former;
+  FormedBatch batch;
+  std::vector<FlyPtr> retired;
+  int avg_prefill, avg_decode;
+  nf_batch_former(int pages, int page, int gb, int n1, int k1, int k3, int ap, int ad)
+      : former(pages, page, gb, n1, k1, k3, ap, ad), avg_prefill(ap), avg_decode(ad) {}
+};
+
+extern "C" {
+
+nf_batch_former* pllm_sched_create(int kv_pages, int page_size, int global_batch_size,
+                                   int nanobatch_1_size, int kqv1_size, int kqv3_size,
+                                   int average_prefill_length, int average_decode_length) {
+  if (kv_pages <= 0 || page_size <= 0 || global_batch_size <= 0 || nanobatch_1_size < 0 ||
+      kqv1_size < 0 || kqv1_size > nanobatch_1_size || kqv3_size < 0 || average_prefill_length < 0 ||
+      average_decode_length < 0) {
+    fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_create: bad sizes");
+    return nullptr;
+  }
+  return new nf_batch_former(kv_pages, page_size, global_batch_size, nanobatch_1_size, kqv1_size,
+                             kqv3_size, average_prefill_length, average_decode_length);
+}
+
+void pllm_sched_destroy(nf_batch_former* f) { delete f; }
+
+int pllm_sched_add_request(nf_batch_former* f, int req_idx, const int32_t* prompt, int prompt_len,
+                           int output_len, double start_time) {
+  if (!f || !prompt || prompt_len <= 0 || output_len <= 0)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_add_request: bad request");
+  SchedRequest r;
+  r.req_idx = req_idx;
+  r.prompt.assign(prompt, prompt + prompt_len);
+  r.output_len = output_len;
+  r.start_time = start_time;
+  f->former.add_request(std::move(r));
+  return NF_PLLM_OK;
+}
+
+int pllm_sched_schedule(nf_batch_former* f) {
+  if (!f) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_schedule: null");
+  try {
+    f->former.schedule();
+  } catch (const std::exception& e) {
+    return fail(NF_PLLM_ERR_STATE, "pllm_sched_schedule: %s", e.what());
+  }
+  return NF_PLLM_OK;
+}
+
+int pllm_sched_form(nf_batch_former* f, nf_vortex_update_data* out) {
+  if (!f || !out) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_form: null");
+  try {
+    f->former.form(f->batch);
+  } catch (const std::exception& e) {
+    return fail(NF_PLLM_ERR_STATE, "pllm_sched_form: %s", e.what());
+  }
+  FormedBatch& b = f->batch;
+  out->decodePrefillBorder = b.decodePrefillBorder;
+  out->prefillNum = b.prefillNum;
+  out->prefillTokensNum = b.prefillTokensNum;
+  out->keepTokenListLength = b.keepTokenListLength;
+  out->input_tokens = b.input_tokens.data();
+  out->input_indptr = b.input_indptr.data();
+  out->rev_input_indptr = b.rev_input_indptr.data();
+  out->keep_token_list = b.keep_token_list.data();
+  out->kv_indptr = b.kv_indptr.data();
+  out->kv_indices = b.kv_indices.data();
+  out->kv_last_page_len = b.kv_last_page_len.data();
+  out->per_token_offset = b.per_token_offset.data();
+  out->gemv_batch_size = b.gemv_batch_size;
+  out->gemv_num_blocks = b.gemv_num_blocks;
+  return NF_PLLM_OK;
+}
+
+int pllm_sched_harvest(nf_batch_former* f, const int32_t* ids, int n) {
+  if (!f || (n > 0 && !ids)) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_harvest: null");
+  f->former.harvest(ids, n);
+  return NF_PLLM_OK;
+}
+
+int pllm_sched_advance(nf_batch_former* f, double now, int placeholder_zero, int* n_retired) {
+  if (!f) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_advance: null");
+  const size_t before = f->retired.size();
+  f->former.advance(now, f->retired, placeholder_zero != 0);
+  if (n_retired) *n_retired = (int)(f->retired.size() - before);
+  return NF_PLLM_OK;
+}
+
+int pllm_sched_state(nf_batch_former* f, int counts[5]) {
+  if (!f || !counts) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_state: null");
+  counts[0] = (int)f->former.queued();
+  counts[1] = (int)f->former.decoding();
+  counts[2] = (int)f->former.prefilling();
+  counts[3] = f->former.pool().num_free_pages();
+  counts[4] = (int)f->retired.size();
+  return NF_PLLM_OK;
+}
+
+int pllm_sched_retired_output(nf_batch_former* f, int which, int* req_idx, int32_t* out, int cap) {
+  if (!f || which < 0 || which >= (int)f->retired.size() || (cap > 0 && !out))
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_retired_output: bad index %d", which);
+  const FlyRequest& r = *f->retired[which];
+  if (req_idx) *req_idx = r.req_idx;
+  const int n = std::min<int>(cap, (int)r.output.size());
+  for (int i = 0; i < n; ++i) out[i] = r.output[i];
+  return n;
+}
+
+int pllm_sched_future_page_usage(nf_batch_former* f, int64_t* out, int cap) {
+  if (!f || (cap > 0 && !out)) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_future_page_usage: null");
+  std::vector<long long> u = f->former.future_page_usage();
+  for (int i = 0; i < cap && i < (int)u.size(); ++i) out[i] = u[i];
+  return (int)u.size();
+}
+
+int pllm_serve(nf_batch_former* f, int skip_cycles, int run_cycles, nf_serve_stats* stats) {
+  if (!f || !stats) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_serve: null");
+  if (!g_configured) return fail(NF_PLLM_ERR_STATE, "pllm_serve: call pllm_init and pllm_config first");
+  if (g_running) return fail(NF_PLLM_ERR_STATE, "pllm_serve: a run is in flight");
+  ServeStats s;
+  try {
+    s = serveLoop(f->former, skip_cycles, run_cycles, &f->retired);
+  } catch (const std::exception& e) {
+    g_updated = false;
+    return fail(NF_PLLM_ERR_STATE, "pllm_serve: %s", e.what());
+  }
+  stats->cycles = s.cycles;
+  stats->retired = s.retired;
+  stats->wall_s = s.wall_s;
+  stats->tokens_per_s = s.wall_s > 0 ? s.retired * double(f->avg_prefill + f->avg_decode) / s.wall_s : 0;
+  stats->cycle_ms = s.cycle_ms;
+  stats->form_ms = s.form_ms;
+  stats->wait_ms = s.wait_ms;
+  stats->update_ms = s.update_ms;
+  stats->gpu_iter_ms = s.gpu_iter_ms;
+  stats->tokens_processed = s.tokens_processed;
+  g_updated = false;
+  return NF_PLLM_OK;
+}
+
+}  // extern "C"

@@ -14,11 +14,16 @@
 // Online softmax runs in the exp2 domain with fp32 state per column; masked keys contribute
 // exactly zero (the reference's -5e4 mask underflows to zero in fp32 as well).
 //
+// The key loop is software-pipelined on the operand registers themselves: the K loads of step
+// i+1 are issued as soon as the score MFMAs of step i have consumed K, the V loads of step
+// i+1 as soon as the transposes of step i have consumed V, and the page ids of step i+1 are
+// fetched (scalar) at the top of step i -- every wavefront keeps a K and a V tile in flight.
+//
 // Decode mode: a workgroup's 4 wavefronts split the request's pages (32 keys per step each)
-// and merge (m, l, O) through LDS.  Prefill mode: each wavefront owns its own query tile.
-// Work items are (tile, kv head) with the head fastest, so concurrently running workgroups
-// stream the same pages.  Tiles are planned on the device from qo_indptr (prefix of tiles per
-// request), no host round trip.
+// and merge (m, l, O) through LDS; work item = (request, kv head), head fastest, so that
+// concurrently running workgroups stream the same 64 KiB pages.  Prefill mode: each wavefront
+// owns its own query tile; tiles are planned on the device from qo_indptr (prefix of tiles per
+// request) -- no host round trip in either mode.
 #include "common.h"
 
 namespace nf {
@@ -39,6 +44,18 @@ union H8 {
   uint32_t w[4];
 };
 
+// KV pages are read exactly once per launch: load them with the non-temporal hint so the
+// stream does not displace the working set of kernels running beside this one.
+typedef uint32_t nt_vec4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4 load_stream16(const uint16_t* p) {
+#ifdef NF_ATTN_TEMPORAL_LOADS
+  return *reinterpret_cast<const u32x4*>(p);
+#else
+  nt_vec4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_vec4*>(p));
+  return u32x4{v.x, v.y, v.z, v.w};
+#endif
+}
+
 // tile_start[i] = number of tiles of requests < i; tile_start[batch] = total.
 __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restrict__ qo_indptr,
                                                         int32_t* __restrict__ tile_start, int batch,
@@ -53,17 +70,15 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restric
   }
   s_sum[threadIdx.x] = sum;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int t = 0; t < 256; ++t) {
-      int v = s_sum[t];
-      s_sum[t] = run;
-      run += v;
-    }
-    tile_start[batch] = run;
+  // inclusive scan over the 256 partial sums (Hillis-Steele)
+  for (int off = 1; off < 256; off <<= 1) {
+    int v = threadIdx.x >= off ? s_sum[threadIdx.x - off] : 0;
+    __syncthreads();
+    s_sum[threadIdx.x] += v;
+    __syncthreads();
   }
-  __syncthreads();
-  int run = s_sum[threadIdx.x];
+  int run = s_sum[threadIdx.x] - sum;  // exclusive prefix of this thread's range
+  if (threadIdx.x == 255) tile_start[batch] = s_sum[255];
   for (int i = lo; i < hi; ++i) {
     tile_start[i] = run;
     int len = qo_indptr[i + 1] - qo_indptr[i];
@@ -71,8 +86,10 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restric
   }
 }
 
+// SPLIT (decode mode): one tile per request (tile index == request index, no plan needed),
+// the 4 wavefronts split the KV range.  !SPLIT (prefill mode): tiles from tile_start.
 template <int GROUP, int NQB, bool SPLIT>
-__global__ __launch_bounds__(256) void attn_paged_kernel(
+__global__ __launch_bounds__(256, SPLIT ? 2 : 1) void attn_paged_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ o, const int32_t* __restrict__ qo_indptr,
     const uint16_t* __restrict__ kv_data, const int32_t* __restrict__ kv_indptr,
     const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_last_page_len,
@@ -87,27 +104,39 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(
   __shared__ float s_m[SPLIT ? 4 * 64 : 1];
   __shared__ float s_l[SPLIT ? 4 * 64 : 1];
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform by construction
   const int c16 = lane & 15, g = lane >> 4;
-  const int total_tiles = tile_start[batch];
+  const int total_tiles = SPLIT ? batch : tile_start[batch];
   const size_t page_halves = (size_t)2 * PAGE * Hkv * D;
   const size_t v_off = (size_t)PAGE * Hkv * D;
 
   for (long long w = blockIdx.x; w < (long long)total_tiles * Hkv; w += gridDim.x) {
     const int tile = (int)(w / Hkv), kvh = (int)(w % Hkv);
-    // request = largest i with tile_start[i] <= tile
-    int lo = 0, hi = batch;
-    while (hi - lo > 1) {
-      int mid = (lo + hi) >> 1;
-      if (tile_start[mid] <= tile) lo = mid; else hi = mid;
+    int req, tile_in_req0;
+    if constexpr (SPLIT) {
+      req = tile;
+      tile_in_req0 = 0;
+    } else {
+      // request = largest i with tile_start[i] <= tile
+      int lo = 0, hi = batch;
+      while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (tile_start[mid] <= tile) lo = mid; else hi = mid;
+      }
+      req = lo;
+      tile_in_req0 = tile - tile_start[req];
     }
-    const int req = lo;
     const int qo0 = qo_indptr[req];
     const int qo_len = qo_indptr[req + 1] - qo0;
     const int pg0 = kv_indptr[req];
     const int npages = kv_indptr[req + 1] - pg0;
     const int kv_len = npages > 0 ? (npages - 1) * PAGE + kv_last_page_len[req] : 0;
-    const int tok0 = (tile - tile_start[req]) * WG_TOK + (SPLIT ? 0 : wave * WAVE_TOK);
+    // decode mode walks all row blocks of its request itself (one block when qo_len == 1)
+    const int n_sub = SPLIT ? (qo_len + WG_TOK - 1) / WG_TOK : 1;
+    for (int sub = 0; sub < n_sub; ++sub) {
+    const int tile_in_req = tile_in_req0 + sub;
+    const int tok0 = tile_in_req * WG_TOK + (SPLIT ? 0 : wave * WAVE_TOK);
     const bool wave_active = tok0 < qo_len;
 
     float4_t oacc[NQB][8];
@@ -139,28 +168,69 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(
       const int tok_last = min(tok0 + WAVE_TOK, qo_len) - 1;
       const int kv_end = causal ? min(kv_len, kv_len - qo_len + tok_last + 1) : kv_len;
       const int npairs = (kv_end + 31) >> 5;
+      constexpr int PSTEP = SPLIT ? 4 : 1;
+      const int pp0 = SPLIT ? wave : 0;
 
-      for (int pp = SPLIT ? wave : 0; pp < npairs; pp += SPLIT ? 4 : 1) {
-        const int t_base = pp * 32;
-        H8 kf[2][4], vf[2][4];
+      // lane's offsets inside a page: K row c16 (16 B at feature g*8 + 32j), V rows 4g+r
+      const size_t k_lane = ((size_t)c16 * Hkv + kvh) * D + g * 8;
+      const size_t v_lane = v_off + ((size_t)(g * 4) * Hkv + kvh) * D + c16 * 8;
+      const size_t v_row = (size_t)Hkv * D;
+
+      H8 kf[2][4], vf[2][4];
+      auto page_of = [&](int pidx) -> int {   // uniform: becomes a scalar load
+        return kv_indices[pg0 + (pidx < npages ? pidx : 0)];
+      };
+      auto load_k = [&](int page_a, int page_b) {
+        const uint16_t* ka = kv_data + (size_t)page_a * page_halves + k_lane;
+        const uint16_t* kb = kv_data + (size_t)page_b * page_halves + k_lane;
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-          const int pidx = 2 * pp + blk;
-          const bool page_ok = pidx < npages;
-          const int page = kv_indices[pg0 + (page_ok ? pidx : 0)];
-          const uint16_t* kp = kv_data + (size_t)page * page_halves;
-          const uint16_t* krow = kp + ((size_t)c16 * Hkv + kvh) * D + g * 8;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) kf[blk][j].u = *reinterpret_cast<const u32x4*>(krow + j * 32);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int t = t_base + blk * 16 + g * 4 + r;
-            const uint16_t* vrow = kp + v_off + ((size_t)(g * 4 + r) * Hkv + kvh) * D + c16 * 8;
-            // entries past kv_len may hold anything (NaN x 0 = NaN): feed zeros instead
-            vf[blk][r].u = (t < kv_len) ? *reinterpret_cast<const u32x4*>(vrow) : u32x4{0, 0, 0, 0};
-          }
+        for (int j = 0; j < 4; ++j) {
+          kf[0][j].u = load_stream16(ka + j * 32);
+          kf[1][j].u = load_stream16(kb + j * 32);
         }
-        // V^T operands: vt[i] = {V[tok a0..a3][d], V[tok b0..b3][d]} with d = c16*8 + i
+      };
+      auto load_v = [&](int page_a, int page_b, int t_base) {
+        const uint16_t* va = kv_data + (size_t)page_a * page_halves + v_lane;
+        const uint16_t* vb = kv_data + (size_t)page_b * page_halves + v_lane;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          // entries past kv_len may hold anything (NaN x 0 = NaN): feed zeros instead
+          const int t = t_base + g * 4 + r;
+          vf[0][r].u = (t < kv_len) ? load_stream16(va + r * v_row) : u32x4{0, 0, 0, 0};
+          vf[1][r].u = (t + 16 < kv_len) ? load_stream16(vb + r * v_row) : u32x4{0, 0, 0, 0};
+        }
+      };
+
+      int page_a = 0, page_b = 0;
+      if (pp0 < npairs) {
+        page_a = page_of(2 * pp0);
+        page_b = page_of(2 * pp0 + 1);
+        load_k(page_a, page_b);
+        load_v(page_a, page_b, pp0 * 32);
+      }
+      for (int pp = pp0; pp < npairs; pp += PSTEP) {
+        const int t_base = pp * 32;
+        const int pn = pp + PSTEP;
+        const bool have_next = pn < npairs;
+        int next_a = 0, next_b = 0;
+        if (have_next) {
+          next_a = page_of(2 * pn);
+          next_b = page_of(2 * pn + 1);
+        }
+        // ---- scores for every column block, then K is free
+        float4_t s[NQB][2];
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk) {
+            s[nb][blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              s[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[blk][j].h, qf[nb][j].h, s[nb][blk], 0, 0, 0);
+          }
+        if (have_next) load_k(next_a, next_b);
+
+        // ---- V^T operands: vt[i] = {V[tok a0..a3][d], V[tok b0..b3][d]} with d = c16*8 + i
         H8 vt[8];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -171,16 +241,11 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(
           vt[2 * k].u = u32x4{pk_lo(a0, a1), pk_lo(a2, a3), pk_lo(b0, b1), pk_lo(b2, b3)};
           vt[2 * k + 1].u = u32x4{pk_hi(a0, a1), pk_hi(a2, a3), pk_hi(b0, b1), pk_hi(b2, b3)};
         }
+        if (have_next) load_v(next_a, next_b, pn * 32);
+
+        // ---- online softmax + P.V per column block
 #pragma unroll
         for (int nb = 0; nb < NQB; ++nb) {
-          float4_t s[2];
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk) {
-            s[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              s[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[blk][j].h, qf[nb][j].h, s[blk], 0, 0, 0);
-          }
           // lane holds keys t_base + blk*16 + g*4 + r of column c16
           float mx = -1e30f;
           bool ok[2][4];
@@ -190,8 +255,8 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(
             for (int r = 0; r < 4; ++r) {
               const int t = t_base + blk * 16 + g * 4 + r;
               ok[blk][r] = t <= key_limit[nb] && t < kv_len;
-              s[blk][r] *= scale_log2;
-              if (ok[blk][r]) mx = fmaxf(mx, s[blk][r]);
+              s[nb][blk][r] *= scale_log2;
+              if (ok[blk][r]) mx = fmaxf(mx, s[nb][blk][r]);
             }
           mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
           mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -205,9 +270,9 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(
           for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
             for (int rr = 0; rr < 2; ++rr) {
-              float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[blk][2 * rr] - m_new) : 0.f;
-              float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[blk][2 * rr + 1] - m_new) : 0.f;
-              // the reference rounds P to fp16 before P.V and sums the unrounded values
+              float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr] - m_new) : 0.f;
+              float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr + 1] - m_new) : 0.f;
+              // P is rounded to fp16 for P.V; the row sum uses the unrounded values
               psum += p0 + p1;
               pw[blk * 2 + rr] = f2h_bits(p0) | (f2h_bits(p1) << 16);
             }
@@ -238,8 +303,7 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(
       s_m[wave * 64 + lane] = m_run[0];
       s_l[wave * 64 + lane] = l_run[0];
       __syncthreads();
-      const int tq = c16 / GROUP;  // tok0 == tile token base in split mode
-      const int tok = (tile - tile_start[req]) * WG_TOK + tq;
+      const int tok = tok0 + c16 / GROUP;
       float M = -1e30f;
 #pragma unroll
       for (int ww = 0; ww < 4; ++ww) M = fmaxf(M, s_m[ww * 64 + lane]);
@@ -286,6 +350,7 @@ __global__ __launch_bounds__(256) void attn_paged_kernel(
         }
       }
     }
+    }  // sub
   }
 }
 
@@ -297,11 +362,18 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
                        hipStream_t stream) {
   const float scale_log2 = 1.4426950408889634f / sqrtf((float)D);
   constexpr int TPB = 16 / GROUP;
+  // Decode mode (KV split over the wavefronts, one workgroup per request and kv head) is the
+  // right shape when requests carry about one row each; it stays correct for any row count.
   const bool decode_mode = max_qo_rows <= batch;
   constexpr int NQB_PREFILL = 4;
-  const int wg_tok = decode_mode ? TPB : 4 * NQB_PREFILL * TPB;
-  attn_plan_kernel<<<1, 256, 0, stream>>>(qo_indptr, tile_start, batch, wg_tok);
-  long long bound = ((long long)batch + max_qo_rows / wg_tok) * Hkv;
+  long long bound;
+  if (decode_mode) {
+    bound = (long long)batch * Hkv;
+  } else {
+    const int wg_tok = 4 * NQB_PREFILL * TPB;
+    attn_plan_kernel<<<1, 256, 0, stream>>>(qo_indptr, tile_start, batch, wg_tok);
+    bound = ((long long)batch + max_qo_rows / wg_tok) * Hkv;
+  }
   if (num_blocks > 0 && bound > num_blocks) bound = num_blocks;
   if (bound > 0x7fffffffLL) bound = 0x7fffffffLL;
   if (bound < 1) bound = 1;

@@ -43,6 +43,18 @@ __device__ __forceinline__ uint32_t pack_hi(uint32_t x, uint32_t y) {
   return __builtin_amdgcn_perm(y, x, 0x07060302u);  // {x.hi, y.hi}
 }
 
+// Raw buffer loads: an offset at or past the descriptor's byte count reads as zero, so tile
+// edges need no branches -- out-of-range chunks just get the kOob offset.
+constexpr uint32_t kOob = 0xFFFFFFF0u;
+typedef uint32_t bufvec4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)(uint32_t)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+  bufvec4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
+  return u32x4{v.x, v.y, v.z, v.w};
+}
+
 // SiLU(g)*u on values already rounded to fp16, as the reference's dual epilogue computes it.
 __device__ __forceinline__ float swiglu_rounded(float g_acc, float u_acc) {
   float g = __half2float(__float2half_rn(g_acc));
@@ -92,74 +104,88 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[b][i][j][r] = 0.f;
 
+  // ---- staging registers: one slab's worth of this thread's global chunks
+  constexpr int B_UNITS = kBCol ? BC_CHUNKS : B_BLOCKS;  // per weight matrix
+  constexpr int B_LOADS = kBCol ? 1 : 4;                  // 16-byte loads per B unit
   u32x4 a_reg[A_CHUNKS];
-  u32x4 b_reg[NB][kBCol ? BC_CHUNKS : B_BLOCKS * 4];
+  u32x4 b_reg[NB][B_UNITS * B_LOADS];
 
-  auto load_global = [&](int k0) {
+  // Per-thread byte offsets of the chunks it stages, at k0 = 0 (kOob when the row / column is
+  // outside the matrix); the slab offset is added per iteration.
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K * 2);
+  __amdgpu_buffer_rsrc_t b_rsrc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) b_rsrc[b] = make_rsrc(b ? B1 : B0, (size_t)N * K * 2);
+  uint32_t a_off[A_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < A_CHUNKS; ++i) {
+    const int id = tid + 256 * i;
+    const int gm = m_base + (id >> 3);
+    a_off[i] = gm < M ? ((uint32_t)gm * (uint32_t)K + (id & 7) * 8) * 2u : kOob;
+  }
+  uint32_t b_off[B_UNITS];
+#pragma unroll
+  for (int i = 0; i < B_UNITS; ++i) {
+    const int id = tid + 256 * i;
+    if constexpr (kBCol) {
+      const int gn = n_base + (id >> 3);
+      b_off[i] = gn < N ? ((uint32_t)gn * (uint32_t)K + (id & 7) * 8) * 2u : kOob;
+    } else {
+      const int gn = n_base + (id % (BN / 8)) * 8;
+      b_off[i] = gn < N ? ((uint32_t)(id / (BN / 8)) * 4u * (uint32_t)N + gn) * 2u : kOob;
+    }
+  }
+
+  // The staging work of a slab is cut into 3 parts (quarter q of the MFMA loop handles the
+  // A chunks with i % 3 == q and the B units with (2 - u % 3) == q); part < 0 = everything.
+  auto load_part = [&](int k0, int part) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-      const int id = tid + 256 * i;
-      const int row = id >> 3, kc = id & 7;
-      const int gm = m_base + row, gk = k0 + kc * 8;
-      a_reg[i] = (gm < M && gk < K)
-                     ? *reinterpret_cast<const u32x4*>(A + (size_t)gm * K + gk)
-                     : u32x4{0, 0, 0, 0};
+      if (part >= 0 && i % 3 != part) continue;
+      const bool ok = a_off[i] != kOob && k0 + ((tid + 256 * i) & 7) * 8 < K;
+      a_reg[i] = buf_load16(a_rsrc, ok ? a_off[i] + (uint32_t)k0 * 2u : kOob);
     }
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      const uint16_t* Bp = b ? B1 : B0;
-      if constexpr (kBCol) {
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int i = 0; i < BC_CHUNKS; ++i) {
-          const int id = tid + 256 * i;
-          const int n = id >> 3, kc = id & 7;
-          const int gn = n_base + n, gk = k0 + kc * 8;
-          b_reg[b][i] = (gn < N && gk < K)
-                            ? *reinterpret_cast<const u32x4*>(Bp + (size_t)gn * K + gk)
-                            : u32x4{0, 0, 0, 0};
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < B_BLOCKS; ++i) {
-          const int id = tid + 256 * i;
-          const int nb = id % (BN / 8), kq = id / (BN / 8);
-          const int gn = n_base + nb * 8;
+      for (int i = 0; i < B_UNITS; ++i) {
+        if (part >= 0 && 2 - (b * B_UNITS + i) % 3 != part) continue;
+        if constexpr (kBCol) {
+          const bool ok = b_off[i] != kOob && k0 + ((tid + 256 * i) & 7) * 8 < K;
+          b_reg[b][i] = buf_load16(b_rsrc[b], ok ? b_off[i] + (uint32_t)k0 * 2u : kOob);
+        } else {
+          const int kq = (tid + 256 * i) / (BN / 8);
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int gk = k0 + kq * 4 + r;
-            b_reg[b][i * 4 + r] = (gn < N && gk < K)
-                                      ? *reinterpret_cast<const u32x4*>(Bp + (size_t)gk * N + gn)
-                                      : u32x4{0, 0, 0, 0};
+            const bool ok = b_off[i] != kOob && k0 + kq * 4 + r < K;
+            b_reg[b][i * 4 + r] =
+                buf_load16(b_rsrc[b], ok ? b_off[i] + ((uint32_t)(k0 + r) * (uint32_t)N) * 2u : kOob);
           }
         }
       }
-    }
   };
 
-  auto store_lds = [&](int stage) {
+  auto store_part = [&](int stage, int part) {
     uint16_t* As = smem + stage * SM::stage_halves;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
+      if (part >= 0 && i % 3 != part) continue;
       const int id = tid + 256 * i;
-      const int row = id >> 3, kc = id & 7;
-      *reinterpret_cast<u32x4*>(As + row * A_LD + kc * 8) = a_reg[i];
+      *reinterpret_cast<u32x4*>(As + (id >> 3) * A_LD + (id & 7) * 8) = a_reg[i];
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
       uint16_t* Bs = As + SM::a_halves + b * SM::b_halves;
-      if constexpr (kBCol) {
 #pragma unroll
-        for (int i = 0; i < BC_CHUNKS; ++i) {
-          const int id = tid + 256 * i;
+      for (int i = 0; i < B_UNITS; ++i) {
+        if (part >= 0 && 2 - (b * B_UNITS + i) % 3 != part) continue;
+        const int id = tid + 256 * i;
+        if constexpr (kBCol) {
           const int n = id >> 3, kc = id & 7;
           const u32x4 v = b_reg[b][i];
           *reinterpret_cast<u32x2*>(Bs + ((2 * kc) * B_LD + n) * 4) = u32x2{v.x, v.y};
           *reinterpret_cast<u32x2*>(Bs + ((2 * kc + 1) * B_LD + n) * 4) = u32x2{v.z, v.w};
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < B_BLOCKS; ++i) {
-          const int id = tid + 256 * i;
+        } else {
           const int nb = id % (BN / 8), kq = id / (BN / 8);
           const u32x4 r0 = b_reg[b][i * 4 + 0], r1 = b_reg[b][i * 4 + 1];
           const u32x4 r2 = b_reg[b][i * 4 + 2], r3 = b_reg[b][i * 4 + 3];
@@ -180,44 +206,71 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
     }
   };
 
-  auto compute = [&](int stage) {
+  // ---- MFMA operand fragments, double-buffered across the 4 k-steps of a slab
+  half8_t af[2][TM];
+  half8_t bf[2][NB][TN];
+  auto read_frags = [&](int stage, int kk, int buf) {
     const uint16_t* As = smem + stage * SM::stage_halves;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      half8_t af[TM];
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm * (BM / WM) + i * 32 + l32;
+      af[buf][i] = *reinterpret_cast<const half8_t*>(As + row * A_LD + kk * 16 + lg * 8);
+    }
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = wm * (BM / WM) + i * 32 + l32;
-        af[i] = *reinterpret_cast<const half8_t*>(As + row * A_LD + kk * 16 + lg * 8);
+    for (int b = 0; b < NB; ++b) {
+      const uint16_t* Bs = As + SM::a_halves + b * SM::b_halves;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = wn * (BN / WN) + j * 32 + l32;
+        const int q = kk * 4 + lg * 2;
+        half4_t lo = *reinterpret_cast<const half4_t*>(Bs + (q * B_LD + n) * 4);
+        half4_t hi = *reinterpret_cast<const half4_t*>(Bs + ((q + 1) * B_LD + n) * 4);
+        bf[buf][b][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
+    }
+  };
+  auto mfma_step = [&](int buf) {
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        const uint16_t* Bs = As + SM::a_halves + b * SM::b_halves;
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const int n = wn * (BN / WN) + j * 32 + l32;
-          const int q = kk * 4 + lg * 2;
-          half4_t lo = *reinterpret_cast<const half4_t*>(Bs + (q * B_LD + n) * 4);
-          half4_t hi = *reinterpret_cast<const half4_t*>(Bs + ((q + 1) * B_LD + n) * 4);
-          half8_t bf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-          for (int i = 0; i < TM; ++i)
-            acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf, af[i], acc[b][i][j], 0, 0, 0);
-        }
+        for (int i = 0; i < TM; ++i)
+          acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[buf][b][j], af[buf][i], acc[b][i][j], 0, 0, 0);
+  };
+
+  // One slab of the steady state.  While the MFMAs of slab s run out of LDS stage s&1:
+  //   quarters 0-2: prefetch the next k-step's fragments; write slab s+1 (already in
+  //                 registers) into the other stage; refill those registers with slab s+2;
+  //   quarter 3:    barrier, then prefetch slab s+1's first fragments under the last MFMAs.
+  auto slab = [&](int s, bool do_store, bool do_load) {
+    const int cur = s & 1;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      if (kk == 3) __syncthreads();
+      if (kk < 3) read_frags(cur, kk + 1, (kk + 1) & 1);
+      else if (do_store) read_frags(cur ^ 1, 0, 0);
+      if (kk < 3) {
+        if (do_store) store_part(cur ^ 1, kk);
+        if (do_load) load_part((s + 2) * BK, kk);
       }
+      mfma_step(kk & 1);
     }
   };
 
   const int nslab = (K + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
+  load_part(0, -1);
+  store_part(0, -1);
+  if (nslab > 1) load_part(BK, -1);
   __syncthreads();
-  for (int s = 0; s < nslab; ++s) {
-    if (s + 1 < nslab) load_global((s + 1) * BK);
-    compute(s & 1);
-    if (s + 1 < nslab) store_lds((s + 1) & 1);
-    __syncthreads();
+  read_frags(0, 0, 0);
+  int s = 0;
+  for (; s + 2 < nslab; ++s) slab(s, true, true);
+  if (s + 1 < nslab) {
+    slab(s, true, false);
+    ++s;
   }
+  slab(s, false, false);
 
   // Epilogue.  acc[.][i][j][r] holds D[m][n] with m = tile row l32 and
   // n = (r/4)*8 + lg*4 + r%4 of the 32x32 tile: 4 consecutive n per register quad.
@@ -302,6 +355,9 @@ static int check_gemm_args(const char* who, const void* A, const void* B, const 
   NF_REQUIRE(M == 0 || (A && B && D), "%s: null pointer", who);
   NF_REQUIRE(((uintptr_t)A | (uintptr_t)B | (uintptr_t)D) % 16 == 0,
              "%s: operands must be 16-byte aligned", who);
+  // operands are addressed through 32-bit buffer offsets
+  NF_REQUIRE((size_t)M * K * 2 < 0xFFFFFF00ull && (size_t)N * K * 2 < 0xFFFFFF00ull,
+             "%s: an operand of %d x %d x %d exceeds the 4 GiB buffer-addressing limit", who, M, N, K);
   return NF_OK;
 }
 

@@ -322,3 +322,123 @@ def debugBuffer(name: str):
     p, r, c = C.c_void_p(), C.c_int(), C.c_int()
     _check(lib().pllm_debug_buffer(name.encode(), C.byref(p), C.byref(r), C.byref(c)), "debugBuffer")
     return p.value, r.value, c.value
+
+
+# ---------------------------------------------------------------- batch former / serve loop
+
+class ServeStats(C.Structure):
+    _fields_ = [("cycles", C.c_int), ("retired", C.c_int), ("wall_s", C.c_double),
+                ("tokens_per_s", C.c_double), ("cycle_ms", C.c_double), ("form_ms", C.c_double),
+                ("wait_ms", C.c_double), ("update_ms", C.c_double), ("gpu_iter_ms", C.c_double),
+                ("tokens_processed", C.c_longlong)]
+
+
+SYMBOLS += [
+    "pllm_sched_create", "pllm_sched_destroy", "pllm_sched_add_request", "pllm_sched_schedule",
+    "pllm_sched_form", "pllm_sched_harvest", "pllm_sched_advance", "pllm_sched_state",
+    "pllm_sched_retired_output", "pllm_sched_future_page_usage", "pllm_serve",
+]
+
+
+def _sched_lib():
+    l = lib()
+    if not getattr(l, "_sched_declared", False):
+        l.pllm_sched_create.restype = C.c_void_p
+        l.pllm_sched_create.argtypes = [C.c_int] * 8
+        l.pllm_sched_destroy.restype = None
+        l.pllm_sched_destroy.argtypes = [C.c_void_p]
+        l.pllm_sched_add_request.argtypes = [C.c_void_p, C.c_int, _i32p, C.c_int, C.c_int, C.c_double]
+        l.pllm_sched_schedule.argtypes = [C.c_void_p]
+        l.pllm_sched_form.argtypes = [C.c_void_p, C.POINTER(_CUpdateData)]
+        l.pllm_sched_harvest.argtypes = [C.c_void_p, _i32p, C.c_int]
+        l.pllm_sched_advance.argtypes = [C.c_void_p, C.c_double, C.c_int, C.POINTER(C.c_int)]
+        l.pllm_sched_state.argtypes = [C.c_void_p, C.POINTER(C.c_int * 5)]
+        l.pllm_sched_retired_output.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), _i32p, C.c_int]
+        l.pllm_sched_future_page_usage.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int]
+        l.pllm_serve.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(ServeStats)]
+        l._sched_declared = True
+    return l
+
+
+class BatchFormer:
+    """The C++ batch former (scheduler + paged-KV bookkeeping) behind the C ABI."""
+
+    def __init__(self, kv_pages, page_size, global_bsz, nano1, kqv1, kqv3, avg_prefill, avg_decode):
+        self._l = _sched_lib()
+        self._h = self._l.pllm_sched_create(kv_pages, page_size, global_bsz, nano1, kqv1, kqv3,
+                                            avg_prefill, avg_decode)
+        if not self._h:
+            raise NanoflowPipelineError(self._l.pllm_last_error().decode())
+
+    def close(self):
+        if self._h:
+            self._l.pllm_sched_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def add_request(self, req_idx, prompt, output_len, start_time=0.0):
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        _check(self._l.pllm_sched_add_request(self._h, req_idx, p.ctypes.data_as(_i32p), len(p),
+                                              output_len, start_time), "sched_add_request")
+
+    def schedule(self):
+        _check(self._l.pllm_sched_schedule(self._h), "sched_schedule")
+
+    def form(self) -> dict:
+        """Forms the next batch; returns copies of its arrays (numpy int32) and scalars."""
+        u = _CUpdateData()
+        _check(self._l.pllm_sched_form(self._h, C.byref(u)), "sched_form")
+        req = u.decodePrefillBorder + u.prefillNum
+        tok = u.decodePrefillBorder + u.prefillTokensNum
+
+        def arr(addr, n):
+            if n == 0 or not addr:
+                return np.zeros(0, np.int32)
+            return np.ctypeslib.as_array(C.cast(addr, _i32p), shape=(n,)).copy()
+
+        kv_indptr = arr(u.kv_indptr, req + 1)
+        return dict(decodePrefillBorder=u.decodePrefillBorder, prefillNum=u.prefillNum,
+                    prefillTokensNum=u.prefillTokensNum, keepTokenListLength=u.keepTokenListLength,
+                    input_tokens=arr(u.input_tokens, u.prefillTokensNum),
+                    input_indptr=arr(u.input_indptr, req + 1),
+                    rev_input_indptr=arr(u.rev_input_indptr, tok),
+                    per_token_offset=arr(u.per_token_offset, tok), kv_indptr=kv_indptr,
+                    kv_indices=arr(u.kv_indices, int(kv_indptr[-1]) if len(kv_indptr) else 0),
+                    kv_last_page_len=arr(u.kv_last_page_len, req),
+                    keep_token_list=arr(u.keep_token_list, u.keepTokenListLength),
+                    gemv_batch_size=arr(u.gemv_batch_size, 4))
+
+    def harvest(self, ids):
+        a = np.ascontiguousarray(ids, dtype=np.int32)
+        _check(self._l.pllm_sched_harvest(self._h, a.ctypes.data_as(_i32p), len(a)), "sched_harvest")
+
+    def advance(self, now=0.0, placeholder_zero=False) -> int:
+        n = C.c_int()
+        _check(self._l.pllm_sched_advance(self._h, now, int(placeholder_zero), C.byref(n)), "sched_advance")
+        return n.value
+
+    def state(self) -> dict:
+        c = (C.c_int * 5)()
+        _check(self._l.pllm_sched_state(self._h, C.byref(c)), "sched_state")
+        return dict(queued=c[0], decoding=c[1], prefilling=c[2], free_pages=c[3], retired=c[4])
+
+    def retired_output(self, which, cap=65536):
+        out = np.empty(cap, np.int32)
+        idx = C.c_int()
+        n = self._l.pllm_sched_retired_output(self._h, which, C.byref(idx), out.ctypes.data_as(_i32p), cap)
+        if n < 0:
+            _check(n, "sched_retired_output")
+        return idx.value, out[:n].copy()
+
+    def future_page_usage(self):
+        n = self._l.pllm_sched_future_page_usage(self._h, None, 0)
+        out = np.empty(n, np.int64)
+        self._l.pllm_sched_future_page_usage(self._h, out.ctypes.data_as(C.POINTER(C.c_int64)), n)
+        return out
+
+    def serve(self, skip_cycles, run_cycles) -> ServeStats:
+        st = ServeStats()
+        _check(self._l.pllm_serve(self._h, skip_cycles, run_cycles, C.byref(st)), "serve")
+        return st

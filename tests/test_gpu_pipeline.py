@@ -145,3 +145,98 @@ def test_unsupported_pipeline_types_are_rejected():
     with pytest.raises(P.NanoflowPipelineError, match="tensor-parallel"):
         engine.Engine(shape, P.PipelineType.PLLM, global_batch=32, nano1=16, kv_pages=64)
     P.finalize()
+
+
+def _serve_requests(n=14, seed=3):
+    rng = np.random.default_rng(seed)
+    return [(i, rng.integers(2, 1000, size=int(rng.integers(3, 70))).astype(np.int32), int(rng.integers(3, 9)))
+            for i in range(n)]
+
+
+@pytest.mark.parametrize("pt_name", ["LOCAL", "NON_OVERLAP_LOCAL"])
+def test_serving_loop_matches_oracle_and_stepwise_driver(oracle, pt_name):
+    """The C++ serving loop (batch former + asynchronous run) against (a) the same former driven
+    step by step from Python with the oracle checking every iteration on the same inputs, and
+    (b) itself: the retired requests' outputs must be identical both ways."""
+    from nanoflow_amd import engine, pllm_python as P
+    pt = P.PipelineType[pt_name]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=2)
+    T, nano1, kqv1, kqv3, pages = 96, 40, 20, 28, 128
+    reqs = _serve_requests()
+    mk_former = lambda: P.BatchFormer(pages, 16, T, nano1, kqv1, kqv3, 70, 8)
+
+    # ---- (a) step-by-step, every iteration checked by the oracle on the GPU's own token feed
+    former = mk_former()
+    for i, prompt, olen in reqs:
+        former.add_request(i, prompt, olen)
+    pools_ref = [np.zeros((pages, 2, 16, shape.Hkv, shape.d), np.float16) for _ in range(shape.layers)]
+    prev = None
+    checked = 0
+    with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=kqv1, kqv3=kqv3, kv_pages=pages,
+                       weights=w, kv_fill="zeros") as e:
+        for cycle in range(200):
+            st = former.state()
+            if st["queued"] + st["decoding"] + st["prefilling"] == 0:
+                break
+            former.schedule()
+            b = former.form()
+            nd = b["decodePrefillBorder"]
+            dec = prev[b["keep_token_list"] == 1] if nd else np.zeros(0, np.int32)
+            assert len(dec) == nd
+            tokens = np.concatenate([dec, b["input_tokens"]]).astype(np.int32)
+            pages_per = np.diff(b["kv_indptr"])
+            batch = synth.Batch(decodePrefillBorder=nd, prefillNum=b["prefillNum"],
+                                prefillTokensNum=b["prefillTokensNum"], input_tokens=tokens,
+                                input_indptr=b["input_indptr"], rev_input_indptr=b["rev_input_indptr"],
+                                per_token_offset=b["per_token_offset"], kv_indptr=b["kv_indptr"],
+                                kv_indices=b["kv_indices"], kv_last_page_len=b["kv_last_page_len"],
+                                kv_len=((pages_per - 1) * 16 + b["kv_last_page_len"]).astype(np.int32),
+                                num_pages=pages)
+            print(f"serve {pt_name} cycle={cycle} decode={nd} prefill={b['prefillTokensNum']}", flush=True)
+            e.update(batch, keep_token_list=b["keep_token_list"])
+            out = e.run()
+            _, log_ref, samp_ref = oracle.decoder_forward(shape.as_dict(), w, pools_ref, batch.as_dict(),
+                                                          want_logits=True)
+            lg = log_ref.astype(np.float32)
+            top2 = np.sort(lg, axis=1)[:, -2:]
+            clear = (top2[:, 1] - top2[:, 0]) > 2 * E2E_RTOL * np.abs(lg).max()
+            assert np.array_equal(out[clear], samp_ref[clear]), (cycle, "samples")
+            checked += int(clear.sum())
+            if prev is not None:
+                former.harvest(prev)
+            former.advance(0.0)
+            prev = out
+    assert former.state()["retired"] == len(reqs) and checked > 50
+    stepwise = dict(former.retired_output(k) for k in range(len(reqs)))
+    for i, prompt, olen in reqs:
+        # olen - 1 sampled tokens are recorded; the last one is never harvested (placeholder)
+        assert len(stepwise[i]) == olen - 1 and stepwise[i][-1] == -1
+        assert (stepwise[i][:-1] >= 0).all()
+
+    # ---- (b) the C++ loop end to end
+    former2 = mk_former()
+    for i, prompt, olen in reqs:
+        former2.add_request(i, prompt, olen)
+    with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=kqv1, kqv3=kqv3, kv_pages=pages,
+                       weights=w, kv_fill="zeros"):
+        stats = former2.serve(0, 200)
+    assert stats.retired == len(reqs) and stats.cycles > 0 and stats.tokens_per_s > 0
+    served = dict(former2.retired_output(k) for k in range(len(reqs)))
+    for i, _, _ in reqs:
+        assert np.array_equal(served[i], stepwise[i]), (i, served[i], stepwise[i])
+
+
+def test_serve_skip_cycles_reach_steady_state_without_gpu_work():
+    from nanoflow_amd import engine, pllm_python as P
+    shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)
+    T = 64
+    former = P.BatchFormer(256, 16, T, 32, 16, 16, 24, 12)
+    for i in range(40):
+        former.add_request(i, np.arange(24) + 2, 12)
+    with engine.Engine(shape, P.PipelineType.LOCAL, global_batch=T, nano1=32, kqv1=16, kqv3=16,
+                       kv_pages=256, kv_fill="zeros"):
+        stats = former.serve(10, 8)
+    assert stats.cycles == 8
+    assert stats.tokens_processed > 6 * T       # the timed cycles run (nearly) full batches
+    assert stats.gpu_iter_ms > 0 and stats.cycle_ms > 0
