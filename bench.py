@@ -1,17 +1,24 @@
 #!/usr/bin/env python3
-"""Benchmark of the single-GPU nano-batch pipeline on one MI355X.
+"""Benchmark of the single-GPU nano-batch pipeline on one MI355X (Llama-3-8B shape: 32
+layers, vocab 128256, fp16 random-init weights, paged KV with page 16).
 
-A step is ONE dense iteration of the Llama-3-8B-shaped model (32 layers executed, vocab
-128256, fp16 random-init weights): 2048 tokens = 1792 decode tokens (KV length uniform in
-[1024, 1536], paged KV, page 16, permuted page table) + one 256-token prefill chunk, run by
-the overlapped LocalPipeline through the control-plane C ABI.  The iteration's update data is
-staged once before the timed region (inputs resident in HBM); each timed step is one
-``run()`` = embedding ... sampler, ending with the sampled ids on the host.
+--workload offline (default): the offline-throughput job the headline metric is quoted on --
+  4096 requests, constant 1024-token prompts (ids uniform over the vocab) and 512 output
+  tokens, greedy, EOS ignored, served by the C++ batch former + asynchronous loop through the
+  control-plane C ABI at <= 2048 tokens per iteration (steady state: ~682 decode rows + ~1366
+  chunked-prefill rows).  As in the reference's own evaluation the scheduler is first advanced
+  to steady state by simulated cycles (no GPU work), then W warm-up cycles run untimed and K
+  cycles run timed; a step is one serving cycle (form batch i+1 on the CPU while the GPU runs
+  batch i).  tokens/s = retired requests x 1536 / wall time (the reference's definition).
+  --full-run times the whole job from the first request to the last instead.
+--workload iteration: ONE dense 2048-token iteration = 1792 decode tokens (KV length uniform
+  in [1024, 1536], permuted page table) + one 256-token prefill chunk, update data staged once
+  before the timed region; a step is one ``run()`` = embedding ... sampler.
 
-Prints one JSON line: tokens/s (2048 tokens / step time), the roofline record of the
-dominant kernel (paged decode attention, HBM-bound; durations from HIP events recorded on the
-attention stream inside the timed region) and a CPU baseline (the oracle, a port of the
-reference math, timed on the host cores on a bounded sample of the same workload).
+Prints one JSON line: tokens/s, the roofline record of the dominant kernel (offline: the dense
+MFMA GEMMs; iteration: paged decode attention, HBM-bound -- durations from HIP events recorded
+on the kernels' own streams inside the timed region), and a CPU baseline (the oracle, a port
+of the reference math, timed on the host cores on a bounded sample of the same workload).
 """
 from __future__ import annotations
 
@@ -28,6 +35,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0       # dense fp16
+A100_PUBLISHED_TOKENS_PER_S = 12756.0   # reference, 1x A100 80GB, same offline workload
 # HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # as a ratio to the algorithmic bytes of the same launch; None until measured
 # (see profiles/decode_attention_config2_pmc.txt when present).
@@ -49,65 +57,86 @@ def gemm_flops_per_iteration(shape, T, logits_rows, layers) -> float:
     return per_tok * T * layers + 2.0 * logits_rows * shape.hidden * shape.vocab
 
 
-def cpu_baseline(shape, batch, n_sample: int, seed: int):
+def cpu_baseline(shape, decode_lens_after, prefill_chunks, total_decode, seed: int):
     """Times the oracle on a bounded sample of the same iteration: ONE decoder layer plus the
-    LM head over the first n_sample decode requests of the batch (their real KV lengths),
-    and scales to the 32-layer model: tokens/s = n / (layers * t_layer + t_head)."""
+    LM head over a sample of the batch's requests (decode requests with their real KV
+    lengths, prefill chunks of the same proportion), and scales to the full depth:
+    tokens/s = rows / (layers * t_layer + t_head)."""
     from nanoflow_amd import synth
     from oracle import nf_oracle as O
-    nd = n_sample
-    lens_after = batch.kv_len[:nd]
-    b = synth.make_batch(lens_after - 1, [], vocab=shape.vocab, seed=seed)
+    decode_lens_after = np.asarray(decode_lens_after)
+    b = synth.make_batch(decode_lens_after - 1, prefill_chunks, vocab=shape.vocab, seed=seed)
+    rows = b.tokens
     rng = np.random.default_rng(seed + 1)
     one = synth.ModelShape(**{**shape.as_dict(), "layers": 1})
     w = synth.make_weights(one, seed=seed)
     pool = [synth.make_kv_pool(b.num_pages, one, rng)]
-    x = synth.normal_f16(rng, (nd, shape.hidden))
+    x = synth.normal_f16(rng, (rows, shape.hidden))
     O.lib()
     t0 = time.perf_counter()
     hid, _, _ = O.decoder_forward(one.as_dict(), w, pool, b.as_dict(), hidden_in=x,
                                   want_sampled=False)
     t_layer = time.perf_counter() - t0
     t0 = time.perf_counter()
-    kept = O.keep_token(hid, b.input_indptr, nd)
+    kept = O.keep_token(hid, b.input_indptr, b.req_num)
     logits = O.gemm(O.rmsnorm(kept, w["model_norm"]), w["lm_head"])
     O.argmax(logits)
     t_head = time.perf_counter() - t0
     total = shape.layers * t_layer + t_head
+    nd = len(decode_lens_after)
     return {
-        "value": nd / total, "unit": "tokens/s", "cores": O.num_threads(), "kind": "port",
+        "value": rows / total, "unit": "tokens/s", "cores": O.num_threads(), "kind": "port",
         "sample": (f"oracle (C + OpenMP restatement of the reference math): 1 of {shape.layers} layers "
-                   f"+ LM head + sampler on {nd} of the {batch.decodePrefillBorder} decode requests "
-                   f"(KV {int(lens_after.min())}-{int(lens_after.max())}); layer {t_layer:.2f} s, head "
-                   f"{t_head:.2f} s, scaled to {shape.layers} layers"),
+                   f"+ LM head + sampler on {nd} of the {total_decode} decode requests "
+                   f"(KV {int(decode_lens_after.min())}-{int(decode_lens_after.max())})"
+                   + (f" and prefill chunks (prev, len) {list(prefill_chunks)}" if prefill_chunks else "")
+                   + f"; layer {t_layer:.2f} s, head {t_head:.2f} s, scaled to {shape.layers} layers"),
     }
 
 
-def main():
-    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--pipeline", default="LOCAL", choices=["LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL"])
-    ap.add_argument("--nano1", type=int, default=640, help="rows of nano-batch 1")
-    ap.add_argument("--kqv1", type=int, default=256)
-    ap.add_argument("--kqv3", type=int, default=768)
-    ap.add_argument("--distinct-layers", type=int, default=0,
-                    help="distinct weight/KV layers held in HBM (0 = as many of the 32 as fit)")
-    ap.add_argument("--cpu-sample", type=int, default=128, help="decode requests in the CPU baseline (0 = skip)")
-    ap.add_argument("--seed", type=int, default=0)
-    args = ap.parse_args()
-
+def _check_single_gpu(args):
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the single-device pipeline on ONE GPU; --gpus N>1 is not "
               "supported (no collectives are part of this path).", file=sys.stderr)
         sys.exit(2)
 
+
+def _attention_roofline(tm, bytes_per_launch, name="roofline"):
+    n_launch = max(tm.decode_attn_launches, 1)
+    avg_launch_ms = tm.decode_attn_ms / n_launch
+    achieved = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9 if avg_launch_ms > 0 else 0.0
+    return {
+        "kernel": "attn_paged_kernel (paged decode attention)", "bound": "hbm",
+        "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+        "traffic": (None if DECODE_ATTN_TRAFFIC_RATIO is None
+                    else bytes_per_launch * DECODE_ATTN_TRAFFIC_RATIO),
+        "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": avg_launch_ms,
+        "launches_timed": int(tm.decode_attn_launches),
+    }
+
+
+def _gemm_roofline(tm):
+    n = max(tm.gemm_launches, 1)
+    avg_ms = tm.gemm_ms / n
+    flop_per_launch = tm.gemm_flop / n
+    achieved = flop_per_launch / (avg_ms * 1e-3) / 1e12 if avg_ms > 0 else 0.0
+    return {
+        "kernel": "gemm_f16_kernel / dual_swiglu_f16_kernel (all dense GEMM launches of the iteration)",
+        "bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+        "algorithmic_flop_per_launch": flop_per_launch, "avg_launch_ms": avg_ms,
+        "launches_timed": int(tm.gemm_launches),
+    }
+
+
+def run_iteration(args):
     import torch
     from nanoflow_amd import engine, synth, pllm_python as P
     assert torch.cuda.is_available(), "bench.py needs the MI355X (no CPU path)"
     shape = synth.LLAMA3_8B
     T = 2048
+    steps = args.steps or 5
+    warmup = 2 if args.warmup is None else args.warmup
     batch = synth.config2_batch(seed=args.seed)
     assert batch.tokens == T
     pages = batch.num_pages
@@ -123,44 +152,40 @@ def main():
     t_setup = time.perf_counter()
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, run_layer=shape.layers,
-                        distinct_layers=distinct, seed=args.seed, profiling=True)
+                        distinct_layers=distinct, seed=args.seed, profiling=args.profile_level)
     eng.update(batch)
     torch.cuda.synchronize()
     t_setup = time.perf_counter() - t_setup
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         eng.run()
     P.resetTimings()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         out = eng.run()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     tm = P.getTimings()
-    ms_per_step = dt * 1e3 / args.steps
+    ms_per_step = dt * 1e3 / steps
 
     # per-iteration PCIe-inclusive variant: stage the update data every step
     t0 = time.perf_counter()
-    for _ in range(max(1, args.steps // 2)):
+    for _ in range(max(1, steps // 2)):
         eng.update(batch)
         eng.run()
     torch.cuda.synchronize()
-    ms_with_update = (time.perf_counter() - t0) * 1e3 / max(1, args.steps // 2)
+    ms_with_update = (time.perf_counter() - t0) * 1e3 / max(1, steps // 2)
 
     nd = batch.decodePrefillBorder
     groups = synth.gemv_batch_split(nd, args.kqv1, args.nano1, args.kqv3) if args.pipeline != "NON_OVERLAP_LOCAL" else [nd]
     launches_per_layer = sum(1 for g in groups if g > 0)
     bytes_per_layer = decode_attention_bytes(batch.kv_len[:nd])
-    n_launch = max(tm.decode_attn_launches, 1)
-    avg_launch_ms = tm.decode_attn_ms / n_launch
-    bytes_per_launch = bytes_per_layer / launches_per_layer
-    achieved = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9 if avg_launch_ms > 0 else 0.0
     flops = gemm_flops_per_iteration(shape, T, min((batch.req_num + 127) // 128 * 128, T), shape.layers)
 
     rec = {
         "metric": "tokens/s/GPU", "value": T / (ms_per_step * 1e-3), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {
@@ -171,26 +196,159 @@ def main():
             "distinct_layers_in_hbm": distinct, "kv_pages_per_layer": int(pages),
             "decode_attention_launches_per_layer": launches_per_layer,
         },
-        "roofline": {
-            "kernel": "attn_paged_kernel (paged decode attention)", "bound": "hbm",
-            "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": (None if DECODE_ATTN_TRAFFIC_RATIO is None
-                        else bytes_per_launch * DECODE_ATTN_TRAFFIC_RATIO),
-            "algorithmic_bytes_per_launch": bytes_per_launch, "avg_launch_ms": avg_launch_ms,
-            "launches_timed": int(tm.decode_attn_launches),
-        },
+        "roofline": _attention_roofline(tm, bytes_per_layer / launches_per_layer),
         "iteration": {
             "device_ms_last": tm.iter_ms, "ms_per_step_with_update": ms_with_update,
-            "decode_attention_ms_per_step": tm.decode_attn_ms / args.steps,
-            "prefill_attention_ms_per_step": tm.prefill_attn_ms / args.steps,
+            "decode_attention_ms_per_step": tm.decode_attn_ms / steps,
+            "prefill_attention_ms_per_step": tm.prefill_attn_ms / steps,
             "gemm_tflop_per_step": flops / 1e12,
-            "gemm_mfma_frac_if_serial": (flops / 1e12) / (max(ms_per_step - 0.0, 1e-9) * 1e-3) / MFMA_PEAK_TFLOPS,
+            "gemm_mfma_frac_if_serial": (flops / 1e12) / (max(ms_per_step, 1e-9) * 1e-3) / MFMA_PEAK_TFLOPS,
             "setup_s": t_setup, "sampled_tokens": int(out.shape[0]),
         },
     }
+    if tm.gemm_launches:
+        rec["roofline_gemm"] = _gemm_roofline(tm)
+        rec["iteration"]["gemm_ms_per_step"] = tm.gemm_ms / steps
     eng.close()
     if args.cpu_sample > 0:
-        rec["cpu_baseline"] = cpu_baseline(shape, batch, args.cpu_sample, args.seed)
+        rec["cpu_baseline"] = cpu_baseline(shape, batch.kv_len[:args.cpu_sample], [], nd, args.seed)
+    return rec
+
+
+def run_offline(args):
+    import torch
+    from nanoflow_amd import engine, synth, pllm_python as P
+    assert torch.cuda.is_available(), "bench.py needs the MI355X (no CPU path)"
+    shape = synth.LLAMA3_8B
+    T, n_req, in_len, out_len = 2048, args.requests, 1024, 512
+    steps = args.steps or 256
+    warmup = 8 if args.warmup is None else args.warmup
+
+    # KV pool: every layer distinct; 2 MiB per page over the 32 layers.  The trace peaks near
+    # 66k pages in flight; the pool is sized to HBM with headroom, capped at 128 Ki pages.
+    free_b, _ = torch.cuda.mem_get_info()
+    weight_b = 2 * (shape.layers * (shape.hidden * (shape.kqv_n + shape.Hq * shape.d + 2 * shape.ffn)
+                                    + shape.ffn * shape.hidden) + 2 * shape.vocab * shape.hidden)
+    page_b = shape.layers * 2 * 16 * shape.Hkv * shape.d * 2
+    pages = args.kv_pages or int(min(131072, (free_b * 0.90 - weight_b - (6 << 30)) // page_b))
+    pages = pages // 64 * 64
+    assert pages >= 4096, f"not enough free HBM for the KV pool ({free_b / 2**30:.0f} GiB free)"
+
+    t_setup = time.perf_counter()
+    eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
+                        kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, seed=args.seed,
+                        profiling=args.profile_level, kv_fill="zeros")
+    former = P.BatchFormer(pages, shape.page_size, T, args.nano1, args.kqv1, args.kqv3, in_len, out_len)
+    rng = np.random.default_rng(args.seed)
+    for i in range(n_req):
+        former.add_request(i, rng.integers(0, shape.vocab, size=in_len, dtype=np.int32), out_len)
+    torch.cuda.synchronize()
+    t_setup = time.perf_counter() - t_setup
+
+    if args.full_run:
+        skip, warmup, steps = 0, 0, 1 << 30
+    else:
+        skip = args.skip_cycles
+    st = former.serve(skip, steps, warmup_cycles=warmup)
+    tm = P.getTimings()
+    state = former.state()
+    steps = st.cycles
+    rows_per_req = in_len + out_len - 1          # dense-batch rows a request occupies in its life
+    by_retired = st.retired * (in_len + out_len) / st.wall_s
+    by_rows = st.tokens_processed / rows_per_req * (in_len + out_len) / st.wall_s
+    # the reference's definition counts whole retired requests; over a short window that is
+    # quantised (about 1.33 requests retire per cycle), so below 200 retirements the same
+    # quantity is taken from the rows processed instead
+    use_retired = st.retired >= 200
+    value = by_retired if use_retired else by_rows
+
+    # steady-state decode set for the byte accounting: the requests now decoding
+    former.schedule()
+    nxt = former.form()
+    nd = nxt["decodePrefillBorder"]
+    kv_len = ((np.diff(nxt["kv_indptr"]) - 1) * shape.page_size + nxt["kv_last_page_len"])[:nd]
+    groups = [g for g in nxt["gemv_batch_size"].tolist() if g > 0] if args.pipeline != "NON_OVERLAP_LOCAL" else [nd]
+    launches_per_layer = max(len(groups), 1)
+    bytes_per_layer = decode_attention_bytes(kv_len) if nd else 0
+    prefill_chunks = [(int(nxt["per_token_offset"][nxt["input_indptr"][nd + j]]),
+                       int(nxt["input_indptr"][nd + j + 1] - nxt["input_indptr"][nd + j]))
+                      for j in range(nxt["prefillNum"])]
+
+    rec = {
+        "metric": "tokens/s/GPU", "value": value, "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": st.cycle_ms,
+        "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": value / A100_PUBLISHED_TOKENS_PER_S, "dtype": "f16", "data": "synthetic",
+        "config": {
+            "workload": (f"Llama-3-8B shape, offline throughput: {n_req} requests, constant {in_len}-token "
+                         f"prompts (ids uniform over the vocab) / {out_len} output tokens, greedy, EOS "
+                         f"ignored, <= {T} tokens per iteration with chunked prefill; "
+                         + ("whole job timed" if args.full_run else
+                            f"{skip} simulated scheduler cycles to steady state, then {warmup} warm-up and "
+                            f"{steps} timed serving cycles")),
+            "pipeline": args.pipeline, "global_batch": T, "nanobatch_1_size": args.nano1,
+            "kqv1_size": args.kqv1, "kqv3_size": args.kqv3, "layers_executed": shape.layers,
+            "distinct_layers_in_hbm": shape.layers, "kv_pages_per_layer": int(pages),
+            "kv_pool_gib": pages * page_b / 2**30,
+            "value_formula": ("retired_requests * 1536 / wall_s" if use_retired else
+                              "dense_rows_processed / 1535 * 1536 / wall_s (fewer than 200 retirements in the window)"),
+            "baseline": "12756 tokens/s/GPU published by the reference for this workload on 1x A100 80GB",
+        },
+        "roofline": _gemm_roofline(tm) if tm.gemm_launches else _attention_roofline(
+            tm, bytes_per_layer / launches_per_layer),
+        "serving": {
+            "cycles": st.cycles, "retired_requests": st.retired, "wall_s": st.wall_s,
+            "tokens_per_s_by_retired_requests": by_retired, "tokens_per_s_by_rows": by_rows,
+            "dense_rows_processed": int(st.tokens_processed),
+            "cycle_ms": st.cycle_ms, "gpu_iteration_ms": st.gpu_iter_ms,
+            "cpu_form_ms": st.form_ms, "cpu_wait_for_gpu_ms": st.wait_ms, "cpu_update_ms": st.update_ms,
+            # cycle time not covered by the device's iteration: update (staging + H2D), launch
+            # latency and whatever part of batch formation did not overlap the GPU
+            "cpu_exposed_ms_per_cycle": max(0.0, st.cycle_ms - st.gpu_iter_ms),
+            "cpu_form_hidden_fraction": (1.0 - min(1.0, max(0.0, st.cycle_ms - st.gpu_iter_ms - st.update_ms)
+                                                   / st.form_ms) if st.form_ms > 0 else None),
+            "steady_state_decode_rows": int(nd), "steady_state_prefill_rows": int(nxt["prefillTokensNum"]),
+            "decode_attention_ms_per_cycle": tm.decode_attn_ms / max(st.cycles, 1),
+            "prefill_attention_ms_per_cycle": tm.prefill_attn_ms / max(st.cycles, 1),
+            "gemm_ms_per_cycle": tm.gemm_ms / max(st.cycles, 1),
+            "requests_left": state["queued"] + state["decoding"] + state["prefilling"],
+            "setup_s": t_setup,
+        },
+    }
+    if tm.gemm_launches and tm.decode_attn_launches and nd:
+        rec["roofline_decode_attention"] = _attention_roofline(tm, bytes_per_layer / launches_per_layer)
+    eng.close()
+    if args.cpu_sample > 0 and nd:
+        n = min(args.cpu_sample, nd)
+        sample_chunks = [(p, max(1, l * n // nd)) for p, l in prefill_chunks]
+        rec["cpu_baseline"] = cpu_baseline(shape, kv_len[:n], sample_chunks, nd, args.seed)
+    return rec
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: offline 256, iteration 5)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps (default: offline 8, iteration 2)")
+    ap.add_argument("--workload", default="offline", choices=["offline", "iteration"])
+    ap.add_argument("--pipeline", default="LOCAL", choices=["LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL"])
+    ap.add_argument("--nano1", type=int, default=1024, help="rows of nano-batch 1")
+    ap.add_argument("--kqv1", type=int, default=512)
+    ap.add_argument("--kqv3", type=int, default=512)
+    ap.add_argument("--distinct-layers", type=int, default=0,
+                    help="iteration workload: distinct weight/KV layers held in HBM (0 = as many of the 32 as fit)")
+    ap.add_argument("--requests", type=int, default=4096, help="offline workload: requests in the trace")
+    ap.add_argument("--skip-cycles", type=int, default=1280,
+                    help="offline workload: simulated scheduler cycles before the GPU runs")
+    ap.add_argument("--full-run", action="store_true", help="offline workload: time the whole job")
+    ap.add_argument("--kv-pages", type=int, default=0, help="offline workload: KV pool pages (0 = sized to HBM)")
+    ap.add_argument("--profile-level", type=int, default=2, choices=[0, 1, 2],
+                    help="per-launch events: 1 attention, 2 attention and GEMMs")
+    ap.add_argument("--cpu-sample", type=int, default=96, help="decode requests in the CPU baseline (0 = skip)")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    _check_single_gpu(args)
+    rec = run_offline(args) if args.workload == "offline" else run_iteration(args)
     print(json.dumps(rec))
 
 

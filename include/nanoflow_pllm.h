@@ -200,13 +200,18 @@ typedef struct nf_serve_stats {
   long long tokens_processed;
 } nf_serve_stats;
 /* The serving loop of serve_8B.py:655-700 over an initialised and configured pipeline:
- * skip_cycles simulated cycles (scheduler only), then run_cycles executed and timed cycles in
- * which batch i+1 is formed on the CPU while the GPU runs batch i. */
-NF_PLLM_API int pllm_serve(nf_batch_former* f, int skip_cycles, int run_cycles, nf_serve_stats* stats);
+ * skip_cycles simulated cycles (scheduler only), warmup_cycles executed but untimed cycles,
+ * then run_cycles executed and timed cycles; batch i+1 is formed on the CPU while the GPU runs
+ * batch i.  The timed region starts and ends with the GPU idle and resets the accumulated
+ * pipeline timings at its start. */
+NF_PLLM_API int pllm_serve(nf_batch_former* f, int skip_cycles, int warmup_cycles, int run_cycles,
+                           nf_serve_stats* stats);
 
 /* Measurement (no counterpart in the reference, which only logs the iteration time,
- * pipeline_local.cu:444-463).  With profiling on, every attention launch is bracketed by
- * events on its own stream.  pllm_get_timings returns the last iteration's time and the
+ * pipeline_local.cu:444-463).  pllm_set_profiling level 1 brackets every attention launch with
+ * events on its own stream; level 2 also every dense GEMM launch; 0 switches it off.
+ * Schedules of 8 or more layers time every 4th layer only (the event records cost device
+ * time); the launch counts returned are the launches actually timed.  pllm_get_timings returns the last iteration's time and the
  * durations accumulated since the last pllm_reset_timings. */
 typedef struct nf_pipeline_timings {
   double iter_ms;
@@ -214,6 +219,9 @@ typedef struct nf_pipeline_timings {
   long decode_attn_launches;
   double prefill_attn_ms;
   long prefill_attn_launches;
+  double gemm_ms;    /* dense GEMM launches (level 2): summed duration, count, flops */
+  long gemm_launches;
+  double gemm_flop;
 } nf_pipeline_timings;
 NF_PLLM_API int pllm_set_profiling(int on);
 NF_PLLM_API int pllm_get_timings(nf_pipeline_timings* out);

@@ -144,7 +144,8 @@ struct ServeStats {
 // The asynchronous serving loop (pipeline/utils/serve_8B.py:348-569, 655-700): batch i+1 is
 // scheduled and formed on the CPU while the GPU runs batch i; outputs are harvested one
 // iteration late.  skip_cycles advance the scheduler without touching the GPU (the reference's
-// simulated warm-up), run_cycles are executed and timed.  Requires an initialised and configured
-// pipeline (init() + config()).
-ServeStats serveLoop(BatchFormer& former, int skip_cycles, int run_cycles,
+// simulated warm-up), warmup_cycles are executed untimed, run_cycles are executed and timed (the
+// timed region starts and ends with the GPU idle; the pipeline's accumulated timings are reset
+// at its start).  Requires an initialised and configured pipeline (init() + config()).
+ServeStats serveLoop(BatchFormer& former, int skip_cycles, int warmup_cycles, int run_cycles,
                      std::vector<FlyPtr>* retired_out = nullptr);

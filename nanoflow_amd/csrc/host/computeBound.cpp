@@ -19,7 +19,7 @@ static SharedState shared_state;
 static std::unique_ptr<SimpleThreadSync> global_sync;  // workers + the caller's thread
 static vortexInitData* persistant_input = nullptr;
 static std::vector<int> complete_input_tokens;
-static bool g_profiling = false;
+static int g_profiling = 0;
 
 int buildInputTokens(const int* prev_output, int prev_count, const int32_t* keep_token_list,
                      int keep_token_list_length, const int* prefill_tokens, int prefill_tokens_num,
@@ -122,9 +122,9 @@ void finalize() {
 
 PipelineBase* currentPipeline() { return workers.empty() ? nullptr : workers[0]->getPipeline(); }
 
-void setPipelineProfiling(bool on) {
-  g_profiling = on;
-  if (auto* p = currentPipeline()) p->setProfiling(on);
+void setPipelineProfiling(int level) {
+  g_profiling = level;
+  if (auto* p = currentPipeline()) p->setProfiling(level);
 }
 
 Worker::PipelineType Worker::PipeTy = Worker::PipelineType::LOCAL;
@@ -149,7 +149,7 @@ void Worker::init() {
     pipeline = std::make_unique<NonOverlapLocalPipeline>(input, rank, nranks, vnranks);
   else
     NF_LOG_ERROR("Unknown pipeline type %d", static_cast<int>(PipeTy));
-  if (pipeline && g_profiling) pipeline->setProfiling(true);
+  if (pipeline && g_profiling) pipeline->setProfiling(g_profiling);
 }
 
 void Worker::run_pipeline() { *output = pipeline->run(); }

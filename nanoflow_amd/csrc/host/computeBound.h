@@ -114,4 +114,4 @@ int buildInputTokens(const int* prev_output, int prev_count, const int32_t* keep
 
 // Access for measurement code: the rank-0 pipeline (nullptr before init()).
 PipelineBase* currentPipeline();
-void setPipelineProfiling(bool on);
+void setPipelineProfiling(int level);

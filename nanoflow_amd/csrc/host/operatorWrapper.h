@@ -20,6 +20,7 @@ struct OperatorWrapper {
   // per-launch timing (off by default)
   std::vector<hipEvent_t> prof_events;  // 2 per launch: start, end
   size_t prof_used = 0;
+  unsigned prof_stride = 1, prof_seq = 0;
 
   OperatorWrapper(bool create_start = false, bool create_end = true) {
     if (create_start) HIP_CHECK(hipEventCreate(&start_event));
@@ -67,7 +68,7 @@ struct OperatorWrapper {
       return *this;
     }
     recordStartEvent();
-    const bool prof = prof_used + 2 <= prof_events.size();
+    const bool prof = prof_used + 2 <= prof_events.size() && (prof_seq++ % prof_stride) == 0;
     if (prof) HIP_CHECK(hipEventRecord(prof_events[prof_used], stream));
     work();
     if (prof) {
@@ -110,7 +111,10 @@ struct OperatorWrapper {
   OperatorWrapper& log() { return *this; }
 
   // Time up to max_launches launches per iteration with event pairs on the op's own stream.
-  void enableProfiling(size_t max_launches) {
+  // Every stride-th launch is timed (event records cost device time, so long schedules sample).
+  void enableProfiling(size_t max_launches, unsigned stride = 1) {
+    prof_stride = stride ? stride : 1;
+    prof_seq = 0;
     for (auto e : prof_events) (void)hipEventDestroy(e);
     prof_events.assign(2 * max_launches, nullptr);
     for (auto& e : prof_events) HIP_CHECK(hipEventCreate(&e));

@@ -31,8 +31,9 @@ struct PipelineTimings {
   long decode_attn_launches = 0;
   double prefill_attn_ms = 0;
   long prefill_attn_launches = 0;
-  double gemm_ms = 0;        // sum over the timed dense GEMM launches (when enabled)
+  double gemm_ms = 0;        // sum of dense GEMM launch durations (profiling level 2)
   long gemm_launches = 0;
+  double gemm_flop = 0;      // flops of those launches (2*M*N*K each; the fused gate/up pair 4*M*N*K)
 };
 
 class PipelineBase {
@@ -52,6 +53,7 @@ protected:
   EventManager ev;
   std::vector<hipEvent_t>& events = ev.events;
   bool profiling = false;
+  bool profile_gemms = false;
   PipelineTimings timings;
 
 public:
@@ -61,7 +63,9 @@ public:
   virtual void setName() {}
   // stream on which update data must be uploaded so that it is ordered before run()
   virtual hipStream_t uploadStream() = 0;
-  virtual void setProfiling(bool on) { profiling = on; }
+  // level 0: off; 1: attention launches; 2: attention and dense GEMM launches
+  virtual void setProfiling(int level) { profiling = level > 0; profile_gemms = level > 1; }
+  int profilingLevel() const { return profiling ? (profile_gemms ? 2 : 1) : 0; }
   const PipelineTimings& getTimings() const { return timings; }
   void resetTimings() { timings = PipelineTimings(); }
   void setHostUpdate(const vortexUpdateData& h) { host_update_data = h; }
@@ -131,7 +135,7 @@ public:
   void GEMVOpUpdate();
   void setName() override;
   hipStream_t uploadStream() override { return stream_gemm; }
-  void setProfiling(bool on) override;
+  void setProfiling(int level) override;
 
 private:
   void init();
@@ -182,7 +186,7 @@ public:
   void GEMVOpUpdate();
   void setName() override;
   hipStream_t uploadStream() override { return stream_all; }
-  void setProfiling(bool on) override;
+  void setProfiling(int level) override;
 
 private:
   double totalCompute();

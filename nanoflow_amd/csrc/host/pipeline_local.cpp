@@ -116,12 +116,20 @@ void LocalPipeline::assignSameStream() {
   prefill2.setStream(stream_gemm);
 }
 
-void LocalPipeline::setProfiling(bool on) {
-  profiling = on;
-  const size_t n = on ? (size_t)ModelConfig.run_layer : 0;
-  for (auto gemv : gemvs) gemv->enableProfiling(n);
-  prefill1.enableProfiling(n);
-  prefill2.enableProfiling(n);
+void LocalPipeline::setProfiling(int level) {
+  profiling = level > 0;
+  profile_gemms = level > 1;
+  // long schedules time every 4th layer: the event records themselves cost device time
+  const unsigned stride = ModelConfig.run_layer >= 8 ? 4 : 1;
+  const size_t n = profiling ? (size_t)ModelConfig.run_layer : 0;
+  for (auto gemv : gemvs) gemv->enableProfiling(n, stride);
+  prefill1.enableProfiling(n, stride);
+  prefill2.enableProfiling(n, stride);
+  const size_t ng = profile_gemms ? (size_t)ModelConfig.run_layer : 0;
+  for (auto g : gemms)
+    if (g) g->enableProfiling(ng, stride);
+  dual1.enableProfiling(ng, stride);
+  dual2.enableProfiling(ng, stride);
 }
 
 void LocalPipeline::setWeight(int layer) {
@@ -390,6 +398,17 @@ vortexOutputData LocalPipeline::run() {
     prefill1.collectProfile(timings.prefill_attn_ms, timings.prefill_attn_launches);
     prefill2.collectProfile(timings.prefill_attn_ms, timings.prefill_attn_launches);
   }
+  if (profile_gemms) {
+    auto add = [&](OperatorWrapper& op, double flop) {
+      const long before = timings.gemm_launches;
+      op.collectProfile(timings.gemm_ms, timings.gemm_launches);
+      timings.gemm_flop += flop * double(timings.gemm_launches - before);
+    };
+    for (auto g : gemms)
+      if (g) add(*g, g->totalCompute());
+    add(dual1, dual1.totalCompute());
+    add(dual2, dual2.totalCompute());
+  }
   NF_LOG_INFO("Total running cost (ms) of one microbatch is %f (%.1f token/s)", runtime_ms,
               config_data.global_batch_size / (runtime_ms / 1000.0));
   return output_data;
@@ -611,5 +630,5 @@ void LocalPipeline::config(vortexConfigData* config_data_) {
   HIP_CHECK(hipHostMalloc(&prefill1_staging.input_indptr, sizeof(int) * n, hipHostMallocDefault));
   HIP_CHECK(hipHostMalloc(&prefill1_staging.kv_indptr, sizeof(int) * n, hipHostMallocDefault));
   HIP_CHECK(hipHostMalloc(&prefill1_staging.kv_last_page_len, sizeof(int) * n, hipHostMallocDefault));
-  if (profiling) setProfiling(true);
+  if (profiling) setProfiling(profilingLevel());
 }

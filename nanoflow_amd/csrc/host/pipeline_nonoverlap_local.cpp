@@ -17,11 +17,18 @@ NonOverlapLocalPipeline::~NonOverlapLocalPipeline() {
   if (stream_all) (void)hipStreamDestroy(stream_all);
 }
 
-void NonOverlapLocalPipeline::setProfiling(bool on) {
-  profiling = on;
-  const size_t n = on ? (size_t)ModelConfig.run_layer : 0;
-  GEMV.enableProfiling(n);
-  prefill.enableProfiling(n);
+void NonOverlapLocalPipeline::setProfiling(int level) {
+  profiling = level > 0;
+  profile_gemms = level > 1;
+  // long schedules time every 4th layer: the event records themselves cost device time
+  const unsigned stride = ModelConfig.run_layer >= 8 ? 4 : 1;
+  const size_t n = profiling ? (size_t)ModelConfig.run_layer : 0;
+  GEMV.enableProfiling(n, stride);
+  prefill.enableProfiling(n, stride);
+  const size_t ng = profile_gemms ? (size_t)ModelConfig.run_layer : 0;
+  for (auto g : gemms)
+    if (g) g->enableProfiling(ng, stride);
+  dual.enableProfiling(ng, stride);
 }
 
 vortexOutputData NonOverlapLocalPipeline::run() {
@@ -56,6 +63,16 @@ vortexOutputData NonOverlapLocalPipeline::run() {
   if (profiling) {
     GEMV.collectProfile(timings.decode_attn_ms, timings.decode_attn_launches);
     prefill.collectProfile(timings.prefill_attn_ms, timings.prefill_attn_launches);
+  }
+  if (profile_gemms) {
+    auto add = [&](OperatorWrapper& op, double flop) {
+      const long before = timings.gemm_launches;
+      op.collectProfile(timings.gemm_ms, timings.gemm_launches);
+      timings.gemm_flop += flop * double(timings.gemm_launches - before);
+    };
+    for (auto g : gemms)
+      if (g) add(*g, g->totalCompute());
+    add(dual, dual.totalCompute());
   }
   NF_LOG_INFO("Total running cost (ms) of one microbatch is %f", runtime_ms);
   return output_data;
@@ -111,7 +128,7 @@ void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
   output_data = vortexOutputData();
   output_data.sampled_token_array = new int[globalbatch];
   output_data.global_batch_size = globalbatch;
-  if (profiling) setProfiling(true);
+  if (profiling) setProfiling(profilingLevel());
 }
 
 void NonOverlapLocalPipeline::setName() {

@@ -285,7 +285,7 @@ int pllm_build_input_tokens(const int32_t* prev_output, int prev_count, const in
 }
 
 int pllm_set_profiling(int on) {
-  setPipelineProfiling(on != 0);
+  setPipelineProfiling(on < 0 ? 0 : on > 2 ? 2 : on);
   return NF_PLLM_OK;
 }
 
@@ -298,6 +298,9 @@ int pllm_get_timings(nf_pipeline_timings* out) {
   out->decode_attn_launches = t.decode_attn_launches;
   out->prefill_attn_ms = t.prefill_attn_ms;
   out->prefill_attn_launches = t.prefill_attn_launches;
+  out->gemm_ms = t.gemm_ms;
+  out->gemm_launches = t.gemm_launches;
+  out->gemm_flop = t.gemm_flop;
   return NF_PLLM_OK;
 }
 
@@ -447,13 +450,13 @@ int pllm_sched_future_page_usage(nf_batch_former* f, int64_t* out, int cap) {
   return (int)u.size();
 }
 
-int pllm_serve(nf_batch_former* f, int skip_cycles, int run_cycles, nf_serve_stats* stats) {
+int pllm_serve(nf_batch_former* f, int skip_cycles, int warmup_cycles, int run_cycles, nf_serve_stats* stats) {
   if (!f || !stats) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_serve: null");
   if (!g_configured) return fail(NF_PLLM_ERR_STATE, "pllm_serve: call pllm_init and pllm_config first");
   if (g_running) return fail(NF_PLLM_ERR_STATE, "pllm_serve: a run is in flight");
   ServeStats s;
   try {
-    s = serveLoop(f->former, skip_cycles, run_cycles, &f->retired);
+    s = serveLoop(f->former, skip_cycles, warmup_cycles, run_cycles, &f->retired);
   } catch (const std::exception& e) {
     g_updated = false;
     return fail(NF_PLLM_ERR_STATE, "pllm_serve: %s", e.what());

@@ -24,57 +24,67 @@ static void to_update(FormedBatch& b, vortexUpdateData& u) {
   u.gemv_num_blocks = b.gemv_num_blocks;
 }
 
-ServeStats serveLoop(BatchFormer& former, int skip_cycles, int run_cycles, std::vector<FlyPtr>* retired_out) {
+ServeStats serveLoop(BatchFormer& former, int skip_cycles, int warmup_cycles, int run_cycles,
+                     std::vector<FlyPtr>* retired_out) {
   ServeStats st;
   std::vector<FlyPtr> retired_local;
   std::vector<FlyPtr>& retired = retired_out ? *retired_out : retired_local;
   FormedBatch batch;
   std::vector<vortexUpdateData> upd(1);
+  auto busy = [&] { return former.queued() + former.decoding() + former.prefilling() > 0; };
 
   // simulated warm-up: the scheduler advances, the GPU does not run
-  for (int c = 0; c < skip_cycles && (former.queued() + former.decoding() + former.prefilling()) > 0; ++c) {
+  for (int c = 0; c < skip_cycles && busy(); ++c) {
     former.schedule();
     former.form(batch);
     former.advance(now_s(), retired, /*placeholder_zero=*/true);
   }
-  const size_t retired_before = retired.size();
 
-  enum { SKIP, FIRST, RUNNING } state = SKIP;
-  double t_form = 0, t_wait = 0, t_update = 0, t_gpu = 0;
-  const double t1 = now_s();
+  bool in_flight = false;     // an iteration is running on the worker thread
+  bool have_outputs = false;  // aggregated_output holds the samples of the former's previous iteration
+  size_t retired_before = retired.size();
+  double t_form = 0, t_wait = 0, t_update = 0, t_gpu = 0, t1 = now_s();
+  auto wait_iteration = [&] {
+    run_async_wait();
+    in_flight = false;
+    have_outputs = true;
+    if (auto* p = currentPipeline()) t_gpu += p->getTimings().iter_ms;
+  };
   try {
-  for (int c = 0; c < run_cycles && (former.queued() + former.decoding() + former.prefilling()) > 0; ++c) {
-    const double a = now_s();
-    former.schedule();
-    former.form(batch);
-    const double b = now_s();
-    if (batch.decodePrefillBorder + batch.prefillTokensNum == 0) break;  // nothing left to run
-    if (state != SKIP) {
-      run_async_wait();  // iteration c-1 is done; its samples feed the decode rows below
-      if (auto* p = currentPipeline()) t_gpu += p->getTimings().iter_ms;
+    for (int c = 0; c < warmup_cycles + run_cycles && busy(); ++c) {
+      if (c == warmup_cycles) {  // the timed region starts with the GPU idle
+        if (in_flight) wait_iteration();
+        if (auto* p = currentPipeline()) p->resetTimings();
+        retired_before = retired.size();
+        t_form = t_wait = t_update = t_gpu = 0;
+        st = ServeStats();
+        t1 = now_s();
+      }
+      const double a = now_s();
+      former.schedule();
+      former.form(batch);
+      const double b = now_s();
+      if (batch.decodePrefillBorder + batch.prefillTokensNum == 0) break;  // nothing left to run
+      if (in_flight) wait_iteration();  // iteration c-1 is done; its samples feed the decode rows below
+      const double w = now_s();
+      to_update(batch, upd[0]);
+      update(1, upd);
+      const double u = now_s();
+      run_async();
+      in_flight = true;
+      if (have_outputs) former.harvest(aggregated_output.data(), (int)aggregated_output.size());
+      former.advance(now_s(), retired, false);
+      t_form += b - a;
+      t_wait += w - b;
+      t_update += u - w;
+      st.tokens_processed += batch.decodePrefillBorder + batch.prefillTokensNum;
+      ++st.cycles;
     }
-    const double w = now_s();
-    to_update(batch, upd[0]);
-    update(1, upd);
-    const double u = now_s();
-    run_async();
-    state = state == SKIP ? FIRST : RUNNING;
-    if (state == RUNNING) former.harvest(aggregated_output.data(), (int)aggregated_output.size());
-    former.advance(now_s(), retired, false);
-    t_form += b - a;
-    t_wait += w - b;
-    t_update += u - w;
-    st.tokens_processed += batch.decodePrefillBorder + batch.prefillTokensNum;
-    ++st.cycles;
-  }
   } catch (...) {
-    if (state != SKIP) run_async_wait();  // never leave an iteration in flight behind an error
+    if (in_flight) run_async_wait();  // never leave an iteration in flight behind an error
     throw;
   }
-  if (state != SKIP) {
-    run_async_wait();
-    if (auto* p = currentPipeline()) t_gpu += p->getTimings().iter_ms;
-  }
+  if (in_flight) wait_iteration();
   const double t2 = now_s();
   st.wall_s = t2 - t1;
   st.retired = (int)(retired.size() - retired_before);

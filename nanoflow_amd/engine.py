@@ -136,8 +136,7 @@ class Engine:
         init.setWeight(mw, H * H * 3)
         init.setTmpBuffer(self.tmp.data_ptr(), self.tmp.numel())
         torch.cuda.synchronize()
-        if profiling:
-            P.setProfiling(True)
+        P.setProfiling(int(profiling))
         P.init([init], pipeline_type)
         cfg = P.VortexConfigData()
         cfg.setGemmOpTag([DEFAULT_TAG] * n_tags)

@@ -170,7 +170,8 @@ class VortexConfigData:
 class PipelineTimings(C.Structure):
     _fields_ = [("iter_ms", C.c_double), ("decode_attn_ms", C.c_double),
                 ("decode_attn_launches", C.c_long), ("prefill_attn_ms", C.c_double),
-                ("prefill_attn_launches", C.c_long)]
+                ("prefill_attn_launches", C.c_long), ("gemm_ms", C.c_double),
+                ("gemm_launches", C.c_long), ("gemm_flop", C.c_double)]
 
 
 SYMBOLS = [
@@ -304,8 +305,9 @@ def buildInputTokens(prev_output, keep_token_list, prefill_tokens) -> np.ndarray
     return out[:n]
 
 
-def setProfiling(on: bool):
-    _check(lib().pllm_set_profiling(int(on)), "setProfiling")
+def setProfiling(level):
+    """0/False: off; 1/True: attention launches are timed; 2: dense GEMM launches as well."""
+    _check(lib().pllm_set_profiling(int(level)), "setProfiling")
 
 
 def getTimings() -> PipelineTimings:
@@ -355,7 +357,7 @@ def _sched_lib():
         l.pllm_sched_state.argtypes = [C.c_void_p, C.POINTER(C.c_int * 5)]
         l.pllm_sched_retired_output.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), _i32p, C.c_int]
         l.pllm_sched_future_page_usage.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int]
-        l.pllm_serve.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(ServeStats)]
+        l.pllm_serve.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(ServeStats)]
         l._sched_declared = True
     return l
 
@@ -438,7 +440,7 @@ class BatchFormer:
         self._l.pllm_sched_future_page_usage(self._h, out.ctypes.data_as(C.POINTER(C.c_int64)), n)
         return out
 
-    def serve(self, skip_cycles, run_cycles) -> ServeStats:
+    def serve(self, skip_cycles, run_cycles, warmup_cycles=0) -> ServeStats:
         st = ServeStats()
-        _check(self._l.pllm_serve(self._h, skip_cycles, run_cycles, C.byref(st)), "serve")
+        _check(self._l.pllm_serve(self._h, skip_cycles, warmup_cycles, run_cycles, C.byref(st)), "serve")
         return st
