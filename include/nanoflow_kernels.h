@@ -65,12 +65,27 @@ NF_API int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, 
 NF_API int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
                        int M, int N, int K, nf_stream_t stream);
 
-/* D = half(alpha * scale[n] * A.dequant(Bq) + beta * C) with Bq [K,N] OCP fp8 e4m3
- * bytes and one fp32 scale per output channel.  No counterpart in the reference
- * (its GEMM wrappers are half-only, pipeline/include/cutlassGemmWrapperImpl.cuh:24-27);
- * same operand roles as nf_gemm_f16. */
-NF_API int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* scale, const uint16_t* C,
-                    uint16_t* D, int M, int N, int K, float alpha, float beta, nf_stream_t stream);
+/* fp8 GEMM family (OCP e4m3: bias 7, no infinities, max 448) on the fp8 matrix cores.  No
+ * counterpart in the reference (its GEMM wrappers are half-only,
+ * pipeline/include/cutlassGemmWrapperImpl.cuh:24-27); operand roles as in nf_gemm_f16.
+ *
+ * nf_quantize_rows_e4m3: row_scale[m] = max_k |X[m][k]| / 448 (1 for an all-zero row),
+ *   Xq[m][k] = e4m3(X[m][k] / row_scale[m]), round to nearest even.  X fp16 [M,K], K % 16 == 0.
+ * nf_gemm_f8_f16: D = half(alpha * a_scale[m] * b_scale[n] * sum_k Aq[m][k] * Bq[n][k] + beta * C)
+ *   with Aq [M,K] and Bq [N,K] e4m3 bytes (weights stored one row per output channel, k
+ *   contiguous), fp32 accumulation.  K % 16 == 0, N % 8 == 0.
+ * nf_gemm_f8w_f16: fp16 activations against fp8 weights = the two calls above, the quantised
+ *   activations and their scales living in `workspace` (nf_gemm_f8w_workspace_bytes(M, K)
+ *   bytes, 16-byte aligned). */
+NF_API int nf_quantize_rows_e4m3(const uint16_t* X, uint8_t* Xq, float* row_scale, int M, int K,
+                                 nf_stream_t stream);
+NF_API int nf_gemm_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, const float* b_scale,
+                          const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha, float beta,
+                          nf_stream_t stream);
+NF_API size_t nf_gemm_f8w_workspace_bytes(int M, int K);
+NF_API int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* b_scale, const uint16_t* C,
+                           uint16_t* D, int M, int N, int K, float alpha, float beta, void* workspace,
+                           size_t workspace_bytes, nf_stream_t stream);
 
 /* Per token t of kqv [n_tokens,(Hq+2Hkv)*d] (columns K | V | Q): request
  * r = rev_input_indptr[t], position p = per_token_offset[t],

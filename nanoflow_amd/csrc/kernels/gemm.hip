@@ -391,12 +391,4 @@ int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t*
   return launch_gemm<128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
 }
 
-int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* scale, const uint16_t* C,
-                    uint16_t* D, int M, int N, int K, float alpha, float beta, nf_stream_t stream) {
-  (void)A; (void)Bq; (void)scale; (void)C; (void)D; (void)M; (void)N; (void)K; (void)alpha;
-  (void)beta; (void)stream;
-  set_error("nf_gemm_f8w_f16: fp8-weight GEMM kernel not built yet");
-  return NF_ERR_UNSUPPORTED;
-}
-
 }  // extern "C"

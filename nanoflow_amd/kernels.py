@@ -16,7 +16,8 @@ LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
 
 SYMBOLS = [
     "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16",
-    "nf_dual_swiglu_f16", "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
+    "nf_dual_swiglu_f16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
+    "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
 ]
 
@@ -44,7 +45,11 @@ def lib() -> C.CDLL:
         l.nf_rmsnorm_f16.argtypes = [vp, vp, vp, i32, i32, f32, vp]
         l.nf_gemm_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
-        l.nf_gemm_f8w_f16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp]
+        l.nf_quantize_rows_e4m3.argtypes = [vp, vp, vp, i32, i32, vp]
+        l.nf_gemm_f8_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp]
+        l.nf_gemm_f8w_workspace_bytes.restype = C.c_size_t
+        l.nf_gemm_f8w_workspace_bytes.argtypes = [i32, i32]
+        l.nf_gemm_f8w_f16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp, C.c_size_t, vp]
         l.nf_rope_append_f16.argtypes = [vp] * 7 + [i32] * 5 + [f32] * 4 + [vp]
         l.nf_attention_workspace_bytes.restype = sz
         l.nf_attention_workspace_bytes.argtypes = [i32, i32, i32]
@@ -123,15 +128,44 @@ def dual_swiglu(A, Bg, Bu, out=None):
     return out
 
 
-def gemm_f8w(A, Bq, scale, Cmat=None, alpha=1.0, beta=0.0, out=None):
+def quantize_rows_e4m3(X):
+    """fp16 [M,K] -> (e4m3 bytes [M,K], fp32 row scales [M])."""
+    _f16(X)
+    M, K = X.shape
+    Xq = torch.empty((M, K), dtype=torch.uint8, device=X.device)
+    scale = torch.empty((M,), dtype=torch.float32, device=X.device)
+    _check(lib().nf_quantize_rows_e4m3(_p(X), _p(Xq), _p(scale), M, K, _stream()), "nf_quantize_rows_e4m3")
+    return Xq, scale
+
+
+def gemm_f8(Aq, a_scale, Bq_nk, b_scale, Cmat=None, alpha=1.0, beta=0.0, out=None):
+    """Aq e4m3 bytes [M,K], Bq_nk e4m3 bytes [N,K] (one row per output channel)."""
+    assert Aq.dtype == torch.uint8 and Bq_nk.dtype == torch.uint8
+    assert a_scale.dtype == torch.float32 and b_scale.dtype == torch.float32
+    M, K = Aq.shape
+    N = Bq_nk.shape[0]
+    assert tuple(Bq_nk.shape) == (N, K) and a_scale.numel() == M and b_scale.numel() == N
+    assert Aq.is_contiguous() and Bq_nk.is_contiguous()
+    out = torch.empty((M, N), dtype=torch.float16, device=Aq.device) if out is None else out
+    _check(lib().nf_gemm_f8_f16(_p(Aq), _p(a_scale), _p(Bq_nk), _p(b_scale), _p(Cmat), _p(out), M, N, K,
+                                alpha, beta, _stream()), "nf_gemm_f8_f16")
+    return out
+
+
+def gemm_f8w(A, Bq_nk, b_scale, Cmat=None, alpha=1.0, beta=0.0, out=None, workspace=None):
+    """fp16 activations [M,K] against e4m3 weights [N,K] with per-output-channel scales."""
     _f16(A)
-    assert Bq.dtype in (torch.uint8, torch.float8_e4m3fn) and scale.dtype == torch.float32
+    assert Bq_nk.dtype == torch.uint8 and b_scale.dtype == torch.float32 and Bq_nk.is_contiguous()
     M, K = A.shape
-    N = Bq.shape[1]
-    assert tuple(Bq.shape) == (K, N) and scale.numel() == N
+    N = Bq_nk.shape[0]
+    assert tuple(Bq_nk.shape) == (N, K) and b_scale.numel() == N
+    need = lib().nf_gemm_f8w_workspace_bytes(M, K)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
     out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
-    _check(lib().nf_gemm_f8w_f16(_p(A), _p(Bq), _p(scale), _p(Cmat), _p(out), M, N, K, alpha, beta,
-                                 _stream()), "nf_gemm_f8w_f16")
+    _check(lib().nf_gemm_f8w_f16(_p(A), _p(Bq_nk), _p(b_scale), _p(Cmat), _p(out), M, N, K, alpha, beta,
+                                 _p(workspace), workspace.numel() * workspace.element_size(), _stream()),
+           "nf_gemm_f8w_f16")
     return out
 
 

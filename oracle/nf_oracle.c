@@ -229,6 +229,57 @@ static inline float e4m3_to_float(uint8_t v) {
 }
 NFO_API float nfo_e4m3_to_float(uint8_t v) { return e4m3_to_float(v); }
 
+/* Nearest e4m3 code, ties to the even code, saturating at +-448 (NaN also lands there).
+ * Written as a search over the 127 finite magnitudes so that it shares nothing with the
+ * arithmetic encoders it checks. */
+static inline uint8_t float_to_e4m3(float x) {
+  uint8_t sign = signbit(x) ? 0x80 : 0;
+  float a = fabsf(x);
+  if (!(a < 448.f)) return sign | 0x7E;
+  int lo = 0, hi = 0x7E; /* decode(lo) <= a < decode(hi) */
+  while (hi - lo > 1) {
+    int mid = (lo + hi) / 2;
+    if (e4m3_to_float((uint8_t)mid) <= a) lo = mid; else hi = mid;
+  }
+  double dl = (double)a - (double)e4m3_to_float((uint8_t)lo);
+  double dh = (double)e4m3_to_float((uint8_t)hi) - (double)a;
+  int code = dl < dh ? lo : dh < dl ? hi : ((lo & 1) ? hi : lo);
+  return sign | (uint8_t)code;
+}
+NFO_API uint8_t nfo_float_to_e4m3(float x) { return float_to_e4m3(x); }
+
+/* Per-row dynamic activation quantisation: scale = amax / 448 (1 for a zero row),
+ * q = e4m3(x / scale), both in fp32. */
+NFO_API void nfo_quantize_rows_e4m3(const uint16_t* X, uint8_t* Xq, float* scale, int M, int K) {
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; ++m) {
+    float amax = 0.f;
+    for (int k = 0; k < K; ++k) amax = fmaxf(amax, fabsf(h2f(X[(size_t)m * K + k])));
+    float s = amax > 0.f ? amax / 448.f : 1.f;
+    scale[m] = s;
+    for (int k = 0; k < K; ++k) Xq[(size_t)m * K + k] = float_to_e4m3(h2f(X[(size_t)m * K + k]) / s);
+  }
+}
+
+/* D = half(alpha * sa[m] * sb[n] * sum_k Aq[m][k] * Bq[n][k] + beta * C); both operands e4m3
+ * with k contiguous.  The products are exact in binary; the sum is taken in double. */
+NFO_API void nfo_gemm_f8f8_f16(const uint8_t* Aq, const float* sa, const uint8_t* Bq, const float* sb,
+                               const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha,
+                               float beta) {
+  float lut[256];
+  for (int i = 0; i < 256; ++i) lut[i] = e4m3_to_float((uint8_t)i);
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int m = 0; m < M; ++m)
+    for (int n = 0; n < N; ++n) {
+      double acc = 0.0;
+      for (int k = 0; k < K; ++k)
+        acc += (double)lut[Aq[(size_t)m * K + k]] * (double)lut[Bq[(size_t)n * K + k]];
+      float v = alpha * sa[m] * sb[n] * (float)acc;
+      if (beta != 0.f) v += beta * h2f(C[(size_t)m * N + n]);
+      D[(size_t)m * N + n] = f2h(v);
+    }
+}
+
 NFO_API void nfo_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* scale,
                               const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha,
                               float beta) {

@@ -94,6 +94,13 @@ def _declare(l):
     l.nfo_dual_swiglu_f16.restype = None
     l.nfo_dual_swiglu_f16.argtypes = [_u16p, _u16p, _u16p, _u16p, _u16p, _u16p, C.c_int, C.c_int,
                                       C.c_int]
+    l.nfo_float_to_e4m3.restype = C.c_uint8
+    l.nfo_float_to_e4m3.argtypes = [C.c_float]
+    l.nfo_quantize_rows_e4m3.restype = None
+    l.nfo_quantize_rows_e4m3.argtypes = [_u16p, _u8p, _f32p, C.c_int, C.c_int]
+    l.nfo_gemm_f8f8_f16.restype = None
+    l.nfo_gemm_f8f8_f16.argtypes = [_u8p, _f32p, _u8p, _f32p, _u16p, _u16p, C.c_int, C.c_int, C.c_int,
+                                    C.c_float, C.c_float]
     l.nfo_gemm_f8w_f16.restype = None
     l.nfo_gemm_f8w_f16.argtypes = [_u16p, _u8p, _f32p, _u16p, _u16p, C.c_int, C.c_int, C.c_int,
                                    C.c_float, C.c_float]
@@ -162,6 +169,32 @@ def gemm_f8w(A, Bq, scale, Cmat=None, alpha=1.0, beta=0.0):
 
 def e4m3_to_float(v: int) -> float:
     return lib().nfo_e4m3_to_float(v)
+
+
+def float_to_e4m3(x: float) -> int:
+    return int(lib().nfo_float_to_e4m3(float(x)))
+
+
+def quantize_rows_e4m3(X):
+    """X fp16 [M,K] -> (Xq uint8 [M,K], scale fp32 [M])."""
+    M, K = X.shape
+    Xq = np.empty((M, K), np.uint8)
+    scale = np.empty((M,), np.float32)
+    lib().nfo_quantize_rows_e4m3(_h(X), Xq.ctypes.data_as(_u8p), scale.ctypes.data_as(_f32p), M, K)
+    return Xq, scale
+
+
+def gemm_f8f8(Aq, sa, Bq_nk, sb, Cmat=None, alpha=1.0, beta=0.0):
+    """Aq uint8 [M,K], Bq_nk uint8 [N,K] (one row per output channel), fp32 scales."""
+    M, K = Aq.shape
+    N = Bq_nk.shape[0]
+    assert Aq.dtype == np.uint8 and Bq_nk.dtype == np.uint8 and Bq_nk.shape == (N, K)
+    Aq, Bq_nk = np.ascontiguousarray(Aq), np.ascontiguousarray(Bq_nk)
+    sa, sb = np.ascontiguousarray(sa, np.float32), np.ascontiguousarray(sb, np.float32)
+    D = np.empty((M, N), np.float16)
+    lib().nfo_gemm_f8f8_f16(Aq.ctypes.data_as(_u8p), sa.ctypes.data_as(_f32p), Bq_nk.ctypes.data_as(_u8p),
+                            sb.ctypes.data_as(_f32p), _h(Cmat), _h(D), M, N, K, alpha, beta)
+    return D
 
 
 def rmsnorm(x, w, eps=1e-5):

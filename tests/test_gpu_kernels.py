@@ -156,6 +156,75 @@ def test_dual_known_answer_inputs(K, oracle):
 
 # ---------------------------------------------------------------- RoPE + paged append
 
+F8_RTOL = 3e-2   # fp8 path: activations rounded to e4m3 (3 mantissa bits) on the way in
+
+
+def _quantize_weights_nk(W):
+    """fp32 [N,K] -> (e4m3 bytes [N,K], per-output-channel fp32 scales), scale = amax / 448."""
+    sc = (np.abs(W).max(axis=1) / 448.0).astype(np.float32)
+    q = torch.from_numpy(W / sc[:, None]).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    return q, sc
+
+
+@pytest.mark.parametrize("M,K_", [(1, 16), (5, 4096), (33, 144), (64, 28672)])
+def test_quantize_rows_e4m3_bit_exact(K, oracle, M, K_):
+    rng = np.random.default_rng(M * 7 + K_)
+    X = (rng.normal(0, 1, (M, K_)) * rng.uniform(0.01, 20, (M, 1))).astype(np.float16)
+    if M > 2:
+        X[2] = 0                                  # all-zero row: scale 1, codes 0
+        X[1, ::3] = 0
+    q_ref, s_ref = oracle.quantize_rows_e4m3(X)
+    q, s = K.quantize_rows_e4m3(dev(X))
+    assert np.array_equal(host(s), s_ref)
+    assert np.array_equal(host(q), q_ref)
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 8, 16), (37, 136, 144), (130, 520, 1040), (300, 264, 4096),
+                                     (64, 1024, 512), (256, 256, 128), (512, 2048, 384)])
+def test_gemm_f8_exact_products(K, oracle, M, N, K_):
+    """fp8 x fp8 with fp32 accumulation: the products are exact, so the result matches the
+    oracle (double accumulation) to fp16 rounding."""
+    rng = np.random.default_rng(M + N + K_)
+    fin = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], np.uint8)
+    Aq, Bq = rng.choice(fin, (M, K_)), rng.choice(fin, (N, K_))
+    # keep magnitudes moderate so that the sum does not ride on a few 448*448 products
+    Aq, Bq = (Aq & 0xBF).astype(np.uint8), (Bq & 0xBF).astype(np.uint8)
+    sa = rng.uniform(0.5, 2, M).astype(np.float32)
+    sb = rng.uniform(0.5, 2, N).astype(np.float32)
+    Cm = rng.normal(0, 1, (M, N)).astype(np.float16)
+    for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+        ref = oracle.gemm_f8f8(Aq, sa, Bq, sb, Cm if beta else None, alpha=alpha, beta=beta)
+        got = K.gemm_f8(dev(Aq), dev(sa), dev(Bq), dev(sb), dev(Cm) if beta else None, alpha=alpha, beta=beta)
+        assert_close(host(got), ref, what=f"gemm_f8 {M}x{N}x{K_} a={alpha} b={beta}")
+
+
+@pytest.mark.parametrize("M,N,K_", [(48, 256, 512), (200, 1024, 4096), (1, 4096, 4096)])
+def test_gemm_f8w_within_fp8_tolerance_of_dequantised_reference(K, oracle, M, N, K_):
+    rng = np.random.default_rng(N + K_)
+    A = rng.normal(0, 1, (M, K_)).astype(np.float16)
+    W = rng.normal(0, 0.02, (N, K_)).astype(np.float32)
+    Wq, sc = _quantize_weights_nk(W)
+    Cm = rng.normal(0, 1, (M, N)).astype(np.float16)
+    ref = oracle.gemm_f8w(A, np.ascontiguousarray(Wq.T), sc, Cm, alpha=1.0, beta=1.0)   # oracle takes [K,N]
+    got = host(K.gemm_f8w(dev(A), dev(Wq), dev(sc), dev(Cm), alpha=1.0, beta=1.0))
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    assert np.isfinite(got).all()
+    assert err.max() <= F8_RTOL * np.abs(ref).max(), (err.max(), np.abs(ref).max())
+    # and the two-step form gives the same bits as the fused entry point
+    q, s = K.quantize_rows_e4m3(dev(A))
+    two = host(K.gemm_f8(q, s, dev(Wq), dev(sc), dev(Cm), alpha=1.0, beta=1.0))
+    assert np.array_equal(two, got)
+
+
+def test_gemm_f8w_rejects_short_workspace(K):
+    from nanoflow_amd import kernels
+    A = torch.zeros((8, 64), dtype=torch.float16, device="cuda")
+    Wq = torch.zeros((16, 64), dtype=torch.uint8, device="cuda")
+    sc = torch.ones(16, dtype=torch.float32, device="cuda")
+    with pytest.raises(kernels.NanoflowKernelError, match="workspace"):
+        K.gemm_f8w(A, Wq, sc, workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+
+
 @pytest.mark.parametrize("Hq,Hkv,theta,scale,sa,sb", [
     (32, 8, 5e5, 1.0, 0.0, 0.0),
     (8, 2, 1e4, 1.0, 0.0, 0.0),

@@ -155,6 +155,74 @@ def test_gemm_f8w_is_dequantise_then_gemm(oracle):
 
 # ------------------------------------------------------------------ row ops
 
+def _finite_codes():
+    return [c for c in range(256) if (c & 0x7F) != 0x7F]
+
+
+def test_e4m3_encode_roundtrip_ties_and_saturation(oracle):
+    dec = {c: oracle.e4m3_to_float(c) for c in _finite_codes()}
+    # every finite code is a fixed point of decode -> encode (the sign of zero included)
+    for c, v in dec.items():
+        assert oracle.float_to_e4m3(v) == c, hex(c)
+    # between neighbours: nearest wins, the midpoint goes to the even code
+    for c in range(0, 0x7E):
+        lo, hi = dec[c], dec[c + 1]
+        mid = (lo + hi) / 2                           # exact in binary
+        even = c if c % 2 == 0 else c + 1
+        assert oracle.float_to_e4m3(mid) == even, hex(c)
+        assert oracle.float_to_e4m3(np.nextafter(np.float32(mid), np.float32(0))) == c
+        assert oracle.float_to_e4m3(np.nextafter(np.float32(mid), np.float32(1e9))) == c + 1
+        assert oracle.float_to_e4m3(-mid) == 0x80 | even
+    # saturation instead of NaN codes
+    for x, want in [(448.0, 0x7E), (463.9, 0x7E), (464.0, 0x7E), (1e6, 0x7E), (-1e6, 0xFE),
+                    (float("inf"), 0x7E), (2.0 ** -10, 0x00), (2.0 ** -10 * 1.01, 0x01), (1.0, 0x38)]:
+        assert oracle.float_to_e4m3(x) == want, x
+    # agrees with torch's converter wherever that one does not produce NaN
+    import torch
+    xs = np.random.default_rng(0).normal(0, 50, size=4000).astype(np.float32)
+    xs = xs[np.abs(xs) < 448]
+    t = torch.from_numpy(xs).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert [oracle.float_to_e4m3(float(x)) for x in xs] == t.tolist()
+
+
+def test_quantize_rows_e4m3_closed_form(oracle):
+    # a row made of representable values times a power of two, with 448 * 2^j present, quantises
+    # exactly: scale = 2^j and the codes are the values' own codes
+    codes = np.array([0x7E, 0x38, 0xB8, 0x01, 0x00, 0x45, 0xC9, 0x08] * 2, np.uint8)
+    vals = np.array([oracle.e4m3_to_float(int(c)) for c in codes], np.float32)
+    X = np.stack([vals * 2.0 ** -5, vals * 2.0 ** 3, np.zeros_like(vals)]).astype(np.float16)
+    assert np.array_equal(X[0].astype(np.float32), vals * 2.0 ** -5)      # fp16 holds them exactly
+    Xq, sc = oracle.quantize_rows_e4m3(X)
+    assert sc.tolist() == [2.0 ** -5, 2.0 ** 3, 1.0]
+    assert np.array_equal(Xq[0], codes) and np.array_equal(Xq[1], codes)
+    assert not Xq[2].any()
+    # general rows: |x - scale * decode(q)| <= half a step of the code's binade, max maps to 448
+    rng = np.random.default_rng(1)
+    X = (rng.normal(0, 1, (5, 64)) * np.array([[1e-3], [1], [30], [0.2], [7]])).astype(np.float16)
+    Xq, sc = oracle.quantize_rows_e4m3(X)
+    deq = np.vectorize(oracle.e4m3_to_float)(Xq) * sc[:, None]
+    assert np.array_equal((Xq & 0x7F).max(axis=1), np.full(5, 0x7E))
+    rel = np.abs(deq - X.astype(np.float32)) / np.maximum(np.abs(X.astype(np.float32)), sc[:, None] * 2.0 ** -6)
+    assert rel.max() <= 2.0 ** -4 + 1e-6
+
+
+def test_gemm_f8f8_matches_float64(oracle):
+    rng = np.random.default_rng(2)
+    M, N, K = 9, 24, 80
+    fin = np.array(_finite_codes(), np.uint8)
+    Aq, Bq = rng.choice(fin, (M, K)), rng.choice(fin, (N, K))
+    sa, sb = rng.uniform(0.01, 0.1, M).astype(np.float32), rng.uniform(0.001, 0.01, N).astype(np.float32)
+    Cm = rng.normal(0, 1, (M, N)).astype(np.float16)
+    lut = np.array([oracle.e4m3_to_float(c) if (c & 0x7F) != 0x7F else 0.0 for c in range(256)])
+    ref = 0.5 * (sa[:, None] * sb[None, :]).astype(np.float64) * (lut[Aq] @ lut[Bq].T) + 2.0 * Cm.astype(np.float64)
+    got = oracle.gemm_f8f8(Aq, sa, Bq, sb, Cm, alpha=0.5, beta=2.0).astype(np.float64)
+    assert np.abs(got - ref).max() <= 1e-3 * np.abs(ref).max()
+    # transposing the roles of the operands transposes the result
+    g1 = oracle.gemm_f8f8(Aq, sa, Bq, sb)
+    g2 = oracle.gemm_f8f8(Bq, sb, Aq, sa)
+    assert np.array_equal(g1, g2.T)
+
+
 def test_rmsnorm_closed_form(oracle):
     rng = np.random.default_rng(5)
     x = synth.normal_f16(rng, (11, 256), 3.0)
