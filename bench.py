@@ -153,6 +153,7 @@ def run_iteration(args):
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, run_layer=shape.layers,
                         distinct_layers=distinct, seed=args.seed, profiling=args.profile_level)
+    P.setGraphMode(args.graph)
     eng.update(batch)
     torch.cuda.synchronize()
     t_setup = time.perf_counter() - t_setup
@@ -238,6 +239,7 @@ def run_offline(args):
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, seed=args.seed,
                         profiling=args.profile_level, kv_fill="zeros")
+    P.setGraphMode(args.graph)
     former = P.BatchFormer(pages, shape.page_size, T, args.nano1, args.kqv1, args.kqv3, in_len, out_len)
     rng = np.random.default_rng(args.seed)
     for i in range(n_req):
@@ -311,6 +313,7 @@ def run_offline(args):
             "decode_attention_ms_per_cycle": tm.decode_attn_ms / max(st.cycles, 1),
             "prefill_attention_ms_per_cycle": tm.prefill_attn_ms / max(st.cycles, 1),
             "gemm_ms_per_cycle": tm.gemm_ms / max(st.cycles, 1),
+            "graph_counters": P.getGraphCounters(),
             "requests_left": state["queued"] + state["decoding"] + state["prefilling"],
             "setup_s": t_setup,
         },
@@ -344,10 +347,14 @@ def main():
     ap.add_argument("--kv-pages", type=int, default=0, help="offline workload: KV pool pages (0 = sized to HBM)")
     ap.add_argument("--profile-level", type=int, default=2, choices=[0, 1, 2],
                     help="per-launch events: 1 attention, 2 attention and GEMMs")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay iterations from captured hipGraphs (disables per-launch profiling)")
     ap.add_argument("--cpu-sample", type=int, default=96, help="decode requests in the CPU baseline (0 = skip)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     _check_single_gpu(args)
+    if args.graph:
+        args.profile_level = 0
     rec = run_offline(args) if args.workload == "offline" else run_iteration(args)
     print(json.dumps(rec))
 

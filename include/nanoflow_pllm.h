@@ -225,6 +225,14 @@ typedef struct nf_pipeline_timings {
 } nf_pipeline_timings;
 NF_PLLM_API int pllm_set_profiling(int on);
 NF_PLLM_API int pllm_get_timings(nf_pipeline_timings* out);
+/* hipGraph replay (the reference carries a graph switch that is compiled off, `constexpr bool
+ * enableGraph = false`, pipeline_local.cu:319-327, and only its capture events remain).  With graph mode on, an iteration whose launch signature
+ * (decode rows, prefill requests and tokens, the four attention group sizes and block caps) has
+ * been seen before is captured once and replayed afterwards; the first occurrence of a
+ * signature runs eagerly.  Profiling (level > 0) takes precedence and disables replay.
+ * counters = {iterations run eagerly, graphs captured, iterations replayed}. */
+NF_PLLM_API int pllm_set_graph_mode(int on);
+NF_PLLM_API int pllm_get_graph_counters(long counters[3]);
 NF_PLLM_API int pllm_reset_timings(void);
 /* Device address of an intermediate of the current pipeline, for parity checks:
  * name in {"hidden" (residual stream after the last layer, [T, hidden]),

@@ -20,6 +20,7 @@ static std::unique_ptr<SimpleThreadSync> global_sync;  // workers + the caller's
 static vortexInitData* persistant_input = nullptr;
 static std::vector<int> complete_input_tokens;
 static int g_profiling = 0;
+static bool g_graph_mode = false;
 
 int buildInputTokens(const int* prev_output, int prev_count, const int32_t* keep_token_list,
                      int keep_token_list_length, const int* prefill_tokens, int prefill_tokens_num,
@@ -122,6 +123,11 @@ void finalize() {
 
 PipelineBase* currentPipeline() { return workers.empty() ? nullptr : workers[0]->getPipeline(); }
 
+void setPipelineGraphMode(bool on) {
+  g_graph_mode = on;
+  if (auto* p = currentPipeline()) p->setGraphMode(on);
+}
+
 void setPipelineProfiling(int level) {
   g_profiling = level;
   if (auto* p = currentPipeline()) p->setProfiling(level);
@@ -150,6 +156,7 @@ void Worker::init() {
   else
     NF_LOG_ERROR("Unknown pipeline type %d", static_cast<int>(PipeTy));
   if (pipeline && g_profiling) pipeline->setProfiling(g_profiling);
+  if (pipeline && g_graph_mode) pipeline->setGraphMode(true);
 }
 
 void Worker::run_pipeline() { *output = pipeline->run(); }

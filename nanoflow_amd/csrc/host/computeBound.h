@@ -115,3 +115,6 @@ int buildInputTokens(const int* prev_output, int prev_count, const int32_t* keep
 // Access for measurement code: the rank-0 pipeline (nullptr before init()).
 PipelineBase* currentPipeline();
 void setPipelineProfiling(int level);
+// Replay iterations from captured hipGraphs (one per launch signature) instead of enqueueing
+// every launch; takes effect for the current and for later pipelines.
+void setPipelineGraphMode(bool on);

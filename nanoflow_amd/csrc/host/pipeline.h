@@ -20,6 +20,9 @@
 #include "otherWrapper.h"
 #include "vortexData.h"
 
+#include <map>
+#include <set>
+
 #define SET_NAME_PTR(var) (var)->name = #var;
 #define SET_NAME_REF(var) (var).name = #var;
 #define GEMM_ALIAS(x) BaseGEMMWrapper*& x = gemms[static_cast<int>(GEMM_NAME::x)]
@@ -56,6 +59,61 @@ protected:
   bool profile_gemms = false;
   PipelineTimings timings;
 
+  // hipGraph replay of an iteration.  Everything that shapes a launch (grid sizes, row counts,
+  // which operators are skipped) is a function of the configuration and of a few integers of
+  // the update data; those integers form the signature a captured graph is filed under.  A
+  // signature runs eagerly the first time it is seen (one-time kernel attribute calls must not
+  // happen inside a capture), is captured the second time, and is replayed from then on.
+  // Per-launch profiling brackets cannot be read back from a replay, so profiling disables it.
+  bool graph_mode = false;
+  std::map<std::vector<int>, hipGraphExec_t> graph_execs;
+  std::set<std::vector<int>> graph_seen;
+  long graph_replays = 0, graph_captures = 0, graph_eager = 0;
+  static constexpr size_t kMaxGraphs = 64;
+
+  template <class F>
+  void runIteration(hipStream_t origin, const std::vector<int>& sig, F&& enqueue) {
+    if (!graph_mode || profiling) {
+      ++graph_eager;
+      enqueue();
+      return;
+    }
+    auto it = graph_execs.find(sig);
+    if (it == graph_execs.end()) {
+      if (!graph_seen.count(sig) || graph_execs.size() >= kMaxGraphs) {
+        graph_seen.insert(sig);
+        ++graph_eager;
+        enqueue();
+        return;
+      }
+      hipGraph_t graph = nullptr;
+      HIP_CHECK(hipStreamBeginCapture(origin, hipStreamCaptureModeRelaxed));
+      enqueue();
+      HIP_CHECK(hipStreamEndCapture(origin, &graph));
+      hipGraphExec_t exec = nullptr;
+      HIP_CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+      HIP_CHECK(hipGraphDestroy(graph));
+      it = graph_execs.emplace(sig, exec).first;
+      ++graph_captures;
+    }
+    HIP_CHECK(hipGraphLaunch(it->second, origin));
+    ++graph_replays;
+  }
+  void clearGraphs() {
+    for (auto& kv : graph_execs) (void)hipGraphExecDestroy(kv.second);
+    graph_execs.clear();
+    graph_seen.clear();
+  }
+  std::vector<int> baseSignature() const {
+    std::vector<int> s = {host_update_data.decodePrefillBorder, host_update_data.prefillNum,
+                          host_update_data.prefillTokensNum};
+    for (int i = 0; i < 4; ++i) {
+      s.push_back(host_update_data.gemv_batch_size ? host_update_data.gemv_batch_size[i] : 0);
+      s.push_back(host_update_data.gemv_num_blocks ? host_update_data.gemv_num_blocks[i] : 0);
+    }
+    return s;
+  }
+
 public:
   virtual vortexOutputData run() = 0;
   virtual void update(vortexUpdateData* update_data) = 0;
@@ -68,6 +126,15 @@ public:
   int profilingLevel() const { return profiling ? (profile_gemms ? 2 : 1) : 0; }
   const PipelineTimings& getTimings() const { return timings; }
   void resetTimings() { timings = PipelineTimings(); }
+  void setGraphMode(bool on) {
+    graph_mode = on;
+    if (!on) clearGraphs();
+  }
+  void graphCounters(long out[3]) const {
+    out[0] = graph_eager;
+    out[1] = graph_captures;
+    out[2] = graph_replays;
+  }
   void setHostUpdate(const vortexUpdateData& h) { host_update_data = h; }
 };
 

@@ -58,6 +58,7 @@ LocalPipeline::LocalPipeline(vortexInitData* input_data, int nrank, int nranks, 
 }
 
 LocalPipeline::~LocalPipeline() {
+  clearGraphs();
   for (auto g : gemms) delete g;
   delete[] output_data.sampled_token_array;
   if (prefill1_update.input_indptr) (void)hipFree(prefill1_update.input_indptr);
@@ -374,13 +375,16 @@ void LocalPipeline::enqueueIteration() {
   layerNormModel.run();
   LOGITS->run();
   maxSampler.run();
+  // the attention stream rejoins the dense stream (all of its launches are already ordered
+  // before O1/O2; a capture needs the join to be explicit)
   HIP_CHECK(hipEventRecord(events[EventManager::CAPTURE_GEMV_END], stream_gemv));
+  HIP_CHECK(hipStreamWaitEvent(stream_gemm, events[EventManager::CAPTURE_GEMV_END], 0));
 }
 
 vortexOutputData LocalPipeline::run() {
   setWeight(0);
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_START], stream_gemm));
-  enqueueIteration();
+  runIteration(stream_gemm, baseSignature(), [this] { enqueueIteration(); });
   // the sampler (stream_gemm) depends on every attention launch through O1/O2
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_END], stream_gemm));
   HIP_CHECK(hipMemcpyAsync(output_data.sampled_token_array, maxSampler.d_argMax.ptr,
@@ -580,6 +584,7 @@ double LocalPipeline::totalCompute() {
 
 void LocalPipeline::config(vortexConfigData* config_data_) {
   NF_LOG_INFO("Config local pipeline");
+  clearGraphs();  // the buffer plan below may move every operand
   this->config_data = *config_data_;
   for (int i = 0; i < gemmNum; ++i) {
     const std::string& tag =

@@ -12,6 +12,7 @@ NonOverlapLocalPipeline::NonOverlapLocalPipeline(vortexInitData* input_data, int
 }
 
 NonOverlapLocalPipeline::~NonOverlapLocalPipeline() {
+  clearGraphs();
   for (auto g : gemms) delete g;
   delete[] output_data.sampled_token_array;
   if (stream_all) (void)hipStreamDestroy(stream_all);
@@ -34,23 +35,25 @@ void NonOverlapLocalPipeline::setProfiling(int level) {
 vortexOutputData NonOverlapLocalPipeline::run() {
   setWeight(0);
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_START], stream_all));
-  genEmbedding.run();
-  for (int iter = 0; iter < ModelConfig.run_layer; ++iter) {
-    setWeight(iter % ModelConfig.model_layer);
-    layerNormAttention.run();
-    KQV->run();
-    roPEAppend.run();
-    if (GEMV.batch_size > 0) GEMV.run();
-    if (update_data.prefillNum > 0) prefill.run();
-    O->run();
-    layerNormFFN.run();
-    dual.run();
-    D->run();
-  }
-  keepToken.run();
-  layerNormModel.run();
-  LOGITS->run();
-  maxSampler.run();
+  runIteration(stream_all, baseSignature(), [this] {
+    genEmbedding.run();
+    for (int iter = 0; iter < ModelConfig.run_layer; ++iter) {
+      setWeight(iter % ModelConfig.model_layer);
+      layerNormAttention.run();
+      KQV->run();
+      roPEAppend.run();
+      if (GEMV.batch_size > 0) GEMV.run();
+      if (update_data.prefillNum > 0) prefill.run();
+      O->run();
+      layerNormFFN.run();
+      dual.run();
+      D->run();
+    }
+    keepToken.run();
+    layerNormModel.run();
+    LOGITS->run();
+    maxSampler.run();
+  });
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_END], stream_all));
   HIP_CHECK(hipMemcpyAsync(output_data.sampled_token_array, maxSampler.d_argMax.ptr,
                            output_data.sampled_tokens * sizeof(int), hipMemcpyDeviceToHost,
@@ -95,6 +98,7 @@ void NonOverlapLocalPipeline::update(vortexUpdateData* update_data_) {
 
 void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
   NF_LOG_INFO("Config non-overlap local pipeline");
+  clearGraphs();  // the buffer plan below may move every operand
   this->config_data = *config_data_;
   for (int i = 0; i < gemmNum; ++i) {
     const std::string& tag =

@@ -289,6 +289,19 @@ int pllm_set_profiling(int on) {
   return NF_PLLM_OK;
 }
 
+int pllm_set_graph_mode(int on) {
+  if (g_running) return fail(NF_PLLM_ERR_STATE, "pllm_set_graph_mode: a run is in flight");
+  setPipelineGraphMode(on != 0);
+  return NF_PLLM_OK;
+}
+
+int pllm_get_graph_counters(long counters[3]) {
+  PipelineBase* p = currentPipeline();
+  if (!p || !counters) return fail(NF_PLLM_ERR_STATE, "pllm_get_graph_counters: no pipeline");
+  p->graphCounters(counters);
+  return NF_PLLM_OK;
+}
+
 int pllm_get_timings(nf_pipeline_timings* out) {
   PipelineBase* p = currentPipeline();
   if (!p || !out) return fail(NF_PLLM_ERR_STATE, "pllm_get_timings: no pipeline");

@@ -179,7 +179,7 @@ SYMBOLS = [
     "pllm_max_page_num", "pllm_init", "pllm_model_weight_to_gpu", "pllm_config", "pllm_update",
     "pllm_run", "pllm_run_async", "pllm_run_async_wait", "pllm_get_pipeline_output",
     "pllm_finalize", "pllm_build_input_tokens", "pllm_set_profiling", "pllm_get_timings",
-    "pllm_reset_timings", "pllm_debug_buffer",
+    "pllm_reset_timings", "pllm_debug_buffer", "pllm_set_graph_mode", "pllm_get_graph_counters",
 ]
 
 _lib = None
@@ -308,6 +308,17 @@ def buildInputTokens(prev_output, keep_token_list, prefill_tokens) -> np.ndarray
 def setProfiling(level):
     """0/False: off; 1/True: attention launches are timed; 2: dense GEMM launches as well."""
     _check(lib().pllm_set_profiling(int(level)), "setProfiling")
+
+
+def setGraphMode(on: bool):
+    """Replay iterations from captured hipGraphs (one per launch signature)."""
+    _check(lib().pllm_set_graph_mode(int(bool(on))), "setGraphMode")
+
+
+def getGraphCounters() -> dict:
+    c = (C.c_long * 3)()
+    _check(lib().pllm_get_graph_counters(c), "getGraphCounters")
+    return dict(eager=c[0], captured=c[1], replayed=c[2])
 
 
 def getTimings() -> PipelineTimings:

@@ -240,3 +240,49 @@ def test_serve_skip_cycles_reach_steady_state_without_gpu_work():
     assert stats.cycles == 8
     assert stats.tokens_processed > 6 * T       # the timed cycles run (nearly) full batches
     assert stats.gpu_iter_ms > 0 and stats.cycle_ms > 0
+
+
+@pytest.mark.parametrize("pt_name", ["LOCAL", "NON_OVERLAP_LOCAL"])
+def test_graph_replay_is_identical_to_eager(pt_name):
+    """The same sequence of iterations, eagerly and with hipGraph replay (two launch signatures,
+    several replays each, with other device work and synchronisations in between): sampled ids
+    and the residual stream must be identical step by step."""
+    from nanoflow_amd import engine, pllm_python as P
+    pt = P.PipelineType[pt_name]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=4)
+    T, nano1 = 96, 40
+    b1 = synth.make_batch([5, 17, 33, 64, 20, 9], [(0, 50)], vocab=shape.vocab, seed=31, extra_pages=8)
+    b2 = synth.make_batch([7, 12, 40, 3, 28], [(16, 30), (0, 21)], vocab=shape.vocab, seed=32, extra_pages=8)
+    pages = max(b1.num_pages, b2.num_pages)
+    rng = np.random.default_rng(9)
+    big = synth.ModelShape(**{**shape.as_dict()})
+    pools0 = [synth.make_kv_pool(pages, big, rng) for _ in range(shape.layers)]
+    keep = {id(b1): np.array([1, 1, 1, 1, 1, 1, 0], np.int32), id(b2): np.array([1, 1, 1, 1, 1, 0, 0], np.int32)}
+    order = [b1, b1, b1, b2, b2, b1, b2, b2, b1, b1]
+
+    def run_sequence(graph):
+        outs = []
+        with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=20, kqv3=28, kv_pages=pages,
+                           weights=w, kv_pools=pools0) as e:
+            P.setGraphMode(graph)
+            scratch = torch.zeros(1 << 16, device="cuda")
+            for i, b in enumerate(order):
+                print(f"graph={graph} {pt_name} step={i}", flush=True)
+                e.update(b, keep_token_list=np.ones(b.decodePrefillBorder, np.int32) if i == 0 else keep[id(b)])
+                s = e.run()
+                h = e.buffer("hidden").cpu().numpy()[:b.tokens]
+                outs.append((s.copy(), h))
+                scratch.add_(1.0)                       # unrelated eager work between replays
+                torch.cuda.synchronize()
+            counters = P.getGraphCounters()
+            P.setGraphMode(False)
+        return outs, counters
+
+    eager, c0 = run_sequence(False)
+    replay, c1 = run_sequence(True)
+    assert c0["captured"] == 0 and c0["replayed"] == 0 and c0["eager"] == len(order)
+    assert c1["captured"] == 2 and c1["eager"] == 2 and c1["replayed"] == len(order) - 2, c1
+    for i, ((s0, h0), (s1, h1)) in enumerate(zip(eager, replay)):
+        assert np.array_equal(s0, s1), (i, "sampled ids")
+        assert np.array_equal(h0, h1), (i, "residual stream")
