@@ -200,8 +200,8 @@ def run_iteration(args):
         "roofline": _attention_roofline(tm, bytes_per_layer / launches_per_layer),
         "iteration": {
             "device_ms_last": tm.iter_ms, "ms_per_step_with_update": ms_with_update,
-            "decode_attention_ms_per_step": tm.decode_attn_ms / steps,
-            "prefill_attention_ms_per_step": tm.prefill_attn_ms / steps,
+            "decode_attention_ms_per_step": tm.decode_attn_ms * tm.layer_stride / steps,
+            "prefill_attention_ms_per_step": tm.prefill_attn_ms * tm.layer_stride / steps,
             "gemm_tflop_per_step": flops / 1e12,
             "gemm_mfma_frac_if_serial": (flops / 1e12) / (max(ms_per_step, 1e-9) * 1e-3) / MFMA_PEAK_TFLOPS,
             "setup_s": t_setup, "sampled_tokens": int(out.shape[0]),
@@ -209,7 +209,7 @@ def run_iteration(args):
     }
     if tm.gemm_launches:
         rec["roofline_gemm"] = _gemm_roofline(tm)
-        rec["iteration"]["gemm_ms_per_step"] = tm.gemm_ms / steps
+        rec["iteration"]["gemm_ms_per_step"] = tm.gemm_ms * tm.layer_stride / steps
     eng.close()
     if args.cpu_sample > 0:
         rec["cpu_baseline"] = cpu_baseline(shape, batch.kv_len[:args.cpu_sample], [], nd, args.seed)
@@ -310,9 +310,10 @@ def run_offline(args):
             "cpu_form_hidden_fraction": (1.0 - min(1.0, max(0.0, st.cycle_ms - st.gpu_iter_ms - st.update_ms)
                                                    / st.form_ms) if st.form_ms > 0 else None),
             "steady_state_decode_rows": int(nd), "steady_state_prefill_rows": int(nxt["prefillTokensNum"]),
-            "decode_attention_ms_per_cycle": tm.decode_attn_ms / max(st.cycles, 1),
-            "prefill_attention_ms_per_cycle": tm.prefill_attn_ms / max(st.cycles, 1),
-            "gemm_ms_per_cycle": tm.gemm_ms / max(st.cycles, 1),
+            "decode_attention_ms_per_cycle": tm.decode_attn_ms * tm.layer_stride / max(st.cycles, 1),
+            "prefill_attention_ms_per_cycle": tm.prefill_attn_ms * tm.layer_stride / max(st.cycles, 1),
+            "gemm_ms_per_cycle": tm.gemm_ms * tm.layer_stride / max(st.cycles, 1),   # LM head: timed 1 iteration in layer_stride
+            "timed_layer_stride": tm.layer_stride,
             "graph_counters": P.getGraphCounters(),
             "requests_left": state["queued"] + state["decoding"] + state["prefilling"],
             "setup_s": t_setup,

@@ -222,6 +222,7 @@ typedef struct nf_pipeline_timings {
   double gemm_ms;    /* dense GEMM launches (level 2): summed duration, count, flops */
   long gemm_launches;
   double gemm_flop;
+  int layer_stride;  /* every layer_stride-th layer is timed: totals per iteration = sums * layer_stride */
 } nf_pipeline_timings;
 NF_PLLM_API int pllm_set_profiling(int on);
 NF_PLLM_API int pllm_get_timings(nf_pipeline_timings* out);

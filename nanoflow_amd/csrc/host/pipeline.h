@@ -37,6 +37,7 @@ struct PipelineTimings {
   double gemm_ms = 0;        // sum of dense GEMM launch durations (profiling level 2)
   long gemm_launches = 0;
   double gemm_flop = 0;      // flops of those launches (2*M*N*K each; the fused gate/up pair 4*M*N*K)
+  int layer_stride = 1;      // every layer_stride-th layer's launches are the timed ones
 };
 
 class PipelineBase {
@@ -125,7 +126,11 @@ public:
   virtual void setProfiling(int level) { profiling = level > 0; profile_gemms = level > 1; }
   int profilingLevel() const { return profiling ? (profile_gemms ? 2 : 1) : 0; }
   const PipelineTimings& getTimings() const { return timings; }
-  void resetTimings() { timings = PipelineTimings(); }
+  void resetTimings() {
+    const int stride = timings.layer_stride;
+    timings = PipelineTimings();
+    timings.layer_stride = stride;
+  }
   void setGraphMode(bool on) {
     graph_mode = on;
     if (!on) clearGraphs();

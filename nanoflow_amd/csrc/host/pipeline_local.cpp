@@ -122,6 +122,7 @@ void LocalPipeline::setProfiling(int level) {
   profile_gemms = level > 1;
   // long schedules time every 4th layer: the event records themselves cost device time
   const unsigned stride = ModelConfig.run_layer >= 8 ? 4 : 1;
+  timings.layer_stride = (int)stride;
   const size_t n = profiling ? (size_t)ModelConfig.run_layer : 0;
   for (auto gemv : gemvs) gemv->enableProfiling(n, stride);
   prefill1.enableProfiling(n, stride);

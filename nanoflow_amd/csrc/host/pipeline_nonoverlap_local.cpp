@@ -23,6 +23,7 @@ void NonOverlapLocalPipeline::setProfiling(int level) {
   profile_gemms = level > 1;
   // long schedules time every 4th layer: the event records themselves cost device time
   const unsigned stride = ModelConfig.run_layer >= 8 ? 4 : 1;
+  timings.layer_stride = (int)stride;
   const size_t n = profiling ? (size_t)ModelConfig.run_layer : 0;
   GEMV.enableProfiling(n, stride);
   prefill.enableProfiling(n, stride);

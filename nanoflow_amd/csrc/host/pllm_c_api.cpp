@@ -314,6 +314,7 @@ int pllm_get_timings(nf_pipeline_timings* out) {
   out->gemm_ms = t.gemm_ms;
   out->gemm_launches = t.gemm_launches;
   out->gemm_flop = t.gemm_flop;
+  out->layer_stride = t.layer_stride;
   return NF_PLLM_OK;
 }
 

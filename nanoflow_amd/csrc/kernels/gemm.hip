@@ -5,54 +5,70 @@
 //
 // Workgroup = 256 threads = 4 wavefronts in a WM x WN grid; each wavefront owns a
 // (BM/WM) x (BN/WN) block of 32x32 MFMA tiles.  K is walked in slabs of 64 through two LDS
-// stages: while the MFMAs of slab i run out of LDS stage i&1, the global loads of slab i+1
-// are in flight into registers and are written to the other stage afterwards (one barrier per
-// slab).
+// stages.
 //
-// LDS layouts (both conflict-free for the accesses used):
-//   A slab  As[BM][64+8]           row = m, k contiguous; 16-byte fragment reads.
-//   B slab  Bs[16][BN+2][4]        "k-quad major": quad q holds k = 4q..4q+3 for every n as one
-//                                  8-byte cell.  A row-major [K,N] weight tile is loaded as
-//                                  4(k) x 8(n) register blocks (four coalesced 16-byte loads),
-//                                  transposed in registers with 16 byte-permutes and stored as
-//                                  64 contiguous bytes; an MFMA operand is two 8-byte reads.
+// Operands go from global memory STRAIGHT INTO LDS (buffer_load_dwordx4 ... lds): a CU moves
+// about 38 GB/s through the load-to-register path but well over 100 GB/s through this one, and
+// a 256x256 tile needs ~60 GB/s per CU to keep the matrix pipe busy.  One such instruction
+// writes 64 lanes x 16 bytes to 1 KB of consecutive LDS, so the LDS image cannot be padded;
+// bank conflicts are avoided by choosing WHICH 16-byte chunk each lane fetches (an XOR swizzle
+// applied on the global side):
+//   A slab (and [N][K] weights)  rows of 128 bytes (64 k), 8 rows per instruction; row r keeps
+//       logical chunk c at position c ^ (r & 7).  An MFMA fragment is one 16-byte read; the 8
+//       lanes of a read phase hit 8 different positions.
+//   [K][N] weights               kept row-major, 64 rows of BN*2 bytes; row r keeps chunk c at
+//       position c ^ ((r & 3) << 1).  The k-contiguous MFMA operand is produced by the
+//       transposing LDS read (ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(n) block row-wise
+//       and receive it column-wise), two per operand; the 4 rows of a block sit in 4 different
+//       32-byte bank groups.
+// No staging registers, no permutes, no LDS stores.  While the MFMAs of slab i run out of one
+// stage, the loads of slab i+1 are in flight into the other; one barrier per slab.
 //
 // The MFMA is issued as D^T = B^T.A^T (weights as the first operand) so that each lane ends up
 // with 4 consecutive output columns of one row -> 8-byte stores/loads for D and C.
+#include <type_traits>
+
 #include "common.h"
 
 namespace nf {
 
-constexpr int BK = 64;                 // K slab
-constexpr int A_LD = BK + 8;           // halves per As row (144 B: 16-byte aligned, bank-skewed)
-constexpr int NQ = BK / 4;             // k-quads per slab
+constexpr int BK = 64;  // K slab (halves); an A-style LDS row is 128 bytes
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
 
 template <int BM, int BN, int NB>
 struct GemmSmem {
-  static constexpr int B_LD = BN + 2;  // 8-byte cells per quad row (+2 cells = 16 B skew)
-  static constexpr int a_halves = BM * A_LD;
-  static constexpr int b_halves = NQ * B_LD * 4;
-  static constexpr int stage_halves = a_halves + NB * b_halves;
-  static constexpr size_t bytes = 2 * (size_t)stage_halves * sizeof(uint16_t);
+  static constexpr int a_bytes = BM * 128;
+  static constexpr int b_bytes = BN * 128;  // 64 rows x BN*2 bytes, or BN rows x 128 bytes
+  static constexpr int stage_bytes = a_bytes + NB * b_bytes;
+  // as many stages as fit 144 KB (of the CU's 160 KB), at most 4: the loads of a slab are issued
+  // stages-1 slabs before they are needed
+  static constexpr int stages = (144 * 1024) / stage_bytes > 4 ? 4 : (144 * 1024) / stage_bytes;
+  static_assert(stages >= 2, "tile too large for two LDS stages");
+  static constexpr size_t bytes = (size_t)stages * stage_bytes;
 };
 
-__device__ __forceinline__ uint32_t pack_lo(uint32_t x, uint32_t y) {
-  return __builtin_amdgcn_perm(y, x, 0x05040100u);  // {x.lo, y.lo}
-}
-__device__ __forceinline__ uint32_t pack_hi(uint32_t x, uint32_t y) {
-  return __builtin_amdgcn_perm(y, x, 0x07060302u);  // {x.hi, y.hi}
-}
-
-// Raw buffer loads: an offset at or past the descriptor's byte count reads as zero, so tile
-// edges need no branches -- out-of-range chunks just get the kOob offset.
+// Out-of-range per-lane offsets read as zero (also into LDS), so tile edges need no branches:
+// out-of-range chunks just get the kOob offset.  Only the per-lane offset is range-checked by
+// the hardware, so the whole address stays in it.
 constexpr uint32_t kOob = 0xFFFFFFF0u;
-typedef uint32_t bufvec4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, size_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)(uint32_t)bytes, 0x00020000);
+typedef uint32_t rsrc_t __attribute__((ext_vector_type(4)));  // raw buffer descriptor (4 SGPRs)
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
+  const uint64_t a = (uint64_t)p;
+  return rsrc_t{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)bytes, 0x00020000u};
 }
-__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
-  bufvec4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
-  return u32x4{v.x, v.y, v.z, v.w};
+// 64 lanes x 16 bytes -> LDS [lds_addr, lds_addr + 1024); lds_addr (a byte address inside LDS)
+// must be the same for the whole wavefront.  Written as inline assembly on purpose: for the
+// builtin form the compiler makes every later LDS read wait for ALL outstanding loads
+// (vmcnt(0)), because it cannot tell the stage being filled from the stage being read, and
+// that serialises the loads with the MFMAs.  The kernel waits itself (wait_loads below).
+// M0 carries the LDS address; nothing else in these kernels uses M0.
+__device__ __forceinline__ void load16_to_lds(rsrc_t r, uint32_t byte_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(lds_addr), "v"(byte_off), "s"(r) : "memory");
+}
+__device__ __forceinline__ short4_t lds_read_tr16(const uint8_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p);
 }
 
 // SiLU(g)*u on values already rounded to fp16, as the reference's dual epilogue computes it.
@@ -70,16 +86,18 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
     int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n) {
   constexpr int NB = kDual ? 2 : 1;
   using SM = GemmSmem<BM, BN, NB>;
-  constexpr int B_LD = SM::B_LD;
   constexpr int TM = BM / WM / 32;  // MFMA tiles per wave along M
   constexpr int TN = BN / WN / 32;
   static_assert(WM * WN == 4, "four wavefronts");
-  constexpr int A_CHUNKS = BM * (BK / 8) / 256;     // 16-byte chunks per thread per slab
-  constexpr int B_BLOCKS = (BK / 4) * (BN / 8) / 256;  // 4x8 blocks per thread per slab (row-major B)
-  constexpr int BC_CHUNKS = BN * (BK / 8) / 256;    // 16-byte chunks per thread (col-major B)
-  static_assert(A_CHUNKS >= 1 && B_BLOCKS >= 1, "tile too small for 256 threads");
+  static_assert((BN / WN) % 64 == 0 && BM % 32 == 0 && BN % 64 == 0, "tile shape");
+  constexpr int A_LOADS = BM / 32;   // 1 KB load instructions per wave per slab
+  constexpr int B_LOADS = BN / 32;   // ... per weight matrix
+  constexpr int ROWB = BN * 2;       // bytes per k row of a [K][N] weight slab
+  constexpr int B_CPR = BN / 8;      // 16-byte chunks per such row
+  constexpr int B_RPI = 64 / B_CPR;  // rows covered by one load instruction
 
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
 
   // XCD-aware tile order: consecutive workgroup ids land on different XCDs (8 of them), so
   // give each XCD one contiguous range of tiles, M fastest, to share weight panels in its L2.
@@ -90,7 +108,8 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
   const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
   const int m_base = tile_m * BM, n_base = tile_n * BN;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int l32 = lane & 31, lg = lane >> 5;
 
@@ -104,128 +123,107 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[b][i][j][r] = 0.f;
 
-  // ---- staging registers: one slab's worth of this thread's global chunks
-  constexpr int B_UNITS = kBCol ? BC_CHUNKS : B_BLOCKS;  // per weight matrix
-  constexpr int B_LOADS = kBCol ? 1 : 4;                  // 16-byte loads per B unit
-  u32x4 a_reg[A_CHUNKS];
-  u32x4 b_reg[NB][B_UNITS * B_LOADS];
-
-  // Per-thread byte offsets of the chunks it stages, at k0 = 0 (kOob when the row / column is
-  // outside the matrix); the slab offset is added per iteration.
-  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K * 2);
-  __amdgpu_buffer_rsrc_t b_rsrc[NB];
+  // ---- global -> LDS: per-lane byte offsets of the chunks this lane fetches
+  const rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K * 2);
+  rsrc_t b_rsrc[NB];
 #pragma unroll
   for (int b = 0; b < NB; ++b) b_rsrc[b] = make_rsrc(b ? B1 : B0, (size_t)N * K * 2);
-  uint32_t a_off[A_CHUNKS];
+  // A-style rows: lane -> (row lane/8 of the instruction's 8 rows, position lane%8), fetching
+  // logical chunk position ^ row.
+  const int a_kc = ((lane & 7) ^ (lane >> 3)) * 8;  // k of that chunk inside the slab
+  uint32_t a_off[A_LOADS];
 #pragma unroll
-  for (int i = 0; i < A_CHUNKS; ++i) {
-    const int id = tid + 256 * i;
-    const int gm = m_base + (id >> 3);
-    a_off[i] = gm < M ? ((uint32_t)gm * (uint32_t)K + (id & 7) * 8) * 2u : kOob;
+  for (int t = 0; t < A_LOADS; ++t) {
+    const int gm = m_base + (t * 4 + wave) * 8 + (lane >> 3);
+    a_off[t] = gm < M ? ((uint32_t)gm * (uint32_t)K + a_kc) * 2u : kOob;
   }
-  uint32_t b_off[B_UNITS];
+  // [K][N] weights: one running offset per load, advanced by a slab (64 rows) after use.  Rows
+  // k >= K lie at or past the end of the buffer and read as zero, so K needs no test there.
+  uint32_t b_off[NB][B_LOADS];
+  const uint32_t b_slab = (uint32_t)BK * (uint32_t)N * 2u;
 #pragma unroll
-  for (int i = 0; i < B_UNITS; ++i) {
-    const int id = tid + 256 * i;
+  for (int t = 0; t < B_LOADS; ++t) {
+    uint32_t off;
     if constexpr (kBCol) {
-      const int gn = n_base + (id >> 3);
-      b_off[i] = gn < N ? ((uint32_t)gn * (uint32_t)K + (id & 7) * 8) * 2u : kOob;
+      const int gn = n_base + (t * 4 + wave) * 8 + (lane >> 3);
+      off = gn < N ? ((uint32_t)gn * (uint32_t)K + a_kc) * 2u : kOob;
     } else {
-      const int gn = n_base + (id % (BN / 8)) * 8;
-      b_off[i] = gn < N ? ((uint32_t)(id / (BN / 8)) * 4u * (uint32_t)N + gn) * 2u : kOob;
+      const int row = (t * 4 + wave) * B_RPI + lane / B_CPR;
+      const int c = (lane % B_CPR) ^ ((row & 3) << 1);
+      const int gn = n_base + c * 8;
+      off = gn < N ? ((uint32_t)row * (uint32_t)N + gn) * 2u : kOob;
     }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) b_off[b][t] = off;
   }
 
-  // The staging work of a slab is cut into 3 parts (quarter q of the MFMA loop handles the
-  // A chunks with i % 3 == q and the B units with (2 - u % 3) == q); part < 0 = everything.
-  auto load_part = [&](int k0, int part) {
+  // The loads of one slab, or (part >= 0) the share of them with index % parts == part.
+  constexpr int NS = SM::stages;
+  constexpr int LOADS = A_LOADS + NB * B_LOADS;  // per wave per slab
+  constexpr int PARTS = NS == 2 ? 2 : 4;         // k-steps of a slab the loads are spread over
+  auto issue_loads = [&](int stage, int k0, int part) {
+    const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::stage_bytes + wave * 1024);
+    const bool k_ok = k0 + a_kc < K;
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      if (part >= 0 && i % 3 != part) continue;
-      const bool ok = a_off[i] != kOob && k0 + ((tid + 256 * i) & 7) * 8 < K;
-      a_reg[i] = buf_load16(a_rsrc, ok ? a_off[i] + (uint32_t)k0 * 2u : kOob);
+    for (int t = 0; t < A_LOADS; ++t) {
+      if (part >= 0 && t % PARTS != part) continue;
+      load16_to_lds(a_rsrc, (k_ok && a_off[t] != kOob) ? a_off[t] + (uint32_t)k0 * 2u : kOob,
+                    st + t * 4096);
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-      for (int i = 0; i < B_UNITS; ++i) {
-        if (part >= 0 && 2 - (b * B_UNITS + i) % 3 != part) continue;
+      for (int t = 0; t < B_LOADS; ++t) {
+        if (part >= 0 && (A_LOADS + b * B_LOADS + t) % PARTS != part) continue;
+        const uint32_t dst = st + SM::a_bytes + b * SM::b_bytes + t * 4096;
         if constexpr (kBCol) {
-          const bool ok = b_off[i] != kOob && k0 + ((tid + 256 * i) & 7) * 8 < K;
-          b_reg[b][i] = buf_load16(b_rsrc[b], ok ? b_off[i] + (uint32_t)k0 * 2u : kOob);
+          load16_to_lds(b_rsrc[b], (k_ok && b_off[b][t] != kOob) ? b_off[b][t] + (uint32_t)k0 * 2u : kOob, dst);
         } else {
-          const int kq = (tid + 256 * i) / (BN / 8);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const bool ok = b_off[i] != kOob && k0 + kq * 4 + r < K;
-            b_reg[b][i * 4 + r] =
-                buf_load16(b_rsrc[b], ok ? b_off[i] + ((uint32_t)(k0 + r) * (uint32_t)N) * 2u : kOob);
-          }
+          load16_to_lds(b_rsrc[b], b_off[b][t], dst);
+          if (b_off[b][t] != kOob) b_off[b][t] += b_slab;
         }
       }
   };
 
-  auto store_part = [&](int stage, int part) {
-    uint16_t* As = smem + stage * SM::stage_halves;
+  // ---- LDS -> MFMA operand fragments, double-buffered across the 4 k-steps of a slab
+  // A-style: row r = l32 (+ tile offsets), logical chunk kk*2+lg sits at position chunk ^ (r&7).
+  const uint32_t a_rd = (uint32_t)(wm * (BM / WM) + l32) * 128u;
+  const uint32_t bc_rd = (uint32_t)(wn * (BN / WN) + l32) * 128u;  // [N][K] weights
+  uint32_t swz[4];
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      if (part >= 0 && i % 3 != part) continue;
-      const int id = tid + 256 * i;
-      *reinterpret_cast<u32x4*>(As + (id >> 3) * A_LD + (id & 7) * 8) = a_reg[i];
-    }
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      uint16_t* Bs = As + SM::a_halves + b * SM::b_halves;
-#pragma unroll
-      for (int i = 0; i < B_UNITS; ++i) {
-        if (part >= 0 && 2 - (b * B_UNITS + i) % 3 != part) continue;
-        const int id = tid + 256 * i;
-        if constexpr (kBCol) {
-          const int n = id >> 3, kc = id & 7;
-          const u32x4 v = b_reg[b][i];
-          *reinterpret_cast<u32x2*>(Bs + ((2 * kc) * B_LD + n) * 4) = u32x2{v.x, v.y};
-          *reinterpret_cast<u32x2*>(Bs + ((2 * kc + 1) * B_LD + n) * 4) = u32x2{v.z, v.w};
-        } else {
-          const int nb = id % (BN / 8), kq = id / (BN / 8);
-          const u32x4 r0 = b_reg[b][i * 4 + 0], r1 = b_reg[b][i * 4 + 1];
-          const u32x4 r2 = b_reg[b][i * 4 + 2], r3 = b_reg[b][i * 4 + 3];
-          // cell(n) = {B[k0][n], B[k1][n], B[k2][n], B[k3][n]}; n = nb*8 + 0..7
-          u32x4 o0, o1, o2, o3;
-          o0.x = pack_lo(r0.x, r1.x); o0.y = pack_lo(r2.x, r3.x);  // n+0
-          o0.z = pack_hi(r0.x, r1.x); o0.w = pack_hi(r2.x, r3.x);  // n+1
-          o1.x = pack_lo(r0.y, r1.y); o1.y = pack_lo(r2.y, r3.y);  // n+2
-          o1.z = pack_hi(r0.y, r1.y); o1.w = pack_hi(r2.y, r3.y);  // n+3
-          o2.x = pack_lo(r0.z, r1.z); o2.y = pack_lo(r2.z, r3.z);  // n+4
-          o2.z = pack_hi(r0.z, r1.z); o2.w = pack_hi(r2.z, r3.z);  // n+5
-          o3.x = pack_lo(r0.w, r1.w); o3.y = pack_lo(r2.w, r3.w);  // n+6
-          o3.z = pack_hi(r0.w, r1.w); o3.w = pack_hi(r2.w, r3.w);  // n+7
-          u32x4* dst = reinterpret_cast<u32x4*>(Bs + (kq * B_LD + nb * 8) * 4);
-          dst[0] = o0; dst[1] = o1; dst[2] = o2; dst[3] = o3;
-        }
-      }
-    }
-  };
+  for (int kk = 0; kk < 4; ++kk) swz[kk] = (uint32_t)(((kk * 2 + lg) ^ (l32 & 7)) << 4);
+  // [K][N] weights: 16-lane group g reads the 4(k) x 16(n) block at rows lg*8 + 4h.., columns
+  // (g&1)*16.. of the MFMA tile, lane i of the group addressing row i/4, columns (i&3)*4..+3.
+  // 32-byte unit u of a row sits at u ^ (row & 3); with u = 2*jt + (g&1) that is
+  // 2*(jt ^ x1) + ((g&1) ^ x0) for x = row & 3 = (i/4) & 3.
+  const int i16 = lane & 15, x0 = (i16 >> 2) & 1, x1 = (i16 >> 3) & 1, g1 = (lane >> 4) & 1;
+  const uint32_t br_common = (uint32_t)(lg * 8 + (i16 >> 2)) * ROWB + (uint32_t)(wn * (BN / WN)) * 2u +
+                             (uint32_t)(i16 & 3) * 8u + (uint32_t)((g1 ^ x0) * 32);
+  const uint32_t br_even = br_common + (uint32_t)x1 * 64u;        // jt even: unit pair jt + x1
+  const uint32_t br_odd = br_common + (uint32_t)(1 - x1) * 64u;   // jt odd:  unit pair jt - x1 (+ (jt-1)*64 below)
 
-  // ---- MFMA operand fragments, double-buffered across the 4 k-steps of a slab
   half8_t af[2][TM];
   half8_t bf[2][NB][TN];
   auto read_frags = [&](int stage, int kk, int buf) {
-    const uint16_t* As = smem + stage * SM::stage_halves;
+    const uint8_t* st = smem + stage * SM::stage_bytes;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int row = wm * (BM / WM) + i * 32 + l32;
-      af[buf][i] = *reinterpret_cast<const half8_t*>(As + row * A_LD + kk * 16 + lg * 8);
-    }
+    for (int i = 0; i < TM; ++i)
+      af[buf][i] = *reinterpret_cast<const half8_t*>(st + a_rd + swz[kk] + i * 32 * 128);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-      const uint16_t* Bs = As + SM::a_halves + b * SM::b_halves;
+      const uint8_t* bs = st + SM::a_bytes + b * SM::b_bytes;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int n = wn * (BN / WN) + j * 32 + l32;
-        const int q = kk * 4 + lg * 2;
-        half4_t lo = *reinterpret_cast<const half4_t*>(Bs + (q * B_LD + n) * 4);
-        half4_t hi = *reinterpret_cast<const half4_t*>(Bs + ((q + 1) * B_LD + n) * 4);
-        bf[buf][b][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        if constexpr (kBCol) {
+          bf[buf][b][j] = *reinterpret_cast<const half8_t*>(bs + bc_rd + swz[kk] + j * 32 * 128);
+        } else {
+          const uint8_t* p = bs + ((j & 1) ? br_odd + (j - 1) * 64 : br_even + j * 64) + kk * 16 * ROWB;
+          const short4_t lo = lds_read_tr16(p);
+          const short4_t hi = lds_read_tr16(p + 4 * ROWB);
+          typedef short short8_t __attribute__((ext_vector_type(8)));
+          const short8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          bf[buf][b][j] = __builtin_bit_cast(half8_t, v);
+        }
       }
     }
   };
@@ -239,38 +237,62 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
           acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[buf][b][j], af[buf][i], acc[b][i][j], 0, 0, 0);
   };
 
-  // One slab of the steady state.  While the MFMAs of slab s run out of LDS stage s&1:
-  //   quarters 0-2: prefetch the next k-step's fragments; write slab s+1 (already in
-  //                 registers) into the other stage; refill those registers with slab s+2;
-  //   quarter 3:    barrier, then prefetch slab s+1's first fragments under the last MFMAs.
-  auto slab = [&](int s, bool do_store, bool do_load) {
-    const int cur = s & 1;
+  // Slab s lives in LDS stage s % NS.  While its four k-steps run (next step's fragments
+  // prefetched), the loads of slab s+NS-1 are issued, spread over the k-steps, into the stage
+  // that slab s-1 has just left (every wavefront is past the barrier that ended slab s-1).  At
+  // the end the wavefront waits until its loads of slab s+1 have landed -- the younger loads it
+  // has issued since may stay in flight -- and meets the others at the barrier.
+  auto slab = [&](auto issue_c, int s, int cs, int ls) {
+    constexpr bool issue = decltype(issue_c)::value;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      if (kk == 3) __syncthreads();
-      if (kk < 3) read_frags(cur, kk + 1, (kk + 1) & 1);
-      else if (do_store) read_frags(cur ^ 1, 0, 0);
-      if (kk < 3) {
-        if (do_store) store_part(cur ^ 1, kk);
-        if (do_load) load_part((s + 2) * BK, kk);
-      }
+#if !defined(NF_EXP_NOLOAD)
+      if (issue && kk < PARTS) issue_loads(ls, (s + NS - 1) * BK, kk);
+#endif
+#if !defined(NF_EXP_NOFRAG)
+      if (kk < 3) read_frags(cs, kk + 1, (kk + 1) & 1);
+#endif
+      __builtin_amdgcn_sched_barrier(0);  // the fragment reads go out before this step's MFMAs
+#if !defined(NF_EXP_NOMFMA)
       mfma_step(kk & 1);
+#endif
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
+  auto wait_loads = [&](int younger) {  // vmcnt(younger): encoded in bits [3:0] and [15:14]
+    if (younger == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS * (NS - 2) & 15) | (((LOADS * (NS - 2)) >> 4) << 14));
+  };
+  static_assert(LOADS * (NS - 2) < 64, "vmcnt range");
+  auto next = [](int st) { return st + 1 == NS ? 0 : st + 1; };
 
   const int nslab = (K + BK - 1) / BK;
-  load_part(0, -1);
-  store_part(0, -1);
-  if (nslab > 1) load_part(BK, -1);
+#pragma unroll
+  for (int p = 0; p < NS - 1; ++p)
+    if (p < nslab) issue_loads(p, p * BK, -1);
+  // slab 0 must have landed; later prologue loads may still be in flight (exact count only
+  // matters for speed: waiting for everything is always correct)
+  if (nslab >= NS - 1) wait_loads(1); else wait_loads(0);
   __syncthreads();
   read_frags(0, 0, 0);
-  int s = 0;
-  for (; s + 2 < nslab; ++s) slab(s, true, true);
-  if (s + 1 < nslab) {
-    slab(s, true, false);
-    ++s;
+  int cs = 0, ls = NS - 1, s = 0;
+  for (; s + NS - 1 < nslab; ++s) {  // steady state: one slab's loads issued per slab
+    slab(std::true_type{}, s, cs, ls);
+    wait_loads(1);
+    __syncthreads();
+    cs = next(cs);
+    ls = next(ls);
+    read_frags(cs, 0, 0);
   }
-  slab(s, false, false);
+  for (; s < nslab; ++s) {           // drain: nothing left to issue
+    slab(std::false_type{}, s, cs, ls);
+    if (s + 1 < nslab) {
+      wait_loads(0);
+      __syncthreads();
+      cs = next(cs);
+      read_frags(cs, 0, 0);
+    }
+  }
 
   // Epilogue.  acc[.][i][j][r] holds D[m][n] with m = tile row l32 and
   // n = (r/4)*8 + lg*4 + r%4 of the 32x32 tile: 4 consecutive n per register quad.
@@ -332,15 +354,16 @@ static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1
   return check_launch("gemm launch");
 }
 
-// Tile choice: the largest tile that still yields at least ~one workgroup per CU (256 CUs);
-// short M uses a 64-row tile so the padding rows do not dominate.
+// Tile choice (256 CUs, one workgroup each): the largest tile that still gives most CUs a
+// workgroup -- measured on the pipeline's shapes, 192 tiles of the bigger kind beat 1.5 rounds
+// of the smaller one; short M uses a 64-row tile so the padding rows do not dominate.
 template <bool kBCol>
 static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
                           int M, int N, int K, float alpha, float beta, hipStream_t s) {
   auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (M <= 64) return launch_gemm<64, 256, 1, 4, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (tiles(256, 256) >= 224) return launch_gemm<256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (tiles(128, 256) >= 224 || M <= 128) return launch_gemm<128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (tiles(256, 256) >= 192) return launch_gemm<256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (tiles(128, 256) >= 192 || M <= 128) return launch_gemm<128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
   return launch_gemm<128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
 }
 
@@ -356,7 +379,8 @@ static int check_gemm_args(const char* who, const void* A, const void* B, const 
   NF_REQUIRE(((uintptr_t)A | (uintptr_t)B | (uintptr_t)D) % 16 == 0,
              "%s: operands must be 16-byte aligned", who);
   // operands are addressed through 32-bit buffer offsets
-  NF_REQUIRE((size_t)M * K * 2 < 0xFFFFFF00ull && (size_t)N * K * 2 < 0xFFFFFF00ull,
+  // (the weight offsets run up to two slabs past K before they are discarded)
+  NF_REQUIRE((size_t)M * K * 2 < 0xFFFFFF00ull && (size_t)N * ((size_t)K + 128) * 2 < 0xFFFFFF00ull,
              "%s: an operand of %d x %d x %d exceeds the 4 GiB buffer-addressing limit", who, M, N, K);
   return NF_OK;
 }
@@ -384,9 +408,10 @@ int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t*
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
   if (M <= 64)
-    return launch_gemm<64, 128, 1, 4, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+    return launch_gemm<64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
   const long long t256 = (long long)((M + 255) / 256) * ((N + 127) / 128);
-  if (t256 >= 224)
+  const int tail = M % 256;  // rows in the last 256-row tile: half-empty tiles go to the 128-row kernel
+  if (t256 >= 192 && (tail == 0 || tail > 128))
     return launch_gemm<256, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
   return launch_gemm<128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
 }

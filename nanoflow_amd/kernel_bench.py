@@ -1,0 +1,114 @@
+#!/usr/bin/env python3
+"""Kernel-level throughput of the HIP operators at the pipeline's own shapes (one MI355X).
+
+    python -m nanoflow_amd.kernel_bench --op gemm --m 2048            # KQV, O, down, LM head
+    python -m nanoflow_amd.kernel_bench --op dual --m 1024
+    python -m nanoflow_amd.kernel_bench --op gemm_f8 --m 2048
+    python -m nanoflow_amd.kernel_bench --op attn --requests 1792 --kv-lo 1024 --kv-hi 1536
+    python -m nanoflow_amd.kernel_bench --op copy                     # counter-calibration kernel
+
+Each line reports the average launch time over --iters launches (HIP events on the launch
+stream) and the algorithmic rate: 2*M*N*K flops (4*M*N*K for the fused gate/up pair), or the
+decode-attention bytes of gemv/src/bench_batch_decode.cu:77-81 (K and V once, q and o, page
+indices).  --iters 1 --warm 0 gives one launch per shape, for counter collection.
+"""
+from __future__ import annotations
+
+import argparse
+import os
+import sys
+
+import numpy as np
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+from nanoflow_amd import kernels as K, synth  # noqa: E402
+
+DEV = "cuda"
+
+
+def timeit(fn, iters, warm):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def layer_shapes(shape: synth.ModelShape, M: int):
+    return [("kqv", M, shape.kqv_n, shape.hidden), ("o", M, shape.hidden, shape.Hq * shape.d),
+            ("down", M, shape.hidden, shape.ffn), ("lm_head", (M + 127) // 128 * 128, shape.vocab, shape.hidden)]
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--op", required=True, choices=["gemm", "dual", "gemm_f8", "attn", "copy"])
+    ap.add_argument("--model", default="8b", choices=["8b", "70b"])
+    ap.add_argument("--m", type=int, default=2048, help="rows (tokens) of the GEMM operand")
+    ap.add_argument("--only", default="", help="gemm: run only this role (kqv, o, down, lm_head)")
+    ap.add_argument("--requests", type=int, default=1792)
+    ap.add_argument("--kv-lo", type=int, default=1024)
+    ap.add_argument("--kv-hi", type=int, default=1536)
+    ap.add_argument("--num-blocks", type=int, default=0, help="attn: cap on resident workgroups (0 = none)")
+    ap.add_argument("--mib", type=int, default=1024, help="copy: MiB moved")
+    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--warm", type=int, default=3)
+    a = ap.parse_args()
+    assert torch.cuda.is_available(), "needs the MI355X"
+    shape = synth.LLAMA3_8B if a.model == "8b" else synth.LLAMA3_70B
+    g = torch.Generator(device=DEV).manual_seed(0)
+    rnd = lambda *s, std=1.0: torch.empty(s, dtype=torch.float16, device=DEV).normal_(0, std, generator=g)
+
+    if a.op in ("gemm", "gemm_f8"):
+        for name, M, N, Kd in layer_shapes(shape, a.m):
+            if a.only and name != a.only:
+                continue
+            out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+            if a.op == "gemm":
+                A, B = rnd(M, Kd), rnd(Kd, N, std=0.02)
+                fn = lambda: K.gemm(A, B, out=out)
+            else:
+                Aq = torch.randint(0, 120, (M, Kd), dtype=torch.uint8, device=DEV)
+                Bq = torch.randint(0, 120, (N, Kd), dtype=torch.uint8, device=DEV)
+                sa, sb = torch.ones(M, device=DEV), torch.ones(N, device=DEV)
+                fn = lambda: K.gemm_f8(Aq, sa, Bq, sb, out=out)
+            ms = timeit(fn, a.iters, a.warm)
+            print(f"{a.op} {name:8s} {M}x{N}x{Kd}: {ms * 1e3:9.1f} us  {2.0 * M * N * Kd / ms / 1e9:8.1f} TFLOP/s", flush=True)
+    elif a.op == "dual":
+        A, Bg, Bu = rnd(a.m, shape.hidden), rnd(shape.hidden, shape.ffn, std=0.02), rnd(shape.hidden, shape.ffn, std=0.02)
+        out = torch.empty(a.m, shape.ffn, dtype=torch.float16, device=DEV)
+        ms = timeit(lambda: K.dual_swiglu(A, Bg, Bu, out=out), a.iters, a.warm)
+        print(f"dual gate/up {a.m}x{shape.ffn}x{shape.hidden}: {ms * 1e3:9.1f} us  "
+              f"{4.0 * a.m * shape.ffn * shape.hidden / ms / 1e9:8.1f} TFLOP/s", flush=True)
+    elif a.op == "attn":
+        b = synth.config2_batch(seed=0, n_decode=a.requests, lo=a.kv_lo, hi=a.kv_hi, prefill_chunk=16)
+        nd = b.decodePrefillBorder
+        pool = rnd(b.num_pages, 2, shape.page_size, shape.Hkv, shape.d)
+        q = rnd(b.tokens, shape.Hq * shape.d)
+        o = torch.zeros_like(q)
+        t = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(DEV)
+        qi, kvp, kvi, kvl = t(b.input_indptr[:nd + 1]), t(b.kv_indptr[:nd + 1]), t(b.kv_indices), t(b.kv_last_page_len[:nd])
+        ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+        fn = lambda: K.attention_paged(q, qi, pool, kvp, kvi, kvl, shape.Hq, shape.Hkv, causal=False, out=o,
+                                       batch=nd, max_qo_rows=nd, workspace=ws, num_blocks=a.num_blocks)
+        ms = timeit(fn, a.iters, a.warm)
+        L = b.kv_len[:nd].astype(np.int64)
+        nbytes = int((2 * L * shape.Hkv * shape.d * 2 + 2 * shape.Hq * shape.d * 2 + 4 * ((L + 15) // 16 + 2)).sum())
+        print(f"decode attention {nd} requests, KV [{a.kv_lo},{a.kv_hi}]: {ms * 1e3:9.1f} us  "
+              f"{nbytes / ms / 1e6:8.1f} GB/s  ({nbytes} algorithmic bytes per launch)", flush=True)
+    else:
+        n = a.mib << 20
+        src = torch.empty(n, dtype=torch.uint8, device=DEV).random_(generator=g)
+        dst = torch.empty_like(src)
+        ms = timeit(lambda: dst.copy_(src), a.iters, a.warm)
+        print(f"copy {a.mib} MiB: {ms * 1e3:9.1f} us  {2 * n / ms / 1e6:8.1f} GB/s (read + write; "
+              f"{n} bytes read, {n} bytes written per launch)", flush=True)
+
+
+if __name__ == "__main__":
+    main()

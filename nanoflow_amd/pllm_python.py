@@ -171,7 +171,7 @@ class PipelineTimings(C.Structure):
     _fields_ = [("iter_ms", C.c_double), ("decode_attn_ms", C.c_double),
                 ("decode_attn_launches", C.c_long), ("prefill_attn_ms", C.c_double),
                 ("prefill_attn_launches", C.c_long), ("gemm_ms", C.c_double),
-                ("gemm_launches", C.c_long), ("gemm_flop", C.c_double)]
+                ("gemm_launches", C.c_long), ("gemm_flop", C.c_double), ("layer_stride", C.c_int)]
 
 
 SYMBOLS = [
