@@ -354,6 +354,267 @@ __global__ __launch_bounds__(256, SPLIT ? 2 : 1) void attn_paged_kernel(
   }
 }
 
+// Decode attention (one query row per request, or few): the HBM-bound kernel.  Same
+// formulation and column packing as attn_paged_kernel; what differs is how K and V travel:
+//
+//   * K and V pages go from global memory STRAIGHT INTO LDS (buffer_load ... lds), not through
+//     registers: the load-to-register path of a CU saturates near 38 GB/s, the direct path
+//     carries half again as much from HBM, and the data in flight no longer costs registers.
+//   * A workgroup is (request, kv head); its 4 wavefronts take every 4th 32-key step and merge
+//     (m, l, O) at the end.  Every wavefront owns a private LDS ring (2 K tiles + 2 V tiles of
+//     32 keys x 256 bytes), so no barrier is needed while streaming: a wavefront only waits
+//     for its own loads (s_waitcnt vmcnt), and refills a tile as soon as its MFMAs have read it
+//     -- the K tile of step i+2 is requested right after the score MFMAs of step i.
+//   * Layout in LDS = the page layout (one 256-byte row per key), with the 16-byte chunks of a
+//     row permuted on the way in so that operand reads are bank-conflict free: K row r keeps
+//     chunk c at c ^ (r & 15) (16-byte A-operand reads), V row r keeps chunk c at
+//     c ^ ((r & 3) << 1) and is read with the transposing LDS read (ds_read_b64_tr_b16), which
+//     hands each lane 4 consecutive keys of one feature: the V^T operand with no permutes.
+//   * A page is addressed through its own buffer descriptor (base = page, 64 KiB range), so
+//     pools larger than 4 GiB need no 64-bit per-lane arithmetic and out-of-page offsets
+//     (used to zero-fill V rows past the end of the sequence) read as zero.
+template <int GROUP>
+__global__ __launch_bounds__(256, 1) void attn_decode_kernel(
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ o, const int32_t* __restrict__ qo_indptr,
+    const uint16_t* __restrict__ kv_data, const int32_t* __restrict__ kv_indptr,
+    const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_last_page_len, int batch,
+    int Hq, int Hkv, int causal, float scale_log2) {
+  constexpr int TPB = 16 / GROUP;  // tokens per 16-column block = tokens per work item pass
+  constexpr int WAVE_LDS = 32768;  // per wavefront: K0 K1 V0 V1, 8 KB each
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c16 = lane & 15, g = lane >> 4;
+  const uint32_t wlds = __builtin_amdgcn_readfirstlane(lds0 + wave * WAVE_LDS);  // DMA destination base
+  uint8_t* const wptr = lds + wave * WAVE_LDS;                                   // same, for reads
+  const uint32_t page_bytes = (uint32_t)(2 * PAGE * Hkv * D * 2);
+  const uint32_t v_half = (uint32_t)(PAGE * Hkv * D * 2);  // byte offset of the V half of a page
+
+  // operand read offsets inside a tile (constant per lane)
+  uint32_t kx[4];  // K: row blk*16 + c16, logical chunk 4j + g
+#pragma unroll
+  for (int j = 0; j < 4; ++j) kx[j] = (uint32_t)(c16 * 256 + (((j * 4 + g) ^ c16) << 4));
+  // V: lanes 16g..16g+15 read the 4(key) x 16(feature) block of keys 4g.. and features 16i..;
+  // lane i16 addresses key 4g + i16/4, features 16i + 4(i16&3)..+3; 32-byte unit u of a row
+  // sits at u ^ (key & 3), which for u = 2i + .. is (i ^ x) in the 32-byte index, x = (i16/4) & 3.
+  const int i16 = lane & 15, vx_x = (i16 >> 2) & 3;
+  uint32_t vx[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    vx[k] = (uint32_t)((g * 4 + (i16 >> 2)) * 256 + ((k ^ vx_x) * 32) + (i16 & 3) * 8);
+
+  for (long long w = blockIdx.x; w < (long long)batch * Hkv; w += gridDim.x) {
+    const int req = (int)(w / Hkv), kvh = (int)(w % Hkv);
+    const int qo0 = qo_indptr[req];
+    const int qo_len = qo_indptr[req + 1] - qo0;
+    const int pg0 = kv_indptr[req];
+    const int npages = kv_indptr[req + 1] - pg0;
+    const int kv_len = npages > 0 ? (npages - 1) * PAGE + kv_last_page_len[req] : 0;
+    // DMA source offsets inside a page: instruction t4 moves keys 4*t4 .. 4*t4+3 of a page
+    // (64 lanes x 16 bytes = 4 rows), lane -> key 4*t4 + lane/16, position lane%16.
+    uint32_t k_src[4], v_src[4];
+#pragma unroll
+    for (int t4 = 0; t4 < 4; ++t4) {
+      const int key = 4 * t4 + (lane >> 4), pos = lane & 15;
+      const uint32_t row = (uint32_t)((key * Hkv + kvh) * D * 2);
+      k_src[t4] = row + (uint32_t)(((pos ^ key) & 15) << 4);
+      v_src[t4] = v_half + row + (uint32_t)((pos ^ ((key & 3) << 1)) << 4);
+    }
+    const int n_sub = (qo_len + TPB - 1) / TPB;
+    for (int sub = 0; sub < n_sub; ++sub) {
+      const int tok0 = sub * TPB;
+      float4_t oacc[8];
+      float m_run = -1e30f, l_run = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) oacc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+      // Q operand: column c16 = (token tok0 + c16/GROUP, head c16%GROUP)
+      H8 qf[4];
+      const int tq = tok0 + c16 / GROUP;
+      const bool live = tq < qo_len;
+      {
+        const uint16_t* qp = q + ((size_t)(qo0 + (live ? tq : 0)) * Hq + kvh * GROUP + c16 % GROUP) * D + g * 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          qf[j].u = live ? *reinterpret_cast<const u32x4*>(qp + j * 32) : u32x4{0, 0, 0, 0};
+      }
+      int key_limit = causal ? kv_len - qo_len + tq : kv_len - 1;
+      if (!live) key_limit = -1;
+      const int tok_last = min(tok0 + TPB, qo_len) - 1;
+      const int kv_end = causal ? min(kv_len, kv_len - qo_len + tok_last + 1) : kv_len;
+      const int npairs = (kv_end + 31) >> 5;  // 32-key steps; this wavefront takes wave, wave+4, ...
+
+      auto page_rsrc = [&](int pidx) -> rsrc_t {  // uniform: scalar loads and arithmetic
+        const int page = kv_indices[pg0 + (pidx < npages ? pidx : 0)];
+        return make_rsrc(kv_data + (size_t)page * (page_bytes / 2), page_bytes);
+      };
+      auto dma_k = [&](int pp, int buf) {
+        const rsrc_t ra = page_rsrc(2 * pp), rb = page_rsrc(2 * pp + 1);
+        const uint32_t dst = wlds + buf * 8192;
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4) load16_to_lds(ra, k_src[t4], dst + t4 * 1024);
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4) load16_to_lds(rb, k_src[t4], dst + 4096 + t4 * 1024);
+      };
+      auto dma_v = [&](int pp, int buf) {
+        const rsrc_t ra = page_rsrc(2 * pp), rb = page_rsrc(2 * pp + 1);
+        const uint32_t dst = wlds + 16384 + buf * 8192;
+        // rows past the end of the sequence may hold anything (NaN x 0 = NaN): zero-fill them
+        const int first_key = pp * 32 + (lane >> 4);
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4)
+          load16_to_lds(ra, first_key + 4 * t4 < kv_len ? v_src[t4] : kOob, dst + t4 * 1024);
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4)
+          load16_to_lds(rb, first_key + 16 + 4 * t4 < kv_len ? v_src[t4] : kOob, dst + 4096 + t4 * 1024);
+      };
+      // vmcnt(n): everything but the n youngest load instructions of this wavefront has landed
+      auto wait_but = [&](int younger) {
+        if (younger >= 24) __builtin_amdgcn_s_waitcnt(0x0F70 | (24 & 15) | ((24 >> 4) << 14));
+        else if (younger >= 16) __builtin_amdgcn_s_waitcnt(0x0F70 | (16 & 15) | ((16 >> 4) << 14));
+        else if (younger >= 8) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+      };
+
+      // two steps in flight before the loop
+      if (wave < npairs) {
+        dma_k(wave, 0);
+        dma_v(wave, 0);
+      }
+      if (wave + 4 < npairs) {
+        dma_k(wave + 4, 1);
+        dma_v(wave + 4, 1);
+      }
+      int buf = 0;
+      for (int pp = wave; pp < npairs; pp += 4, buf ^= 1) {
+        const int t_base = pp * 32;
+        const bool n1 = pp + 4 < npairs, n2 = pp + 8 < npairs;
+        const uint8_t* kt = wptr + buf * 8192;
+        const uint8_t* vt = wptr + 16384 + buf * 8192;
+
+        // ---- scores: K(pp) has landed once only V(pp), K(pp+4), V(pp+4) may still be in flight
+        wait_but(n1 ? 24 : 8);
+        float4_t s[2];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+          s[blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const half8_t kf = *reinterpret_cast<const half8_t*>(kt + blk * 4096 + kx[j]);
+            s[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[j].h, s[blk], 0, 0, 0);
+          }
+        }
+        // the K tile is free as soon as those reads have returned: s depends on them
+        if (n2) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          dma_k(pp + 8, buf);
+        }
+
+        // ---- online softmax; lane holds keys t_base + blk*16 + g*4 + r of column c16
+        float mx = -1e30f;
+        bool ok[2][4];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int t = t_base + blk * 16 + g * 4 + r;
+            ok[blk][r] = t <= key_limit && t < kv_len;
+            s[blk][r] *= scale_log2;
+            if (ok[blk][r]) mx = fmaxf(mx, s[blk][r]);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.f;
+        uint32_t pw[4];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int rr = 0; rr < 2; ++rr) {
+            float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[blk][2 * rr] - m_new) : 0.f;
+            float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[blk][2 * rr + 1] - m_new) : 0.f;
+            psum += p0 + p1;  // the row sum uses the unrounded values, P.V the fp16 ones
+            pw[blk * 2 + rr] = f2h_bits(p0) | (f2h_bits(p1) << 16);
+          }
+        H8 pf;
+        pf.u = u32x4{pw[0], pw[1], pw[2], pw[3]};
+        l_run = l_run * alpha + psum;
+
+        // ---- P.V: V(pp) has landed once only K(pp+4), V(pp+4), K(pp+8) may still be in flight
+        wait_but((n1 ? 16 : 0) + (n2 ? 8 : 0));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const uint8_t* vp = vt + vx[i & 3] + (i >> 2) * 128;
+          const short4_t lo = lds_read_tr16(vp);         // keys 4g..4g+3 of the first page
+          const short4_t hi = lds_read_tr16(vp + 4096);  // ... of the second page
+          typedef short short8_t __attribute__((ext_vector_type(8)));
+          const short8_t v8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          oacc[i] *= alpha;
+          oacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, v8), pf.h, oacc[i], 0, 0, 0);
+        }
+        if (n2) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          dma_v(pp + 8, buf);
+        }
+      }
+      l_run += __shfl_xor(l_run, 16, 64);
+      l_run += __shfl_xor(l_run, 32, 64);
+
+      // ---- merge the 4 wavefronts.  oacc[i][r] = O[column c16][feature 16i + 4g + r].  Each
+      // wavefront parks its partial result in its own LDS region (its streaming is over).
+      float* s_o = reinterpret_cast<float*>(wptr);             // [8][4][64]
+      float* s_m = reinterpret_cast<float*>(wptr + 8192);      // [64]
+      float* s_l = reinterpret_cast<float*>(wptr + 8192 + 256);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s_o[(i * 4 + r) * 64 + lane] = oacc[i][r];
+      s_m[lane] = m_run;
+      s_l[lane] = l_run;
+      __syncthreads();
+      float M = -1e30f, mw[4];
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        mw[ww] = *reinterpret_cast<const float*>(lds + ww * WAVE_LDS + 8192 + lane * 4);
+        M = fmaxf(M, mw[ww]);
+      }
+      float wgt[4], L = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        wgt[ww] = __builtin_amdgcn_exp2f(mw[ww] - M);
+        L += wgt[ww] * *reinterpret_cast<const float*>(lds + ww * WAVE_LDS + 8192 + 256 + lane * 4);
+      }
+      const float inv = L > 0.f ? 1.0f / L : 0.f;
+      if (live) {
+        // wavefront w finishes features 32w .. 32w+31 (i = 2w, 2w+1): 4 consecutive per lane and i
+        uint16_t* op = o + ((size_t)(qo0 + tq) * Hq + kvh * GROUP + c16 % GROUP) * D;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int i = 2 * wave + e;
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float acc = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < 4; ++ww)
+              acc += wgt[ww] * *reinterpret_cast<const float*>(lds + ww * WAVE_LDS + ((i * 4 + r) * 64 + lane) * 4);
+            v[r] = acc * inv;
+          }
+          u32x2 out;
+          out.x = f2h_bits(v[0]) | (f2h_bits(v[1]) << 16);
+          out.y = f2h_bits(v[2]) | (f2h_bits(v[3]) << 16);
+          *reinterpret_cast<u32x2*>(op + 16 * i + 4 * g) = out;
+        }
+      }
+      __syncthreads();  // the merge reads are done before the next pass streams into the rings
+    }
+  }
+}
+
 template <int GROUP>
 static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
                        const uint16_t* kv_data, const int32_t* kv_indptr, const int32_t* kv_indices,
@@ -377,11 +638,22 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
   if (num_blocks > 0 && bound > num_blocks) bound = num_blocks;
   if (bound > 0x7fffffffLL) bound = 0x7fffffffLL;
   if (bound < 1) bound = 1;
-  if (decode_mode)
-    attn_paged_kernel<GROUP, 1, true><<<(int)bound, 256, 0, stream>>>(
-        q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, batch, Hq,
-        Hkv, causal, scale_log2);
-  else
+  if (decode_mode) {
+    constexpr int kDecodeLds = 4 * 32768;
+    auto kern = attn_decode_kernel<GROUP>;
+    static bool attr_set = false;  // benign race: the call is idempotent
+    if (!attr_set) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLds);
+      if (e != hipSuccess) {
+        set_error("attention: cannot reserve %d bytes of LDS: %s", kDecodeLds, hipGetErrorString(e));
+        return NF_ERR_RUNTIME;
+      }
+      attr_set = true;
+    }
+    kern<<<(int)bound, 256, kDecodeLds, stream>>>(q, o, qo_indptr, kv_data, kv_indptr, kv_indices,
+                                                  kv_last_page_len, batch, Hq, Hkv, causal, scale_log2);
+  } else
     attn_paged_kernel<GROUP, NQB_PREFILL, false><<<(int)bound, 256, 0, stream>>>(
         q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, batch, Hq,
         Hkv, causal, scale_log2);

@@ -59,4 +59,29 @@ __device__ __forceinline__ uint32_t f2h_bits(float f) {
   return (uint32_t)__half_as_ushort(__float2half_rn(f));
 }
 
+// ---- global memory -> LDS without passing through registers (gfx950 buffer_load ... lds)
+typedef short short4_t __attribute__((ext_vector_type(4)));
+// Out-of-range per-lane offsets read as zero (also into LDS), so tile edges need no branches:
+// out-of-range chunks just get the kOob offset.  Only the per-lane offset is range-checked by
+// the hardware, so the whole address stays in it.
+constexpr uint32_t kOob = 0xFFFFFFF0u;
+typedef uint32_t rsrc_t __attribute__((ext_vector_type(4)));  // raw buffer descriptor (4 SGPRs)
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
+  const uint64_t a = (uint64_t)p;
+  return rsrc_t{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)bytes, 0x00020000u};
+}
+// 64 lanes x 16 bytes -> LDS [lds_addr, lds_addr + 1024); lds_addr (a byte address inside LDS)
+// must be the same for the whole wavefront.  Written as inline assembly on purpose: for the
+// builtin form the compiler makes every later LDS read wait for ALL outstanding loads
+// (vmcnt(0)), because it cannot tell the stage being filled from the stage being read, and
+// that serialises the loads with the MFMAs.  The kernel waits itself (wait_loads below).
+// M0 carries the LDS address; nothing else in these kernels uses M0.
+__device__ __forceinline__ void load16_to_lds(rsrc_t r, uint32_t byte_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(lds_addr), "v"(byte_off), "s"(r) : "memory");
+}
+__device__ __forceinline__ short4_t lds_read_tr16(const uint8_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p);
+}
+
 }  // namespace nf
