@@ -368,7 +368,7 @@ __global__ __launch_bounds__(256, SPLIT ? 2 : 1) void attn_paged_kernel(
 //   * Layout in LDS = the page layout (one 256-byte row per key), with the 16-byte chunks of a
 //     row permuted on the way in so that operand reads are bank-conflict free: K row r keeps
 //     chunk c at c ^ (r & 15) (16-byte A-operand reads), V row r keeps chunk c at
-//     c ^ ((r & 3) << 1) and is read with the transposing LDS read (ds_read_b64_tr_b16), which
+//     c ^ ((r & 7) << 1) and is read with the transposing LDS read (ds_read_b64_tr_b16), which
 //     hands each lane 4 consecutive keys of one feature: the V^T operand with no permutes.
 //   * A page is addressed through its own buffer descriptor (base = page, 64 KiB range), so
 //     pools larger than 4 GiB need no 64-bit per-lane arithmetic and out-of-page offsets
@@ -397,13 +397,13 @@ __global__ __launch_bounds__(256, 1) void attn_decode_kernel(
 #pragma unroll
   for (int j = 0; j < 4; ++j) kx[j] = (uint32_t)(c16 * 256 + (((j * 4 + g) ^ c16) << 4));
   // V: lanes 16g..16g+15 read the 4(key) x 16(feature) block of keys 4g.. and features 16i..;
-  // lane i16 addresses key 4g + i16/4, features 16i + 4(i16&3)..+3; 32-byte unit u of a row
-  // sits at u ^ (key & 3), which for u = 2i + .. is (i ^ x) in the 32-byte index, x = (i16/4) & 3.
-  const int i16 = lane & 15, vx_x = (i16 >> 2) & 3;
-  uint32_t vx[4];
+  // lane i16 addresses key 4g + i16/4, features 16i + 4(i16&3)..+3; 32-byte unit i of a row
+  // sits at i ^ (key & 7) (the 8 keys x 32 bytes of a read cycle then cover all 64 banks).
+  const int i16 = lane & 15, vx_x = ((g & 1) << 2) | ((i16 >> 2) & 3);
+  uint32_t vx[8];
 #pragma unroll
-  for (int k = 0; k < 4; ++k)
-    vx[k] = (uint32_t)((g * 4 + (i16 >> 2)) * 256 + ((k ^ vx_x) * 32) + (i16 & 3) * 8);
+  for (int i = 0; i < 8; ++i)
+    vx[i] = (uint32_t)((g * 4 + (i16 >> 2)) * 256 + ((i ^ vx_x) * 32) + (i16 & 3) * 8);
 
   for (long long w = blockIdx.x; w < (long long)batch * Hkv; w += gridDim.x) {
     const int req = (int)(w / Hkv), kvh = (int)(w % Hkv);
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(256, 1) void attn_decode_kernel(
       const int key = 4 * t4 + (lane >> 4), pos = lane & 15;
       const uint32_t row = (uint32_t)((key * Hkv + kvh) * D * 2);
       k_src[t4] = row + (uint32_t)(((pos ^ key) & 15) << 4);
-      v_src[t4] = v_half + row + (uint32_t)((pos ^ ((key & 3) << 1)) << 4);
+      v_src[t4] = v_half + row + (uint32_t)((pos ^ ((key & 7) << 1)) << 4);
     }
     const int n_sub = (qo_len + TPB - 1) / TPB;
     for (int sub = 0; sub < n_sub; ++sub) {
@@ -548,7 +548,7 @@ __global__ __launch_bounds__(256, 1) void attn_decode_kernel(
         wait_but((n1 ? 16 : 0) + (n2 ? 8 : 0));
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const uint8_t* vp = vt + vx[i & 3] + (i >> 2) * 128;
+          const uint8_t* vp = vt + vx[i];
           const short4_t lo = lds_read_tr16(vp);         // keys 4g..4g+3 of the first page
           const short4_t hi = lds_read_tr16(vp + 4096);  // ... of the second page
           typedef short short8_t __attribute__((ext_vector_type(8)));
@@ -626,7 +626,7 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
   // Decode mode (KV split over the wavefronts, one workgroup per request and kv head) is the
   // right shape when requests carry about one row each; it stays correct for any row count.
   const bool decode_mode = max_qo_rows <= batch;
-  constexpr int NQB_PREFILL = 4;
+  constexpr int NQB_PREFILL = 2;
   long long bound;
   if (decode_mode) {
     bound = (long long)batch * Hkv;

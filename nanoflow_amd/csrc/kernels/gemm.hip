@@ -13,14 +13,17 @@
 // writes 64 lanes x 16 bytes to 1 KB of consecutive LDS, so the LDS image cannot be padded;
 // bank conflicts are avoided by choosing WHICH 16-byte chunk each lane fetches (an XOR swizzle
 // applied on the global side):
+// (LDS has 64 banks of 4 bytes: a 16-byte read is served 16 lanes per cycle, an 8-byte read 32
+// lanes per cycle, each cycle covering 256 bytes of distinct banks when conflict-free.)
 //   A slab (and [N][K] weights)  rows of 128 bytes (64 k), 8 rows per instruction; row r keeps
-//       logical chunk c at position c ^ (r & 7).  An MFMA fragment is one 16-byte read; the 8
-//       lanes of a read phase hit 8 different positions.
+//       logical chunk c at position c ^ ((r >> 1) & 7).  An MFMA fragment is one 16-byte read;
+//       the 16 rows of a read cycle (two per 256 bytes) land on 16 different 16-byte slots.
 //   [K][N] weights               kept row-major, 64 rows of BN*2 bytes; row r keeps chunk c at
-//       position c ^ ((r & 3) << 1).  The k-contiguous MFMA operand is produced by the
+//       position c ^ ((r & 3) << 2).  The k-contiguous MFMA operand is produced by the
 //       transposing LDS read (ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(n) block row-wise
-//       and receive it column-wise), two per operand; the 4 rows of a block sit in 4 different
-//       32-byte bank groups.
+//       and receive it column-wise), two per operand; the 4 rows x 64 bytes a read cycle
+//       touches sit in 4 different 64-byte bank groups.
+// With these two permutations SQ_LDS_BANK_CONFLICT reads zero for the kernel.
 // No staging registers, no permutes, no LDS stores.  While the MFMAs of slab i run out of one
 // stage, the loads of slab i+1 are in flight into the other; one barrier per slab.
 //
@@ -104,8 +107,8 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
 #pragma unroll
   for (int b = 0; b < NB; ++b) b_rsrc[b] = make_rsrc(b ? B1 : B0, (size_t)N * K * 2);
   // A-style rows: lane -> (row lane/8 of the instruction's 8 rows, position lane%8), fetching
-  // logical chunk position ^ row.
-  const int a_kc = ((lane & 7) ^ (lane >> 3)) * 8;  // k of that chunk inside the slab
+  // logical chunk position ^ ((row >> 1) & 7); bit 3 of the row number is the wave's parity.
+  const int a_kc = ((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2))) * 8;
   uint32_t a_off[A_LOADS];
 #pragma unroll
   for (int t = 0; t < A_LOADS; ++t) {
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
       off = gn < N ? ((uint32_t)gn * (uint32_t)K + a_kc) * 2u : kOob;
     } else {
       const int row = (t * 4 + wave) * B_RPI + lane / B_CPR;
-      const int c = (lane % B_CPR) ^ ((row & 3) << 1);
+      const int c = (lane % B_CPR) ^ ((row & 3) << 2);
       const int gn = n_base + c * 8;
       off = gn < N ? ((uint32_t)row * (uint32_t)N + gn) * 2u : kOob;
     }
@@ -161,21 +164,23 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
   };
 
   // ---- LDS -> MFMA operand fragments, double-buffered across the 4 k-steps of a slab
-  // A-style: row r = l32 (+ tile offsets), logical chunk kk*2+lg sits at position chunk ^ (r&7).
+  // A-style: row r = l32 (+ multiples of 32), logical chunk kk*2+lg sits at chunk ^ ((r>>1)&7).
   const uint32_t a_rd = (uint32_t)(wm * (BM / WM) + l32) * 128u;
   const uint32_t bc_rd = (uint32_t)(wn * (BN / WN) + l32) * 128u;  // [N][K] weights
   uint32_t swz[4];
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) swz[kk] = (uint32_t)(((kk * 2 + lg) ^ (l32 & 7)) << 4);
+  for (int kk = 0; kk < 4; ++kk) swz[kk] = (uint32_t)(((kk * 2 + lg) ^ ((l32 >> 1) & 7)) << 4);
   // [K][N] weights: 16-lane group g reads the 4(k) x 16(n) block at rows lg*8 + 4h.., columns
   // (g&1)*16.. of the MFMA tile, lane i of the group addressing row i/4, columns (i&3)*4..+3.
-  // 32-byte unit u of a row sits at u ^ (row & 3); with u = 2*jt + (g&1) that is
-  // 2*(jt ^ x1) + ((g&1) ^ x0) for x = row & 3 = (i/4) & 3.
-  const int i16 = lane & 15, x0 = (i16 >> 2) & 1, x1 = (i16 >> 3) & 1, g1 = (lane >> 4) & 1;
-  const uint32_t br_common = (uint32_t)(lg * 8 + (i16 >> 2)) * ROWB + (uint32_t)(wn * (BN / WN)) * 2u +
-                             (uint32_t)(i16 & 3) * 8u + (uint32_t)((g1 ^ x0) * 32);
-  const uint32_t br_even = br_common + (uint32_t)x1 * 64u;        // jt even: unit pair jt + x1
-  const uint32_t br_odd = br_common + (uint32_t)(1 - x1) * 64u;   // jt odd:  unit pair jt - x1 (+ (jt-1)*64 below)
+  // 32-byte unit u of a row sits at u ^ ((row & 3) << 1), row & 3 = (i/4) & 3.
+  const int i16 = lane & 15, bx = (i16 >> 2) & 3, g1 = (lane >> 4) & 1;
+  const uint32_t br_row = (uint32_t)(lg * 8 + (i16 >> 2)) * ROWB + (uint32_t)(i16 & 3) * 8u;
+  uint32_t br_tbl[TN];  // byte offset inside the row of this lane's 8 bytes, per MFMA tile j
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int unit = (wn * (BN / WN)) / 16 + 2 * j + g1;  // logical 32-byte unit
+    br_tbl[j] = (uint32_t)((unit ^ (bx << 1)) * 32);
+  }
 
   half8_t af[2][TM];
   half8_t bf[2][NB][TN];
@@ -192,7 +197,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
         if constexpr (kBCol) {
           bf[buf][b][j] = *reinterpret_cast<const half8_t*>(bs + bc_rd + swz[kk] + j * 32 * 128);
         } else {
-          const uint8_t* p = bs + ((j & 1) ? br_odd + (j - 1) * 64 : br_even + j * 64) + kk * 16 * ROWB;
+          const uint8_t* p = bs + br_row + br_tbl[j] + kk * 16 * ROWB;
           const short4_t lo = lds_read_tr16(p);
           const short4_t hi = lds_read_tr16(p + 4 * ROWB);
           typedef short short8_t __attribute__((ext_vector_type(8)));

@@ -7,38 +7,31 @@
 //   sa[m] = max_k |x[m][k]| / 448 (1 when the row is all zero),  Aq = e4m3_rne(x / sa[m]).
 //
 // Both operands are stored with k contiguous (Aq [M][K], Bq [N][K]: one row per output
-// channel), so both are staged the same way: a slab is 128 k-bytes per row, written to LDS rows
-// of 144 bytes (16-byte skew: conflict-free 16-byte fragment reads).  Workgroup = 256 threads
-// = 4 wavefronts in a WM x WN grid; two LDS stages; while the two MFMA k-steps of slab i run,
-// slab i+1 moves from registers to the other stage and slab i+2 is loaded into registers.
-// The MFMA is issued as D^T = B.A^T so that a lane owns 4 consecutive output columns.
+// channel), so both are staged the same way: a slab is 128 k-bytes per row, moved from global
+// memory straight into LDS (buffer_load ... lds, XOR-swizzled rows, multi-stage ring -- the
+// scheme of gemm.hip with both operands in its row form).  Workgroup = 256 threads = 4
+// wavefronts in a WM x WN grid.  The MFMA is issued as D^T = B.A^T so that a lane owns 4
+// consecutive output columns.
 //
 // A dot product does not depend on which k a lane slot holds as long as both operands use the
 // same assignment; lane (l32, lg) slot s of k-step kk holds k = kk*64 + lg*32 + s for both.
+#include <type_traits>
+
 #include "common.h"
 
 namespace nf {
 
-constexpr int F8_BK = 128;          // k-bytes per slab
-constexpr int F8_LD = F8_BK + 16;   // LDS row pitch in bytes
-constexpr uint32_t kOob8 = 0xFFFFFFF0u;
+constexpr int F8_BK = 128;  // k-bytes per slab = one 128-byte LDS row per matrix row
 
 typedef int v8i32 __attribute__((ext_vector_type(8)));
-typedef uint32_t bufvec4_8 __attribute__((ext_vector_type(4)));
 
 template <int BM, int BN>
 struct F8Smem {
-  static constexpr int stage_bytes = (BM + BN) * F8_LD;
-  static constexpr size_t bytes = 2 * (size_t)stage_bytes;
+  static constexpr int stage_bytes = (BM + BN) * 128;
+  static constexpr int stages = (144 * 1024) / stage_bytes > 4 ? 4 : (144 * 1024) / stage_bytes;
+  static_assert(stages >= 2, "tile too large for two LDS stages");
+  static constexpr size_t bytes = (size_t)stages * stage_bytes;
 };
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc8(const void* p, size_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)(uint32_t)bytes, 0x00020000);
-}
-__device__ __forceinline__ u32x4 buf_load16_8(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
-  bufvec4_8 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
-  return u32x4{v.x, v.y, v.z, v.w};
-}
 
 // Round-to-nearest-even OCP e4m3 (bias 7, no infinities, max 448), saturating.
 __device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
@@ -107,11 +100,14 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   using SM = F8Smem<BM, BN>;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(WM * WN == 4, "four wavefronts");
-  constexpr int A_CHUNKS = BM * 8 / 256;  // 16-byte chunks per thread per slab
-  constexpr int B_CHUNKS = BN * 8 / 256;
-  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for 256 threads");
+  constexpr int A_LOADS = BM / 32;  // 1 KB (8 rows) load instructions per wave per slab
+  constexpr int B_LOADS = BN / 32;
+  constexpr int NS = SM::stages;
+  constexpr int LOADS = A_LOADS + B_LOADS;
+  constexpr int PARTS = 2;          // the loads of a slab are spread over its two k-steps
 
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem8[];
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem8[];
+  const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem8;
 
   // XCD-aware tile order (workgroup ids round-robin over 8 XCDs): each XCD walks one
   // contiguous range of tiles, M fastest, so a weight panel stays in that XCD's L2.
@@ -122,7 +118,8 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
   const int m_base = tile_m * BM, n_base = tile_n * BN;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int l32 = lane & 31, lg = lane >> 5;
 
@@ -134,66 +131,58 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc8(A, (size_t)M * K);
-  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc8(B, (size_t)N * K);
-  u32x4 a_reg[A_CHUNKS], b_reg[B_CHUNKS];
-  uint32_t a_off[A_CHUNKS], b_off[B_CHUNKS];
-  const int kc = tid & 7;  // this thread's 16-byte column within a slab row
+  // Both operands are rows of 128 k-bytes; they go from global memory straight into LDS
+  // (see gemm.hip): 8 rows per load instruction, row r keeping its logical 16-byte chunk c at
+  // position c ^ ((r >> 1) & 7) (bit 3 of the row number is the wave's parity).
+  const rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K);
+  const rsrc_t b_rsrc = make_rsrc(B, (size_t)N * K);
+  const int kc = ((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2))) * 16;  // k-byte of this lane's chunk inside the slab
+  uint32_t a_off[A_LOADS], b_off[B_LOADS];
 #pragma unroll
-  for (int i = 0; i < A_CHUNKS; ++i) {
-    const int gm = m_base + ((tid + 256 * i) >> 3);
-    a_off[i] = gm < M ? (uint32_t)gm * (uint32_t)K + kc * 16 : kOob8;
+  for (int t = 0; t < A_LOADS; ++t) {
+    const int gm = m_base + (t * 4 + wave) * 8 + (lane >> 3);
+    a_off[t] = gm < M ? (uint32_t)gm * (uint32_t)K + kc : kOob;
   }
 #pragma unroll
-  for (int i = 0; i < B_CHUNKS; ++i) {
-    const int gn = n_base + ((tid + 256 * i) >> 3);
-    b_off[i] = gn < N ? (uint32_t)gn * (uint32_t)K + kc * 16 : kOob8;
+  for (int t = 0; t < B_LOADS; ++t) {
+    const int gn = n_base + (t * 4 + wave) * 8 + (lane >> 3);
+    b_off[t] = gn < N ? (uint32_t)gn * (uint32_t)K + kc : kOob;
   }
-
-  // part 0 / 1 = even / odd chunks (one half of the staging work per MFMA k-step); < 0 = all
-  auto load_part = [&](int k0, int part) {
-    const bool k_ok = k0 + kc * 16 < K;
+  auto issue_loads = [&](int stage, int k0, int part) {
+    const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::stage_bytes + wave * 1024);
+    const bool k_ok = k0 + kc < K;
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      if (part >= 0 && (i & 1) != part) continue;
-      a_reg[i] = buf_load16_8(a_rsrc, (k_ok && a_off[i] != kOob8) ? a_off[i] + (uint32_t)k0 : kOob8);
+    for (int t = 0; t < A_LOADS; ++t) {
+      if (part >= 0 && t % PARTS != part) continue;
+      load16_to_lds(a_rsrc, (k_ok && a_off[t] != kOob) ? a_off[t] + (uint32_t)k0 : kOob, st + t * 4096);
     }
 #pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      if (part >= 0 && (i & 1) != part) continue;
-      b_reg[i] = buf_load16_8(b_rsrc, (k_ok && b_off[i] != kOob8) ? b_off[i] + (uint32_t)k0 : kOob8);
-    }
-  };
-  auto store_part = [&](int stage, int part) {
-    uint8_t* As = smem8 + stage * SM::stage_bytes;
-    uint8_t* Bs = As + BM * F8_LD;
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      if (part >= 0 && (i & 1) != part) continue;
-      *reinterpret_cast<u32x4*>(As + ((tid + 256 * i) >> 3) * F8_LD + kc * 16) = a_reg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      if (part >= 0 && (i & 1) != part) continue;
-      *reinterpret_cast<u32x4*>(Bs + ((tid + 256 * i) >> 3) * F8_LD + kc * 16) = b_reg[i];
+    for (int t = 0; t < B_LOADS; ++t) {
+      if (part >= 0 && (A_LOADS + t) % PARTS != part) continue;
+      load16_to_lds(b_rsrc, (k_ok && b_off[t] != kOob) ? b_off[t] + (uint32_t)k0 : kOob,
+                    st + BM * 128 + t * 4096);
     }
   };
 
+  // MFMA operand of k-step kk: 32 bytes of row r = the logical chunks 4kk + 2lg and + 1, which
+  // sit at positions p and p ^ 1 with p = (4kk + 2lg) ^ ((r >> 1) & 7).
+  const uint32_t a_rd = (uint32_t)(wm * (BM / WM) + l32) * 128u;
+  const uint32_t b_rd = (uint32_t)(BM * 128 + (wn * (BN / WN) + l32) * 128);
+  uint32_t swz[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) swz[kk] = (uint32_t)(((kk * 4 + lg * 2) ^ ((l32 >> 1) & 7)) << 4);
   v8i32 af[2][TM], bf[2][TN];
-  auto read32 = [&](const uint8_t* p) {
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(p);
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(p + 16);
+  auto read32 = [&](const uint8_t* p, uint32_t pos) {
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(p + pos);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(p + (pos ^ 16u));
     return v8i32{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
   };
   auto read_frags = [&](int stage, int kk, int buf) {
-    const uint8_t* As = smem8 + stage * SM::stage_bytes;
-    const uint8_t* Bs = As + BM * F8_LD;
+    const uint8_t* st = smem8 + stage * SM::stage_bytes;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
-      af[buf][i] = read32(As + (wm * (BM / WM) + i * 32 + l32) * F8_LD + kk * 64 + lg * 32);
+    for (int i = 0; i < TM; ++i) af[buf][i] = read32(st + a_rd + i * 32 * 128, swz[kk]);
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-      bf[buf][j] = read32(Bs + (wn * (BN / WN) + j * 32 + l32) * F8_LD + kk * 64 + lg * 32);
+    for (int j = 0; j < TN; ++j) bf[buf][j] = read32(st + b_rd + j * 32 * 128, swz[kk]);
   };
   auto mfma_step = [&](int buf) {
 #pragma unroll
@@ -204,36 +193,52 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
                                                                     0, 0, 0, 0, 0, 0);
   };
 
-  // Steady state of slab s (LDS stage s&1), two k-steps:
-  //   step 0: prefetch step 1's fragments; write half of slab s+1 (held in registers) to the
-  //           other stage and refill those registers from slab s+2;
-  //   step 1: write the other half, barrier, prefetch slab s+1's first fragments, refill.
-  auto slab = [&](int s, bool do_store, bool do_load) {
-    const int cur = s & 1;
-    read_frags(cur, 1, 1);
-    if (do_store) store_part(cur ^ 1, 0);
-    if (do_load) load_part((s + 2) * F8_BK, 0);
-    mfma_step(0);
-    if (do_store) store_part(cur ^ 1, 1);
-    __syncthreads();
-    if (do_store) read_frags(cur ^ 1, 0, 0);
-    if (do_load) load_part((s + 2) * F8_BK, 1);
-    mfma_step(1);
+  // Slab s lives in LDS stage s % NS; while its two k-steps run, the loads of slab s+NS-1 go
+  // into the stage slab s-1 has left; at the end the wavefront waits for its loads of slab s+1
+  // (younger ones may stay in flight) and meets the others at the barrier.
+  auto slab = [&](auto issue_c, int s, int cs, int ls) {
+    constexpr bool issue = decltype(issue_c)::value;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      if (issue) issue_loads(ls, (s + NS - 1) * F8_BK, kk);
+      if (kk < 1) read_frags(cs, kk + 1, (kk + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_step(kk & 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
+  auto wait_loads = [&](int younger) {  // vmcnt(younger): bits [3:0] and [15:14]
+    if (younger == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS * (NS - 2) & 15) | (((LOADS * (NS - 2)) >> 4) << 14));
+  };
+  static_assert(LOADS * (NS - 2) < 64, "vmcnt range");
+  auto next = [](int st) { return st + 1 == NS ? 0 : st + 1; };
 
   const int nslab = (K + F8_BK - 1) / F8_BK;
-  load_part(0, -1);
-  store_part(0, -1);
-  if (nslab > 1) load_part(F8_BK, -1);
+#pragma unroll
+  for (int p = 0; p < NS - 1; ++p)
+    if (p < nslab) issue_loads(p, p * F8_BK, -1);
+  if (nslab >= NS - 1) wait_loads(1); else wait_loads(0);
   __syncthreads();
   read_frags(0, 0, 0);
-  int s = 0;
-  for (; s + 2 < nslab; ++s) slab(s, true, true);
-  if (s + 1 < nslab) {
-    slab(s, true, false);
-    ++s;
+  int cs = 0, ls = NS - 1, s = 0;
+  for (; s + NS - 1 < nslab; ++s) {
+    slab(std::true_type{}, s, cs, ls);
+    wait_loads(1);
+    __syncthreads();
+    cs = next(cs);
+    ls = next(ls);
+    read_frags(cs, 0, 0);
   }
-  slab(s, false, false);
+  for (; s < nslab; ++s) {
+    slab(std::false_type{}, s, cs, ls);
+    if (s + 1 < nslab) {
+      wait_loads(0);
+      __syncthreads();
+      cs = next(cs);
+      read_frags(cs, 0, 0);
+    }
+  }
 
   // Epilogue: acc[i][j][r] is D[m][n] with m = tile row l32, n = (r/4)*8 + lg*4 + r%4.
 #pragma unroll
@@ -247,10 +252,10 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
       for (int qd = 0; qd < 4; ++qd) {
         const int gn = n_base + wn * (BN / WN) + j * 32 + qd * 8 + lg * 4;
         if (gn >= N) continue;  // N % 8 == 0 and gn % 4 == 0: the whole quad is in or out
-        const float4_t cs = *reinterpret_cast<const float4_t*>(sb + gn);
+        const float4_t cs4 = *reinterpret_cast<const float4_t*>(sb + gn);
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = row_scale * cs[e] * acc[i][j][qd * 4 + e];
+        for (int e = 0; e < 4; ++e) v[e] = row_scale * cs4[e] * acc[i][j][qd * 4 + e];
         if (beta != 0.f) {
           const u32x2 c = *reinterpret_cast<const u32x2*>(C + (size_t)gm * N + gn);
           v[0] += beta * h2f_bits(c.x & 0xffffu);

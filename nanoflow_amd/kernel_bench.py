@@ -5,6 +5,7 @@
     python -m nanoflow_amd.kernel_bench --op dual --m 1024
     python -m nanoflow_amd.kernel_bench --op gemm_f8 --m 2048
     python -m nanoflow_amd.kernel_bench --op attn --requests 1792 --kv-lo 1024 --kv-hi 1536
+    python -m nanoflow_amd.kernel_bench --op prefill --chunks 755:269,0:1024,0:74
     python -m nanoflow_amd.kernel_bench --op copy                     # counter-calibration kernel
 
 Each line reports the average launch time over --iters launches (HIP events on the launch
@@ -47,7 +48,9 @@ def layer_shapes(shape: synth.ModelShape, M: int):
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--op", required=True, choices=["gemm", "dual", "gemm_f8", "attn", "copy"])
+    ap.add_argument("--op", required=True, choices=["gemm", "dual", "gemm_f8", "attn", "prefill", "copy"])
+    ap.add_argument("--chunks", default="755:269,0:1024,0:74",
+                    help="prefill: prev_len:chunk_len per request (default: a steady-state offline iteration)")
     ap.add_argument("--model", default="8b", choices=["8b", "70b"])
     ap.add_argument("--m", type=int, default=2048, help="rows (tokens) of the GEMM operand")
     ap.add_argument("--only", default="", help="gemm: run only this role (kqv, o, down, lm_head)")
@@ -101,6 +104,21 @@ def main():
         nbytes = int((2 * L * shape.Hkv * shape.d * 2 + 2 * shape.Hq * shape.d * 2 + 4 * ((L + 15) // 16 + 2)).sum())
         print(f"decode attention {nd} requests, KV [{a.kv_lo},{a.kv_hi}]: {ms * 1e3:9.1f} us  "
               f"{nbytes / ms / 1e6:8.1f} GB/s  ({nbytes} algorithmic bytes per launch)", flush=True)
+    elif a.op == "prefill":
+        chunks = [tuple(int(x) for x in c.split(":")) for c in a.chunks.split(",")]
+        b = synth.make_batch([], chunks, vocab=shape.vocab, seed=0)
+        pool = rnd(b.num_pages, 2, shape.page_size, shape.Hkv, shape.d)
+        q = rnd(b.tokens, shape.Hq * shape.d)
+        o = torch.zeros_like(q)
+        t = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(DEV)
+        qi, kvp, kvi, kvl = t(b.input_indptr), t(b.kv_indptr), t(b.kv_indices), t(b.kv_last_page_len)
+        ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+        fn = lambda: K.attention_paged(q, qi, pool, kvp, kvi, kvl, shape.Hq, shape.Hkv, causal=True, out=o,
+                                       batch=len(chunks), max_qo_rows=b.tokens, workspace=ws)
+        ms = timeit(fn, a.iters, a.warm)
+        flops = sum(l * (2 * (p + l) - l) * 2 * shape.Hq * shape.d for p, l in chunks)
+        print(f"chunked-prefill attention {chunks}: {ms * 1e3:9.1f} us  {flops / ms / 1e9:8.1f} TFLOP/s "
+              f"(causal flops of gemv/src/bench_batch_prefill.cu:133-134)", flush=True)
     else:
         n = a.mib << 20
         src = torch.empty(n, dtype=torch.uint8, device=DEV).random_(generator=g)
