@@ -36,10 +36,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0       # dense fp16
 A100_PUBLISHED_TOKENS_PER_S = 12756.0   # reference, 1x A100 80GB, same offline workload
-# HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
-# as a ratio to the algorithmic bytes of the same launch; None until measured
-# (see profiles/decode_attention_config2_pmc.txt when present).
-DECODE_ATTN_TRAFFIC_RATIO = None
+# HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
+# by what the same counter reads for a 1 GiB device copy), as a ratio to the algorithmic bytes of
+# the same launch: profiles/decode_attention_config2_pmc.txt.
+DECODE_ATTN_TRAFFIC_RATIO = 1.0072
 
 
 def decode_attention_bytes(kv_len: np.ndarray, Hq=32, Hkv=8, d=128, page=16) -> int:
@@ -335,7 +335,9 @@ def main():
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default: offline 256, iteration 5)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps (default: offline 8, iteration 2)")
     ap.add_argument("--workload", default="offline", choices=["offline", "iteration"])
-    ap.add_argument("--pipeline", default="LOCAL", choices=["LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL"])
+    ap.add_argument("--pipeline", default="auto", choices=["auto", "LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL"],
+                    help="auto = the faster schedule measured on MI355X for the workload: NON_OVERLAP_LOCAL for\n"
+                         "offline, LOCAL (two streams) for iteration")
     ap.add_argument("--nano1", type=int, default=1024, help="rows of nano-batch 1")
     ap.add_argument("--kqv1", type=int, default=512)
     ap.add_argument("--kqv3", type=int, default=512)
@@ -354,6 +356,8 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     _check_single_gpu(args)
+    if args.pipeline == "auto":
+        args.pipeline = "NON_OVERLAP_LOCAL" if args.workload == "offline" else "LOCAL"
     if args.graph:
         args.profile_level = 0
     rec = run_offline(args) if args.workload == "offline" else run_iteration(args)
