@@ -55,7 +55,10 @@ struct vortexModelConfig {
     kqv_n = model_hidden_dim_pergpu + 2 * model_hidden_dim_pergpu / model_gqa;
     page_mem_size = (size_t)frame_page_size * model_kv_heads_gpu * model_head_dim * 2 * 2;
     max_page_num = (size_t)allocate_kv_data_batch * ((1024 + frame_page_size - 1) / frame_page_size);
-    k_temp_size = (size_t)max_batch_size * model_hidden_dim * 16 + (size_t)max_batch_size * vocab_size * 2;
+    // the reference's figure (config.h:100) plus room for the FFN activation rows, which it only
+    // covers when the vocabulary term is large
+    k_temp_size = (size_t)max_batch_size * model_hidden_dim * 16 + (size_t)max_batch_size * vocab_size * 2 +
+                  (size_t)max_batch_size * model_ff_dim + 65536;
     if (!rope_3_1) {
       smooth_a = 0;
       smooth_b = 0;

@@ -373,8 +373,8 @@ __global__ __launch_bounds__(256, SPLIT ? 2 : 1) void attn_paged_kernel(
 //   * A page is addressed through its own buffer descriptor (base = page, 64 KiB range), so
 //     pools larger than 4 GiB need no 64-bit per-lane arithmetic and out-of-page offsets
 //     (used to zero-fill V rows past the end of the sequence) read as zero.
-template <int GROUP>
-__global__ __launch_bounds__(256, 1) void attn_decode_kernel(
+template <int GROUP, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ o, const int32_t* __restrict__ qo_indptr,
     const uint16_t* __restrict__ kv_data, const int32_t* __restrict__ kv_indptr,
     const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_last_page_len, int batch,
@@ -483,14 +483,14 @@ __global__ __launch_bounds__(256, 1) void attn_decode_kernel(
         dma_k(wave, 0);
         dma_v(wave, 0);
       }
-      if (wave + 4 < npairs) {
-        dma_k(wave + 4, 1);
-        dma_v(wave + 4, 1);
+      if (wave + NW < npairs) {
+        dma_k(wave + NW, 1);
+        dma_v(wave + NW, 1);
       }
       int buf = 0;
-      for (int pp = wave; pp < npairs; pp += 4, buf ^= 1) {
+      for (int pp = wave; pp < npairs; pp += NW, buf ^= 1) {
         const int t_base = pp * 32;
-        const bool n1 = pp + 4 < npairs, n2 = pp + 8 < npairs;
+        const bool n1 = pp + NW < npairs, n2 = pp + 2 * NW < npairs;
         const uint8_t* kt = wptr + buf * 8192;
         const uint8_t* vt = wptr + 16384 + buf * 8192;
 
@@ -509,7 +509,7 @@ __global__ __launch_bounds__(256, 1) void attn_decode_kernel(
         // the K tile is free as soon as those reads have returned: s depends on them
         if (n2) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          dma_k(pp + 8, buf);
+          dma_k(pp + 2 * NW, buf);
         }
 
         // ---- online softmax; lane holds keys t_base + blk*16 + g*4 + r of column c16
@@ -558,7 +558,7 @@ __global__ __launch_bounds__(256, 1) void attn_decode_kernel(
         }
         if (n2) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          dma_v(pp + 8, buf);
+          dma_v(pp + 2 * NW, buf);
         }
       }
       l_run += __shfl_xor(l_run, 16, 64);
@@ -576,31 +576,31 @@ __global__ __launch_bounds__(256, 1) void attn_decode_kernel(
       s_m[lane] = m_run;
       s_l[lane] = l_run;
       __syncthreads();
-      float M = -1e30f, mw[4];
+      float M = -1e30f, mw[NW];
 #pragma unroll
-      for (int ww = 0; ww < 4; ++ww) {
+      for (int ww = 0; ww < NW; ++ww) {
         mw[ww] = *reinterpret_cast<const float*>(lds + ww * WAVE_LDS + 8192 + lane * 4);
         M = fmaxf(M, mw[ww]);
       }
-      float wgt[4], L = 0.f;
+      float wgt[NW], L = 0.f;
 #pragma unroll
-      for (int ww = 0; ww < 4; ++ww) {
+      for (int ww = 0; ww < NW; ++ww) {
         wgt[ww] = __builtin_amdgcn_exp2f(mw[ww] - M);
         L += wgt[ww] * *reinterpret_cast<const float*>(lds + ww * WAVE_LDS + 8192 + 256 + lane * 4);
       }
       const float inv = L > 0.f ? 1.0f / L : 0.f;
       if (live) {
-        // wavefront w finishes features 32w .. 32w+31 (i = 2w, 2w+1): 4 consecutive per lane and i
+        // wavefront w finishes 8/NW of the 16-feature blocks: 4 consecutive features per lane and i
         uint16_t* op = o + ((size_t)(qo0 + tq) * Hq + kvh * GROUP + c16 % GROUP) * D;
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int i = 2 * wave + e;
+        for (int e = 0; e < 8 / NW; ++e) {
+          const int i = (8 / NW) * wave + e;
           float v[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float acc = 0.f;
 #pragma unroll
-            for (int ww = 0; ww < 4; ++ww)
+            for (int ww = 0; ww < NW; ++ww)
               acc += wgt[ww] * *reinterpret_cast<const float*>(lds + ww * WAVE_LDS + ((i * 4 + r) * 64 + lane) * 4);
             v[r] = acc * inv;
           }
@@ -639,8 +639,9 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
   if (bound > 0x7fffffffLL) bound = 0x7fffffffLL;
   if (bound < 1) bound = 1;
   if (decode_mode) {
-    constexpr int kDecodeLds = 4 * 32768;
-    auto kern = attn_decode_kernel<GROUP>;
+    constexpr int kWaves = 4;  // wavefronts per (request, kv head) workgroup
+    constexpr int kDecodeLds = kWaves * 32768;
+    auto kern = attn_decode_kernel<GROUP, kWaves>;
     static bool attr_set = false;  // benign race: the call is idempotent
     if (!attr_set) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -651,7 +652,7 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
       }
       attr_set = true;
     }
-    kern<<<(int)bound, 256, kDecodeLds, stream>>>(q, o, qo_indptr, kv_data, kv_indptr, kv_indices,
+    kern<<<(int)bound, kWaves * 64, kDecodeLds, stream>>>(q, o, qo_indptr, kv_data, kv_indptr, kv_indices,
                                                   kv_last_page_len, batch, Hq, Hkv, causal, scale_log2);
   } else
     attn_paged_kernel<GROUP, NQB_PREFILL, false><<<(int)bound, 256, 0, stream>>>(

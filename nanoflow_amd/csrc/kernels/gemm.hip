@@ -226,16 +226,10 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
     constexpr bool issue = decltype(issue_c)::value;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-#if !defined(NF_EXP_NOLOAD)
       if (issue && kk < PARTS) issue_loads(ls, (s + NS - 1) * BK, kk);
-#endif
-#if !defined(NF_EXP_NOFRAG)
       if (kk < 3) read_frags(cs, kk + 1, (kk + 1) & 1);
-#endif
       __builtin_amdgcn_sched_barrier(0);  // the fragment reads go out before this step's MFMAs
-#if !defined(NF_EXP_NOMFMA)
       mfma_step(kk & 1);
-#endif
       __builtin_amdgcn_sched_barrier(0);
     }
   };

@@ -137,14 +137,19 @@ class Engine:
         init.setTmpBuffer(self.tmp.data_ptr(), self.tmp.numel())
         torch.cuda.synchronize()
         P.setProfiling(int(profiling))
-        P.init([init], pipeline_type)
-        cfg = P.VortexConfigData()
-        cfg.setGemmOpTag([DEFAULT_TAG] * n_tags)
-        cfg.globalBatchSize, cfg.nanobatch1Size = global_batch, nano1
-        cfg.kqv1Size, cfg.kqv3Size = self.kqv1, self.kqv3
-        P.config([cfg])
-        self._open = True
+        self._open = False
         self._hold = None
+        P.init([init], pipeline_type)
+        self._open = True
+        try:
+            cfg = P.VortexConfigData()
+            cfg.setGemmOpTag([DEFAULT_TAG] * n_tags)
+            cfg.globalBatchSize, cfg.nanobatch1Size = global_batch, nano1
+            cfg.kqv1Size, cfg.kqv3Size = self.kqv1, self.kqv3
+            P.config([cfg])
+        except Exception:
+            self.close()        # never leave the worker thread waiting behind a failed set-up
+            raise
 
     # ------------------------------------------------------------------ per iteration
     def update(self, b: synth.Batch, keep_token_list=None, num_blocks=(0, 0, 0, 0)):

@@ -10,6 +10,7 @@ There is no fallback: a missing ``libnf_pipeline.so`` raises.
 """
 from __future__ import annotations
 
+import atexit
 import ctypes as C
 import enum
 import os
@@ -193,6 +194,7 @@ def lib() -> C.CDLL:
                 f"{LIB_PATH} is missing: build it with `make -C nanoflow_amd/csrc` (no fallback)")
         # the host library resolves libnf_kernels.so through its $ORIGIN rpath
         l = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+        atexit.register(l.pllm_finalize)   # a pipeline left open must not keep the process alive
         l.pllm_last_error.restype = C.c_char_p
         l.pllm_set_model_config.argtypes = [C.c_char_p]
         l.pllm_set_rank.argtypes = [C.c_int, C.c_int]

@@ -193,3 +193,33 @@ def test_pool_exhaustion_is_reported_not_fatal():
     with pytest.raises(AssertionError, match="Out of memory"):
         py.form()
     assert cpp.state()["queued"] == len(py.queue)
+
+
+def test_offline_trace_at_full_scale():
+    # the offline-throughput workload itself: 4096 requests, 1024-token prompts, 512 outputs,
+    # 2048 tokens per iteration; scheduler only (no GPU)
+    f = P.BatchFormer(120000, 16, 2048, 1024, 512, 512, 1024, 512)
+    rng = np.random.default_rng(0)
+    for i in range(4096):
+        f.add_request(i, rng.integers(0, 128256, 1024), 512)
+    cycles, full, steady = 0, 0, []
+    while True:
+        st = f.state()
+        if st["queued"] + st["decoding"] + st["prefilling"] == 0:
+            break
+        f.schedule()
+        b = f.form()
+        tok = b["decodePrefillBorder"] + b["prefillTokensNum"]
+        assert tok <= 2048
+        full += tok == 2048
+        if 1300 <= cycles < 2800:
+            steady.append(b["decodePrefillBorder"])
+        assert int(np.sum(b["gemv_batch_size"])) == b["decodePrefillBorder"]
+        f.advance(0.0, True)
+        cycles += 1
+    st = f.state()
+    assert st["retired"] == 4096 and st["free_pages"] == 120000
+    # every request occupies 1024 prefill rows + 511 decode rows
+    assert cycles >= 4096 * 1535 // 2048
+    assert full > 2900                                   # the batch is full until the trace drains
+    assert 675 < np.mean(steady) < 690                   # steady state: ~682 decode rows per iteration
