@@ -183,6 +183,12 @@ NF_PLLM_API int pllm_sched_retired_output(nf_batch_former* f, int which, int* re
                                           int cap);
 /* check_future_page_usage (serve_8B.py:177-203): out[0..n) pages in use i iterations ahead;
  * returns the forecast length (average_prefill + average_decode + 2). */
+/* Bookkeeping of retired request `which` as the reference writes it to its .req_time file
+ * (serve_8B.py:795-797): times = {request_comein_time, encode_latency, decode_start_at,
+ * decode_latency}, in the seconds of the `now` values passed to pllm_sched_advance (pllm_serve
+ * uses a monotonic clock). */
+NF_PLLM_API int pllm_sched_retired_info(nf_batch_former* f, int which, int* req_idx, int* input_len,
+                                        int* output_len, double times[4]);
 NF_PLLM_API int pllm_sched_future_page_usage(nf_batch_former* f, int64_t* out, int cap);
 
 /* What the reference prints to its .stat file (serve_8B.py:755-793) plus the CPU-side split

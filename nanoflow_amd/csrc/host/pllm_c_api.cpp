@@ -457,6 +457,23 @@ int pllm_sched_retired_output(nf_batch_former* f, int which, int* req_idx, int32
   return n;
 }
 
+int pllm_sched_retired_info(nf_batch_former* f, int which, int* req_idx, int* input_len, int* output_len,
+                            double times[4]) {
+  if (!f || which < 0 || which >= (int)f->retired.size())
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_retired_info: bad index %d", which);
+  const FlyRequest& r = *f->retired[which];
+  if (req_idx) *req_idx = r.req_idx;
+  if (input_len) *input_len = r.input_len;
+  if (output_len) *output_len = r.output_len;
+  if (times) {
+    times[0] = r.request_comein_time;
+    times[1] = r.encode_latency;
+    times[2] = r.decode_start_at;
+    times[3] = r.decode_latency;
+  }
+  return NF_PLLM_OK;
+}
+
 int pllm_sched_future_page_usage(nf_batch_former* f, int64_t* out, int cap) {
   if (!f || (cap > 0 && !out)) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_sched_future_page_usage: null");
   std::vector<long long> u = f->former.future_page_usage();

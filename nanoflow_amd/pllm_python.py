@@ -351,7 +351,7 @@ class ServeStats(C.Structure):
 SYMBOLS += [
     "pllm_sched_create", "pllm_sched_destroy", "pllm_sched_add_request", "pllm_sched_schedule",
     "pllm_sched_form", "pllm_sched_harvest", "pllm_sched_advance", "pllm_sched_state",
-    "pllm_sched_retired_output", "pllm_sched_future_page_usage", "pllm_serve",
+    "pllm_sched_retired_output", "pllm_sched_retired_info", "pllm_sched_future_page_usage", "pllm_serve",
 ]
 
 
@@ -369,6 +369,8 @@ def _sched_lib():
         l.pllm_sched_advance.argtypes = [C.c_void_p, C.c_double, C.c_int, C.POINTER(C.c_int)]
         l.pllm_sched_state.argtypes = [C.c_void_p, C.POINTER(C.c_int * 5)]
         l.pllm_sched_retired_output.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), _i32p, C.c_int]
+        l.pllm_sched_retired_info.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                              C.POINTER(C.c_int), C.POINTER(C.c_double * 4)]
         l.pllm_sched_future_page_usage.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.c_int]
         l.pllm_serve.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(ServeStats)]
         l._sched_declared = True
@@ -446,6 +448,13 @@ class BatchFormer:
         if n < 0:
             _check(n, "sched_retired_output")
         return idx.value, out[:n].copy()
+
+    def retired_info(self, which) -> dict:
+        idx, il, ol, t = C.c_int(), C.c_int(), C.c_int(), (C.c_double * 4)()
+        _check(self._l.pllm_sched_retired_info(self._h, which, C.byref(idx), C.byref(il), C.byref(ol), C.byref(t)),
+               "sched_retired_info")
+        return dict(req_idx=idx.value, input_len=il.value, output_len=ol.value, request_comein_time=t[0],
+                    encode_latency=t[1], decode_start_at=t[2], decode_latency=t[3])
 
     def future_page_usage(self):
         n = self._l.pllm_sched_future_page_usage(self._h, None, 0)

@@ -286,3 +286,39 @@ def test_graph_replay_is_identical_to_eager(pt_name):
     for i, ((s0, h0), (s1, h1)) in enumerate(zip(eager, replay)):
         assert np.array_equal(s0, s1), (i, "sampled ids")
         assert np.array_equal(h0, h1), (i, "residual stream")
+
+
+@pytest.mark.parametrize("online", [False, True])
+def test_serve_command_line_writes_the_reference_result_files(tmp_path, online):
+    """nanoflow_amd.serve with the reference's flags on a tiny model: offline trace (whole loop in
+    the library) and a trace with arrival times (loop driven per phase)."""
+    import subprocess, sys, os, csv
+    from nanoflow_amd import engine, pllm_python as P
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    cfg = tmp_path / "tiny.json"
+    engine.write_config(str(cfg), shape, global_batch=96, nano1=40, kqv1=20, kqv3=28,
+                        pipeline_type=P.PipelineType.LOCAL, kv_pages=256)
+    trace = tmp_path / "trace.csv"
+    with open(trace, "w") as f:
+        f.write("idx,input_len,output_len,arrival\n")
+        for i in range(16):
+            f.write(f"{i},{20 + 3 * i},{4 + i % 5},{0.02 * i if online else 0}\n")
+    prefix = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, "-m", "nanoflow_amd.serve", "-t", str(trace), "-c", str(cfg), "-r", "400",
+           "-s", "2" if online else "0", "--est_cycle_time", "0.05", "--empty_weight", "True", "-o", str(prefix)]
+    print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    rows = list(csv.DictReader(open(str(prefix) + ".stat.csv")))
+    assert list(rows[0].keys()) == ["total_time", "token_per_second", "token_per_second_per_gpu", "total_cycle",
+                                    "cycle_time", "average_ttft", "average_tpot", "average_normalize_latency"]
+    assert float(rows[0]["token_per_second"]) > 0 and int(rows[0]["total_cycle"]) > 0
+    times = list(csv.DictReader(open(str(prefix) + ".req_time")))
+    # requests admitted during the skip cycles are left out of the latency file (as in the reference)
+    got = sorted(int(t["req_idx"]) for t in times)
+    assert got == list(range(got[0], 16)) and (len(got) == 16 if not online else len(got) >= 8)
+    for t in times:
+        assert int(t["input_len"]) == 20 + 3 * int(t["req_idx"])
+        assert float(t["encode_latency"]) >= 0 and float(t["decode_latency"]) >= 0
+    assert "Token per second" in open(str(prefix) + ".stat").read()
