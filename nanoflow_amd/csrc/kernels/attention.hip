@@ -1,5 +1,5 @@
-// Paged-KV attention for gfx950: decode (one query row per request, HBM-bound) and
-// chunked prefill (causal, many rows) from one kernel template on v_mfma_f32_16x16x32_f16.
+// Paged-KV attention for gfx950: decode (one query row per request, HBM-bound) and chunked
+// prefill (causal, many rows) on v_mfma_f32_16x16x32_f16.
 //
 // Formulation per (request, kv head):   S^T = K . Q^T   then   O^T = V^T . P^T
 //   * the MFMA "column" dimension (16 wide) carries query rows: column c of a block is
@@ -7,23 +7,16 @@
 //     uses 4 live columns and a prefill block packs 16 / GROUP tokens;
 //   * S^T comes out of the first MFMA with a lane holding 4 consecutive kv positions of one
 //     column -- exactly the B-operand layout of the second MFMA, so P never leaves registers;
-//   * K rows are loaded straight into A-operand registers (16 bytes per lane per MFMA);
-//   * V^T operands are built from eight 16-byte row loads by an 8x8 half transpose in
-//     registers (32 byte-permutes); the output row order is chosen so that each lane ends with
-//     8 consecutive features per register quad (16-byte stores).
+//   * K and V pages go from global memory straight into LDS (buffer_load ... lds); K rows are
+//     read back as 16-byte A operands, V^T operands come from the transposing LDS read.
 // Online softmax runs in the exp2 domain with fp32 state per column; masked keys contribute
 // exactly zero (the reference's -5e4 mask underflows to zero in fp32 as well).
 //
-// The key loop is software-pipelined on the operand registers themselves: the K loads of step
-// i+1 are issued as soon as the score MFMAs of step i have consumed K, the V loads of step
-// i+1 as soon as the transposes of step i have consumed V, and the page ids of step i+1 are
-// fetched (scalar) at the top of step i -- every wavefront keeps a K and a V tile in flight.
-//
-// Decode mode: a workgroup's 4 wavefronts split the request's pages (32 keys per step each)
-// and merge (m, l, O) through LDS; work item = (request, kv head), head fastest, so that
-// concurrently running workgroups stream the same 64 KiB pages.  Prefill mode: each wavefront
-// owns its own query tile; tiles are planned on the device from qo_indptr (prefix of tiles per
-// request) -- no host round trip in either mode.
+// Decode: a workgroup's 4 wavefronts split the request's pages (32 keys per step each) and
+// merge (m, l, O) through LDS; work item = (request, kv head), head fastest, so that
+// concurrently running workgroups stream the same 64 KiB pages.  Prefill: a workgroup is a
+// 16-token tile (for GQA 4) whose wavefronts share the streamed K/V tiles; tiles are planned
+// on the device from qo_indptr (prefix of tiles per request) -- no host round trip in either mode.
 #include "common.h"
 
 namespace nf {
@@ -31,30 +24,11 @@ namespace nf {
 constexpr int D = 128;      // head_dim
 constexpr int PAGE = 16;    // kv entries per page
 
-__device__ __forceinline__ uint32_t pk_lo(uint32_t x, uint32_t y) {
-  return __builtin_amdgcn_perm(y, x, 0x05040100u);
-}
-__device__ __forceinline__ uint32_t pk_hi(uint32_t x, uint32_t y) {
-  return __builtin_amdgcn_perm(y, x, 0x07060302u);
-}
-
 union H8 {
   u32x4 u;
   half8_t h;
   uint32_t w[4];
 };
-
-// KV pages are read exactly once per launch: load them with the non-temporal hint so the
-// stream does not displace the working set of kernels running beside this one.
-typedef uint32_t nt_vec4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ u32x4 load_stream16(const uint16_t* p) {
-#ifdef NF_ATTN_TEMPORAL_LOADS
-  return *reinterpret_cast<const u32x4*>(p);
-#else
-  nt_vec4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_vec4*>(p));
-  return u32x4{v.x, v.y, v.z, v.w};
-#endif
-}
 
 // tile_start[i] = number of tiles of requests < i; tile_start[batch] = total.
 __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restrict__ qo_indptr,
@@ -83,274 +57,6 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restric
     tile_start[i] = run;
     int len = qo_indptr[i + 1] - qo_indptr[i];
     run += len > 0 ? (len + wg_tok - 1) / wg_tok : 0;
-  }
-}
-
-// SPLIT (decode mode): one tile per request (tile index == request index, no plan needed),
-// the 4 wavefronts split the KV range.  !SPLIT (prefill mode): tiles from tile_start.
-template <int GROUP, int NQB, bool SPLIT>
-__global__ __launch_bounds__(256, SPLIT ? 2 : 1) void attn_paged_kernel(
-    const uint16_t* __restrict__ q, uint16_t* __restrict__ o, const int32_t* __restrict__ qo_indptr,
-    const uint16_t* __restrict__ kv_data, const int32_t* __restrict__ kv_indptr,
-    const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_last_page_len,
-    const int32_t* __restrict__ tile_start, int batch, int Hq, int Hkv, int causal,
-    float scale_log2) {
-  constexpr int TPB = 16 / GROUP;        // tokens per 16-column block
-  constexpr int WAVE_TOK = NQB * TPB;    // tokens per wavefront tile
-  constexpr int WG_TOK = SPLIT ? WAVE_TOK : 4 * WAVE_TOK;
-  static_assert(!SPLIT || NQB == 1, "split-KV merge is written for one column block");
-
-  __shared__ float s_o[SPLIT ? 4 * 8 * 4 * 64 : 1];
-  __shared__ float s_m[SPLIT ? 4 * 64 : 1];
-  __shared__ float s_l[SPLIT ? 4 * 64 : 1];
-
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform by construction
-  const int c16 = lane & 15, g = lane >> 4;
-  const int total_tiles = SPLIT ? batch : tile_start[batch];
-  const size_t page_halves = (size_t)2 * PAGE * Hkv * D;
-  const size_t v_off = (size_t)PAGE * Hkv * D;
-
-  for (long long w = blockIdx.x; w < (long long)total_tiles * Hkv; w += gridDim.x) {
-    const int tile = (int)(w / Hkv), kvh = (int)(w % Hkv);
-    int req, tile_in_req0;
-    if constexpr (SPLIT) {
-      req = tile;
-      tile_in_req0 = 0;
-    } else {
-      // request = largest i with tile_start[i] <= tile
-      int lo = 0, hi = batch;
-      while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (tile_start[mid] <= tile) lo = mid; else hi = mid;
-      }
-      req = lo;
-      tile_in_req0 = tile - tile_start[req];
-    }
-    const int qo0 = qo_indptr[req];
-    const int qo_len = qo_indptr[req + 1] - qo0;
-    const int pg0 = kv_indptr[req];
-    const int npages = kv_indptr[req + 1] - pg0;
-    const int kv_len = npages > 0 ? (npages - 1) * PAGE + kv_last_page_len[req] : 0;
-    // decode mode walks all row blocks of its request itself (one block when qo_len == 1)
-    const int n_sub = SPLIT ? (qo_len + WG_TOK - 1) / WG_TOK : 1;
-    for (int sub = 0; sub < n_sub; ++sub) {
-    const int tile_in_req = tile_in_req0 + sub;
-    const int tok0 = tile_in_req * WG_TOK + (SPLIT ? 0 : wave * WAVE_TOK);
-    const bool wave_active = tok0 < qo_len;
-
-    float4_t oacc[NQB][8];
-    float m_run[NQB], l_run[NQB];
-#pragma unroll
-    for (int nb = 0; nb < NQB; ++nb) {
-      m_run[nb] = -1e30f;
-      l_run[nb] = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) oacc[nb][i] = float4_t{0.f, 0.f, 0.f, 0.f};
-    }
-
-    if (wave_active) {
-      // Q operands: column c16 of block nb = (token tok0 + nb*TPB + c16/GROUP, head c16%GROUP)
-      H8 qf[NQB][4];
-      int key_limit[NQB];  // last visible key index for this lane's column
-#pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) {
-        const int tq = tok0 + nb * TPB + c16 / GROUP;
-        const bool live = tq < qo_len;
-        const uint16_t* qp =
-            q + ((size_t)(qo0 + (live ? tq : 0)) * Hq + kvh * GROUP + c16 % GROUP) * D + g * 8;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          qf[nb][j].u = live ? *reinterpret_cast<const u32x4*>(qp + j * 32) : u32x4{0, 0, 0, 0};
-        key_limit[nb] = causal ? kv_len - qo_len + tq : kv_len - 1;
-        if (!live) key_limit[nb] = -1;
-      }
-      const int tok_last = min(tok0 + WAVE_TOK, qo_len) - 1;
-      const int kv_end = causal ? min(kv_len, kv_len - qo_len + tok_last + 1) : kv_len;
-      const int npairs = (kv_end + 31) >> 5;
-      constexpr int PSTEP = SPLIT ? 4 : 1;
-      const int pp0 = SPLIT ? wave : 0;
-
-      // lane's offsets inside a page: K row c16 (16 B at feature g*8 + 32j), V rows 4g+r
-      const size_t k_lane = ((size_t)c16 * Hkv + kvh) * D + g * 8;
-      const size_t v_lane = v_off + ((size_t)(g * 4) * Hkv + kvh) * D + c16 * 8;
-      const size_t v_row = (size_t)Hkv * D;
-
-      H8 kf[2][4], vf[2][4];
-      auto page_of = [&](int pidx) -> int {   // uniform: becomes a scalar load
-        return kv_indices[pg0 + (pidx < npages ? pidx : 0)];
-      };
-      auto load_k = [&](int page_a, int page_b) {
-        const uint16_t* ka = kv_data + (size_t)page_a * page_halves + k_lane;
-        const uint16_t* kb = kv_data + (size_t)page_b * page_halves + k_lane;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          kf[0][j].u = load_stream16(ka + j * 32);
-          kf[1][j].u = load_stream16(kb + j * 32);
-        }
-      };
-      auto load_v = [&](int page_a, int page_b, int t_base) {
-        const uint16_t* va = kv_data + (size_t)page_a * page_halves + v_lane;
-        const uint16_t* vb = kv_data + (size_t)page_b * page_halves + v_lane;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          // entries past kv_len may hold anything (NaN x 0 = NaN): feed zeros instead
-          const int t = t_base + g * 4 + r;
-          vf[0][r].u = (t < kv_len) ? load_stream16(va + r * v_row) : u32x4{0, 0, 0, 0};
-          vf[1][r].u = (t + 16 < kv_len) ? load_stream16(vb + r * v_row) : u32x4{0, 0, 0, 0};
-        }
-      };
-
-      int page_a = 0, page_b = 0;
-      if (pp0 < npairs) {
-        page_a = page_of(2 * pp0);
-        page_b = page_of(2 * pp0 + 1);
-        load_k(page_a, page_b);
-        load_v(page_a, page_b, pp0 * 32);
-      }
-      for (int pp = pp0; pp < npairs; pp += PSTEP) {
-        const int t_base = pp * 32;
-        const int pn = pp + PSTEP;
-        const bool have_next = pn < npairs;
-        int next_a = 0, next_b = 0;
-        if (have_next) {
-          next_a = page_of(2 * pn);
-          next_b = page_of(2 * pn + 1);
-        }
-        // ---- scores for every column block, then K is free
-        float4_t s[NQB][2];
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb)
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk) {
-            s[nb][blk] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              s[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[blk][j].h, qf[nb][j].h, s[nb][blk], 0, 0, 0);
-          }
-        if (have_next) load_k(next_a, next_b);
-
-        // ---- V^T operands: vt[i] = {V[tok a0..a3][d], V[tok b0..b3][d]} with d = c16*8 + i
-        H8 vt[8];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const uint32_t a0 = vf[0][0].w[k], a1 = vf[0][1].w[k];
-          const uint32_t a2 = vf[0][2].w[k], a3 = vf[0][3].w[k];
-          const uint32_t b0 = vf[1][0].w[k], b1 = vf[1][1].w[k];
-          const uint32_t b2 = vf[1][2].w[k], b3 = vf[1][3].w[k];
-          vt[2 * k].u = u32x4{pk_lo(a0, a1), pk_lo(a2, a3), pk_lo(b0, b1), pk_lo(b2, b3)};
-          vt[2 * k + 1].u = u32x4{pk_hi(a0, a1), pk_hi(a2, a3), pk_hi(b0, b1), pk_hi(b2, b3)};
-        }
-        if (have_next) load_v(next_a, next_b, pn * 32);
-
-        // ---- online softmax + P.V per column block
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-          // lane holds keys t_base + blk*16 + g*4 + r of column c16
-          float mx = -1e30f;
-          bool ok[2][4];
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int t = t_base + blk * 16 + g * 4 + r;
-              ok[blk][r] = t <= key_limit[nb] && t < kv_len;
-              s[nb][blk][r] *= scale_log2;
-              if (ok[blk][r]) mx = fmaxf(mx, s[nb][blk][r]);
-            }
-          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-          const float m_new = fmaxf(m_run[nb], mx);
-          const float alpha = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
-          m_run[nb] = m_new;
-          float psum = 0.f;
-          H8 pf;
-          uint32_t pw[4];
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int rr = 0; rr < 2; ++rr) {
-              float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr] - m_new) : 0.f;
-              float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr + 1] - m_new) : 0.f;
-              // P is rounded to fp16 for P.V; the row sum uses the unrounded values
-              psum += p0 + p1;
-              pw[blk * 2 + rr] = f2h_bits(p0) | (f2h_bits(p1) << 16);
-            }
-          pf.u = u32x4{pw[0], pw[1], pw[2], pw[3]};
-          l_run[nb] = l_run[nb] * alpha + psum;
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            oacc[nb][i] *= alpha;
-            oacc[nb][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt[i].h, pf.h, oacc[nb][i], 0, 0, 0);
-          }
-        }
-      }
-      // row sums were kept per lane; columns are spread over the 4 lane groups
-#pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) {
-        l_run[nb] += __shfl_xor(l_run[nb], 16, 64);
-        l_run[nb] += __shfl_xor(l_run[nb], 32, 64);
-      }
-    }
-
-    // oacc[nb][i][r] = O[column c16][feature (4g + r)*8 + i]
-    if constexpr (SPLIT) {
-      __syncthreads();  // previous work item's merge reads are done
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) s_o[((wave * 8 + i) * 4 + r) * 64 + lane] = oacc[0][i][r];
-      s_m[wave * 64 + lane] = m_run[0];
-      s_l[wave * 64 + lane] = l_run[0];
-      __syncthreads();
-      const int tok = tok0 + c16 / GROUP;
-      float M = -1e30f;
-#pragma unroll
-      for (int ww = 0; ww < 4; ++ww) M = fmaxf(M, s_m[ww * 64 + lane]);
-      float wgt[4], L = 0.f;
-#pragma unroll
-      for (int ww = 0; ww < 4; ++ww) {
-        wgt[ww] = __builtin_amdgcn_exp2f(s_m[ww * 64 + lane] - M);
-        L += wgt[ww] * s_l[ww * 64 + lane];
-      }
-      const float inv = L > 0.f ? 1.0f / L : 0.f;
-      if (tok < qo_len) {
-        uint16_t* op = o + ((size_t)(qo0 + tok) * Hq + kvh * GROUP + c16 % GROUP) * D;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v[2];
-#pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            const int i = 2 * wave + e;
-            float acc = 0.f;
-#pragma unroll
-            for (int ww = 0; ww < 4; ++ww) acc += wgt[ww] * s_o[((ww * 8 + i) * 4 + r) * 64 + lane];
-            v[e] = acc * inv;
-          }
-          *reinterpret_cast<uint32_t*>(op + (4 * g + r) * 8 + 2 * wave) =
-              f2h_bits(v[0]) | (f2h_bits(v[1]) << 16);
-        }
-      }
-    } else {
-      if (wave_active) {
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-          const int tq = tok0 + nb * TPB + c16 / GROUP;
-          if (tq >= qo_len) continue;
-          const float inv = l_run[nb] > 0.f ? 1.0f / l_run[nb] : 0.f;
-          uint16_t* op = o + ((size_t)(qo0 + tq) * Hq + kvh * GROUP + c16 % GROUP) * D;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            uint32_t pwd[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-              pwd[k] = f2h_bits(oacc[nb][2 * k][r] * inv) | (f2h_bits(oacc[nb][2 * k + 1][r] * inv) << 16);
-            *reinterpret_cast<u32x4*>(op + (4 * g + r) * 8) = u32x4{pwd[0], pwd[1], pwd[2], pwd[3]};
-          }
-        }
-      }
-    }
-    }  // sub
   }
 }
 
@@ -615,6 +321,209 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
   }
 }
 
+// Chunked-prefill attention (causal, many rows per request).  A workgroup is one tile of
+// 4 * NQB * (16 / GROUP) query tokens of one request and one kv head; each wavefront owns
+// NQB column blocks of it.  The K and V pages are streamed ONCE per workgroup, straight into
+// two LDS stages (32 keys x 256 bytes each for K and for V) that all four wavefronts read:
+// every wavefront issues a quarter of a tile's load instructions, waits for its own, and one
+// barrier per 32-key step makes the tile visible and frees the other stage for the next loads.
+// LDS layout and operand reads are those of attn_decode_kernel.  Wavefronts whose tokens cannot
+// see a step's keys (causal) skip its MFMAs but keep loading and meeting at the barrier.
+template <int GROUP, int NQB>
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ o, const int32_t* __restrict__ qo_indptr,
+    const uint16_t* __restrict__ kv_data, const int32_t* __restrict__ kv_indptr,
+    const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_last_page_len,
+    const int32_t* __restrict__ tile_start, int batch, int Hq, int Hkv, int causal, float scale_log2) {
+  constexpr int TPB = 16 / GROUP;
+  constexpr int WAVE_TOK = NQB * TPB;
+  constexpr int WG_TOK = 4 * WAVE_TOK;
+  constexpr int STAGE = 16384;  // K tile 8 KB + V tile 8 KB
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c16 = lane & 15, g = lane >> 4;
+  const uint32_t page_bytes = (uint32_t)(2 * PAGE * Hkv * D * 2);
+  const uint32_t v_half = (uint32_t)(PAGE * Hkv * D * 2);
+
+  uint32_t kx[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) kx[j] = (uint32_t)(c16 * 256 + (((j * 4 + g) ^ c16) << 4));
+  const int i16 = lane & 15, vx_x = ((g & 1) << 2) | ((i16 >> 2) & 3);
+  uint32_t vx[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    vx[i] = (uint32_t)((g * 4 + (i16 >> 2)) * 256 + ((i ^ vx_x) * 32) + (i16 & 3) * 8);
+
+  const int total_tiles = tile_start[batch];
+  for (long long w = blockIdx.x; w < (long long)total_tiles * Hkv; w += gridDim.x) {
+    const int tile = (int)(w / Hkv), kvh = (int)(w % Hkv);
+    int lo = 0, hi = batch;  // request = largest i with tile_start[i] <= tile
+    while (hi - lo > 1) {
+      int mid = (lo + hi) >> 1;
+      if (tile_start[mid] <= tile) lo = mid; else hi = mid;
+    }
+    const int req = lo, tile_in_req = tile - tile_start[req];
+    const int qo0 = qo_indptr[req];
+    const int qo_len = qo_indptr[req + 1] - qo0;
+    const int pg0 = kv_indptr[req];
+    const int npages = kv_indptr[req + 1] - pg0;
+    const int kv_len = npages > 0 ? (npages - 1) * PAGE + kv_last_page_len[req] : 0;
+    const int wg_tok0 = tile_in_req * WG_TOK;
+    const int tok0 = wg_tok0 + wave * WAVE_TOK;
+    const bool wave_active = tok0 < qo_len;
+
+    // this wavefront's load instructions: 2 of the 8 of a K tile and of a V tile (instruction
+    // t8 = keys 4*t8 .. 4*t8+3 of the 32-key step; t8 < 4 is the first page, else the second)
+    uint32_t k_src[2], v_src[2];
+    int key_in_step[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int t8 = wave * 2 + e;
+      const int key = 4 * (t8 & 3) + (lane >> 4), pos = lane & 15;
+      const uint32_t row = (uint32_t)((key * Hkv + kvh) * D * 2);
+      k_src[e] = row + (uint32_t)(((pos ^ key) & 15) << 4);
+      v_src[e] = v_half + row + (uint32_t)((pos ^ ((key & 7) << 1)) << 4);
+      key_in_step[e] = (t8 >> 2) * 16 + key;
+    }
+
+    float4_t oacc[NQB][8];
+    float m_run[NQB], l_run[NQB];
+    H8 qf[NQB][4];
+    int key_limit[NQB];
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb) {
+      m_run[nb] = -1e30f;
+      l_run[nb] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) oacc[nb][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+      const int tq = tok0 + nb * TPB + c16 / GROUP;
+      const bool live = wave_active && tq < qo_len;
+      const uint16_t* qp = q + ((size_t)(qo0 + (live ? tq : 0)) * Hq + kvh * GROUP + c16 % GROUP) * D + g * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        qf[nb][j].u = live ? *reinterpret_cast<const u32x4*>(qp + j * 32) : u32x4{0, 0, 0, 0};
+      key_limit[nb] = causal ? kv_len - qo_len + tq : kv_len - 1;
+      if (!live) key_limit[nb] = -1;
+    }
+    // keys the workgroup / this wavefront can see at all
+    const int wg_last = min(wg_tok0 + WG_TOK, qo_len) - 1;
+    const int wg_end = causal ? min(kv_len, kv_len - qo_len + wg_last + 1) : kv_len;
+    const int wave_last = min(tok0 + WAVE_TOK, qo_len) - 1;
+    const int wave_end = !wave_active ? 0 : (causal ? min(kv_len, kv_len - qo_len + wave_last + 1) : kv_len);
+    const int npairs = (wg_end + 31) >> 5;
+
+    auto dma = [&](int pp, int stage) {
+      const int pidx = 2 * pp + (wave >> 1);  // waves 0,1 load the first page of the step, 2,3 the second
+      const int page = kv_indices[pg0 + (pidx < npages ? pidx : 0)];
+      const rsrc_t r = make_rsrc(kv_data + (size_t)page * (page_bytes / 2), page_bytes);
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + stage * STAGE + wave * 2048);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) load16_to_lds(r, k_src[e], dst + e * 1024);
+#pragma unroll
+      for (int e = 0; e < 2; ++e)  // rows past the end of the sequence are zero-filled
+        load16_to_lds(r, pp * 32 + key_in_step[e] < kv_len ? v_src[e] : kOob, dst + 8192 + e * 1024);
+    };
+
+    __syncthreads();  // the previous work item's reads of both stages are done
+    if (npairs > 0) dma(0, 0);
+    for (int pp = 0; pp < npairs; ++pp) {
+      const int t_base = pp * 32;
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // this wavefront's share of step pp has landed
+      __syncthreads();                     // ... and everybody else's; stage (pp+1)&1 is free
+      if (pp + 1 < npairs) dma(pp + 1, (pp + 1) & 1);
+      if (t_base >= wave_end) continue;    // nothing visible to this wavefront in this step
+      const uint8_t* kt = lds + (pp & 1) * STAGE;
+      const uint8_t* vt = kt + 8192;
+
+      half8_t kf[2][4];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) kf[blk][j] = *reinterpret_cast<const half8_t*>(kt + blk * 4096 + kx[j]);
+      float4_t s[NQB][2];
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+          s[nb][blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            s[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[blk][j], qf[nb][j].h, s[nb][blk], 0, 0, 0);
+        }
+      H8 pf[NQB];
+      float alpha[NQB];
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) {
+        float mx = -1e30f;
+        bool ok[2][4];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int t = t_base + blk * 16 + g * 4 + r;
+            ok[blk][r] = t <= key_limit[nb] && t < kv_len;
+            s[nb][blk][r] *= scale_log2;
+            if (ok[blk][r]) mx = fmaxf(mx, s[nb][blk][r]);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run[nb], mx);
+        alpha[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+        m_run[nb] = m_new;
+        float psum = 0.f;
+        uint32_t pw[4];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int rr = 0; rr < 2; ++rr) {
+            float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr] - m_new) : 0.f;
+            float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr + 1] - m_new) : 0.f;
+            psum += p0 + p1;
+            pw[blk * 2 + rr] = f2h_bits(p0) | (f2h_bits(p1) << 16);
+          }
+        pf[nb].u = u32x4{pw[0], pw[1], pw[2], pw[3]};
+        l_run[nb] = l_run[nb] * alpha[nb] + psum;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const short4_t vlo = lds_read_tr16(vt + vx[i]);
+        const short4_t vhi = lds_read_tr16(vt + vx[i] + 4096);
+        typedef short short8_t __attribute__((ext_vector_type(8)));
+        const half8_t v8 = __builtin_bit_cast(half8_t, __builtin_shufflevector(vlo, vhi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) {
+          oacc[nb][i] *= alpha[nb];
+          oacc[nb][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v8, pf[nb].h, oacc[nb][i], 0, 0, 0);
+        }
+      }
+    }
+
+    // oacc[nb][i][r] = O[column c16][feature 16i + 4g + r]
+    if (wave_active) {
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) {
+        float l = l_run[nb];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        const int tq = tok0 + nb * TPB + c16 / GROUP;
+        if (tq >= qo_len) continue;
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        uint16_t* op = o + ((size_t)(qo0 + tq) * Hq + kvh * GROUP + c16 % GROUP) * D;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          u32x2 out;
+          out.x = f2h_bits(oacc[nb][i][0] * inv) | (f2h_bits(oacc[nb][i][1] * inv) << 16);
+          out.y = f2h_bits(oacc[nb][i][2] * inv) | (f2h_bits(oacc[nb][i][3] * inv) << 16);
+          *reinterpret_cast<u32x2*>(op + 16 * i + 4 * g) = out;
+        }
+      }
+    }
+  }
+}
+
 template <int GROUP>
 static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
                        const uint16_t* kv_data, const int32_t* kv_indptr, const int32_t* kv_indices,
@@ -626,7 +535,7 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
   // Decode mode (KV split over the wavefronts, one workgroup per request and kv head) is the
   // right shape when requests carry about one row each; it stays correct for any row count.
   const bool decode_mode = max_qo_rows <= batch;
-  constexpr int NQB_PREFILL = 2;
+  constexpr int NQB_PREFILL = 1;
   long long bound;
   if (decode_mode) {
     bound = (long long)batch * Hkv;
@@ -655,7 +564,7 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
     kern<<<(int)bound, kWaves * 64, kDecodeLds, stream>>>(q, o, qo_indptr, kv_data, kv_indptr, kv_indices,
                                                   kv_last_page_len, batch, Hq, Hkv, causal, scale_log2);
   } else
-    attn_paged_kernel<GROUP, NQB_PREFILL, false><<<(int)bound, 256, 0, stream>>>(
+    attn_prefill_kernel<GROUP, NQB_PREFILL><<<(int)bound, 256, 2 * 16384, stream>>>(
         q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, batch, Hq,
         Hkv, causal, scale_log2);
   return check_launch("nf_attention_paged_f16");
