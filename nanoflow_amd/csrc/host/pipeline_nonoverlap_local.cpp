@@ -211,10 +211,15 @@ void NonOverlapLocalPipeline::GEMMOpInit() {
   dual.init();
   D->init(1.f);
   KQV->init();
-  for (int i = 0; i < gemmNum; ++i) gemms[i]->setStream(stream_all);
+  // one stream, nobody waits on an operator: no start / end events (each record is a packet
+  // between two kernels)
+  for (int i = 0; i < gemmNum; ++i) {
+    gemms[i]->setStream(stream_all);
+    gemms[i]->updateEventExistance(false, false);
+  }
   LOGITS->set_weight(input_data->weight.lm_head);
   LOGITS->init();
-  dual.setStream(stream_all);
+  dual.setStream(stream_all).updateEventExistance(false, false);
 }
 
 void NonOverlapLocalPipeline::GEMVOpUpdate() {
@@ -242,20 +247,20 @@ void NonOverlapLocalPipeline::GEMVOpUpdate() {
 }
 
 void NonOverlapLocalPipeline::OtherOpInit() {
-  layerNormAttention.setStream(stream_all);
-  layerNormFFN.setStream(stream_all);
-  genEmbedding.setStream(stream_all);
-  layerNormModel.setStream(stream_all);
-  roPEAppend.setStream(stream_all);
-  maxSampler.setStream(stream_all);
-  keepToken.setStream(stream_all);
+  layerNormAttention.setStream(stream_all).updateEventExistance(false, false);
+  layerNormFFN.setStream(stream_all).updateEventExistance(false, false);
+  genEmbedding.setStream(stream_all).updateEventExistance(false, false);
+  layerNormModel.setStream(stream_all).updateEventExistance(false, false);
+  roPEAppend.setStream(stream_all).updateEventExistance(false, false);
+  maxSampler.setStream(stream_all).updateEventExistance(false, false);
+  keepToken.setStream(stream_all).updateEventExistance(false, false);
   genEmbedding.setWeight(input_data->weight.embedding);
   layerNormModel.setWeight(input_data->weight.model_layernorm);
 }
 
 void NonOverlapLocalPipeline::GEMVOpInit() {
-  GEMV.setStream(stream_all);
-  prefill.setStream(stream_all);
+  GEMV.setStream(stream_all).updateEventExistance(false, false);
+  prefill.setStream(stream_all).updateEventExistance(false, false);
 }
 
 double NonOverlapLocalPipeline::totalCompute() {
