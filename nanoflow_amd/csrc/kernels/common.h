@@ -6,6 +6,8 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <type_traits>
+#include <utility>
 
 #include "nanoflow_kernels.h"
 
@@ -80,8 +82,26 @@ __device__ __forceinline__ void load16_to_lds(rsrc_t r, uint32_t byte_off, uint3
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                :: "s"(lds_addr), "v"(byte_off), "s"(r) : "memory");
 }
+// The same with the LDS address given as a wavefront-uniform base plus a compile-time constant.
+template <int kLdsOffset>
+__device__ __forceinline__ void load16_to_lds(rsrc_t r, uint32_t byte_off, uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(lds_base), "v"(byte_off), "s"(r), "n"(kLdsOffset) : "memory", "scc");
+}
 __device__ __forceinline__ short4_t lds_read_tr16(const uint8_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p);
+}
+
+// Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{}).
+template <int V>
+using ic = std::integral_constant<int, V>;
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(ic<I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 }  // namespace nf

@@ -109,14 +109,17 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
   // A-style rows: lane -> (row lane/8 of the instruction's 8 rows, position lane%8), fetching
   // logical chunk position ^ ((row >> 1) & 7); bit 3 of the row number is the wave's parity.
   const int a_kc = ((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2))) * 8;
+  // One running offset per load instruction, advanced by a slab after each use.  Rows past the
+  // operand's last one lie at or past the end of the buffer and read as zero; so do k >= K rows of
+  // [K][N] weights.  Weight columns n >= N of such a slab alias the next row: they only reach
+  // output columns that are never stored.  Left to test: k >= K inside a 128-byte activation (or
+  // [N][K] weight) row, which would read the next row's start.
   uint32_t a_off[A_LOADS];
 #pragma unroll
   for (int t = 0; t < A_LOADS; ++t) {
     const int gm = m_base + (t * 4 + wave) * 8 + (lane >> 3);
-    a_off[t] = gm < M ? ((uint32_t)gm * (uint32_t)K + a_kc) * 2u : kOob;
+    a_off[t] = ((uint32_t)gm * (uint32_t)K + a_kc) * 2u;
   }
-  // [K][N] weights: one running offset per load, advanced by a slab (64 rows) after use.  Rows
-  // k >= K lie at or past the end of the buffer and read as zero, so K needs no test there.
   uint32_t b_off[NB][B_LOADS];
   const uint32_t b_slab = (uint32_t)BK * (uint32_t)N * 2u;
 #pragma unroll
@@ -124,46 +127,46 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
     uint32_t off;
     if constexpr (kBCol) {
       const int gn = n_base + (t * 4 + wave) * 8 + (lane >> 3);
-      off = gn < N ? ((uint32_t)gn * (uint32_t)K + a_kc) * 2u : kOob;
+      off = ((uint32_t)gn * (uint32_t)K + a_kc) * 2u;
     } else {
       const int row = (t * 4 + wave) * B_RPI + lane / B_CPR;
       const int c = (lane % B_CPR) ^ ((row & 3) << 2);
-      const int gn = n_base + c * 8;
-      off = gn < N ? ((uint32_t)row * (uint32_t)N + gn) * 2u : kOob;
+      off = ((uint32_t)row * (uint32_t)N + n_base + c * 8) * 2u;
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b) b_off[b][t] = off;
   }
 
-  // The loads of one slab, or (part >= 0) the share of them with index % parts == part.
+  // ---- global -> LDS, one 1 KB load instruction at a time.  Load t of a slab: t < A_LOADS
+  // fetches activation rows, the rest weight rows.  st = LDS address of the stage + wave * 1024.
   constexpr int NS = SM::stages;
   constexpr int LOADS = A_LOADS + NB * B_LOADS;  // per wave per slab
-  constexpr int PARTS = NS == 2 ? 2 : 4;         // k-steps of a slab the loads are spread over
-  auto issue_loads = [&](int stage, int k0, int part) {
+  constexpr int PARTS = NS == 2 ? 2 : 4;         // k-steps the loads of one slab are spread over
+  // k_ok: this lane's 16 bytes of the slab's 128-byte rows lie below K.
+  auto load_one = [&](auto t_c, uint32_t st, bool k_ok) {
+    constexpr int t = decltype(t_c)::value;
+    if constexpr (t < A_LOADS) {
+      load16_to_lds<t * 4096>(a_rsrc, k_ok ? a_off[t] : kOob, st);
+      a_off[t] += BK * 2;
+    } else {
+      constexpr int b = (t - A_LOADS) / B_LOADS, tt = (t - A_LOADS) % B_LOADS;
+      constexpr int dst = SM::a_bytes + b * SM::b_bytes + tt * 4096;
+      if constexpr (kBCol) {
+        load16_to_lds<dst>(b_rsrc[b], k_ok ? b_off[b][tt] : kOob, st);
+        b_off[b][tt] += BK * 2;
+      } else {
+        load16_to_lds<dst>(b_rsrc[b], b_off[b][tt], st);
+        b_off[b][tt] += b_slab;
+      }
+    }
+  };
+  auto load_slab = [&](int stage, int k0) {  // every load of one slab, back to back
     const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::stage_bytes + wave * 1024);
     const bool k_ok = k0 + a_kc < K;
-#pragma unroll
-    for (int t = 0; t < A_LOADS; ++t) {
-      if (part >= 0 && t % PARTS != part) continue;
-      load16_to_lds(a_rsrc, (k_ok && a_off[t] != kOob) ? a_off[t] + (uint32_t)k0 * 2u : kOob,
-                    st + t * 4096);
-    }
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-      for (int t = 0; t < B_LOADS; ++t) {
-        if (part >= 0 && (A_LOADS + b * B_LOADS + t) % PARTS != part) continue;
-        const uint32_t dst = st + SM::a_bytes + b * SM::b_bytes + t * 4096;
-        if constexpr (kBCol) {
-          load16_to_lds(b_rsrc[b], (k_ok && b_off[b][t] != kOob) ? b_off[b][t] + (uint32_t)k0 * 2u : kOob, dst);
-        } else {
-          load16_to_lds(b_rsrc[b], b_off[b][t], dst);
-          if (b_off[b][t] != kOob) b_off[b][t] += b_slab;
-        }
-      }
+    static_for<LOADS>([&](auto t_c) { load_one(t_c, st, k_ok); });
   };
 
-  // ---- LDS -> MFMA operand fragments, double-buffered across the 4 k-steps of a slab
+  // ---- LDS -> MFMA operand fragments, double-buffered across k-steps
   // A-style: row r = l32 (+ multiples of 32), logical chunk kk*2+lg sits at chunk ^ ((r>>1)&7).
   const uint32_t a_rd = (uint32_t)(wm * (BM / WM) + l32) * 128u;
   const uint32_t bc_rd = (uint32_t)(wn * (BN / WN) + l32) * 128u;  // [N][K] weights
@@ -184,89 +187,115 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
 
   half8_t af[2][TM];
   half8_t bf[2][NB][TN];
-  auto read_frags = [&](int stage, int kk, int buf) {
-    const uint8_t* st = smem + stage * SM::stage_bytes;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-      af[buf][i] = *reinterpret_cast<const half8_t*>(st + a_rd + swz[kk] + i * 32 * 128);
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
+  constexpr int READS = TM + NB * TN;  // fragment reads per k-step: q < TM activations, then weights
+  auto read_one = [&](auto q_c, auto kk_c, auto buf_c, const uint8_t* st) {
+    constexpr int q = decltype(q_c)::value, kk = decltype(kk_c)::value, buf = decltype(buf_c)::value;
+    if constexpr (q < TM) {
+      af[buf][q] = *reinterpret_cast<const half8_t*>(st + a_rd + swz[kk] + q * 32 * 128);
+    } else {
+      constexpr int b = (q - TM) / TN, j = (q - TM) % TN;
       const uint8_t* bs = st + SM::a_bytes + b * SM::b_bytes;
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        if constexpr (kBCol) {
-          bf[buf][b][j] = *reinterpret_cast<const half8_t*>(bs + bc_rd + swz[kk] + j * 32 * 128);
-        } else {
-          const uint8_t* p = bs + br_row + br_tbl[j] + kk * 16 * ROWB;
-          const short4_t lo = lds_read_tr16(p);
-          const short4_t hi = lds_read_tr16(p + 4 * ROWB);
-          typedef short short8_t __attribute__((ext_vector_type(8)));
-          const short8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          bf[buf][b][j] = __builtin_bit_cast(half8_t, v);
-        }
+      if constexpr (kBCol) {
+        bf[buf][b][j] = *reinterpret_cast<const half8_t*>(bs + bc_rd + swz[kk] + j * 32 * 128);
+      } else {
+        const uint8_t* p = bs + br_row + br_tbl[j] + kk * 16 * ROWB;
+        const short4_t lo = lds_read_tr16(p);
+        const short4_t hi = lds_read_tr16(p + 4 * ROWB);
+        typedef short short8_t __attribute__((ext_vector_type(8)));
+        const short8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        bf[buf][b][j] = __builtin_bit_cast(half8_t, v);
       }
     }
   };
-  auto mfma_step = [&](int buf) {
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-          acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[buf][b][j], af[buf][i], acc[b][i][j], 0, 0, 0);
+
+  // One k-step: the MFMAs on fragment buffer kk & 1, with the step's side work dealt out
+  // between them and the order pinned -- a wavefront is alone on its SIMD, so whatever it issues
+  // between two MFMAs must fit into the 32 cycles the first one occupies the matrix pipe:
+  //   loads LP, LP + PARTS, ... of the slab being fetched (LP < 0: none), into stage address ld_st;
+  //   then the fragment reads of k-step RK from stage rd_st into the other buffer (RK < 0: none).
+  constexpr int NM = NB * TN * TM;
+  auto step = [&](auto kk_c, auto lp_c, auto rk_c, uint32_t ld_st, bool ld_ok, const uint8_t* rd_st) {
+    constexpr int kk = decltype(kk_c)::value, LP = decltype(lp_c)::value, RK = decltype(rk_c)::value;
+    constexpr int NL = LP < 0 ? 0 : (LOADS - LP + PARTS - 1) / PARTS;
+    constexpr int NR = RK < 0 ? 0 : READS;
+    constexpr int S = NL + NR;
+    static_for<NM>([&](auto n_c) {
+      constexpr int n = decltype(n_c)::value;
+      constexpr int b = n / (TN * TM), j = (n / TM) % TN, i = n % TM;
+      acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][b][j], af[kk & 1][i], acc[b][i][j], 0, 0, 0);
+      constexpr int lo = n * S / NM, hi = (n + 1) * S / NM;
+      static_for<hi - lo>([&](auto d_c) {
+        constexpr int q = lo + decltype(d_c)::value;
+        if constexpr (q < NL) load_one(ic<(LP < 0 ? 0 : LP) + PARTS * q>{}, ld_st, ld_ok);
+        else read_one(ic<q - NL>{}, ic<(RK < 0 ? 0 : RK)>{}, ic<(kk + 1) & 1>{}, rd_st);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
   };
 
-  // Slab s lives in LDS stage s % NS.  While its four k-steps run (next step's fragments
-  // prefetched), the loads of slab s+NS-1 are issued, spread over the k-steps, into the stage
-  // that slab s-1 has just left (every wavefront is past the barrier that ended slab s-1).  At
-  // the end the wavefront waits until its loads of slab s+1 have landed -- the younger loads it
-  // has issued since may stay in flight -- and meets the others at the barrier.
-  auto slab = [&](auto issue_c, int s, int cs, int ls) {
-    constexpr bool issue = decltype(issue_c)::value;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      if (issue && kk < PARTS) issue_loads(ls, (s + NS - 1) * BK, kk);
-      if (kk < 3) read_frags(cs, kk + 1, (kk + 1) & 1);
-      __builtin_amdgcn_sched_barrier(0);  // the fragment reads go out before this step's MFMAs
-      mfma_step(kk & 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-  auto wait_loads = [&](int younger) {  // vmcnt(younger): encoded in bits [3:0] and [15:14]
-    if (younger == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-    else __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS * (NS - 2) & 15) | (((LOADS * (NS - 2)) >> 4) << 14));
+  // vmcnt(n) with lgkmcnt(0): n in bits [3:0] and [15:14]
+  auto wait_loads = [&](int younger) {
+    if (younger == 0) __builtin_amdgcn_s_waitcnt(0x0070);
+    else __builtin_amdgcn_s_waitcnt(0x0070 | (LOADS * (NS - 2) & 15) | (((LOADS * (NS - 2)) >> 4) << 14));
   };
   static_assert(LOADS * (NS - 2) < 64, "vmcnt range");
   auto next = [](int st) { return st + 1 == NS ? 0 : st + 1; };
 
+  // Slab s lives in LDS stage s % NS.  Its k-steps 0..2 prefetch the fragments of the step after
+  // them; then the wavefront waits until its own loads of slab s+1 have landed and its fragment
+  // reads of this stage have returned, and meets the others at the slab's one barrier.  Past the
+  // barrier slab s+1 is visible to everybody and nobody reads this stage any more, so k-step 3
+  // prefetches the first fragments of slab s+1 and starts refilling this stage with slab s+NS;
+  // the rest of that slab's loads go out during k-steps 0.. of slab s+1.  (With two stages the
+  // loads must land within the same slab and are issued in the first two of those steps only.)
+  //   IA: slab s+NS-1 exists (loads in steps 0..2), IB: slab s+NS exists (loads in step 3),
+  //   LAST: no slab s+1.
+  auto slab = [&](auto ia_c, auto ib_c, auto last_c, int s, int cs, int ls) {
+    constexpr bool IA = decltype(ia_c)::value, IB = decltype(ib_c)::value, LAST = decltype(last_c)::value;
+    const uint8_t* st = smem + cs * SM::stage_bytes;
+    const uint32_t ld_a = __builtin_amdgcn_readfirstlane(smem_lds + ls * SM::stage_bytes + wave * 1024);
+    const bool ok_a = (s + NS - 1) * BK + a_kc < K;
+    step(ic<0>{}, ic<(IA && PARTS > 1) ? 1 : -1>{}, ic<1>{}, ld_a, ok_a, st);
+    step(ic<1>{}, ic<(IA && PARTS > 2) ? 2 : -1>{}, ic<2>{}, ld_a, ok_a, st);
+    step(ic<2>{}, ic<(IA && PARTS > 3) ? 3 : -1>{}, ic<3>{}, ld_a, ok_a, st);
+    if constexpr (!LAST) {
+      wait_loads(IA ? 1 : 0);
+      __syncthreads();
+    }
+    const uint32_t ld_b = __builtin_amdgcn_readfirstlane(smem_lds + cs * SM::stage_bytes + wave * 1024);
+    step(ic<3>{}, ic<IB ? 0 : -1>{}, ic<LAST ? -1 : 0>{}, ld_b, (s + NS) * BK + a_kc < K,
+         smem + next(cs) * SM::stage_bytes);
+  };
+
   const int nslab = (K + BK - 1) / BK;
 #pragma unroll
   for (int p = 0; p < NS - 1; ++p)
-    if (p < nslab) issue_loads(p, p * BK, -1);
+    if (p < nslab) load_slab(p, p * BK);
   // slab 0 must have landed; later prologue loads may still be in flight (exact count only
   // matters for speed: waiting for everything is always correct)
-  if (nslab >= NS - 1) wait_loads(1); else wait_loads(0);
+  wait_loads(nslab >= NS - 1 ? 1 : 0);
   __syncthreads();
-  read_frags(0, 0, 0);
+  static_for<READS>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, smem); });
+  if (NS - 1 < nslab) {  // the share of slab NS-1 that a slab's k-step 3 would have issued
+    const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + (NS - 1) * SM::stage_bytes + wave * 1024);
+    const bool k_ok = (NS - 1) * BK + a_kc < K;
+    static_for<(LOADS + PARTS - 1) / PARTS>([&](auto q_c) { load_one(ic<PARTS * decltype(q_c)::value>{}, st, k_ok); });
+  }
   int cs = 0, ls = NS - 1, s = 0;
-  for (; s + NS - 1 < nslab; ++s) {  // steady state: one slab's loads issued per slab
-    slab(std::true_type{}, s, cs, ls);
-    wait_loads(1);
-    __syncthreads();
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  for (; s + NS < nslab; ++s) {  // steady state
+    slab(T_{}, T_{}, F_{}, s, cs, ls);
     cs = next(cs);
     ls = next(ls);
-    read_frags(cs, 0, 0);
   }
-  for (; s < nslab; ++s) {           // drain: nothing left to issue
-    slab(std::false_type{}, s, cs, ls);
-    if (s + 1 < nslab) {
-      wait_loads(0);
-      __syncthreads();
-      cs = next(cs);
-      read_frags(cs, 0, 0);
-    }
+  for (; s + 1 < nslab; ++s) {   // drain: the last loads, then none
+    if (s + NS - 1 < nslab) slab(T_{}, F_{}, F_{}, s, cs, ls);
+    else slab(F_{}, F_{}, F_{}, s, cs, ls);
+    cs = next(cs);
+    ls = next(ls);
   }
+  slab(F_{}, F_{}, T_{}, s, cs, ls);  // the last slab: nothing left to fetch or prefetch
 
   // Epilogue.  acc[.][i][j][r] holds D[m][n] with m = tile row l32 and
   // n = (r/4)*8 + lg*4 + r%4 of the 32x32 tile: 4 consecutive n per register quad.
@@ -352,9 +381,10 @@ static int check_gemm_args(const char* who, const void* A, const void* B, const 
   NF_REQUIRE(M == 0 || (A && B && D), "%s: null pointer", who);
   NF_REQUIRE(((uintptr_t)A | (uintptr_t)B | (uintptr_t)D) % 16 == 0,
              "%s: operands must be 16-byte aligned", who);
-  // operands are addressed through 32-bit buffer offsets
-  // (the weight offsets run up to two slabs past K before they are discarded)
-  NF_REQUIRE((size_t)M * K * 2 < 0xFFFFFF00ull && (size_t)N * ((size_t)K + 128) * 2 < 0xFFFFFF00ull,
+  // operands are addressed through 32-bit buffer offsets, which run up to a tile past the last
+  // row or column and a few slabs past K before they are discarded
+  NF_REQUIRE(((size_t)M + 256) * ((size_t)K + 512) * 2 < 0xFFFFFF00ull &&
+                 ((size_t)N + 256) * ((size_t)K + 512) * 2 < 0xFFFFFF00ull,
              "%s: an operand of %d x %d x %d exceeds the 4 GiB buffer-addressing limit", who, M, N, K);
   return NF_OK;
 }
