@@ -29,6 +29,7 @@
 //
 // The MFMA is issued as D^T = B^T.A^T (weights as the first operand) so that each lane ends up
 // with 4 consecutive output columns of one row -> 8-byte stores/loads for D and C.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -57,11 +58,12 @@ __device__ __forceinline__ float swiglu_rounded(float g_acc, float u_acc) {
 }
 
 // kDual: two weight matrices, SwiGLU epilogue.  kBCol: weights stored [N][K].
+// One BM x BN output tile at (m_base, n_base), computed by the whole workgroup.
 template <int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
-__global__ __launch_bounds__(256) void gemm_f16_kernel(
+__device__ __forceinline__ void gemm_tile(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
-    int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, float beta, const int m_base, const int n_base) {
   constexpr int NB = kDual ? 2 : 1;
   using SM = GemmSmem<BM, BN, NB>;
   constexpr int TM = BM / WM / 32;  // MFMA tiles per wave along M
@@ -72,19 +74,9 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
   constexpr int B_LOADS = BN / 32;   // ... per weight matrix
   constexpr int ROWB = BN * 2;       // bytes per k row of a [K][N] weight slab
   constexpr int B_CPR = BN / 8;      // 16-byte chunks per such row
-  constexpr int B_RPI = 64 / B_CPR;  // rows covered by one load instruction
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
-
-  // XCD-aware tile order: consecutive workgroup ids land on different XCDs (8 of them), so
-  // give each XCD one contiguous range of tiles, M fastest, to share weight panels in its L2.
-  const int ntiles = tiles_m * tiles_n;
-  const int per_xcd = (ntiles + 7) / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (logical >= ntiles) return;
-  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
-  const int m_base = tile_m * BM, n_base = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -129,8 +121,9 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
       const int gn = n_base + (t * 4 + wave) * 8 + (lane >> 3);
       off = ((uint32_t)gn * (uint32_t)K + a_kc) * 2u;
     } else {
-      const int row = (t * 4 + wave) * B_RPI + lane / B_CPR;
-      const int c = (lane % B_CPR) ^ ((row & 3) << 2);
+      const int g = (t * 4 + wave) * 64 + lane;  // 16-byte slot of the slab's LDS image
+      const int row = g / B_CPR;
+      const int c = (g % B_CPR) ^ ((row & 3) << 2);
       off = ((uint32_t)row * (uint32_t)N + n_base + c * 8) * 2u;
     }
 #pragma unroll
@@ -334,6 +327,50 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
   }
 }
 
+// XCD-aware tile order: consecutive workgroup ids land on different XCDs (8 of them), so give
+// each XCD one contiguous range of the n tiles (M fastest) to share weight panels in its L2.
+__device__ __forceinline__ int xcd_order(int bid, int n) {
+  return (bid % 8) * ((n + 7) / 8) + bid / 8;
+}
+
+template <int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
+__global__ __launch_bounds__(256) void gemm_f16_kernel(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
+    const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
+    int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n) {
+  const int logical = xcd_order(blockIdx.x, tiles_m * tiles_n);
+  if (logical >= tiles_m * tiles_n) return;
+  gemm_tile<BM, BN, WM, WN, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
+                                           (logical % tiles_m) * BM, (logical / tiles_m) * BN);
+}
+
+// Two tile heights in one launch, for shapes whose 256-row tiles fill the 256 CUs a whole number
+// of times plus at most half a round: the first n_big tiles (in M-fastest order) are computed
+// 256 rows high, each of the rest as two 128-row halves by two workgroups, so the last round
+// takes half the time instead of leaving half the CUs idle.
+template <int BN, bool kDual, bool kBCol>
+__global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
+    const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
+    int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n, int n_big) {
+  const int big_grid = (n_big + 7) / 8 * 8;
+  if ((int)blockIdx.x < big_grid) {
+    const int t = xcd_order(blockIdx.x, n_big);
+    if (t >= n_big) return;
+    gemm_tile<256, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
+                                            (t % tiles_m) * 256, (t / tiles_m) * BN);
+  } else {
+    const int n_small = 2 * (tiles_m * tiles_n - n_big);
+    const int u = xcd_order(blockIdx.x - big_grid, n_small);
+    if (u >= n_small) return;
+    const int t = n_big + u / 2;
+    const int m_base = (t % tiles_m) * 256 + (u & 1) * 128;
+    if (m_base >= M) return;
+    gemm_tile<128, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, m_base,
+                                            (t / tiles_m) * BN);
+  }
+}
+
 template <int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1, const uint16_t* C,
                        uint16_t* D, int M, int N, int K, float alpha, float beta,
@@ -357,16 +394,63 @@ static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1
   return check_launch("gemm launch");
 }
 
-// Tile choice (256 CUs, one workgroup each): the largest tile that still gives most CUs a
-// workgroup -- measured on the pipeline's shapes, 192 tiles of the bigger kind beat 1.5 rounds
-// of the smaller one; short M uses a 64-row tile so the padding rows do not dominate.
+template <int BN, bool kDual, bool kBCol>
+static int launch_hybrid(const uint16_t* A, const uint16_t* B0, const uint16_t* B1, const uint16_t* C,
+                         uint16_t* D, int M, int N, int K, float alpha, float beta, int n_big,
+                         hipStream_t stream) {
+  constexpr size_t big = GemmSmem<256, BN, kDual ? 2 : 1>::bytes, small = GemmSmem<128, BN, kDual ? 2 : 1>::bytes;
+  constexpr size_t lds = big > small ? big : small;
+  auto kern = gemm_f16_hybrid_kernel<BN, kDual, kBCol>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) {
+      set_error("gemm: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+      return NF_ERR_RUNTIME;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = (M + 255) / 256, tiles_n = (N + BN - 1) / BN;
+  const int n_small = 2 * (tiles_m * tiles_n - n_big);
+  const int grid = (n_big + 7) / 8 * 8 + (n_small + 7) / 8 * 8;
+  kern<<<grid, 256, lds, stream>>>(A, B0, B1, C, D, M, N, K, alpha, beta, tiles_m, tiles_n, n_big);
+  return check_launch("gemm launch");
+}
+
+// Compute units of the current device (256 on MI355X); one workgroup of these kernels fills one.
+static int cu_count() {
+  static int n = 0;  // benign race: every caller computes the same value
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    n = v;
+  }
+  return n;
+}
+
+// Tile choice.  A launch takes ceil(tiles / CUs) rounds of one tile each, a round costing the
+// tile's area over its relative efficiency (bigger tiles re-read less through LDS); the cheapest
+// candidate wins.  So 192 tiles of 256x256 beat 1.5 rounds of 128x256, and 2048 x 6144 takes
+// 256 tiles of 128x384 rather than 192 of 256x256.  Short M uses a 64-row tile so that padding
+// rows do not dominate.
 template <bool kBCol>
 static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
                           int M, int N, int K, float alpha, float beta, hipStream_t s) {
-  auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (M <= 64) return launch_gemm<64, 256, 1, 4, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (tiles(256, 256) >= 192) return launch_gemm<256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (tiles(128, 256) >= 192 || M <= 128) return launch_gemm<128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  const int cus = cu_count();
+  auto cost = [&](int bm, int bn, double eff) {
+    const long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    return (double)((tiles + cus - 1) / cus) * bm * bn / eff;
+  };
+  const double c256 = cost(256, 256, 1.0), c384 = cost(128, 384, 0.97), c128x256 = cost(128, 256, 0.95),
+               c128 = cost(128, 128, 0.80);
+  const double best = std::min(std::min(c256, c384), std::min(c128x256, c128));
+  if (best == c256) return launch_gemm<256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (best == c384) return launch_gemm<128, 384, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (best == c128x256) return launch_gemm<128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
   return launch_gemm<128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
 }
 
@@ -415,8 +499,13 @@ int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t*
     return launch_gemm<64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
   const long long t256 = (long long)((M + 255) / 256) * ((N + 127) / 128);
   const int tail = M % 256;  // rows in the last 256-row tile: half-empty tiles go to the 128-row kernel
-  if (t256 >= 192 && (tail == 0 || tail > 128))
+  if (t256 >= 192 && (tail == 0 || tail > 128)) {
+    const int cus = cu_count();
+    const int rest = (int)(t256 % cus);  // tiles of the last, partial round
+    if (t256 > cus && rest > 0 && rest <= cus / 2)
+      return launch_hybrid<128, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, (int)(t256 - rest), s);
     return launch_gemm<256, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+  }
   return launch_gemm<128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
 }
 

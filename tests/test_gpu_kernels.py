@@ -96,6 +96,8 @@ GEMM_SHAPES = [
     (257, 512, 128),      # M tail of one row
     (384, 4096, 4096),    # nano-batch O projection
     (1408, 6144, 512),    # 256x256 tiles with an M tail, XCD-remapped grid
+    (2048, 6144, 256),    # one round of 128x384 tiles (the QKV projection of a full batch)
+    (1930, 5000, 264),    # 128x384 tiles with M, N and K tails
 ]
 
 
@@ -123,7 +125,7 @@ def test_gemm_alpha_beta_and_in_place_residual(K, oracle):
 
 def test_gemm_column_major_weights(K, oracle):
     rng = np.random.default_rng(5)
-    for (M, N, K_) in [(64, 512, 256), (300, 384, 320)]:
+    for (M, N, K_) in [(64, 512, 256), (300, 384, 320), (1930, 5000, 264)]:
         A = synth.normal_f16(rng, (M, K_))
         Bt = synth.normal_f16(rng, (N, K_), 0.05)
         assert_close(host(K.gemm(dev(A), dev(Bt), b_col_major=True)),
@@ -137,7 +139,9 @@ def test_gemm_identity_is_exact(K):
     assert np.array_equal(host(K.gemm(dev(A), dev(I))), A)
 
 
-@pytest.mark.parametrize("M,N,K_", [(64, 14336, 4096), (5, 136, 72), (200, 512, 256), (640, 2048, 512)])
+@pytest.mark.parametrize("M,N,K_", [(64, 14336, 4096), (5, 136, 72), (200, 512, 256), (640, 2048, 512),
+                                    (2048, 14336, 128),    # 3.5 rounds of 256-row tiles: two tile heights in one launch
+                                    (1992, 14328, 200)])   # the same with M, N and K tails
 def test_dual_swiglu(K, oracle, M, N, K_):
     rng = np.random.default_rng(7)
     A = synth.normal_f16(rng, (M, K_))
