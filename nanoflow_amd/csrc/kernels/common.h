@@ -60,6 +60,12 @@ __device__ __forceinline__ float h2f_bits(uint32_t bits16) {
 __device__ __forceinline__ uint32_t f2h_bits(float f) {
   return (uint32_t)__half_as_ushort(__float2half_rn(f));
 }
+// Two floats rounded to nearest-even fp16, lo in bits 15:0 (one v_cvt_pk_f16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, f16x2_t));
+}
 
 // ---- global memory -> LDS without passing through registers (gfx950 buffer_load ... lds)
 typedef short short4_t __attribute__((ext_vector_type(4)));

@@ -54,7 +54,8 @@ struct GemmSmem {
 __device__ __forceinline__ float swiglu_rounded(float g_acc, float u_acc) {
   float g = __half2float(__float2half_rn(g_acc));
   float u = __half2float(__float2half_rn(u_acc));
-  return g / (1.0f + __expf(-g)) * u;
+  // hardware reciprocal (1 ulp of fp32): the result is rounded to fp16 afterwards
+  return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
 }
 
 // kDual: two weight matrices, SwiGLU epilogue.  kBCol: weights stored [N][K].
@@ -134,7 +135,7 @@ __device__ __forceinline__ void gemm_tile(
   // fetches activation rows, the rest weight rows.  st = LDS address of the stage + wave * 1024.
   constexpr int NS = SM::stages;
   constexpr int LOADS = A_LOADS + NB * B_LOADS;  // per wave per slab
-  constexpr int PARTS = NS == 2 ? 2 : 4;         // k-steps the loads of one slab are spread over
+  constexpr int PARTS = NS == 2 ? 3 : 4;         // k-steps the loads of one slab are spread over
   // k_ok: this lane's 16 bytes of the slab's 128-byte rows lie below K.
   auto load_one = [&](auto t_c, uint32_t st, bool k_ok) {
     constexpr int t = decltype(t_c)::value;
@@ -216,6 +217,8 @@ __device__ __forceinline__ void gemm_tile(
       constexpr int n = decltype(n_c)::value;
       constexpr int b = n / (TN * TM), j = (n / TM) % TN, i = n % TM;
       acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][b][j], af[kk & 1][i], acc[b][i][j], 0, 0, 0);
+      // front-loaded: the step's last reads should have returned when the step ends
+      constexpr int PER_ = 0;
       constexpr int lo = n * S / NM, hi = (n + 1) * S / NM;
       static_for<hi - lo>([&](auto d_c) {
         constexpr int q = lo + decltype(d_c)::value;
@@ -291,37 +294,80 @@ __device__ __forceinline__ void gemm_tile(
   slab(F_{}, F_{}, T_{}, s, cs, ls);  // the last slab: nothing left to fetch or prefetch
 
   // Epilogue.  acc[.][i][j][r] holds D[m][n] with m = tile row l32 and
-  // n = (r/4)*8 + lg*4 + r%4 of the 32x32 tile: 4 consecutive n per register quad.
+  // n = (r/4)*8 + lg*4 + r%4 of the 32x32 tile: a lane owns 4 consecutive columns of 32 different
+  // rows, which as direct stores would touch 32 cache lines per instruction.  So each wavefront
+  // turns its block around through LDS (free now), 32 rows at a time in fp32: written as the
+  // MFMA left it, read back row by row, so that 64 lanes store (and read C from) whole 512-byte
+  // runs.  Rows are padded by 16 bytes: both directions are free of bank conflicts.
+  constexpr int CW = BN / WN;        // columns of the wavefront's block
+  constexpr int ROWP = CW * 4 + 16;  // bytes per padded fp32 row
+  constexpr int CPR = CW / 4;        // 4-column groups per row
+  static_assert(4 * 32 * ROWP <= (int)SM::bytes && (32 * CPR) % 64 == 0, "epilogue staging");
+  __syncthreads();  // every wavefront has read its last fragments
+  uint8_t* ep = smem + wave * (32 * ROWP);
+  constexpr int ITER = 32 * CPR / 64;  // 4-column groups per lane and pass
+  typedef unsigned int u32v2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int gm = m_base + wm * (BM / WM) + i * 32 + l32;
-    if (gm >= M) continue;
+    // C and D go through buffer descriptors based at the pass's first row and ending with the
+    // matrix (rows >= M fall outside and are dropped by the hardware; columns >= N get an
+    // out-of-range offset), so the pass has no branches and all its loads are in flight together.
+    const int gm0 = m_base + wm * (BM / WM) + i * 32, gn0 = n_base + wn * CW;
+    const int rows = M - gm0 < 32 ? M - gm0 : 32;
+    const int recs = rows > 0 ? rows * N * 2 : 0;
+    const size_t row0 = (size_t)(rows > 0 ? gm0 : 0) * N;
+    const __amdgpu_buffer_rsrc_t d_rsrc = __builtin_amdgcn_make_buffer_rsrc(D + row0, 0, recs, 0x00020000);
+    uint32_t off[ITER];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+    for (int it = 0; it < ITER; ++it) {
+      const int c = it * 64 + lane, gn = gn0 + (c % CPR) * 4;
+      off[it] = gn < N ? (uint32_t)((c / CPR) * N + gn) * 2u : kOob;
+    }
+    u32v2_t cv[ITER];
+    if constexpr (!kDual) {
+      if (beta != 0.f) {  // issued first: the longest latency of the pass
+        const __amdgpu_buffer_rsrc_t c_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(C) + row0, 0, recs, 0x00020000);
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) cv[it] = __builtin_amdgcn_raw_buffer_load_b64(c_rsrc, off[it], 0, 0);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const int gn = n_base + wn * (BN / WN) + j * 32 + qd * 8 + lg * 4;
-        if (gn >= N) continue;  // N % 8 == 0 and gn % 4 == 0: the whole quad is in or out
-        float v[4];
-        if constexpr (kDual) {
+        float4_t v;
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            v[e] = swiglu_rounded(acc[0][i][j][qd * 4 + e], acc[1][i][j][qd * 4 + e]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = alpha * acc[0][i][j][qd * 4 + e];
-          if (beta != 0.f) {
-            const u32x2 c = *reinterpret_cast<const u32x2*>(C + (size_t)gm * N + gn);
-            v[0] += beta * h2f_bits(c.x & 0xffffu);
-            v[1] += beta * h2f_bits(c.x >> 16);
-            v[2] += beta * h2f_bits(c.y & 0xffffu);
-            v[3] += beta * h2f_bits(c.y >> 16);
-          }
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (kDual) v[e] = swiglu_rounded(acc[0][i][j][qd * 4 + e], acc[1][i][j][qd * 4 + e]);
+          else v[e] = acc[0][i][j][qd * 4 + e];
         }
-        u32x2 o;
-        o.x = f2h_bits(v[0]) | (f2h_bits(v[1]) << 16);
-        o.y = f2h_bits(v[2]) | (f2h_bits(v[3]) << 16);
-        *reinterpret_cast<u32x2*>(D + (size_t)gm * N + gn) = o;
+        *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
+      }
+    float4_t a4[ITER];
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      const int c = it * 64 + lane;
+      a4[it] = *reinterpret_cast<const float4_t*>(ep + (c / CPR) * ROWP + (c % CPR) * 16);
+    }
+    auto store_group = [&](int it, float4_t v) {
+      __builtin_amdgcn_raw_buffer_store_b64(u32v2_t{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3])}, d_rsrc, off[it], 0, 0);
+    };
+    if (kDual) {
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) store_group(it, a4[it]);
+    } else if (beta == 0.f) {
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) store_group(it, a4[it] * alpha);
+    } else {
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        float4_t v = a4[it] * alpha;
+        v[0] += beta * h2f_bits(cv[it].x & 0xffffu);
+        v[1] += beta * h2f_bits(cv[it].x >> 16);
+        v[2] += beta * h2f_bits(cv[it].y & 0xffffu);
+        v[3] += beta * h2f_bits(cv[it].y >> 16);
+        store_group(it, v);
       }
     }
   }
