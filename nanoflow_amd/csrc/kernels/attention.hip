@@ -12,7 +12,7 @@
 // Online softmax runs in the exp2 domain with fp32 state per column; masked keys contribute
 // exactly zero (the reference's -5e4 mask underflows to zero in fp32 as well).
 //
-// Decode: a workgroup's 4 wavefronts split the request's pages (32 keys per step each) and
+// Decode: a workgroup's wavefronts split the request's pages (32 keys per step each) and
 // merge (m, l, O) through LDS; work item = (request, kv head), head fastest, so that
 // concurrently running workgroups stream the same 64 KiB pages.  Prefill: a workgroup is a
 // 16-token tile (for GQA 4) whose wavefronts share the streamed K/V tiles; tiles are planned
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restric
 //   * K and V pages go from global memory STRAIGHT INTO LDS (buffer_load ... lds), not through
 //     registers: the load-to-register path of a CU saturates near 38 GB/s, the direct path
 //     carries half again as much from HBM, and the data in flight no longer costs registers.
-//   * A workgroup is (request, kv head); its 4 wavefronts take every 4th 32-key step and merge
+//   * A workgroup is (request, kv head); its NW wavefronts take every NW-th 32-key step and merge
 //     (m, l, O) at the end.  Every wavefront owns a private LDS ring (2 K tiles + 2 V tiles of
 //     32 keys x 256 bytes), so no barrier is needed while streaming: a wavefront only waits
 //     for its own loads (s_waitcnt vmcnt), and refills a tile as soon as its MFMAs have read it
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
       l_run += __shfl_xor(l_run, 16, 64);
       l_run += __shfl_xor(l_run, 32, 64);
 
-      // ---- merge the 4 wavefronts.  oacc[i][r] = O[column c16][feature 16i + 4g + r].  Each
+      // ---- merge the wavefronts.  oacc[i][r] = O[column c16][feature 16i + 4g + r].  Each
       // wavefront parks its partial result in its own LDS region (its streaming is over).
       float* s_o = reinterpret_cast<float*>(wptr);             // [8][4][64]
       float* s_m = reinterpret_cast<float*>(wptr + 8192);      // [64]
@@ -548,7 +548,9 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
   if (bound > 0x7fffffffLL) bound = 0x7fffffffLL;
   if (bound < 1) bound = 1;
   if (decode_mode) {
-    constexpr int kWaves = 4;  // wavefronts per (request, kv head) workgroup
+    // wavefronts per (request, kv head) workgroup: with 2 (64 KB of LDS) two workgroups share a
+    // CU, and one streams while the other starts or merges -- a few percent faster than 4 or 1
+    constexpr int kWaves = 2;
     constexpr int kDecodeLds = kWaves * 32768;
     auto kern = attn_decode_kernel<GROUP, kWaves>;
     static bool attr_set = false;  // benign race: the call is idempotent
