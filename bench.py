@@ -106,7 +106,7 @@ def _attention_roofline(tm, bytes_per_launch, name="roofline"):
     avg_launch_ms = tm.decode_attn_ms / n_launch
     achieved = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9 if avg_launch_ms > 0 else 0.0
     return {
-        "kernel": "attn_paged_kernel (paged decode attention)", "bound": "hbm",
+        "kernel": "attn_decode_kernel (paged decode attention)", "bound": "hbm",
         "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
         "traffic": (None if DECODE_ATTN_TRAFFIC_RATIO is None
                     else bytes_per_launch * DECODE_ATTN_TRAFFIC_RATIO),

@@ -4,8 +4,8 @@
 //   D = half(silu(half(A.Bg)) * half(A.Bu))              (dual; gate/up SwiGLU)
 //
 // Workgroup = 256 threads = 4 wavefronts in a WM x WN grid; each wavefront owns a
-// (BM/WM) x (BN/WN) block of 32x32 MFMA tiles.  K is walked in slabs of 64 through two LDS
-// stages.
+// (BM/WM) x (BN/WN) block of 32x32 MFMA tiles.  K is walked in slabs of 64 through a ring of
+// two to four LDS stages (as many as fit 144 KB).
 //
 // Operands go from global memory STRAIGHT INTO LDS (buffer_load_dwordx4 ... lds): a CU moves
 // about 38 GB/s through the load-to-register path but well over 100 GB/s through this one, and
@@ -24,11 +24,14 @@
 //       and receive it column-wise), two per operand; the 4 rows x 64 bytes a read cycle
 //       touches sit in 4 different 64-byte bank groups.
 // With these two permutations SQ_LDS_BANK_CONFLICT reads zero for the kernel.
-// No staging registers, no permutes, no LDS stores.  While the MFMAs of slab i run out of one
-// stage, the loads of slab i+1 are in flight into the other; one barrier per slab.
+// No staging registers, no permutes, no LDS stores in the main loop.  A wavefront is alone on
+// its SIMD, so nothing hides a stall of its instruction stream: the loads of later slabs and
+// the fragment reads of the next k-step are dealt out one at a time between the MFMAs of the
+// current k-step, in a pinned order; one barrier per slab.
 //
-// The MFMA is issued as D^T = B^T.A^T (weights as the first operand) so that each lane ends up
-// with 4 consecutive output columns of one row -> 8-byte stores/loads for D and C.
+// The MFMA is issued as D^T = B^T.A^T (weights as the first operand): a lane ends up with 4
+// consecutive output columns of 32 rows.  The epilogue turns each wavefront's block around
+// through LDS so that D is stored, and C read, in whole 512-byte runs.
 #include <algorithm>
 #include <type_traits>
 
