@@ -9,10 +9,16 @@ reference's pipeline/utils/serve_8B.py:
   Rows with input_len -1 (prompt text to tokenize) are rejected: no tokenizer ships here.
 * config: the reference's pipeline JSON (pipeline/config_all/llama3-8B/1024.json schema);
   ``serve_configs.pipeline_type`` must be LOCAL, NON_OVERLAP_LOCAL or NANOBATCH_LOCAL.
-* only ``--empty_weight True`` is supported (random-init weights on the device, as the reference's
-  own evaluation runs: pipeline/eval/eval-fix-offline/run.py:42-50); KV pool =
-  ``1024 * allocate_kv_data_batch // 16`` pages per layer (serve_8B.py:643).
-* writes PREFIX.stat, PREFIX.stat.csv (same columns as serve_8B.py:792-793) and PREFIX.req_time.
+* ``--empty_weight True``: random-init weights on the device, as the reference's own evaluation
+  runs (pipeline/eval/eval-fix-offline/run.py:42-50).  Otherwise the weights come from
+  ``serve_configs.weight_path``/weight_rank_0.pt (nanoflow_amd/weights.py; serve_8B.py:611-629);
+  when that file is missing it is first converted from the Hugging Face checkpoint directory
+  ``serve_configs.hf_path``.  Nothing is downloaded.  (The flag is parsed as a truth value here;
+  the reference's ``type=bool`` turns every non-empty string, "False" included, into True.)
+* KV pool = ``1024 * allocate_kv_data_batch // 16`` pages per layer (serve_8B.py:643).
+* writes PREFIX.stat, PREFIX.stat.csv (same columns as serve_8B.py:792-793), PREFIX.req_time and
+  PREFIX.req_tokens (prompt + generated ids of every retired request, one Python list per line,
+  by request index: serve_8B.py:718-721).
 
 Skip cycles advance the scheduler without GPU work and release requests by the estimated cycle
 time; run cycles form batch i+1 on the CPU while the GPU runs batch i.  When every request has
@@ -61,8 +67,7 @@ def main():
     ap.add_argument("--allocate_page_num", type=int, default=740, help="accepted and unused, as in the reference")
     ap.add_argument("--empty_weight", default="True")
     a = ap.parse_args()
-    if str(a.empty_weight).lower() not in ("true", "1"):
-        raise SystemExit("only --empty_weight True is supported (no checkpoint loader here)")
+    empty_weight = str(a.empty_weight).lower() in ("true", "1", "yes")
     prefix = a.output_prefix or a.trace_path[:-4]
 
     import torch
@@ -80,11 +85,29 @@ def main():
     T, nano1, kqv1, kqv3 = pc["global_batch_size"], pc["nanobatch_1_size"], pc["kqv1_size"], pc["kqv3_size"]
     pages = 1024 * mc["allocate_kv_data_batch"] // 16
 
+    weights = None
+    if not empty_weight:
+        from nanoflow_amd import weights as W
+        wdir = sc.get("weight_path")
+        if not wdir:
+            raise SystemExit("serve_configs.weight_path is not set (or pass --empty_weight True)")
+        if not os.path.isfile(os.path.join(wdir, W.FILE_NAME)):
+            hf = sc.get("hf_path")
+            if not hf or not os.path.isdir(hf):
+                raise SystemExit(f"{wdir}/{W.FILE_NAME} not found and serve_configs.hf_path is not a checkpoint "
+                                 "directory to convert it from")
+            print("Saving weights")
+            W.convert_hf_checkpoint(hf, wdir)
+        print("Loading weights")
+        t0 = time.perf_counter()
+        weights = W.load_weight_file(wdir, shape)
+        print("Time taken to load weights: ", time.perf_counter() - t0)
+
     reqs = read_trace(a.trace_path)
     avg_in = sum(r[1] for r in reqs) // len(reqs)
     avg_out = sum(r[2] for r in reqs) // len(reqs)
     eng = engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=kqv1, kqv3=kqv3, kv_pages=pages,
-                        run_layer=mc.get("run_layer", shape.layers), kv_fill="zeros")
+                        run_layer=mc.get("run_layer", shape.layers), kv_fill="zeros", weights=weights)
     former = P.BatchFormer(pages, shape.page_size, T, nano1, kqv1, kqv3, avg_in, avg_out)
 
     pending = list(reqs)                  # not yet released, in arrival order
@@ -160,7 +183,15 @@ def main():
     n_retired = former.state()["retired"]
     done = n_retired - retired_before
     infos = [former.retired_info(k) for k in range(n_retired)]
+    outputs = dict(former.retired_output(k) for k in range(n_retired))
     eng.close()
+    prompt_len = {r[0]: r[1] for r in reqs}
+    with open(prefix + ".req_tokens", "w") as fq:
+        for idx in sorted(outputs):
+            gen = [int(t) for t in outputs[idx]]
+            if gen and gen[-1] == -1:       # the placeholder of a sample that was never harvested
+                gen.pop()
+            fq.write(f"{list(range(prompt_len[idx])) + gen}\n")
     with open(prefix + ".stat", "w") as fs, open(prefix + ".stat.csv", "w") as fc, open(prefix + ".req_time", "w") as ft:
         def out(s):
             print(s)

@@ -288,8 +288,67 @@ def test_graph_replay_is_identical_to_eager(pt_name):
         assert np.array_equal(h0, h1), (i, "residual stream")
 
 
-@pytest.mark.parametrize("online", [False, True])
-def test_serve_command_line_writes_the_reference_result_files(tmp_path, online):
+def _hf_state_dict_from(w, shape):
+    """Engine-format weights written back in the Hugging Face names and [out, in] orientation."""
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a.T))
+    kd = shape.Hkv * shape.d
+    sd = {"model.embed_tokens.weight": torch.from_numpy(w["embedding"].copy()),
+          "lm_head.weight": t(w["lm_head"]), "model.norm.weight": torch.from_numpy(w["model_norm"].copy())}
+    for l in range(shape.layers):
+        p = f"model.layers.{l}."
+        kqv = w["w_kqv"][l]
+        sd.update({p + "self_attn.k_proj.weight": t(kqv[:, :kd]), p + "self_attn.v_proj.weight": t(kqv[:, kd:2 * kd]),
+                   p + "self_attn.q_proj.weight": t(kqv[:, 2 * kd:]), p + "self_attn.o_proj.weight": t(w["w_o"][l]),
+                   p + "mlp.gate_proj.weight": t(w["w_gate"][l]), p + "mlp.up_proj.weight": t(w["w_up"][l]),
+                   p + "mlp.down_proj.weight": t(w["w_down"][l]),
+                   p + "input_layernorm.weight": torch.from_numpy(w["ln_attn"][l].copy()),
+                   p + "post_attention_layernorm.weight": torch.from_numpy(w["ln_ffn"][l].copy())})
+    return sd
+
+
+def _write_hf_checkpoint(dirpath, w, shape):
+    import json, os
+    from safetensors.torch import save_file
+    os.makedirs(dirpath, exist_ok=True)
+    save_file(_hf_state_dict_from(w, shape), os.path.join(dirpath, "model.safetensors"))
+    json.dump({"hidden_size": shape.hidden, "num_attention_heads": shape.Hq, "num_key_value_heads": shape.Hkv,
+               "intermediate_size": shape.ffn, "vocab_size": shape.vocab, "num_hidden_layers": shape.layers,
+               "rms_norm_eps": shape.eps, "rope_theta": shape.rope_theta}, open(os.path.join(dirpath, "config.json"), "w"))
+
+
+def test_weights_loaded_from_a_checkpoint_run_like_the_oracle(oracle, tmp_path):
+    """Hugging Face checkpoint -> weight_rank_0.pt -> pipeline: one mixed iteration gives the oracle's
+    residual stream and samples for the SAME weights in the oracle's own (in-memory) form."""
+    from nanoflow_amd import engine, weights as W, pllm_python as P
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=4)
+    _write_hf_checkpoint(str(tmp_path / "hf"), w, shape)
+    W.convert_hf_checkpoint(str(tmp_path / "hf"), str(tmp_path / "w"))
+    w2 = W.load_weight_file(str(tmp_path / "w"), shape)
+    for k in ("embedding", "lm_head", "model_norm"):
+        assert np.array_equal(w2[k], w[k]), k
+    for k in ("w_kqv", "w_o", "w_gate", "w_up", "w_down", "ln_attn", "ln_ffn"):
+        for l in range(shape.layers):
+            assert np.array_equal(w2[k][l], w[k][l]), (k, l)
+    b = synth.make_batch(list(range(5, 25)), [(7, 30), (0, 46)], vocab=shape.vocab, seed=21, extra_pages=40)
+    rng = np.random.default_rng(5)
+    pools = [synth.make_kv_pool(b.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok = b.input_tokens.copy()
+    tok[:b.decodePrefillBorder] = 1           # first-iteration rule of the decode-token feed
+    d = b.as_dict()
+    d["input_tokens"] = tok
+    hid, _, samp = oracle.decoder_forward(shape.as_dict(), w, [p.copy() for p in pools], d, want_logits=True)
+    with engine.Engine(shape, P.PipelineType.NON_OVERLAP_LOCAL, global_batch=96, nano1=40, kqv1=20, kqv3=28,
+                       kv_pages=b.num_pages, weights=w2, kv_pools=pools) as eng:
+        eng.update(b)
+        got = eng.run()
+        got_hid = eng.buffer("hidden").cpu().numpy()[:b.tokens]
+    assert _max_rel(got_hid, hid) < E2E_RTOL
+    assert np.array_equal(got[:len(samp)], samp)
+
+
+@pytest.mark.parametrize("online,from_file", [(False, False), (True, False), (False, True)])
+def test_serve_command_line_writes_the_reference_result_files(tmp_path, online, from_file):
     """nanoflow_amd.serve with the reference's flags on a tiny model: offline trace (whole loop in
     the library) and a trace with arrival times (loop driven per phase)."""
     import subprocess, sys, os, csv
@@ -303,10 +362,16 @@ def test_serve_command_line_writes_the_reference_result_files(tmp_path, online):
         f.write("idx,input_len,output_len,arrival\n")
         for i in range(16):
             f.write(f"{i},{20 + 3 * i},{4 + i % 5},{0.02 * i if online else 0}\n")
+    if from_file:     # weights from serve_configs.weight_path, converted on the fly from serve_configs.hf_path
+        import json
+        _write_hf_checkpoint(str(tmp_path / "hf"), _scaled_weights(shape, seed=4), shape)
+        c = json.load(open(cfg))
+        c["serve_configs"].update({"weight_path": str(tmp_path / "w"), "hf_path": str(tmp_path / "hf")})
+        json.dump(c, open(cfg, "w"))
     prefix = tmp_path / "out"
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     cmd = [sys.executable, "-m", "nanoflow_amd.serve", "-t", str(trace), "-c", str(cfg), "-r", "400",
-           "-s", "2" if online else "0", "--est_cycle_time", "0.05", "--empty_weight", "True", "-o", str(prefix)]
+           "-s", "2" if online else "0", "--est_cycle_time", "0.05", "--empty_weight", str(not from_file), "-o", str(prefix)]
     print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=110)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
@@ -322,3 +387,13 @@ def test_serve_command_line_writes_the_reference_result_files(tmp_path, online):
         assert int(t["input_len"]) == 20 + 3 * int(t["req_idx"])
         assert float(t["encode_latency"]) >= 0 and float(t["decode_latency"]) >= 0
     assert "Token per second" in open(str(prefix) + ".stat").read()
+    import ast
+    lines = [ast.literal_eval(l) for l in open(str(prefix) + ".req_tokens")]
+    assert len(lines) >= len(got)
+    if len(lines) == 16:     # every request retired: line k is request k (the file is ordered by request index)
+        for k, l in enumerate(lines):
+            n_in, n_out = 20 + 3 * k, 4 + k % 5
+            assert l[:n_in] == list(range(n_in)), k
+            assert len(l) - n_in in (n_out - 1, n_out) and all(0 <= t < shape.vocab for t in l[n_in:]), (k, l[n_in:])
+    if from_file:
+        assert os.path.isfile(str(tmp_path / "w" / "weight_rank_0.pt")) and "Loading weights" in r.stdout

@@ -1,0 +1,124 @@
+"""Weight files in the reference's format (pipeline/utils/weightSaver.py:73-149 and
+weightLoader.py:38-67, single rank): Hugging Face checkpoint -> weight_rank_0.pt -> engine dict.
+The expected tensors are written out here from the Hugging Face [out, in] convention; nothing
+is computed with the converter's own code."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+safetensors_torch = pytest.importorskip("safetensors.torch")
+
+from nanoflow_amd import weights as W  # noqa: E402
+
+CFG = {"hidden_size": 256, "num_attention_heads": 2, "num_key_value_heads": 1, "intermediate_size": 512,
+       "vocab_size": 384, "num_hidden_layers": 2, "rms_norm_eps": 1e-5, "rope_theta": 500000.0}
+
+
+def _hf_state_dict(seed=0, tied=False, bias=False):
+    g = torch.Generator().manual_seed(seed)
+    H, F, V, d = CFG["hidden_size"], CFG["intermediate_size"], CFG["vocab_size"], 128
+    hq, hkv = CFG["num_attention_heads"], CFG["num_key_value_heads"]
+    r = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)
+    sd = {"model.embed_tokens.weight": r(V, H), "model.norm.weight": r(H)}
+    if not tied:
+        sd["lm_head.weight"] = r(V, H)
+    for l in range(CFG["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        sd.update({p + "input_layernorm.weight": r(H), p + "post_attention_layernorm.weight": r(H),
+                   p + "self_attn.q_proj.weight": r(hq * d, H), p + "self_attn.k_proj.weight": r(hkv * d, H),
+                   p + "self_attn.v_proj.weight": r(hkv * d, H), p + "self_attn.o_proj.weight": r(H, hq * d),
+                   p + "mlp.gate_proj.weight": r(F, H), p + "mlp.up_proj.weight": r(F, H),
+                   p + "mlp.down_proj.weight": r(H, F)})
+        if bias:
+            sd.update({p + "self_attn.q_proj.bias": r(hq * d), p + "self_attn.k_proj.bias": r(hkv * d),
+                       p + "self_attn.v_proj.bias": r(hkv * d)})
+    return sd
+
+
+def _write_checkpoint(tmp_path, sd):
+    hf = tmp_path / "hf"
+    hf.mkdir()
+    keys = sorted(sd)
+    half = len(keys) // 2      # two shards, as real checkpoints have
+    safetensors_torch.save_file({k: sd[k].contiguous() for k in keys[:half]}, str(hf / "model-00001-of-00002.safetensors"))
+    safetensors_torch.save_file({k: sd[k].contiguous() for k in keys[half:]}, str(hf / "model-00002-of-00002.safetensors"))
+    json.dump(CFG, open(hf / "config.json", "w"))
+    return str(hf)
+
+
+def _f16(x):
+    return x.to(torch.float16).numpy()
+
+
+def test_convert_and_load_give_the_pipeline_orientation(tmp_path):
+    sd = _hf_state_dict()
+    out_dir = str(tmp_path / "w")
+    path = W.convert_hf_checkpoint(_write_checkpoint(tmp_path, sd), out_dir)
+    assert os.path.basename(path) == "weight_rank_0.pt"
+    shape = W.shape_from_hf_config(CFG)
+    assert (shape.hidden, shape.Hq, shape.Hkv, shape.d, shape.ffn, shape.vocab, shape.layers) == (256, 2, 1, 128, 512, 384, 2)
+    w = W.load_weight_file(out_dir, shape)
+    assert w["embedding"].dtype == np.float16
+    assert np.array_equal(w["embedding"], _f16(sd["model.embed_tokens.weight"]))           # [V, H], as stored
+    assert np.array_equal(w["lm_head"], _f16(sd["lm_head.weight"]).T)                       # [H, V]
+    assert np.array_equal(w["model_norm"], _f16(sd["model.norm.weight"]))
+    for l in range(2):
+        p = f"model.layers.{l}."
+        kqv = w["w_kqv"][l]
+        assert kqv.shape == (256, 128 + 128 + 256)
+        # column blocks K | V | Q, each the transposed projection: y = x . W^T
+        assert np.array_equal(kqv[:, :128], _f16(sd[p + "self_attn.k_proj.weight"]).T)
+        assert np.array_equal(kqv[:, 128:256], _f16(sd[p + "self_attn.v_proj.weight"]).T)
+        assert np.array_equal(kqv[:, 256:], _f16(sd[p + "self_attn.q_proj.weight"]).T)
+        assert np.array_equal(w["w_o"][l], _f16(sd[p + "self_attn.o_proj.weight"]).T)
+        assert np.array_equal(w["w_gate"][l], _f16(sd[p + "mlp.gate_proj.weight"]).T)
+        assert np.array_equal(w["w_up"][l], _f16(sd[p + "mlp.up_proj.weight"]).T)
+        assert np.array_equal(w["w_down"][l], _f16(sd[p + "mlp.down_proj.weight"]).T)
+        assert np.array_equal(w["ln_attn"][l], _f16(sd[p + "input_layernorm.weight"]))
+        assert np.array_equal(w["ln_ffn"][l], _f16(sd[p + "post_attention_layernorm.weight"]))
+        assert all(a.flags["C_CONTIGUOUS"] for a in (kqv, w["w_o"][l], w["w_down"][l]))
+
+
+def test_weight_file_has_the_reference_tensor_names(tmp_path):
+    out_dir = str(tmp_path / "w")
+    W.convert_hf_checkpoint(_write_checkpoint(tmp_path, _hf_state_dict()), out_dir)
+    sd = torch.load(os.path.join(out_dir, "weight_rank_0.pt"), weights_only=True)
+    want = {"ModelNorm", "Embed", "LmHead"}
+    for l in range(2):
+        want |= {f"{n}_{l}" for n in ("O1", "O2", "U", "G", "D", "KQV", "BKQV", "LNATT", "LNFFN")}
+    assert set(sd) == want
+    assert sd["BKQV_0"].shape == (1, 512) and not bool(sd["BKQV_0"].any())
+    assert sd["KQV_1"].dtype == torch.float16 and torch.equal(sd["O1_1"], sd["O2_1"])
+
+
+def test_tied_embeddings_feed_the_lm_head(tmp_path):
+    sd = _hf_state_dict(tied=True)
+    out_dir = str(tmp_path / "w")
+    W.convert_hf_checkpoint(_write_checkpoint(tmp_path, sd), out_dir)
+    w = W.load_weight_file(out_dir)
+    assert np.array_equal(w["lm_head"], _f16(sd["model.embed_tokens.weight"]).T)
+
+
+def test_kqv_bias_is_rejected_not_dropped(tmp_path):
+    out_dir = str(tmp_path / "w")
+    W.convert_hf_checkpoint(_write_checkpoint(tmp_path, _hf_state_dict(bias=True)), out_dir)
+    sd = torch.load(os.path.join(out_dir, "weight_rank_0.pt"), weights_only=True)
+    assert sd["BKQV_0"].shape == (1, 512) and bool(sd["BKQV_0"].any())       # written as K | V | Q like the weights
+    with pytest.raises(ValueError, match="bias"):
+        W.load_weight_file(out_dir)
+
+
+def test_shape_mismatch_and_foreign_files_raise(tmp_path):
+    out_dir = str(tmp_path / "w")
+    W.convert_hf_checkpoint(_write_checkpoint(tmp_path, _hf_state_dict()), out_dir)
+    wrong = W.shape_from_hf_config({**CFG, "intermediate_size": 1024})
+    with pytest.raises(ValueError, match="w_gate"):
+        W.load_weight_file(out_dir, wrong)
+    with pytest.raises(ValueError, match="layers"):
+        W.load_weight_file(out_dir, W.shape_from_hf_config({**CFG, "num_hidden_layers": 3}))
+    torch.save({"something": torch.zeros(3)}, str(tmp_path / "other.pt"))
+    with pytest.raises(ValueError, match="not a pipeline weight file"):
+        W.load_weight_file(str(tmp_path / "other.pt"))
