@@ -336,8 +336,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps (default: offline 8, iteration 2)")
     ap.add_argument("--workload", default="offline", choices=["offline", "iteration"])
     ap.add_argument("--pipeline", default="auto", choices=["auto", "LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL"],
-                    help="auto = the faster schedule measured on MI355X for the workload: NON_OVERLAP_LOCAL for\n"
-                         "offline, LOCAL (two streams) for iteration")
+                    help="auto = the fastest schedule measured on MI355X for both workloads: NON_OVERLAP_LOCAL\n"
+                         "(one stream); LOCAL measures the two-stream overlapped schedule")
     ap.add_argument("--nano1", type=int, default=1024, help="rows of nano-batch 1")
     ap.add_argument("--kqv1", type=int, default=512)
     ap.add_argument("--kqv3", type=int, default=512)
@@ -357,7 +357,7 @@ def main():
     args = ap.parse_args()
     _check_single_gpu(args)
     if args.pipeline == "auto":
-        args.pipeline = "NON_OVERLAP_LOCAL" if args.workload == "offline" else "LOCAL"
+        args.pipeline = "NON_OVERLAP_LOCAL"
     if args.graph:
         args.profile_level = 0
     rec = run_offline(args) if args.workload == "offline" else run_iteration(args)
