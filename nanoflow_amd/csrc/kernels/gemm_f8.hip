@@ -104,7 +104,8 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   constexpr int B_LOADS = BN / 32;
   constexpr int NS = SM::stages;
   constexpr int LOADS = A_LOADS + B_LOADS;
-  constexpr int PARTS = 2;          // the loads of a slab are spread over its two k-steps
+  // k-steps the loads of one slab are spread over; with two stages they must land within one step
+  constexpr int PARTS = NS == 2 ? 1 : 2;
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem8[];
   const uint32_t smem_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem8;
@@ -133,35 +134,35 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
 
   // Both operands are rows of 128 k-bytes; they go from global memory straight into LDS
   // (see gemm.hip): 8 rows per load instruction, row r keeping its logical 16-byte chunk c at
-  // position c ^ ((r >> 1) & 7) (bit 3 of the row number is the wave's parity).
+  // position c ^ ((r >> 1) & 7) (bit 3 of the row number is the wave's parity).  One running
+  // offset per load instruction, advanced by a slab after each use; rows past the operand's last
+  // one lie at or past the end of the buffer and read as zero, which leaves only k >= K inside a
+  // row to be masked.
   const rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K);
   const rsrc_t b_rsrc = make_rsrc(B, (size_t)N * K);
   const int kc = ((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2))) * 16;  // k-byte of this lane's chunk inside the slab
   uint32_t a_off[A_LOADS], b_off[B_LOADS];
 #pragma unroll
-  for (int t = 0; t < A_LOADS; ++t) {
-    const int gm = m_base + (t * 4 + wave) * 8 + (lane >> 3);
-    a_off[t] = gm < M ? (uint32_t)gm * (uint32_t)K + kc : kOob;
-  }
+  for (int t = 0; t < A_LOADS; ++t)
+    a_off[t] = (uint32_t)(m_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)K + kc;
 #pragma unroll
-  for (int t = 0; t < B_LOADS; ++t) {
-    const int gn = n_base + (t * 4 + wave) * 8 + (lane >> 3);
-    b_off[t] = gn < N ? (uint32_t)gn * (uint32_t)K + kc : kOob;
-  }
-  auto issue_loads = [&](int stage, int k0, int part) {
+  for (int t = 0; t < B_LOADS; ++t)
+    b_off[t] = (uint32_t)(n_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)K + kc;
+  auto load_one = [&](auto t_c, uint32_t st, bool k_ok) {
+    constexpr int t = decltype(t_c)::value;
+    if constexpr (t < A_LOADS) {
+      load16_to_lds<t * 4096>(a_rsrc, k_ok ? a_off[t] : kOob, st);
+      a_off[t] += F8_BK;
+    } else {
+      constexpr int tt = t - A_LOADS;
+      load16_to_lds<BM * 128 + tt * 4096>(b_rsrc, k_ok ? b_off[tt] : kOob, st);
+      b_off[tt] += F8_BK;
+    }
+  };
+  auto load_slab = [&](int stage, int k0) {
     const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::stage_bytes + wave * 1024);
     const bool k_ok = k0 + kc < K;
-#pragma unroll
-    for (int t = 0; t < A_LOADS; ++t) {
-      if (part >= 0 && t % PARTS != part) continue;
-      load16_to_lds(a_rsrc, (k_ok && a_off[t] != kOob) ? a_off[t] + (uint32_t)k0 : kOob, st + t * 4096);
-    }
-#pragma unroll
-    for (int t = 0; t < B_LOADS; ++t) {
-      if (part >= 0 && (A_LOADS + t) % PARTS != part) continue;
-      load16_to_lds(b_rsrc, (k_ok && b_off[t] != kOob) ? b_off[t] + (uint32_t)k0 : kOob,
-                    st + BM * 128 + t * 4096);
-    }
+    static_for<LOADS>([&](auto t_c) { load_one(t_c, st, k_ok); });
   };
 
   // MFMA operand of k-step kk: 32 bytes of row r = the logical chunks 4kk + 2lg and + 1, which
@@ -177,96 +178,159 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
     const u32x4 hi = *reinterpret_cast<const u32x4*>(p + (pos ^ 16u));
     return v8i32{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
   };
-  auto read_frags = [&](int stage, int kk, int buf) {
-    const uint8_t* st = smem8 + stage * SM::stage_bytes;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) af[buf][i] = read32(st + a_rd + i * 32 * 128, swz[kk]);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) bf[buf][j] = read32(st + b_rd + j * 32 * 128, swz[kk]);
-  };
-  auto mfma_step = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[buf][j], af[buf][i], acc[i][j],
-                                                                    0, 0, 0, 0, 0, 0);
+  constexpr int READS = TM + TN;
+  auto read_one = [&](auto q_c, auto kk_c, auto buf_c, const uint8_t* st) {
+    constexpr int q = decltype(q_c)::value, kk = decltype(kk_c)::value, buf = decltype(buf_c)::value;
+    if constexpr (q < TM) af[buf][q] = read32(st + a_rd + q * 32 * 128, swz[kk]);
+    else bf[buf][q - TM] = read32(st + b_rd + (q - TM) * 32 * 128, swz[kk]);
   };
 
-  // Slab s lives in LDS stage s % NS; while its two k-steps run, the loads of slab s+NS-1 go
-  // into the stage slab s-1 has left; at the end the wavefront waits for its loads of slab s+1
-  // (younger ones may stay in flight) and meets the others at the barrier.
-  auto slab = [&](auto issue_c, int s, int cs, int ls) {
-    constexpr bool issue = decltype(issue_c)::value;
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      if (issue) issue_loads(ls, (s + NS - 1) * F8_BK, kk);
-      if (kk < 1) read_frags(cs, kk + 1, (kk + 1) & 1);
+  // One k-step: its MFMAs (64 cycles of the matrix pipe each) with the loads LP, LP + PARTS, ...
+  // of the slab being fetched (LP < 0: none) and the fragment reads of k-step RK (RK < 0: none)
+  // dealt out between them, order pinned -- the scheme of gemm.hip.
+  constexpr int NM = TN * TM;
+  auto step = [&](auto kk_c, auto lp_c, auto rk_c, uint32_t ld_st, bool ld_ok, const uint8_t* rd_st) {
+    constexpr int kk = decltype(kk_c)::value, LP = decltype(lp_c)::value, RK = decltype(rk_c)::value;
+    constexpr int NL = LP < 0 ? 0 : (LOADS - LP + PARTS - 1) / PARTS;
+    constexpr int NR = RK < 0 ? 0 : READS;
+    constexpr int S = NL + NR;
+    static_for<NM>([&](auto n_c) {
+      constexpr int n = decltype(n_c)::value;
+      constexpr int j = n / TM, i = n % TM;
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[kk][j], af[kk][i], acc[i][j], 0, 0, 0, 0, 0, 0);
+      constexpr int lo = n * S / NM, hi = (n + 1) * S / NM;
+      static_for<hi - lo>([&](auto d_c) {
+        constexpr int q = lo + decltype(d_c)::value;
+        if constexpr (q < NL) load_one(ic<(LP < 0 ? 0 : LP) + PARTS * q>{}, ld_st, ld_ok);
+        else read_one(ic<q - NL>{}, ic<(RK < 0 ? 0 : RK)>{}, ic<1 - kk>{}, rd_st);
+      });
       __builtin_amdgcn_sched_barrier(0);
-      mfma_step(kk & 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
-  auto wait_loads = [&](int younger) {  // vmcnt(younger): bits [3:0] and [15:14]
-    if (younger == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-    else __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS * (NS - 2) & 15) | (((LOADS * (NS - 2)) >> 4) << 14));
+  // vmcnt(n) with lgkmcnt(0): n in bits [3:0] and [15:14]
+  auto wait_loads = [&](int younger) {
+    if (younger == 0) __builtin_amdgcn_s_waitcnt(0x0070);
+    else __builtin_amdgcn_s_waitcnt(0x0070 | (LOADS * (NS - 2) & 15) | (((LOADS * (NS - 2)) >> 4) << 14));
   };
   static_assert(LOADS * (NS - 2) < 64, "vmcnt range");
   auto next = [](int st) { return st + 1 == NS ? 0 : st + 1; };
 
+  // Slab s lives in LDS stage s % NS and is two k-steps.  Step 0 prefetches the fragments of step
+  // 1; then the wavefront waits for its own loads of slab s+1 and its reads of this stage, and
+  // meets the others at the slab's one barrier; step 1 prefetches the first fragments of slab
+  // s+1 and starts refilling this stage with slab s+NS (the rest of those loads, if spread over
+  // two steps, go out during step 0 of slab s+1).
+  //   IA: slab s+NS-1 exists (loads in step 0), IB: slab s+NS exists (loads in step 1), LAST: no slab s+1.
+  auto slab = [&](auto ia_c, auto ib_c, auto last_c, int s, int cs, int ls) {
+    constexpr bool IA = decltype(ia_c)::value, IB = decltype(ib_c)::value, LAST = decltype(last_c)::value;
+    const uint8_t* st = smem8 + cs * SM::stage_bytes;
+    const uint32_t ld_a = __builtin_amdgcn_readfirstlane(smem_lds + ls * SM::stage_bytes + wave * 1024);
+    step(ic<0>{}, ic<(IA && PARTS > 1) ? 1 : -1>{}, ic<1>{}, ld_a, (s + NS - 1) * F8_BK + kc < K, st);
+    if constexpr (!LAST) {
+      wait_loads(IA ? 1 : 0);
+      __syncthreads();
+    }
+    const uint32_t ld_b = __builtin_amdgcn_readfirstlane(smem_lds + cs * SM::stage_bytes + wave * 1024);
+    step(ic<1>{}, ic<IB ? 0 : -1>{}, ic<LAST ? -1 : 0>{}, ld_b, (s + NS) * F8_BK + kc < K,
+         smem8 + next(cs) * SM::stage_bytes);
+  };
+
   const int nslab = (K + F8_BK - 1) / F8_BK;
 #pragma unroll
   for (int p = 0; p < NS - 1; ++p)
-    if (p < nslab) issue_loads(p, p * F8_BK, -1);
-  if (nslab >= NS - 1) wait_loads(1); else wait_loads(0);
+    if (p < nslab) load_slab(p, p * F8_BK);
+  wait_loads(nslab >= NS - 1 ? 1 : 0);
   __syncthreads();
-  read_frags(0, 0, 0);
+  static_for<READS>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, smem8); });
+  if (NS - 1 < nslab) {  // the share of slab NS-1 that a slab's step 1 would have issued
+    const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + (NS - 1) * SM::stage_bytes + wave * 1024);
+    const bool k_ok = (NS - 1) * F8_BK + kc < K;
+    static_for<(LOADS + PARTS - 1) / PARTS>([&](auto q_c) { load_one(ic<PARTS * decltype(q_c)::value>{}, st, k_ok); });
+  }
   int cs = 0, ls = NS - 1, s = 0;
-  for (; s + NS - 1 < nslab; ++s) {
-    slab(std::true_type{}, s, cs, ls);
-    wait_loads(1);
-    __syncthreads();
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  for (; s + NS < nslab; ++s) {  // steady state
+    slab(T_{}, T_{}, F_{}, s, cs, ls);
     cs = next(cs);
     ls = next(ls);
-    read_frags(cs, 0, 0);
   }
-  for (; s < nslab; ++s) {
-    slab(std::false_type{}, s, cs, ls);
-    if (s + 1 < nslab) {
-      wait_loads(0);
-      __syncthreads();
-      cs = next(cs);
-      read_frags(cs, 0, 0);
-    }
+  for (; s + 1 < nslab; ++s) {   // drain: the last loads, then none
+    if (s + NS - 1 < nslab) slab(T_{}, F_{}, F_{}, s, cs, ls);
+    else slab(F_{}, F_{}, F_{}, s, cs, ls);
+    cs = next(cs);
+    ls = next(ls);
   }
+  slab(F_{}, F_{}, T_{}, s, cs, ls);
 
-  // Epilogue: acc[i][j][r] is D[m][n] with m = tile row l32, n = (r/4)*8 + lg*4 + r%4.
+  // Epilogue, as in gemm.hip: acc[i][j][r] is D[m][n] with m = tile row l32 and
+  // n = (r/4)*8 + lg*4 + r%4; each wavefront turns its block around through LDS, 32 rows at a
+  // time in fp32, and stores (and reads C and the row scales) in whole runs through buffer
+  // descriptors that end with the matrix, so a pass has no branches.
+  constexpr int CW = BN / WN, ROWP = CW * 4 + 16, CPR = CW / 4, ITER = 32 * CPR / 64;
+  static_assert(4 * 32 * ROWP <= (int)SM::bytes && (32 * CPR) % 64 == 0 && 64 % CPR == 0, "epilogue staging");
+  typedef unsigned int u32v2_t __attribute__((ext_vector_type(2)));
+  __syncthreads();  // every wavefront has read its last fragments
+  uint8_t* ep = smem8 + wave * (32 * ROWP);
+  const int gn0 = n_base + wn * CW;
+  const int gn = gn0 + (lane % CPR) * 4;  // the same 4 columns in every pass: 64 % CPR == 0
+  float4_t cs4 = float4_t{0.f, 0.f, 0.f, 0.f};
+  if (gn < N) cs4 = *reinterpret_cast<const float4_t*>(sb + gn);
+  cs4 *= alpha;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int gm = m_base + wm * (BM / WM) + i * 32 + l32;
-    if (gm >= M) continue;
-    const float row_scale = alpha * sa[gm];
+    const int gm0 = m_base + wm * (BM / WM) + i * 32;
+    const int rows = M - gm0 < 32 ? M - gm0 : 32;
+    const int recs = rows > 0 ? rows * N * 2 : 0;
+    const size_t row0 = (size_t)(rows > 0 ? gm0 : 0);
+    const __amdgpu_buffer_rsrc_t d_rsrc = __builtin_amdgcn_make_buffer_rsrc(D + row0 * N, 0, recs, 0x00020000);
+    const __amdgpu_buffer_rsrc_t s_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sa) + row0, 0, rows > 0 ? rows * 4 : 0, 0x00020000);
+    uint32_t off[ITER];
+    float rs[ITER];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+    for (int it = 0; it < ITER; ++it) {
+      const int r = (it * 64 + lane) / CPR;
+      off[it] = gn < N ? (uint32_t)(r * N + gn) * 2u : kOob;
+      rs[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(s_rsrc, r * 4, 0, 0));
+    }
+    u32v2_t cv[ITER];
+    if (beta != 0.f) {
+      const __amdgpu_buffer_rsrc_t c_rsrc =
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(C) + row0 * N, 0, recs, 0x00020000);
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) cv[it] = __builtin_amdgcn_raw_buffer_load_b64(c_rsrc, off[it], 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const int gn = n_base + wn * (BN / WN) + j * 32 + qd * 8 + lg * 4;
-        if (gn >= N) continue;  // N % 8 == 0 and gn % 4 == 0: the whole quad is in or out
-        const float4_t cs4 = *reinterpret_cast<const float4_t*>(sb + gn);
-        float v[4];
+        float4_t v;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = row_scale * cs4[e] * acc[i][j][qd * 4 + e];
-        if (beta != 0.f) {
-          const u32x2 c = *reinterpret_cast<const u32x2*>(C + (size_t)gm * N + gn);
-          v[0] += beta * h2f_bits(c.x & 0xffffu);
-          v[1] += beta * h2f_bits(c.x >> 16);
-          v[2] += beta * h2f_bits(c.y & 0xffffu);
-          v[3] += beta * h2f_bits(c.y >> 16);
-        }
-        u32x2 o;
-        o.x = f2h_bits(v[0]) | (f2h_bits(v[1]) << 16);
-        o.y = f2h_bits(v[2]) | (f2h_bits(v[3]) << 16);
-        *reinterpret_cast<u32x2*>(D + (size_t)gm * N + gn) = o;
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][qd * 4 + e];
+        *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
+      }
+    float4_t a4[ITER];
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      const int c = it * 64 + lane;
+      a4[it] = *reinterpret_cast<const float4_t*>(ep + (c / CPR) * ROWP + (c % CPR) * 16);
+    }
+    auto store_group = [&](int it, float4_t v) {
+      __builtin_amdgcn_raw_buffer_store_b64(u32v2_t{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3])}, d_rsrc, off[it], 0, 0);
+    };
+    if (beta == 0.f) {
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) store_group(it, a4[it] * cs4 * rs[it]);
+    } else {
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        float4_t v = a4[it] * cs4 * rs[it];
+        v[0] += beta * h2f_bits(cv[it].x & 0xffffu);
+        v[1] += beta * h2f_bits(cv[it].x >> 16);
+        v[2] += beta * h2f_bits(cv[it].y & 0xffffu);
+        v[3] += beta * h2f_bits(cv[it].y >> 16);
+        store_group(it, v);
       }
     }
   }
@@ -319,7 +383,8 @@ int nf_gemm_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, c
   NF_REQUIRE(((uintptr_t)Aq | (uintptr_t)Bq | (uintptr_t)b_scale) % 16 == 0 && ((uintptr_t)D | (uintptr_t)C) % 8 == 0,
              "nf_gemm_f8_f16: Aq, Bq, b_scale must be 16-byte and C, D 8-byte aligned");
   NF_REQUIRE(beta == 0.f || C, "nf_gemm_f8_f16: beta=%g needs C", (double)beta);
-  NF_REQUIRE((size_t)M * K < 0xFFFFFF00ull && (size_t)N * K < 0xFFFFFF00ull,
+  // 32-bit buffer offsets run up to a tile past the last row and a few slabs past K
+  NF_REQUIRE(((size_t)M + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull && ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull,
              "nf_gemm_f8_f16: an operand of %d x %d x %d exceeds the 4 GiB buffer-addressing limit", M, N, K);
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
