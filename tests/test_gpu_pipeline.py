@@ -397,3 +397,34 @@ def test_serve_command_line_writes_the_reference_result_files(tmp_path, online, 
             assert len(l) - n_in in (n_out - 1, n_out) and all(0 <= t < shape.vocab for t in l[n_in:]), (k, l[n_in:])
     if from_file:
         assert os.path.isfile(str(tmp_path / "w" / "weight_rank_0.pt")) and "Loading weights" in r.stdout
+
+
+def test_autosearch_writes_a_tuned_pipeline_config(tmp_path):
+    """nanoflow_amd.autosearch on a tiny model: every candidate is measured, the winner lands in the
+    reference's pipeline_configs / serve_configs fields, and the tuned file configures an engine."""
+    import subprocess, sys, os, json
+    from nanoflow_amd import engine, pllm_python as P
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    cfg = tmp_path / "tiny.json"
+    engine.write_config(str(cfg), shape, global_batch=96, nano1=40, kqv1=20, kqv3=28,
+                        pipeline_type=P.PipelineType.LOCAL, kv_pages=256)
+    out = tmp_path / "tuned.json"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, "-m", "nanoflow_amd.autosearch", "-c", str(cfg), "-o", str(out), "--decode", "20",
+           "--kv-lo", "5", "--kv-hi", "60", "--prefill", "7:30,0:40", "--layers", "2", "--step", "24",
+           "--iters", "3", "--warm", "1", "--cu-masks", "4:4"]
+    r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    t = json.load(open(out))
+    rows = t["search"]["measurements"]
+    kinds = {m["pipeline_type"] for m in rows}
+    assert kinds == {"NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL", "LOCAL"}
+    assert any("gemm_xcds" in m for m in rows)
+    best = min(rows, key=lambda m: m["ms"])
+    pc = t["pipeline_configs"]
+    assert t["serve_configs"]["pipeline_type"] == best["pipeline_type"] and best["ms"] > 0
+    assert (pc["nanobatch_1_size"], pc["kqv1_size"], pc["kqv3_size"]) == \
+        (best["nanobatch_1_size"], best["kqv1_size"], best["kqv3_size"])
+    assert pc["global_batch_size"] == 96 and 0 < pc["kqv1_size"] <= pc["nanobatch_1_size"] < 96
+    assert 0 < pc["kqv3_size"] <= 96 - pc["nanobatch_1_size"]
+    assert t["model"] == json.load(open(cfg))["model"]
