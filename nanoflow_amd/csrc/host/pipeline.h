@@ -243,6 +243,11 @@ public:
   pllmTensor<half> gemvInput, gemvOutput;
   vortexOutputData output_data;
   hipStream_t stream_all = nullptr;
+  // Chunked-prefill attention runs beside decode attention (different requests, disjoint rows):
+  // it is bound by the latency of its longest tile, not by bandwidth, and a prefill workgroup
+  // (32 KB of LDS) fits on a CU next to two decode-attention workgroups.
+  hipStream_t stream_prefill = nullptr;
+  hipEvent_t prefill_fork = nullptr, prefill_join = nullptr;
   int update_token_num = 0;
 
   NonOverlapLocalPipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks);

@@ -1,4 +1,5 @@
-// NonOverlapLocalPipeline: the sequential single-stream schedule (no nano-batching).
+// NonOverlapLocalPipeline: the sequential schedule (no nano-batching), on one stream except that
+// chunked-prefill attention is forked onto a side stream while decode attention runs.
 // The plainest statement of the layer math and the baseline the overlapped schedule must
 // agree with.  Operator order follows the reference's
 // pipeline/src/pipeline_nonoverlap_local.cu:25-62, wiring :245-304, update :108-126,327-385.
@@ -8,6 +9,9 @@ NonOverlapLocalPipeline::NonOverlapLocalPipeline(vortexInitData* input_data, int
                                                  int vnranks)
     : PipelineBase(input_data, nrank, nranks, vnranks) {
   stream_all = createPipelineStream(0, 0);
+  stream_prefill = createPipelineStream(0, 0);
+  HIP_CHECK(hipEventCreateWithFlags(&prefill_fork, hipEventDisableTiming));
+  HIP_CHECK(hipEventCreateWithFlags(&prefill_join, hipEventDisableTiming));
   NF_LOG_INFO("Init pipeline (non-overlap local)");
 }
 
@@ -15,6 +19,9 @@ NonOverlapLocalPipeline::~NonOverlapLocalPipeline() {
   clearGraphs();
   for (auto g : gemms) delete g;
   delete[] output_data.sampled_token_array;
+  if (prefill_fork) (void)hipEventDestroy(prefill_fork);
+  if (prefill_join) (void)hipEventDestroy(prefill_join);
+  if (stream_prefill) (void)hipStreamDestroy(stream_prefill);
   if (stream_all) (void)hipStreamDestroy(stream_all);
 }
 
@@ -43,8 +50,22 @@ vortexOutputData NonOverlapLocalPipeline::run() {
       layerNormAttention.run();
       KQV->run();
       roPEAppend.run();
+      // fork: prefill attention beside decode attention; join before the O projection
+      const bool side = update_data.prefillNum > 0 && GEMV.batch_size > 0;
+      if (side) {
+        HIP_CHECK(hipEventRecord(prefill_fork, stream_all));
+        HIP_CHECK(hipStreamWaitEvent(stream_prefill, prefill_fork, 0));
+        prefill.setStream(stream_prefill);
+        prefill.run();
+        HIP_CHECK(hipEventRecord(prefill_join, stream_prefill));
+      }
       if (GEMV.batch_size > 0) GEMV.run();
-      if (update_data.prefillNum > 0) prefill.run();
+      if (side) {
+        HIP_CHECK(hipStreamWaitEvent(stream_all, prefill_join, 0));
+      } else if (update_data.prefillNum > 0) {
+        prefill.setStream(stream_all);
+        prefill.run();
+      }
       O->run();
       layerNormFFN.run();
       dual.run();

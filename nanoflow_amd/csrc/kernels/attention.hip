@@ -17,6 +17,8 @@
 // concurrently running workgroups stream the same 64 KiB pages.  Prefill: a workgroup is a
 // 16-token tile (for GQA 4) whose wavefronts share the streamed K/V tiles; tiles are planned
 // on the device from qo_indptr (prefix of tiles per request) -- no host round trip in either mode.
+#include <type_traits>
+
 #include "common.h"
 
 namespace nf {
@@ -455,38 +457,52 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
         }
       H8 pf[NQB];
       float alpha[NQB];
+      // Steps that lie wholly below the causal limit of the wavefront's first token (and inside
+      // the sequence) need no masks: most steps of a long chunk.  Same arithmetic either way.
+      const bool unmasked = t_base + 31 <= (causal ? kv_len - qo_len + tok0 : kv_len - 1);
+      auto softmax_step = [&](auto masked_c) {
+        constexpr bool kMasked = decltype(masked_c)::value;
 #pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) {
-        float mx = -1e30f;
-        bool ok[2][4];
+        for (int nb = 0; nb < NQB; ++nb) {
+          float mx = -1e30f;
+          bool ok[2][4];
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
+          for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int t = t_base + blk * 16 + g * 4 + r;
-            ok[blk][r] = t <= key_limit[nb] && t < kv_len;
-            s[nb][blk][r] *= scale_log2;
-            if (ok[blk][r]) mx = fmaxf(mx, s[nb][blk][r]);
-          }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[nb], mx);
-        alpha[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
-        m_run[nb] = m_new;
-        float psum = 0.f;
-        uint32_t pw[4];
+            for (int r = 0; r < 4; ++r) {
+              const int t = t_base + blk * 16 + g * 4 + r;
+              ok[blk][r] = !kMasked || (t <= key_limit[nb] && t < kv_len);
+              s[nb][blk][r] *= scale_log2;
+              if (ok[blk][r]) mx = fmaxf(mx, s[nb][blk][r]);
+            }
+          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          const float m_new = fmaxf(m_run[nb], mx);
+          alpha[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+          m_run[nb] = m_new;
+          float psum = 0.f;
+          uint32_t pw[4];
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
+          for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-          for (int rr = 0; rr < 2; ++rr) {
-            float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr] - m_new) : 0.f;
-            float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr + 1] - m_new) : 0.f;
-            psum += p0 + p1;
-            pw[blk * 2 + rr] = f2h_bits(p0) | (f2h_bits(p1) << 16);
-          }
-        pf[nb].u = u32x4{pw[0], pw[1], pw[2], pw[3]};
-        l_run[nb] = l_run[nb] * alpha[nb] + psum;
-      }
+            for (int rr = 0; rr < 2; ++rr) {
+              float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr] - m_new) : 0.f;
+              float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr + 1] - m_new) : 0.f;
+              psum += p0 + p1;
+              pw[blk * 2 + rr] = pack_f16x2(p0, p1);
+            }
+          pf[nb].u = u32x4{pw[0], pw[1], pw[2], pw[3]};
+          l_run[nb] = l_run[nb] * alpha[nb] + psum;
+        }
+      };
+      if (unmasked) softmax_step(std::false_type{});
+      else softmax_step(std::true_type{});
+      // the running maximum settles after a few steps: rescale the accumulators only when some
+      // column's maximum moved (multiplying by exactly 1 changes nothing)
+      bool moved = false;
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb) moved |= alpha[nb] != 1.0f;
+      const bool rescale = __builtin_amdgcn_ballot_w64(moved) != 0;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const short4_t vlo = lds_read_tr16(vt + vx[i]);
@@ -495,7 +511,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
         const half8_t v8 = __builtin_bit_cast(half8_t, __builtin_shufflevector(vlo, vhi, 0, 1, 2, 3, 4, 5, 6, 7));
 #pragma unroll
         for (int nb = 0; nb < NQB; ++nb) {
-          oacc[nb][i] *= alpha[nb];
+          if (rescale) oacc[nb][i] *= alpha[nb];
           oacc[nb][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v8, pf[nb].h, oacc[nb][i], 0, 0, 0);
         }
       }
