@@ -72,6 +72,10 @@ void init(int nranks, int vnranks, std::vector<vortexInitData>& input,
     std::exit(EXIT_FAILURE);
   }
   Worker::PipeTy = pipeTy;
+  // the update mirrors are sized from the model configuration: callers that follow the
+  // reference's order (mirrors first, configuration second: computeMain.cu:37-38) get them
+  // resized here; a no-op when they already fit
+  TensorManager::getInstance().init(nranks, vnranks);
   aggregated_output.clear();
   outputs.clear();
   global_sync = std::make_unique<SimpleThreadSync>(nranks + 1);

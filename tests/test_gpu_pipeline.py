@@ -428,3 +428,29 @@ def test_autosearch_writes_a_tuned_pipeline_config(tmp_path):
     assert pc["global_batch_size"] == 96 and 0 < pc["kqv1_size"] <= pc["nanobatch_1_size"] < 96
     assert 0 < pc["kqv3_size"] <= 96 - pc["nanobatch_1_size"]
     assert t["model"] == json.load(open(cfg))["model"]
+
+
+@pytest.mark.parametrize("pt_name", ["LOCAL", "NON_OVERLAP_LOCAL"])
+def test_cpp_end_to_end_program_runs_the_reference_sequence(tmp_path, pt_name):
+    """nanoflow_amd/test_compute (C++ API only: createModelWeight, createInitData, readConfigData,
+    createUpdateData, init, config, update, run x N, finalize) on a 2-layer model."""
+    import subprocess, os, re
+    from nanoflow_amd import engine, pllm_python as P
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "nanoflow_amd", "test_compute")
+    assert os.path.isfile(exe), "build the package first (make -C nanoflow_amd/csrc)"
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    cfg = tmp_path / "tiny.json"
+    engine.write_config(str(cfg), shape, global_batch=256, nano1=128, kqv1=64, kqv3=64,
+                        pipeline_type=P.PipelineType[pt_name], kv_pages=16384)
+    r = subprocess.run([exe, str(cfg), "3"], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    head = re.search(r"(\d+) tokens per iteration \((\d+) decode requests, (\d+) prefill requests with (\d+) tokens\)", r.stdout)
+    assert head, r.stdout
+    tokens, nd, npf, pf_tok = (int(x) for x in head.groups())
+    assert tokens == 256 == nd + pf_tok and nd > 0 and npf > 0
+    runs = re.findall(r"run (\d+): ([0-9.]+) ms, (\d+) sampled tokens", r.stdout)
+    assert [int(x[0]) for x in runs] == [0, 1, 2]
+    assert all(int(x[2]) == nd + npf and float(x[1]) > 0 for x in runs)
+    bad = subprocess.run([exe, str(tmp_path / "missing.json")], capture_output=True, text=True, timeout=60)
+    assert bad.returncode != 0
