@@ -123,6 +123,16 @@ NF_PLLM_API int pllm_init(const nf_vortex_init_data* input, int pipeline_type);
 NF_PLLM_API int pllm_model_weight_to_gpu(const nf_vortex_model_weight* host_weight,
                                          nf_vortex_model_weight* device_weight,
                                          nf_vortex_layer_weight* device_layers);
+/* pllm_python.createModelWeight (pybind.cu:228, vortexData.cu:386-406): device memory for every
+ * weight of the configured model (zero-filled here; the reference leaves it as allocated), never
+ * freed.  layers must have room for the model's layer count; *weight points at it. */
+NF_PLLM_API int pllm_create_model_weight(nf_vortex_model_weight* weight, nf_vortex_layer_weight* layers,
+                                         int layers_capacity);
+/* pllm_python.createInitData (pybind.cu:229, vortexData.cu:33-56): the tmp buffer and one zeroed
+ * KV pool per layer for the configured model (never freed) around the given weights.  kv_data
+ * must have room for the model's layer count. */
+NF_PLLM_API int pllm_create_init_data(nf_vortex_init_data* data, uint16_t** kv_data, int layers_capacity,
+                                      const nf_vortex_model_weight* weight);
 /* pllm_python.config (pybind.cu:106-108). */
 NF_PLLM_API int pllm_config(const nf_vortex_config_data* config);
 /* pllm_python.update (pybind.cu:100-104 -> update(), computeBound.cu:115-161). */

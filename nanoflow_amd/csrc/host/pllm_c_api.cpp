@@ -118,6 +118,51 @@ int pllm_init(const nf_vortex_init_data* input, int pipeline_type) {
   return NF_PLLM_OK;
 }
 
+static void layers_to_c(const vortexModelWeight& d, nf_vortex_model_weight* out, nf_vortex_layer_weight* layers) {
+  out->lm_head = to_c(d.lm_head);
+  out->embedding = to_c(d.embedding);
+  out->model_layernorm = to_c(d.model_layernorm);
+  out->num_layers = (int)d.layer_weight.size();
+  out->layer_weight = layers;
+  for (size_t i = 0; i < d.layer_weight.size(); ++i) {
+    const auto& s = d.layer_weight[i];
+    layers[i] = nf_vortex_layer_weight{to_c(s.W_O1), to_c(s.W_O2), to_c(s.W_U), to_c(s.W_G),
+                                       to_c(s.W_D), to_c(s.W_KQV), to_c(s.B_KQV),
+                                       to_c(s.W_LN_Attention), to_c(s.W_LN_FFN), to_c(s.W_ROT)};
+  }
+}
+
+int pllm_create_model_weight(nf_vortex_model_weight* weight, nf_vortex_layer_weight* layers,
+                             int layers_capacity) {
+  if (!g_config_loaded) return fail(NF_PLLM_ERR_STATE, "pllm_create_model_weight: call pllm_set_model_config first");
+  if (!weight || !layers || layers_capacity < ModelConfig.model_layer)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_create_model_weight: room for %d layers needed",
+                ModelConfig.model_layer);
+  vortexModelWeight d;
+  createModelWeight(d, 0);
+  layers_to_c(d, weight, layers);
+  return NF_PLLM_OK;
+}
+
+int pllm_create_init_data(nf_vortex_init_data* data, uint16_t** kv_data, int layers_capacity,
+                          const nf_vortex_model_weight* weight) {
+  if (!g_config_loaded) return fail(NF_PLLM_ERR_STATE, "pllm_create_init_data: call pllm_set_model_config first");
+  if (!data || !kv_data || !weight || layers_capacity < ModelConfig.model_layer)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_create_init_data: room for %d layers needed",
+                ModelConfig.model_layer);
+  vortexInitData d;
+  vortexModelWeight w = to_cpp(*weight);
+  createInitData(d, w, 0);
+  for (int i = 0; i < ModelConfig.model_layer; ++i) kv_data[i] = reinterpret_cast<uint16_t*>(d.kv_data[i]);
+  delete[] d.kv_data;
+  data->kv_data = kv_data;
+  data->weight = *weight;
+  data->weight_size = d.weight_size;
+  data->tmp_buffer = reinterpret_cast<uint16_t*>(d.tmp_buffer);
+  data->tmp_buffer_size = d.tmp_buffer_size;
+  return NF_PLLM_OK;
+}
+
 int pllm_model_weight_to_gpu(const nf_vortex_model_weight* host_weight,
                              nf_vortex_model_weight* device_weight,
                              nf_vortex_layer_weight* device_layers) {
@@ -125,17 +170,7 @@ int pllm_model_weight_to_gpu(const nf_vortex_model_weight* host_weight,
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_model_weight_to_gpu: null pointer");
   vortexModelWeight h = to_cpp(*host_weight);
   vortexModelWeight d = modelWeightToGPU(h, 0);
-  device_weight->lm_head = to_c(d.lm_head);
-  device_weight->embedding = to_c(d.embedding);
-  device_weight->model_layernorm = to_c(d.model_layernorm);
-  device_weight->num_layers = (int)d.layer_weight.size();
-  device_weight->layer_weight = device_layers;
-  for (size_t i = 0; i < d.layer_weight.size(); ++i) {
-    const auto& s = d.layer_weight[i];
-    device_layers[i] = nf_vortex_layer_weight{to_c(s.W_O1), to_c(s.W_O2), to_c(s.W_U), to_c(s.W_G),
-                                              to_c(s.W_D), to_c(s.W_KQV), to_c(s.B_KQV),
-                                              to_c(s.W_LN_Attention), to_c(s.W_LN_FFN), to_c(s.W_ROT)};
-  }
+  layers_to_c(d, device_weight, device_layers);
   return NF_PLLM_OK;
 }
 

@@ -177,7 +177,8 @@ class PipelineTimings(C.Structure):
 
 SYMBOLS = [
     "pllm_last_error", "pllm_set_model_config", "pllm_set_rank", "pllm_tmp_buffer_halves",
-    "pllm_max_page_num", "pllm_init", "pllm_model_weight_to_gpu", "pllm_config", "pllm_update",
+    "pllm_max_page_num", "pllm_init", "pllm_model_weight_to_gpu", "pllm_create_model_weight",
+    "pllm_create_init_data", "pllm_config", "pllm_update",
     "pllm_run", "pllm_run_async", "pllm_run_async_wait", "pllm_get_pipeline_output",
     "pllm_finalize", "pllm_build_input_tokens", "pllm_set_profiling", "pllm_get_timings",
     "pllm_reset_timings", "pllm_debug_buffer", "pllm_set_graph_mode", "pllm_get_graph_counters",
@@ -203,6 +204,9 @@ def lib() -> C.CDLL:
         l.pllm_init.argtypes = [C.POINTER(_CInitData), C.c_int]
         l.pllm_model_weight_to_gpu.argtypes = [C.POINTER(_CModelWeight), C.POINTER(_CModelWeight),
                                                C.POINTER(VortexLayerWeight)]
+        l.pllm_create_model_weight.argtypes = [C.POINTER(_CModelWeight), C.POINTER(VortexLayerWeight), C.c_int]
+        l.pllm_create_init_data.argtypes = [C.POINTER(_CInitData), C.POINTER(C.c_void_p), C.c_int,
+                                            C.POINTER(_CModelWeight)]
         l.pllm_config.argtypes = [C.POINTER(_CConfigData)]
         l.pllm_update.argtypes = [C.POINTER(_CUpdateData)]
         l.pllm_get_pipeline_output.argtypes = [C.POINTER(_i32p), C.POINTER(C.c_int)]
@@ -240,6 +244,37 @@ def tmpBufferHalves() -> int:
 
 def maxPageNum() -> int:
     return lib().pllm_max_page_num()
+
+
+_MAX_LAYERS = 1024
+
+
+def createModelWeight(weight: VortexModelWeight, rank: int = 0):
+    """pllm_python.createModelWeight (pybind.cu:228): device memory for every weight of the configured
+    model; fills ``weight`` in place.  The memory lives until the process ends, as in the reference."""
+    if rank != 0:
+        raise NanoflowPipelineError("this build runs one rank")
+    layers = (VortexLayerWeight * _MAX_LAYERS)()
+    c = _CModelWeight()
+    _check(lib().pllm_create_model_weight(C.byref(c), layers, _MAX_LAYERS), "createModelWeight")
+    weight.lm_head, weight.embedding, weight.model_layernorm = c.lm_head, c.embedding, c.model_layernorm
+    weight.layer_weight = [layers[i] for i in range(c.num_layers)]
+    weight._keep = layers
+
+
+def createInitData(data: "VortexInitData", weight: VortexModelWeight, rank: int = 0):
+    """pllm_python.createInitData (pybind.cu:229): tmp buffer and zeroed per-layer KV pools for the
+    configured model around ``weight``; fills ``data`` in place (never freed, as in the reference)."""
+    if rank != 0:
+        raise NanoflowPipelineError("this build runs one rank")
+    cw, keep = weight._to_c()
+    kv = (C.c_void_p * _MAX_LAYERS)()
+    c = _CInitData()
+    _check(lib().pllm_create_init_data(C.byref(c), kv, _MAX_LAYERS, C.byref(cw)), "createInitData")
+    data.setKVdata([kv[i] for i in range(cw.num_layers)])
+    data.setWeight(weight, c.weight_size)
+    data.setTmpBuffer(c.tmp_buffer, c.tmp_buffer_size)
+    data._keep = (keep, kv)
 
 
 def init(data_array, pipeTy):

@@ -454,3 +454,54 @@ def test_cpp_end_to_end_program_runs_the_reference_sequence(tmp_path, pt_name):
     assert all(int(x[2]) == nd + npf and float(x[1]) > 0 for x in runs)
     bad = subprocess.run([exe, str(tmp_path / "missing.json")], capture_output=True, text=True, timeout=60)
     assert bad.returncode != 0
+
+
+def test_python_builders_follow_the_reference_call_sequence(tmp_path):
+    """setModelConfig -> createModelWeight -> createInitData -> init -> config -> update -> run, the
+    sequence of pipeline/utils/serve_8B.py:609-634,131-141 with --empty_weight: the library allocates
+    weights, tmp buffer and KV pools itself."""
+    from nanoflow_amd import engine, pllm_python as P
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    cfg_path = tmp_path / "tiny.json"
+    engine.write_config(str(cfg_path), shape, global_batch=96, nano1=40, kqv1=20, kqv3=28,
+                        pipeline_type=P.PipelineType.LOCAL, kv_pages=256)
+    P.setRank(1, 1)
+    P.setModelConfig(str(cfg_path))
+    weight = P.VortexModelWeight()
+    P.createModelWeight(weight, 0)
+    assert len(weight.layer_weight) == 2 and weight.lm_head.ptr and weight.layer_weight[1].W_KQV.ptr
+    assert weight.layer_weight[0].W_KQV.N * weight.layer_weight[0].W_KQV.K == shape.hidden * shape.kqv_n
+    data = P.VortexInitData()
+    P.createInitData(data, weight, 0)
+    assert len(data.kv_data) == 2 and all(data.kv_data) and data.tmp_buffer and data.tmp_buffer_size == P.tmpBufferHalves()
+    P.init([data], P.PipelineType.LOCAL)
+    try:
+        c = P.VortexConfigData()
+        c.setGemmOpTag([engine.DEFAULT_TAG] * 7)
+        c.globalBatchSize, c.nanobatch1Size, c.kqv1Size, c.kqv3Size = 96, 40, 20, 28
+        P.config([c])
+        b = synth.make_batch(list(range(5, 25)), [(7, 30), (0, 46)], vocab=shape.vocab, seed=21, extra_pages=40)
+        nd = b.decodePrefillBorder
+        arrs = {k: np.ascontiguousarray(v, dtype=np.int32) for k, v in {
+            "tok": b.input_tokens[nd:], "indptr": b.input_indptr, "rev": b.rev_input_indptr,
+            "off": b.per_token_offset, "kvp": b.kv_indptr, "kvi": b.kv_indices, "kvl": b.kv_last_page_len,
+            "keep": np.ones(nd, np.int32)}.items()}
+        u = P.VortexUpdateData()
+        u.decodePrefillBorder, u.prefillNum, u.prefillTokensNum, u.keepTokenListLength = nd, b.prefillNum, b.prefillTokensNum, nd
+        u.setInputEmbedding(arrs["tok"].ctypes.data)
+        u.setInputIndptr(arrs["indptr"].ctypes.data)
+        u.setRevInputIndptr(arrs["rev"].ctypes.data)
+        u.setPerTokenOffset(arrs["off"].ctypes.data)
+        u.setKVIndptr(arrs["kvp"].ctypes.data)
+        u.setKVIndices(arrs["kvi"].ctypes.data)
+        u.setKVLastPageLen(arrs["kvl"].ctypes.data)
+        u.setKeepTokenList(arrs["keep"].ctypes.data)
+        u.setGemvBatchSize(synth.gemv_batch_split(nd, 20, 40, 28))
+        u.setGemvNumBlocks([0, 0, 0, 0])
+        P.update([u])
+        P.run()
+        out = P.getPipelineOutput()
+        # zero weights: every logit is 0 and the sampler's tie rule picks token 0
+        assert len(out) == nd + b.prefillNum and np.array_equal(out, np.zeros(len(out), np.int32))
+    finally:
+        P.finalize()
