@@ -236,6 +236,9 @@ def run_offline(args):
     assert pages >= 4096, f"not enough free HBM for the KV pool ({free_b / 2**30:.0f} GiB free)"
 
     t_setup = time.perf_counter()
+    # hundreds of timed cycles: two timed layers per cycle are plenty, and the event records and
+    # their collection stay below 0.1 ms of a cycle
+    P.setProfilingStride(16 if steps >= 64 else 0)
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, seed=args.seed,
                         profiling=args.profile_level, kv_fill="zeros")

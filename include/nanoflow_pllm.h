@@ -241,6 +241,10 @@ typedef struct nf_pipeline_timings {
   int layer_stride;  /* every layer_stride-th layer is timed: totals per iteration = sums * layer_stride */
 } nf_pipeline_timings;
 NF_PLLM_API int pllm_set_profiling(int on);
+/* Time every stride-th launch of each operator (0 = automatic: 4 on schedules of 8 or more layers,
+ * else 1).  Takes effect at the next pllm_set_profiling / pllm_init.  pllm_get_timings reports the
+ * stride in use as layer_stride. */
+NF_PLLM_API int pllm_set_profiling_stride(int stride);
 NF_PLLM_API int pllm_get_timings(nf_pipeline_timings* out);
 /* hipGraph replay (the reference carries a graph switch that is compiled off, `constexpr bool
  * enableGraph = false`, pipeline_local.cu:319-327, and only its capture events remain).  With graph mode on, an iteration whose launch signature

@@ -124,6 +124,13 @@ public:
   virtual hipStream_t uploadStream() = 0;
   // level 0: off; 1: attention launches; 2: attention and dense GEMM launches
   virtual void setProfiling(int level) { profiling = level > 0; profile_gemms = level > 1; }
+  // every stride-th launch of an operator is timed: the override, else 4 on schedules of 8 or
+  // more layers (the event records themselves cost device time), else 1
+  static inline int profile_stride_override = 0;
+  static unsigned profileStride() {
+    if (profile_stride_override > 0) return (unsigned)profile_stride_override;
+    return ModelConfig.run_layer >= 8 ? 4u : 1u;
+  }
   int profilingLevel() const { return profiling ? (profile_gemms ? 2 : 1) : 0; }
   const PipelineTimings& getTimings() const { return timings; }
   void resetTimings() {

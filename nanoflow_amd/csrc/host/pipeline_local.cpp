@@ -120,8 +120,7 @@ void LocalPipeline::assignSameStream() {
 void LocalPipeline::setProfiling(int level) {
   profiling = level > 0;
   profile_gemms = level > 1;
-  // long schedules time every 4th layer: the event records themselves cost device time
-  const unsigned stride = ModelConfig.run_layer >= 8 ? 4 : 1;
+  const unsigned stride = profileStride();
   timings.layer_stride = (int)stride;
   const size_t n = profiling ? (size_t)ModelConfig.run_layer : 0;
   for (auto gemv : gemvs) gemv->enableProfiling(n, stride);

@@ -319,6 +319,12 @@ int pllm_build_input_tokens(const int32_t* prev_output, int prev_count, const in
                           prefill_tokens_num, out);
 }
 
+int pllm_set_profiling_stride(int stride) {
+  if (stride < 0) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_set_profiling_stride: %d", stride);
+  PipelineBase::profile_stride_override = stride;
+  return NF_PLLM_OK;
+}
+
 int pllm_set_profiling(int on) {
   setPipelineProfiling(on < 0 ? 0 : on > 2 ? 2 : on);
   return NF_PLLM_OK;

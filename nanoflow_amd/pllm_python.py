@@ -180,7 +180,7 @@ SYMBOLS = [
     "pllm_max_page_num", "pllm_init", "pllm_model_weight_to_gpu", "pllm_create_model_weight",
     "pllm_create_init_data", "pllm_config", "pllm_update",
     "pllm_run", "pllm_run_async", "pllm_run_async_wait", "pllm_get_pipeline_output",
-    "pllm_finalize", "pllm_build_input_tokens", "pllm_set_profiling", "pllm_get_timings",
+    "pllm_finalize", "pllm_build_input_tokens", "pllm_set_profiling", "pllm_set_profiling_stride", "pllm_get_timings",
     "pllm_reset_timings", "pllm_debug_buffer", "pllm_set_graph_mode", "pllm_get_graph_counters",
 ]
 
@@ -340,6 +340,11 @@ def buildInputTokens(prev_output, keep_token_list, prefill_tokens) -> np.ndarray
     if n < 0:
         _check(n, "buildInputTokens")
     return out[:n]
+
+
+def setProfilingStride(stride: int):
+    """Time every stride-th launch of each operator (0 = automatic); call before setProfiling / init."""
+    _check(lib().pllm_set_profiling_stride(int(stride)), "setProfilingStride")
 
 
 def setProfiling(level):
