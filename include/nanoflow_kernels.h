@@ -52,18 +52,27 @@ NF_API int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* wei
 /* D = half(alpha * A.B + beta * C), fp16 operands, fp32 accumulate on MFMA.
  * A [M,K] row-major; B [K,N] row-major when b_col_major == 0, [N,K] row-major
  * (K contiguous) when 1; C and D [M,N] row-major; C may alias D or be NULL when
- * beta == 0.  K % 32 == 0, N % 8 == 0.
+ * beta == 0.  K % 8 == 0, N % 8 == 0.
  * Replaces CutlassGEMMWrapper::work / cutlass::gemm::device::Gemm
  * (pipeline/include/cutlassGemmWrapperImpl.cuh:68-166). */
 NF_API int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
 
 /* out = half(silu(float(half(A.Bgate))) * float(half(A.Bup))); A [M,K], Bgate/Bup [K,N],
- * out [M,N], all row-major.  K % 32 == 0, N % 8 == 0.
+ * out [M,N], all row-major.  K % 8 == 0, N % 8 == 0.
  * Replaces DualWrapper::work / cutlass DualGemm + LeftSiLUAndMul
  * (pipeline/include/dualWrapper.cuh:95-144,192-194). */
 NF_API int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
                        int M, int N, int K, nf_stream_t stream);
+
+/* The same two operators on bfloat16 storage (bf16 x bf16 -> fp32 -> bf16, products rounded to bf16
+ * before SiLU-mul): same kernels, other element type.  The reference's wrappers are fp16 only
+ * (cutlassGemmWrapperImpl.cuh:24-27); these have no counterpart there and the pipeline does not
+ * use them. */
+NF_API int nf_gemm_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
+                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
+NF_API int nf_dual_swiglu_bf16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
+                        int M, int N, int K, nf_stream_t stream);
 
 /* fp8 GEMM family (OCP e4m3: bias 7, no infinities, max 448) on the fp8 matrix cores.  No
  * counterpart in the reference (its GEMM wrappers are half-only,

@@ -1,4 +1,5 @@
-// fp16 x fp16 -> fp32 -> fp16 GEMM family for gfx950 on v_mfma_f32_32x32x16_f16.
+// 16-bit x 16-bit -> fp32 -> 16-bit GEMM family for gfx950 on v_mfma_f32_32x32x16_f16 (fp16, the
+// pipeline's type) and v_mfma_f32_32x32x16_bf16 (bf16: same kernels, other element type).
 //
 //   D = half(alpha * A.B + beta * C)                     (plain; QKV, O, down, LM head)
 //   D = half(silu(half(A.Bg)) * half(A.Bu))              (dual; gate/up SwiGLU)
@@ -53,17 +54,42 @@ struct GemmSmem {
   static constexpr size_t bytes = (size_t)stages * stage_bytes;
 };
 
-// SiLU(g)*u on values already rounded to fp16, as the reference's dual epilogue computes it.
+// Element types of the family: how 16-bit storage is multiplied, widened and rounded.
+struct F16 {
+  static __device__ __forceinline__ float16_t mfma(half8_t b, half8_t a, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(b, a, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float widen(uint32_t bits) { return h2f_bits(bits); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
+  static __device__ __forceinline__ float rounded(float x) { return __half2float(__float2half_rn(x)); }
+};
+struct BF16 {
+  typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ float16_t mfma(half8_t b, half8_t a, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, b), __builtin_bit_cast(bf16x8_t, a), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float widen(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // round to nearest even
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+  }
+  static __device__ __forceinline__ float rounded(float x) { return widen(pack2(x, 0.f) & 0xffffu); }
+};
+
+// SiLU(g)*u on values already rounded to the storage type, as the reference's dual epilogue
+// computes it (in fp16 there).
+template <class E>
 __device__ __forceinline__ float swiglu_rounded(float g_acc, float u_acc) {
-  float g = __half2float(__float2half_rn(g_acc));
-  float u = __half2float(__float2half_rn(u_acc));
+  float g = E::rounded(g_acc);
+  float u = E::rounded(u_acc);
   // hardware reciprocal (1 ulp of fp32): the result is rounded to fp16 afterwards
   return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
 }
 
 // kDual: two weight matrices, SwiGLU epilogue.  kBCol: weights stored [N][K].
 // One BM x BN output tile at (m_base, n_base), computed by the whole workgroup.
-template <int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
+template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 __device__ __forceinline__ void gemm_tile(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
@@ -219,7 +245,7 @@ __device__ __forceinline__ void gemm_tile(
     static_for<NM>([&](auto n_c) {
       constexpr int n = decltype(n_c)::value;
       constexpr int b = n / (TN * TM), j = (n / TM) % TN, i = n % TM;
-      acc[b][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[kk & 1][b][j], af[kk & 1][i], acc[b][i][j], 0, 0, 0);
+      acc[b][i][j] = E::mfma(bf[kk & 1][b][j], af[kk & 1][i], acc[b][i][j]);
       // front-loaded: the step's last reads should have returned when the step ends
       constexpr int PER_ = 0;
       constexpr int lo = n * S / NM, hi = (n + 1) * S / NM;
@@ -342,7 +368,7 @@ __device__ __forceinline__ void gemm_tile(
         float4_t v;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if constexpr (kDual) v[e] = swiglu_rounded(acc[0][i][j][qd * 4 + e], acc[1][i][j][qd * 4 + e]);
+          if constexpr (kDual) v[e] = swiglu_rounded<E>(acc[0][i][j][qd * 4 + e], acc[1][i][j][qd * 4 + e]);
           else v[e] = acc[0][i][j][qd * 4 + e];
         }
         *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
@@ -354,7 +380,7 @@ __device__ __forceinline__ void gemm_tile(
       a4[it] = *reinterpret_cast<const float4_t*>(ep + (c / CPR) * ROWP + (c % CPR) * 16);
     }
     auto store_group = [&](int it, float4_t v) {
-      __builtin_amdgcn_raw_buffer_store_b64(u32v2_t{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3])}, d_rsrc, off[it], 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b64(u32v2_t{E::pack2(v[0], v[1]), E::pack2(v[2], v[3])}, d_rsrc, off[it], 0, 0);
     };
     if (kDual) {
 #pragma unroll
@@ -366,10 +392,10 @@ __device__ __forceinline__ void gemm_tile(
 #pragma unroll
       for (int it = 0; it < ITER; ++it) {
         float4_t v = a4[it] * alpha;
-        v[0] += beta * h2f_bits(cv[it].x & 0xffffu);
-        v[1] += beta * h2f_bits(cv[it].x >> 16);
-        v[2] += beta * h2f_bits(cv[it].y & 0xffffu);
-        v[3] += beta * h2f_bits(cv[it].y >> 16);
+        v[0] += beta * E::widen(cv[it].x & 0xffffu);
+        v[1] += beta * E::widen(cv[it].x >> 16);
+        v[2] += beta * E::widen(cv[it].y & 0xffffu);
+        v[3] += beta * E::widen(cv[it].y >> 16);
         store_group(it, v);
       }
     }
@@ -382,22 +408,22 @@ __device__ __forceinline__ int xcd_order(int bid, int n) {
   return (bid % 8) * ((n + 7) / 8) + bid / 8;
 }
 
-template <int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
+template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 __global__ __launch_bounds__(256) void gemm_f16_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
     int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n) {
   const int logical = xcd_order(blockIdx.x, tiles_m * tiles_n);
   if (logical >= tiles_m * tiles_n) return;
-  gemm_tile<BM, BN, WM, WN, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
-                                           (logical % tiles_m) * BM, (logical / tiles_m) * BN);
+  gemm_tile<E, BM, BN, WM, WN, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
+                                              (logical % tiles_m) * BM, (logical / tiles_m) * BN);
 }
 
 // Two tile heights in one launch, for shapes whose 256-row tiles fill the 256 CUs a whole number
 // of times plus at most half a round: the first n_big tiles (in M-fastest order) are computed
 // 256 rows high, each of the rest as two 128-row halves by two workgroups, so the last round
 // takes half the time instead of leaving half the CUs idle.
-template <int BN, bool kDual, bool kBCol>
+template <class E, int BN, bool kDual, bool kBCol>
 __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
@@ -406,7 +432,7 @@ __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
   if ((int)blockIdx.x < big_grid) {
     const int t = xcd_order(blockIdx.x, n_big);
     if (t >= n_big) return;
-    gemm_tile<256, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
+    gemm_tile<E, 256, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
                                             (t % tiles_m) * 256, (t / tiles_m) * BN);
   } else {
     const int n_small = 2 * (tiles_m * tiles_n - n_big);
@@ -415,17 +441,17 @@ __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
     const int t = n_big + u / 2;
     const int m_base = (t % tiles_m) * 256 + (u & 1) * 128;
     if (m_base >= M) return;
-    gemm_tile<128, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, m_base,
+    gemm_tile<E, 128, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, m_base,
                                             (t / tiles_m) * BN);
   }
 }
 
-template <int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
+template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1, const uint16_t* C,
                        uint16_t* D, int M, int N, int K, float alpha, float beta,
                        hipStream_t stream) {
   using SM = GemmSmem<BM, BN, kDual ? 2 : 1>;
-  auto kern = gemm_f16_kernel<BM, BN, WM, WN, kDual, kBCol>;
+  auto kern = gemm_f16_kernel<E, BM, BN, WM, WN, kDual, kBCol>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -443,13 +469,13 @@ static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1
   return check_launch("gemm launch");
 }
 
-template <int BN, bool kDual, bool kBCol>
+template <class E, int BN, bool kDual, bool kBCol>
 static int launch_hybrid(const uint16_t* A, const uint16_t* B0, const uint16_t* B1, const uint16_t* C,
                          uint16_t* D, int M, int N, int K, float alpha, float beta, int n_big,
                          hipStream_t stream) {
   constexpr size_t big = GemmSmem<256, BN, kDual ? 2 : 1>::bytes, small = GemmSmem<128, BN, kDual ? 2 : 1>::bytes;
   constexpr size_t lds = big > small ? big : small;
-  auto kern = gemm_f16_hybrid_kernel<BN, kDual, kBCol>;
+  auto kern = gemm_f16_hybrid_kernel<E, BN, kDual, kBCol>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -485,10 +511,10 @@ static int cu_count() {
 // candidate wins.  So 192 tiles of 256x256 beat 1.5 rounds of 128x256, and 2048 x 6144 takes
 // 256 tiles of 128x384 rather than 192 of 256x256.  Short M uses a 64-row tile so that padding
 // rows do not dominate.
-template <bool kBCol>
+template <class E, bool kBCol>
 static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
                           int M, int N, int K, float alpha, float beta, hipStream_t s) {
-  if (M <= 64) return launch_gemm<64, 256, 1, 4, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (M <= 64) return launch_gemm<E, 64, 256, 1, 4, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
   const int cus = cu_count();
   auto cost = [&](int bm, int bn, double eff) {
     const long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
@@ -497,10 +523,10 @@ static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* 
   const double c256 = cost(256, 256, 1.0), c384 = cost(128, 384, 0.97), c128x256 = cost(128, 256, 0.95),
                c128 = cost(128, 128, 0.80);
   const double best = std::min(std::min(c256, c384), std::min(c128x256, c128));
-  if (best == c256) return launch_gemm<256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (best == c384) return launch_gemm<128, 384, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (best == c128x256) return launch_gemm<128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  return launch_gemm<128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (best == c256) return launch_gemm<E, 256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (best == c384) return launch_gemm<E, 128, 384, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (best == c128x256) return launch_gemm<E, 128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  return launch_gemm<E, 128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
 }
 
 }  // namespace nf
@@ -522,40 +548,62 @@ static int check_gemm_args(const char* who, const void* A, const void* B, const 
   return NF_OK;
 }
 
-extern "C" {
-
-int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
-                int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
-  int rc = check_gemm_args("nf_gemm_f16", A, B, D, M, N, K);
+template <class E>
+static int gemm_entry(const char* who, const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                      int M, int N, int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
+  int rc = check_gemm_args(who, A, B, D, M, N, K);
   if (rc) return rc;
-  NF_REQUIRE(beta == 0.f || C, "nf_gemm_f16: beta=%g needs C", (double)beta);
-  NF_REQUIRE(((uintptr_t)C) % 8 == 0, "nf_gemm_f16: C must be 8-byte aligned");
+  NF_REQUIRE(beta == 0.f || C, "%s: beta=%g needs C", who, (double)beta);
+  NF_REQUIRE(((uintptr_t)C) % 8 == 0, "%s: C must be 8-byte aligned", who);
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
-  return b_col_major ? dispatch_plain<true>(A, B, C, D, M, N, K, alpha, beta, s)
-                     : dispatch_plain<false>(A, B, C, D, M, N, K, alpha, beta, s);
+  return b_col_major ? dispatch_plain<E, true>(A, B, C, D, M, N, K, alpha, beta, s)
+                     : dispatch_plain<E, false>(A, B, C, D, M, N, K, alpha, beta, s);
 }
 
-int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
-                       int M, int N, int K, nf_stream_t stream) {
-  int rc = check_gemm_args("nf_dual_swiglu_f16", A, Bgate, out, M, N, K);
+template <class E>
+static int dual_entry(const char* who, const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup,
+                      uint16_t* out, int M, int N, int K, nf_stream_t stream) {
+  int rc = check_gemm_args(who, A, Bgate, out, M, N, K);
   if (rc) return rc;
-  NF_REQUIRE(M == 0 || Bup, "nf_dual_swiglu_f16: null pointer");
-  NF_REQUIRE(((uintptr_t)Bup) % 16 == 0, "nf_dual_swiglu_f16: operands must be 16-byte aligned");
+  NF_REQUIRE(M == 0 || Bup, "%s: null pointer", who);
+  NF_REQUIRE(((uintptr_t)Bup) % 16 == 0, "%s: operands must be 16-byte aligned", who);
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
   if (M <= 64)
-    return launch_gemm<64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+    return launch_gemm<E, 64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
   const long long t256 = (long long)((M + 255) / 256) * ((N + 127) / 128);
   const int tail = M % 256;  // rows in the last 256-row tile: half-empty tiles go to the 128-row kernel
   if (t256 >= 192 && (tail == 0 || tail > 128)) {
     const int cus = cu_count();
     const int rest = (int)(t256 % cus);  // tiles of the last, partial round
     if (t256 > cus && rest > 0 && rest <= cus / 2)
-      return launch_hybrid<128, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, (int)(t256 - rest), s);
-    return launch_gemm<256, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+      return launch_hybrid<E, 128, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, (int)(t256 - rest), s);
+    return launch_gemm<E, 256, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
   }
-  return launch_gemm<128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+  return launch_gemm<E, 128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+}
+
+extern "C" {
+
+int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
+                int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
+  return gemm_entry<F16>("nf_gemm_f16", A, B, C, D, M, N, K, alpha, beta, b_col_major, stream);
+}
+
+int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
+                       int M, int N, int K, nf_stream_t stream) {
+  return dual_entry<F16>("nf_dual_swiglu_f16", A, Bgate, Bup, out, M, N, K, stream);
+}
+
+int nf_gemm_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
+                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
+  return gemm_entry<BF16>("nf_gemm_bf16", A, B, C, D, M, N, K, alpha, beta, b_col_major, stream);
+}
+
+int nf_dual_swiglu_bf16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
+                        int M, int N, int K, nf_stream_t stream) {
+  return dual_entry<BF16>("nf_dual_swiglu_bf16", A, Bgate, Bup, out, M, N, K, stream);
 }
 
 }  // extern "C"

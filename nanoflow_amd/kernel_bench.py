@@ -59,6 +59,7 @@ def main():
     ap.add_argument("--kv-hi", type=int, default=1536)
     ap.add_argument("--num-blocks", type=int, default=0, help="attn: cap on resident workgroups (0 = none)")
     ap.add_argument("--mib", type=int, default=1024, help="copy: MiB moved")
+    ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"], help="gemm, dual: element type")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warm", type=int, default=3)
     a = ap.parse_args()
@@ -66,14 +67,15 @@ def main():
     shape = synth.LLAMA3_8B if a.model == "8b" else synth.LLAMA3_70B
     g = torch.Generator(device=DEV).manual_seed(0)
     rnd = lambda *s, std=1.0: torch.empty(s, dtype=torch.float16, device=DEV).normal_(0, std, generator=g)
+    edt = torch.float16 if a.dtype == "f16" else torch.bfloat16   # element type of the gemm / dual operands
 
     if a.op in ("gemm", "gemm_f8"):
         for name, M, N, Kd in layer_shapes(shape, a.m):
             if a.only and name != a.only:
                 continue
-            out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+            out = torch.empty(M, N, dtype=edt if a.op == "gemm" else torch.float16, device=DEV)
             if a.op == "gemm":
-                A, B = rnd(M, Kd), rnd(Kd, N, std=0.02)
+                A, B = rnd(M, Kd).to(edt), rnd(Kd, N, std=0.02).to(edt)
                 fn = lambda: K.gemm(A, B, out=out)
             else:
                 Aq = torch.randint(0, 120, (M, Kd), dtype=torch.uint8, device=DEV)
@@ -83,8 +85,9 @@ def main():
             ms = timeit(fn, a.iters, a.warm)
             print(f"{a.op} {name:8s} {M}x{N}x{Kd}: {ms * 1e3:9.1f} us  {2.0 * M * N * Kd / ms / 1e9:8.1f} TFLOP/s", flush=True)
     elif a.op == "dual":
-        A, Bg, Bu = rnd(a.m, shape.hidden), rnd(shape.hidden, shape.ffn, std=0.02), rnd(shape.hidden, shape.ffn, std=0.02)
-        out = torch.empty(a.m, shape.ffn, dtype=torch.float16, device=DEV)
+        A, Bg, Bu = (t.to(edt) for t in (rnd(a.m, shape.hidden), rnd(shape.hidden, shape.ffn, std=0.02),
+                                         rnd(shape.hidden, shape.ffn, std=0.02)))
+        out = torch.empty(a.m, shape.ffn, dtype=edt, device=DEV)
         ms = timeit(lambda: K.dual_swiglu(A, Bg, Bu, out=out), a.iters, a.warm)
         print(f"dual gate/up {a.m}x{shape.ffn}x{shape.hidden}: {ms * 1e3:9.1f} us  "
               f"{4.0 * a.m * shape.ffn * shape.hidden / ms / 1e9:8.1f} TFLOP/s", flush=True)

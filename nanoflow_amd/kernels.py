@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
 
 SYMBOLS = [
     "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16",
-    "nf_dual_swiglu_f16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
+    "nf_dual_swiglu_f16", "nf_gemm_bf16", "nf_dual_swiglu_bf16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
 ]
@@ -45,6 +45,8 @@ def lib() -> C.CDLL:
         l.nf_rmsnorm_f16.argtypes = [vp, vp, vp, i32, i32, f32, vp]
         l.nf_gemm_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
+        l.nf_gemm_bf16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
+        l.nf_dual_swiglu_bf16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
         l.nf_quantize_rows_e4m3.argtypes = [vp, vp, vp, i32, i32, vp]
         l.nf_gemm_f8_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp]
         l.nf_gemm_f8w_workspace_bytes.restype = C.c_size_t
@@ -103,28 +105,40 @@ def rmsnorm(x, w, eps=1e-5, out=None):
     return out
 
 
+def _elem(t, dtype):
+    assert t.is_cuda and t.dtype == dtype and t.is_contiguous(), (t.dtype, t.device)
+
+
 def gemm(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None):
-    _f16(A); _f16(B)
+    """fp16 operands run nf_gemm_f16, bfloat16 operands nf_gemm_bf16 (same kernels, other element type)."""
+    dt = A.dtype
+    assert dt in (torch.float16, torch.bfloat16), dt
+    _elem(A, dt); _elem(B, dt)
     M, K = A.shape
     N = B.shape[0] if b_col_major else B.shape[1]
     assert tuple(B.shape) == ((N, K) if b_col_major else (K, N)), (A.shape, B.shape)
     if Cmat is not None:
-        _f16(Cmat)
+        _elem(Cmat, dt)
         assert tuple(Cmat.shape) == (M, N)
-    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
-    _check(lib().nf_gemm_f16(_p(A), _p(B), _p(Cmat), _p(out), M, N, K, alpha, beta,
-                             int(b_col_major), _stream()), "nf_gemm_f16")
+    out = torch.empty((M, N), dtype=dt, device=A.device) if out is None else out
+    _elem(out, dt)
+    fn, name = (lib().nf_gemm_f16, "nf_gemm_f16") if dt == torch.float16 else (lib().nf_gemm_bf16, "nf_gemm_bf16")
+    _check(fn(_p(A), _p(B), _p(Cmat), _p(out), M, N, K, alpha, beta, int(b_col_major), _stream()), name)
     return out
 
 
 def dual_swiglu(A, Bg, Bu, out=None):
-    _f16(A); _f16(Bg); _f16(Bu)
+    dt = A.dtype
+    assert dt in (torch.float16, torch.bfloat16), dt
+    _elem(A, dt); _elem(Bg, dt); _elem(Bu, dt)
     M, K = A.shape
     N = Bg.shape[1]
     assert tuple(Bg.shape) == (K, N) and tuple(Bu.shape) == (K, N)
-    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
-    _check(lib().nf_dual_swiglu_f16(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, _stream()),
-           "nf_dual_swiglu_f16")
+    out = torch.empty((M, N), dtype=dt, device=A.device) if out is None else out
+    _elem(out, dt)
+    fn, name = (lib().nf_dual_swiglu_f16, "nf_dual_swiglu_f16") if dt == torch.float16 else \
+        (lib().nf_dual_swiglu_bf16, "nf_dual_swiglu_bf16")
+    _check(fn(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, _stream()), name)
     return out
 
 

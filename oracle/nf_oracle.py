@@ -157,6 +157,37 @@ def dual_swiglu(A, Bg, Bu, return_parts=False):
     return (out, d0, d1) if return_parts else out
 
 
+# ---- bfloat16 variants of the two GEMM operators.  The reference has no bf16 path (its GEMM
+# wrappers are half only, pipeline/include/cutlassGemmWrapperImpl.cuh:24-27): PARITY UNPINNED
+# against the reference; these are the closed forms D = bf16(alpha*A.B + beta*C) and
+# bf16(silu(bf16(A.Bg)) * bf16(A.Bu)) in float64, on uint16 bit patterns.
+def bf16_to_float(bits: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def float_to_bf16(x: np.ndarray) -> np.ndarray:
+    """Round to nearest, ties to even, on the fp32 bit pattern (finite inputs)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    return u.astype(np.uint16)
+
+
+def gemm_bf16(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False):
+    a = bf16_to_float(A).astype(np.float64)
+    b = bf16_to_float(B).astype(np.float64)
+    d = alpha * (a @ (b.T if b_col_major else b))
+    if Cmat is not None and beta != 0.0:
+        d = d + beta * bf16_to_float(Cmat).astype(np.float64)
+    return float_to_bf16(d.astype(np.float32))
+
+
+def dual_swiglu_bf16(A, Bg, Bu):
+    a = bf16_to_float(A).astype(np.float64)
+    g = bf16_to_float(float_to_bf16((a @ bf16_to_float(Bg).astype(np.float64)).astype(np.float32))).astype(np.float64)
+    u = bf16_to_float(float_to_bf16((a @ bf16_to_float(Bu).astype(np.float64)).astype(np.float32))).astype(np.float64)
+    return float_to_bf16((g / (1.0 + np.exp(-g)) * u).astype(np.float32))
+
+
 def gemm_f8w(A, Bq, scale, Cmat=None, alpha=1.0, beta=0.0):
     M, K = A.shape
     N = Bq.shape[1]

@@ -158,6 +158,57 @@ def test_dual_known_answer_inputs(K, oracle):
     assert_close(host(K.dual_swiglu(dev(X), dev(X), dev(X))), oracle.dual_swiglu(X, X, X), what="dual KAT")
 
 
+# ---------------------------------------------------------------- bf16 variants of the GEMM family
+
+BF16_RTOL = 8e-3   # one bf16 ulp (2^-8 = 3.9e-3 relative) either side of the float64 closed form
+
+
+def _bf16_dev(bits):
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).cuda().view(torch.bfloat16)
+
+
+def _bf16_host(t):
+    torch.cuda.synchronize()
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("M,N,K_", [(64, 512, 256), (33, 136, 200), (300, 384, 320), (2048, 6144, 256), (1408, 6144, 512)])
+def test_gemm_bf16(K, oracle, M, N, K_):
+    rng = np.random.default_rng(31)
+    A = oracle.float_to_bf16(rng.standard_normal((M, K_), dtype=np.float32))
+    B = oracle.float_to_bf16(rng.standard_normal((K_, N), dtype=np.float32) * 0.05)
+    Cm = oracle.float_to_bf16(rng.standard_normal((M, N), dtype=np.float32))
+    got = _bf16_host(K.gemm(_bf16_dev(A), _bf16_dev(B)))
+    assert_close(oracle.bf16_to_float(got), oracle.bf16_to_float(oracle.gemm_bf16(A, B)), BF16_RTOL, "gemm bf16")
+    got = _bf16_host(K.gemm(_bf16_dev(A), _bf16_dev(B), _bf16_dev(Cm), alpha=0.5, beta=1.0))
+    assert_close(oracle.bf16_to_float(got), oracle.bf16_to_float(oracle.gemm_bf16(A, B, Cm, 0.5, 1.0)), BF16_RTOL,
+                 "gemm bf16 beta=1")
+    Bt = np.ascontiguousarray(B.T)
+    got_t = _bf16_host(K.gemm(_bf16_dev(A), _bf16_dev(Bt), b_col_major=True))
+    assert_close(oracle.bf16_to_float(got_t), oracle.bf16_to_float(oracle.gemm_bf16(A, B)), BF16_RTOL, "gemm bf16 col-major B")
+
+
+def test_gemm_bf16_exact_on_small_integers(K, oracle):
+    rng = np.random.default_rng(32)
+    A = rng.integers(-4, 5, (130, 64)).astype(np.float32)
+    B = rng.integers(-4, 5, (64, 264)).astype(np.float32)
+    got = oracle.bf16_to_float(_bf16_host(K.gemm(_bf16_dev(oracle.float_to_bf16(A)), _bf16_dev(oracle.float_to_bf16(B)))))
+    assert np.array_equal(got, oracle.bf16_to_float(oracle.float_to_bf16(A @ B)))
+
+
+@pytest.mark.parametrize("M,N,K_", [(5, 136, 72), (200, 512, 256), (2048, 14336, 128)])
+def test_dual_swiglu_bf16(K, oracle, M, N, K_):
+    rng = np.random.default_rng(33)
+    A = oracle.float_to_bf16(rng.standard_normal((M, K_), dtype=np.float32))
+    Bg = oracle.float_to_bf16(rng.standard_normal((K_, N), dtype=np.float32) * 0.04)
+    Bu = oracle.float_to_bf16(rng.standard_normal((K_, N), dtype=np.float32) * 0.04)
+    got = _bf16_host(K.dual_swiglu(_bf16_dev(A), _bf16_dev(Bg), _bf16_dev(Bu)))
+    # the two products are rounded to bf16 before SiLU-mul: a product that lands on the other side
+    # of a rounding boundary moves the result by up to two ulps
+    assert_close(oracle.bf16_to_float(got), oracle.bf16_to_float(oracle.dual_swiglu_bf16(A, Bg, Bu)), 2 * BF16_RTOL,
+                 "dual swiglu bf16")
+
+
 # ---------------------------------------------------------------- RoPE + paged append
 
 F8_RTOL = 3e-2   # fp8 path: activations rounded to e4m3 (3 mantissa bits) on the way in

@@ -559,3 +559,33 @@ def test_decoder_forward_vs_independent_float64_model(oracle):
     for l in range(shape.layers):
         diff = (pools[l] != pools_in[l]).any(axis=(1, 3, 4))
         assert diff.sum() == b.tokens
+
+
+# ---------------------------------------------------------------- bf16 helpers of the oracle
+
+def test_bf16_conversions_agree_with_torch_and_round_to_even():
+    torch = pytest.importorskip("torch")
+    from oracle import nf_oracle as O
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(20000) * np.exp(rng.uniform(-20, 20, 20000))).astype(np.float32)
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(O.float_to_bf16(x), want)
+    assert np.array_equal(O.bf16_to_float(want), torch.from_numpy(want.view(np.int16)).view(torch.bfloat16).float().numpy())
+    # ties: 1 + 2^-8 lies halfway between 1 and 1 + 2^-7 -> even (1.0); 1 + 3*2^-8 -> 1 + 2^-6
+    assert O.bf16_to_float(O.float_to_bf16(np.array([1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8], np.float32))).tolist() == [1.0, 1 + 2.0 ** -6]
+
+
+def test_bf16_gemm_closed_form_on_exact_inputs():
+    from oracle import nf_oracle as O
+    # small integers are exact in bf16 and so are their dot products: the result is the integer matmul
+    rng = np.random.default_rng(12)
+    A = rng.integers(-4, 5, (9, 16)).astype(np.float32)
+    B = rng.integers(-4, 5, (16, 24)).astype(np.float32)
+    got = O.bf16_to_float(O.gemm_bf16(O.float_to_bf16(A), O.float_to_bf16(B)))
+    assert np.array_equal(got, A @ B)
+    Cm = rng.integers(-3, 4, (9, 24)).astype(np.float32)
+    got = O.bf16_to_float(O.gemm_bf16(O.float_to_bf16(A), O.float_to_bf16(B), O.float_to_bf16(Cm), 0.5, 2.0))
+    assert np.array_equal(got, O.bf16_to_float(O.float_to_bf16((0.5 * (A @ B) + 2.0 * Cm).astype(np.float32))))
+    Bt = np.ascontiguousarray(B.T)
+    assert np.array_equal(O.gemm_bf16(O.float_to_bf16(A), O.float_to_bf16(Bt), b_col_major=True),
+                          O.gemm_bf16(O.float_to_bf16(A), O.float_to_bf16(B)))
