@@ -44,9 +44,9 @@
  *   (oracle/nf_oracle.py) gemm_bf16, dual_swiglu_bf16
  *                           PARITY UNPINNED against the reference (no bf16 path there);
  *                           float64 closed forms, conversions checked against torch's.
- *   (oracle/scheduler_oracle.py) the scheduler restatement: integer formulas pinned by
- *                           hand-derived cases; admission order over long traces PARITY
- *                           UNPINNED (no fixture in the reference; see that file's header).
+ *   (oracle/scheduler_oracle.py) the scheduler restatement: pinned by hand-derived cases and by
+ *                           per-cycle fixtures written from the reference's own scheduler
+ *                           (tests/golden/); see that file's header.
  */
 #include <math.h>
 #include <stdint.h>

@@ -13,10 +13,11 @@ One stated freedom: which free page is handed out.  The reference pops from a Py
 and re-issues the most recently freed page first -- the same rule as the C++ former, so the
 two can be compared bit for bit.
 
-Parity status: the integer formulas are pinned by hand-derived cases in
-tests/test_batch_former.py; the admission order over long traces has no fixture in the
-reference (its scheduler only runs against the compiled extension), so beyond those cases and
-the invariants checked there it is "parity unpinned" against the reference itself.
+Parity status: pinned.  The integer formulas by hand-derived cases in tests/test_batch_former.py;
+the behaviour over whole traces (admission order, chunked prefill, decode order, group split, free
+pages, retirements per cycle) by tests/golden/scheduler_trace_*.json, which
+tests/golden/make_scheduler_fixtures.py wrote by running the reference's own Scheduler in its
+skip-cycle mode (tests/test_scheduler_fixtures.py).  Page ids are outside the fixtures.
 """
 from __future__ import annotations
 
