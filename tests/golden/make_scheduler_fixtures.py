@@ -103,6 +103,10 @@ def run_trace(mods, name, requests, capacity, T, nano1, kqv1, kqv3, cycles):
                 "gemv": list(sch._gemv_batch_size),
                 "free": pool.num_free_pages,
                 "retired": [r.req_idx for r in retired[n_ret:]],
+                # the keep list this cycle leaves for the next update (serve_8B.py:527-560): how many
+                # slots of this iteration's output it covers, and which of them decode again
+                "ktl": sch._old_token_length,
+                "kcrc": zlib.crc32(",".join(str(i) for i, v in enumerate(sch.pinned_keep_token_list.tolist()) if v).encode()),
             }
             if len(out) % 16 == 0:
                 rec["decode"] = dec_ids

@@ -20,6 +20,15 @@ def _crc(ids):
     return zlib.crc32(",".join(map(str, ids)).encode())
 
 
+def _check_keep(c, prev, keep_len, keep_list):
+    """The keep list handed to update c is what cycle c-1 of the reference left behind."""
+    if prev is None:
+        return
+    assert keep_len == prev["ktl"], (c, "keepTokenListLength", keep_len, prev["ktl"])
+    ones = [i for i, v in enumerate(list(keep_list)[:keep_len]) if v]
+    assert _crc(ones) == prev["kcrc"], (c, "keep list", ones[:8])
+
+
 def _check_cycle(c, want, nd, dec_ids, prefill, gemv, free, retired):
     assert nd == want["nd"], (c, "decode rows", nd, want["nd"])
     assert _crc(dec_ids) == want["dcrc"], (c, "decode order", dec_ids[:8])
@@ -42,9 +51,12 @@ def test_python_restatement_follows_the_reference_scheduler(path):
                      t["kqv3_size"], t["avg_prefill"], t["avg_decode"])
     for i, (n_in, n_out) in enumerate(t["requests"]):
         s.add_request(i, [i] * n_in, n_out)
+    prev = None
     for c, want in enumerate(t["cycles"]):
         s.schedule()
         b = s.form()
+        _check_keep(c, prev, b["keepTokenListLength"], b["keep_token_list"])
+        prev = want
         dec_ids = [r.req_idx for r in s.decode]
         nd = b["decodePrefillBorder"]
         ind = b["input_indptr"]
@@ -67,9 +79,12 @@ def test_cpp_batch_former_follows_the_reference_scheduler(path):
         for i, (n_in, n_out) in enumerate(t["requests"]):
             f.add_request(i, np.full(n_in, i, np.int32), n_out)      # the prompt's tokens name the request
         owner = {}                                                   # first KV page -> request
+        prev = None
         for c, want in enumerate(t["cycles"]):
             f.schedule()
             b = f.form()
+            _check_keep(c, prev, b["keepTokenListLength"], b["keep_token_list"])
+            prev = want
             nd, ind, kvp, kvi = b["decodePrefillBorder"], b["input_indptr"], b["kv_indptr"], b["kv_indices"]
             prefill = []
             for j in range(b["prefillNum"]):
