@@ -122,3 +122,29 @@ def test_shape_mismatch_and_foreign_files_raise(tmp_path):
     torch.save({"something": torch.zeros(3)}, str(tmp_path / "other.pt"))
     with pytest.raises(ValueError, match="not a pipeline weight file"):
         W.load_weight_file(str(tmp_path / "other.pt"))
+
+
+# ---- against the reference's own converter -------------------------------------------------
+# tests/golden/weight_file_checksums.json holds names, shapes, dtypes and SHA-256 of the tensors
+# that save_weights of pipeline/utils/weightSaver.py wrote for the synthetic checkpoint built by
+# tests/golden/make_weight_fixture.py:build_checkpoint (the script that produced the file).
+
+def _golden():
+    import importlib.util
+    here = os.path.join(os.path.dirname(__file__), "golden")
+    spec = importlib.util.spec_from_file_location("make_weight_fixture", os.path.join(here, "make_weight_fixture.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod, json.load(open(os.path.join(here, "weight_file_checksums.json")))
+
+
+@pytest.mark.parametrize("case,bias", [("plain", False), ("qkv_bias", True)])
+def test_converted_file_is_the_reference_converters_file(tmp_path, case, bias):
+    mod, want = _golden()
+    hf, out = str(tmp_path / "hf"), str(tmp_path / "w")
+    mod.build_checkpoint(hf, bias)
+    path = W.convert_hf_checkpoint(hf, out)
+    got = mod.describe(path)
+    assert sorted(got) == sorted(want[case])
+    for name in want[case]:
+        assert got[name] == want[case][name], name        # shape, dtype and every byte
