@@ -115,7 +115,28 @@ def _attention_roofline(tm, bytes_per_launch, name="roofline"):
     }
 
 
-def _gemm_roofline(tm):
+# Memory-side bytes per dense GEMM launch over algorithmic bytes (operands once + output), measured
+# with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernels at M = 2048 (LM head: 684 rows) and
+# scaled by the copy-kernel calibration: profiles/gemm_hbm_traffic_pmc.txt.  The activations are
+# fetched once per XCD; most of the repeats hit the Infinity Cache.
+GEMM_TRAFFIC_RATIO = 2.66
+
+
+def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows):
+    """fp16 operands once plus outputs (and the residual operand of O and down) of one cycle's dense
+    GEMMs, averaged over its launches (4 per layer + the LM head)."""
+    H, F, V = shape.hidden, shape.ffn, shape.vocab
+    hq = shape.Hq * shape.d
+    per_layer = (rows * H + H * shape.kqv_n + rows * shape.kqv_n            # QKV
+                 + rows * hq + hq * H + 2 * rows * H                         # O (+ C)
+                 + rows * H + 2 * H * F + rows * F                           # gate/up
+                 + rows * F + F * H + 2 * rows * H)                          # down (+ C)
+    m_lm = (sampled_rows + 127) // 128 * 128
+    total = 2 * (shape.layers * per_layer + m_lm * H + H * V + m_lm * V)
+    return total / (4 * shape.layers + 1)
+
+
+def _gemm_roofline(tm, alg_bytes_per_launch=None):
     n = max(tm.gemm_launches, 1)
     avg_ms = tm.gemm_ms / n
     flop_per_launch = tm.gemm_flop / n
@@ -123,7 +144,9 @@ def _gemm_roofline(tm):
     return {
         "kernel": "gemm_f16_kernel / dual_swiglu_f16_kernel (all dense GEMM launches of the iteration)",
         "bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-        "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+        "frac": achieved / MFMA_PEAK_TFLOPS,
+        "traffic": None if alg_bytes_per_launch is None else alg_bytes_per_launch * GEMM_TRAFFIC_RATIO,
+        "algorithmic_bytes_per_launch": alg_bytes_per_launch,
         "algorithmic_flop_per_launch": flop_per_launch, "avg_launch_ms": avg_ms,
         "launches_timed": int(tm.gemm_launches),
     }
@@ -299,7 +322,8 @@ def run_offline(args):
                               "dense_rows_processed / 1535 * 1536 / wall_s (fewer than 200 retirements in the window)"),
             "baseline": "12756 tokens/s/GPU published by the reference for this workload on 1x A100 80GB",
         },
-        "roofline": _gemm_roofline(tm) if tm.gemm_launches else _attention_roofline(
+        "roofline": _gemm_roofline(tm, _gemm_algorithmic_bytes_per_launch(
+            shape, nd + int(nxt["prefillTokensNum"]), nd + int(nxt["prefillNum"]))) if tm.gemm_launches else _attention_roofline(
             tm, bytes_per_layer / launches_per_layer),
         "serving": {
             "cycles": st.cycles, "retired_requests": st.retired, "wall_s": st.wall_s,
