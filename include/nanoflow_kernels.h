@@ -58,6 +58,14 @@ NF_API int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* wei
 NF_API int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
 
+/* D = half(alpha * A.B + beta * bias[n]): nf_gemm_f16 with one row, bias [N], added to every row
+ * of the product, read in the epilogue instead of from an [M,N] copy of it.
+ * Replaces the QKV GEMM of the *_KQVBIAS pipelines, whose C operand is the bias replicated over
+ * max-batch rows by replicateKQVBias (pipeline/src/small_cuda_operator.cu:254-292; used at
+ * pipeline/src/pipeline.cu:520-533,1048-1058, pipeline_nonoverlap.cu:163-168,209-211). */
+NF_API int nf_gemm_bias_f16(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M,
+                     int N, int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
+
 /* out = half(silu(float(half(A.Bgate))) * float(half(A.Bup))); A [M,K], Bgate/Bup [K,N],
  * out [M,N], all row-major.  K % 8 == 0, N % 8 == 0.
  * Replaces DualWrapper::work / cutlass DualGemm + LeftSiLUAndMul

@@ -36,6 +36,9 @@ enum nf_pipeline_type {
   NF_PIPE_NONOVERLAP = 1,
   NF_PIPE_NANOBATCH = 2,
   NF_PIPE_PLLMOFFLOAD = 3,
+  /* models with a bias on the q/k/v projections (Qwen2; pipeline/src/computeBound.cu:234-242):
+   * on this one device they run as LOCAL / NON_OVERLAP_LOCAL / NANOBATCH_LOCAL with
+   * vortexLayerWeight::B_KQV added by the QKV GEMMs */
   NF_PIPE_KQVBIAS = 4,
   NF_PIPE_NONOVERLAP_KQVBIAS = 5,
   NF_PIPE_NANOBATCH_KQVBIAS = 6,

@@ -63,7 +63,7 @@ void init(int nranks, int vnranks, std::vector<vortexInitData>& input,
   if (!Worker::isSupported(pipeTy)) {
     std::fprintf(stderr,
                  "init: pipeline type %d is a tensor-parallel schedule; this build implements LOCAL, "
-                 "NON_OVERLAP_LOCAL and NANOBATCH_LOCAL\n",
+                 "NON_OVERLAP_LOCAL, NANOBATCH_LOCAL and, as those with a QKV bias, the three *_KQVBIAS types\n",
                  static_cast<int>(pipeTy));
     std::exit(EXIT_FAILURE);
   }
@@ -152,11 +152,19 @@ void Worker::as_thread(int core) {
 
 void Worker::init() {
   HIP_CHECK(hipSetDevice(rank));
+  // The *_KQVBIAS types name the tensor-parallel pipelines with a QKV bias
+  // (pipeline/src/computeBound.cu:234-242); on one device, with no exchange steps left, they are
+  // the local schedules with the bias switched on.
   if (PipeTy == PipelineType::LOCAL || PipeTy == PipelineType::NANOBATCH_LOCAL)
     pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks,
                                                PipeTy == PipelineType::NANOBATCH_LOCAL);
   else if (PipeTy == PipelineType::NON_OVERLAP_LOCAL)
     pipeline = std::make_unique<NonOverlapLocalPipeline>(input, rank, nranks, vnranks);
+  else if ((PipeTy == PipelineType::KQVBIAS || PipeTy == PipelineType::NANOBATCH_KQVBIAS) && nranks == 1)
+    pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks,
+                                               PipeTy == PipelineType::NANOBATCH_KQVBIAS, true);
+  else if (PipeTy == PipelineType::NONOVERLAP_KQVBIAS && nranks == 1)
+    pipeline = std::make_unique<NonOverlapLocalPipeline>(input, rank, nranks, vnranks, true);
   else
     NF_LOG_ERROR("Unknown pipeline type %d", static_cast<int>(PipeTy));
   if (pipeline && g_profiling) pipeline->setProfiling(g_profiling);

@@ -61,7 +61,15 @@ public:
   static PipelineType PipeTy;
   static bool isSupported(PipelineType t) {
     return t == PipelineType::LOCAL || t == PipelineType::NON_OVERLAP_LOCAL ||
-           t == PipelineType::NANOBATCH_LOCAL;
+           t == PipelineType::NANOBATCH_LOCAL || hasKQVBias(t);
+  }
+  // the three bias types run as the local schedules with the QKV bias switched on
+  static bool hasKQVBias(PipelineType t) {
+    return t == PipelineType::KQVBIAS || t == PipelineType::NONOVERLAP_KQVBIAS ||
+           t == PipelineType::NANOBATCH_KQVBIAS;
+  }
+  static bool isSequential(PipelineType t) {
+    return t == PipelineType::NON_OVERLAP_LOCAL || t == PipelineType::NONOVERLAP_KQVBIAS;
   }
 
 private:

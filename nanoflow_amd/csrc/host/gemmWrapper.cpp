@@ -42,6 +42,12 @@ BaseGEMMWrapper* generateGEMM(const std::string& tag) {
 }
 
 void HipGEMMWrapper::work() {
+  if (c_is_row) {
+    NF_KERNEL_CHECK(nf_gemm_bias_f16(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
+                                     pllm_tensor_d.ptr, (int)M, (int)N, (int)K, alpha, beta,
+                                     tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, stream));
+    return;
+  }
   NF_KERNEL_CHECK(nf_gemm_f16(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
                               pllm_tensor_d.ptr, (int)M, (int)N, (int)K, alpha, beta,
                               tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, stream));
@@ -99,7 +105,7 @@ bool HipGEMMWrapper::checkResult() {
     ref *= alpha;
     uint16_t c16 = 0, d16 = 0;
     if (beta != 0.f) {
-      HIP_CHECK(hipMemcpy(&c16, pllm_tensor_c.ptr + m * N + n, 2, hipMemcpyDeviceToHost));
+      HIP_CHECK(hipMemcpy(&c16, pllm_tensor_c.ptr + (c_is_row ? 0 : m * N) + n, 2, hipMemcpyDeviceToHost));
       ref += beta * half_bits_to_float(c16);
     }
     HIP_CHECK(hipMemcpy(&d16, pllm_tensor_d.ptr + m * N + n, 2, hipMemcpyDeviceToHost));

@@ -50,6 +50,10 @@ struct BaseGEMMWrapper : public OperatorWrapper {
   virtual pllmTensor<ElementOutput> getC() = 0;
   virtual void set_alpha(float alpha_) = 0;
   virtual void set_beta(float beta_) = 0;
+  // Not in the reference's interface: C = one row [1, N] added (times beta) to every row of the
+  // product, read by the kernel's epilogue.  Takes the place of setC() with the bias replicated
+  // over max-batch rows (replicateKQVBias, pipeline/src/pipeline.cu:520-533,1048-1058).
+  virtual BaseGEMMWrapper& setCRow(pllmTensor<ElementOutput> row) = 0;
 };
 
 struct GemmTag {
@@ -65,6 +69,7 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   pllmTensor<half> pllm_tensor_a, pllm_tensor_b, pllm_tensor_c, pllm_tensor_d;
   float alpha = 1.f, beta = 0.f;
   bool inited = false;
+  bool c_is_row = false;  // pllm_tensor_c is a [1, N] row added to every row
 
   explicit HipGEMMWrapper(const GemmTag& t) : tag(t) {}
 
@@ -83,6 +88,13 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   HipGEMMWrapper& setC(pllmTensor<half> c) override {
     assert(c.layout == PllmLayout::ROW_MAJOR && c.dim1 == M && c.dim2 == N);
     pllm_tensor_c = c;
+    c_is_row = false;
+    return *this;
+  }
+  HipGEMMWrapper& setCRow(pllmTensor<half> row) override {
+    assert(row.dim1 == 1 && row.dim2 == N);
+    pllm_tensor_c = row;
+    c_is_row = true;
     return *this;
   }
   HipGEMMWrapper& setD(pllmTensor<half> d) override {

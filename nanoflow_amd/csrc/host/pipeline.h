@@ -59,6 +59,19 @@ protected:
   bool profiling = false;
   bool profile_gemms = false;
   PipelineTimings timings;
+  // The *_KQVBIAS pipeline types (models whose q/k/v projections have a bias, Qwen2): the QKV
+  // GEMMs add vortexLayerWeight::B_KQV ([1, kqv_n], columns K|V|Q) to every row, beta = 1
+  // (pipeline/src/pipeline.cu:520-533, pipeline_nonoverlap.cu:209-211).
+  bool kqv_bias = false;
+  bool bindKQVBias(BaseGEMMWrapper* kqv, vortexWeight& bias) {
+    if (!kqv_bias) return true;
+    if (!bias.ptr || bias.size() != kqv->N) {
+      std::fprintf(stderr, "KQV bias size mismatch  %zu %zu\n", bias.size(), kqv->N);
+      return false;
+    }
+    kqv->setCRow(pllmTensor<half>(bias.ptr, 1, (int)kqv->N, PllmLayout::ROW_MAJOR));
+    return true;
+  }
 
   // hipGraph replay of an iteration.  Everything that shapes a launch (grid sizes, row counts,
   // which operators are skipped) is a function of the configuration and of a few integers of
@@ -199,7 +212,7 @@ public:
   bool nanobatch_only = false;
 
   LocalPipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks,
-                bool nanobatch_only = false);
+                bool nanobatch_only = false, bool kqv_bias = false);
   ~LocalPipeline() override;
   void ScheduleInit();
   void GEMMOpInit();
@@ -257,7 +270,8 @@ public:
   hipEvent_t prefill_fork = nullptr, prefill_join = nullptr;
   int update_token_num = 0;
 
-  NonOverlapLocalPipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks);
+  NonOverlapLocalPipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks,
+                          bool kqv_bias = false);
   ~NonOverlapLocalPipeline() override;
   void ScheduleInit();
   void GEMMOpInit();

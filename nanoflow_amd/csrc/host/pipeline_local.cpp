@@ -52,8 +52,9 @@ hipStream_t createPipelineStream(int first_cu, int num_cus) {
 }
 
 LocalPipeline::LocalPipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks,
-                             bool nanobatch_only)
+                             bool nanobatch_only, bool kqv_bias_)
     : PipelineBase(input_data, nrank, nranks, vnranks), nanobatch_only(nanobatch_only) {
+  kqv_bias = kqv_bias_;
   init();
 }
 
@@ -142,6 +143,8 @@ void LocalPipeline::setWeight(int layer) {
   success &= D2->set_weight(lw.W_D);
   success &= KQV1->set_weight(lw.W_KQV);
   success &= KQV2->set_weight(lw.W_KQV);
+  success &= bindKQVBias(KQV1, lw.B_KQV);
+  success &= bindKQVBias(KQV2, lw.B_KQV);
   success &= layerNormAttention1.setWeight(lw.W_LN_Attention);
   success &= layerNormAttention2.setWeight(lw.W_LN_Attention);
   success &= layerNormFFN1.setWeight(lw.W_LN_FFN);
@@ -184,6 +187,8 @@ void LocalPipeline::setWeight_group_LN(int layer) {
   success &= layerNormAttention2.setWeight(lw.W_LN_Attention);
   success &= KQV1->set_weight(lw.W_KQV);
   success &= KQV2->set_weight(lw.W_KQV);
+  success &= bindKQVBias(KQV1, lw.B_KQV);
+  success &= bindKQVBias(KQV2, lw.B_KQV);
   if (!success) NF_LOG_ERROR("Failed to set weight group 2 for layer %d", layer);
   roPEAppends[0].setKVData(input_data->kv_data[layer]);
   roPEAppends[1].setKVData(input_data->kv_data[layer]);
@@ -195,8 +200,8 @@ void LocalPipeline::GEMMOpInit() {
   O2->init(1.f);
   D1->init(1.f);
   D2->init(1.f);
-  KQV1->init();
-  KQV2->init();
+  KQV1->init(kqv_bias ? 1.f : 0.f);
+  KQV2->init(kqv_bias ? 1.f : 0.f);
   LOGITS->set_weight(input_data->weight.lm_head);
   LOGITS->init();
   for (int i = 0; i < gemmNum; ++i) {

@@ -6,8 +6,9 @@
 #include "pipeline.h"
 
 NonOverlapLocalPipeline::NonOverlapLocalPipeline(vortexInitData* input_data, int nrank, int nranks,
-                                                 int vnranks)
+                                                 int vnranks, bool kqv_bias_)
     : PipelineBase(input_data, nrank, nranks, vnranks) {
+  kqv_bias = kqv_bias_;
   stream_all = createPipelineStream(0, 0);
   stream_prefill = createPipelineStream(0, 0);
   HIP_CHECK(hipEventCreateWithFlags(&prefill_fork, hipEventDisableTiming));
@@ -179,6 +180,7 @@ void NonOverlapLocalPipeline::setWeight(int layer) {
   success &= O->set_weight(lw.W_O1);
   success &= D->set_weight(lw.W_D);
   success &= KQV->set_weight(lw.W_KQV);
+  success &= bindKQVBias(KQV, lw.B_KQV);
   success &= layerNormAttention.setWeight(lw.W_LN_Attention);
   success &= layerNormFFN.setWeight(lw.W_LN_FFN);
   success &= dual.set_weight(lw.W_G, lw.W_U);
@@ -230,7 +232,7 @@ void NonOverlapLocalPipeline::GEMMOpInit() {
   O->init(1.f);
   dual.init();
   D->init(1.f);
-  KQV->init();
+  KQV->init(kqv_bias ? 1.f : 0.f);
   // one stream, nobody waits on an operator: no start / end events (each record is a packet
   // between two kernels)
   for (int i = 0; i < gemmNum; ++i) {

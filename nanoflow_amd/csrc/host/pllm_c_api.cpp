@@ -94,10 +94,19 @@ int pllm_init(const nf_vortex_init_data* input, int pipeline_type) {
   if (!Worker::isSupported(ty))
     return fail(NF_PLLM_ERR_UNSUPPORTED,
                 "pllm_init: pipeline type %d is a tensor-parallel schedule; LOCAL(7), "
-                "NON_OVERLAP_LOCAL(8) and NANOBATCH_LOCAL(9) are implemented", pipeline_type);
+                "NON_OVERLAP_LOCAL(8), NANOBATCH_LOCAL(9) and, as those with a QKV bias, KQVBIAS(4), "
+                "NONOVERLAP_KQVBIAS(5), NANOBATCH_KQVBIAS(6) are implemented", pipeline_type);
   if (input->weight.num_layers < ModelConfig.model_layer)
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_init: %d layers of weights, model has %d",
                 input->weight.num_layers, ModelConfig.model_layer);
+  if (Worker::hasKQVBias(ty))
+    for (int i = 0; i < ModelConfig.model_layer; ++i) {
+      const nf_vortex_weight& b = input->weight.layer_weight[i].B_KQV;
+      if (!b.ptr || (size_t)b.N * (size_t)b.K != (size_t)ModelConfig.kqv_n)
+        return fail(NF_PLLM_ERR_INVALID_ARGUMENT,
+                    "pllm_init: pipeline type %d adds a QKV bias; layer %d has B_KQV %d x %d, wants %d elements",
+                    pipeline_type, i, b.N, b.K, ModelConfig.kqv_n);
+    }
   vortexInitData d;
   d.kv_data = new half*[ModelConfig.model_layer];
   for (int i = 0; i < ModelConfig.model_layer; ++i) {
@@ -178,7 +187,7 @@ int pllm_config(const nf_vortex_config_data* c) {
   if (!g_inited) return fail(NF_PLLM_ERR_STATE, "pllm_config: call pllm_init first");
   if (g_configured) return fail(NF_PLLM_ERR_STATE, "pllm_config: already configured");
   if (!c) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: null config");
-  const bool local = Worker::PipeTy != Worker::PipelineType::NON_OVERLAP_LOCAL;
+  const bool local = !Worker::isSequential(Worker::PipeTy);
   if (c->global_batch_size <= 0 || c->global_batch_size > ModelConfig.max_batch_size)
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: global_batch_size %d not in (0, %d]",
                 c->global_batch_size, ModelConfig.max_batch_size);
@@ -235,7 +244,7 @@ int pllm_update(const nf_vortex_update_data* u) {
   if (gsum != u->decodePrefillBorder)
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: gemv_batch_size sums to %d, decode requests %d",
                 gsum, u->decodePrefillBorder);
-  if (Worker::PipeTy != Worker::PipelineType::NON_OVERLAP_LOCAL) {
+  if (!Worker::isSequential(Worker::PipeTy)) {
     // decode groups 0 and 1 are the decode rows of nano-batch 1, groups 2 and 3 those of
     // nano-batch 2 (the O projection of nano-batch 1 waits for groups 0/1 only)
     const int want = std::min(u->decodePrefillBorder, g_cfg[0].nanobatch_1_size);

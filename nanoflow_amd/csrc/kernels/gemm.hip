@@ -93,7 +93,7 @@ template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 __device__ __forceinline__ void gemm_tile(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
-    int M, int N, int K, float alpha, float beta, const int m_base, const int n_base) {
+    int M, int N, int K, float alpha, float beta, const int ldc, const int m_base, const int n_base) {
   constexpr int NB = kDual ? 2 : 1;
   using SM = GemmSmem<BM, BN, NB>;
   constexpr int TM = BM / WM / 32;  // MFMA tiles per wave along M
@@ -355,10 +355,17 @@ __device__ __forceinline__ void gemm_tile(
     u32v2_t cv[ITER];
     if constexpr (!kDual) {
       if (beta != 0.f) {  // issued first: the longest latency of the pass
-        const __amdgpu_buffer_rsrc_t c_rsrc =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(C) + row0, 0, recs, 0x00020000);
+        // C has row stride ldc (N, or 0 when one row is added to every row of the product):
+        // the D offset less the row's share of the difference
+        const int c_recs = rows > 0 ? ((rows - 1) * ldc + N) * 2 : 0;
+        const uint32_t c_skip = (uint32_t)(N - ldc) * 2u;
+        const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(C) + (size_t)(rows > 0 ? gm0 : 0) * ldc, 0, c_recs, 0x00020000);
 #pragma unroll
-        for (int it = 0; it < ITER; ++it) cv[it] = __builtin_amdgcn_raw_buffer_load_b64(c_rsrc, off[it], 0, 0);
+        for (int it = 0; it < ITER; ++it) {
+          const uint32_t r = (uint32_t)((it * 64 + lane) / CPR);
+          cv[it] = __builtin_amdgcn_raw_buffer_load_b64(c_rsrc, off[it] == kOob ? kOob : off[it] - r * c_skip, 0, 0);
+        }
       }
     }
 #pragma unroll
@@ -412,10 +419,10 @@ template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 __global__ __launch_bounds__(256) void gemm_f16_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
-    int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n) {
+    int M, int N, int K, float alpha, float beta, int ldc, int tiles_m, int tiles_n) {
   const int logical = xcd_order(blockIdx.x, tiles_m * tiles_n);
   if (logical >= tiles_m * tiles_n) return;
-  gemm_tile<E, BM, BN, WM, WN, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
+  gemm_tile<E, BM, BN, WM, WN, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc,
                                               (logical % tiles_m) * BM, (logical / tiles_m) * BN);
 }
 
@@ -427,12 +434,12 @@ template <class E, int BN, bool kDual, bool kBCol>
 __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
-    int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n, int n_big) {
+    int M, int N, int K, float alpha, float beta, int ldc, int tiles_m, int tiles_n, int n_big) {
   const int big_grid = (n_big + 7) / 8 * 8;
   if ((int)blockIdx.x < big_grid) {
     const int t = xcd_order(blockIdx.x, n_big);
     if (t >= n_big) return;
-    gemm_tile<E, 256, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta,
+    gemm_tile<E, 256, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc,
                                             (t % tiles_m) * 256, (t / tiles_m) * BN);
   } else {
     const int n_small = 2 * (tiles_m * tiles_n - n_big);
@@ -441,14 +448,14 @@ __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
     const int t = n_big + u / 2;
     const int m_base = (t % tiles_m) * 256 + (u & 1) * 128;
     if (m_base >= M) return;
-    gemm_tile<E, 128, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, m_base,
+    gemm_tile<E, 128, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc, m_base,
                                             (t / tiles_m) * BN);
   }
 }
 
 template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1, const uint16_t* C,
-                       uint16_t* D, int M, int N, int K, float alpha, float beta,
+                       uint16_t* D, int M, int N, int K, float alpha, float beta, int ldc,
                        hipStream_t stream) {
   using SM = GemmSmem<BM, BN, kDual ? 2 : 1>;
   auto kern = gemm_f16_kernel<E, BM, BN, WM, WN, kDual, kBCol>;
@@ -465,13 +472,13 @@ static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int ntiles = tiles_m * tiles_n;
   const int grid = ((ntiles + 7) / 8) * 8;
-  kern<<<grid, 256, SM::bytes, stream>>>(A, B0, B1, C, D, M, N, K, alpha, beta, tiles_m, tiles_n);
+  kern<<<grid, 256, SM::bytes, stream>>>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc, tiles_m, tiles_n);
   return check_launch("gemm launch");
 }
 
 template <class E, int BN, bool kDual, bool kBCol>
 static int launch_hybrid(const uint16_t* A, const uint16_t* B0, const uint16_t* B1, const uint16_t* C,
-                         uint16_t* D, int M, int N, int K, float alpha, float beta, int n_big,
+                         uint16_t* D, int M, int N, int K, float alpha, float beta, int ldc, int n_big,
                          hipStream_t stream) {
   constexpr size_t big = GemmSmem<256, BN, kDual ? 2 : 1>::bytes, small = GemmSmem<128, BN, kDual ? 2 : 1>::bytes;
   constexpr size_t lds = big > small ? big : small;
@@ -489,7 +496,7 @@ static int launch_hybrid(const uint16_t* A, const uint16_t* B0, const uint16_t* 
   const int tiles_m = (M + 255) / 256, tiles_n = (N + BN - 1) / BN;
   const int n_small = 2 * (tiles_m * tiles_n - n_big);
   const int grid = (n_big + 7) / 8 * 8 + (n_small + 7) / 8 * 8;
-  kern<<<grid, 256, lds, stream>>>(A, B0, B1, C, D, M, N, K, alpha, beta, tiles_m, tiles_n, n_big);
+  kern<<<grid, 256, lds, stream>>>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc, tiles_m, tiles_n, n_big);
   return check_launch("gemm launch");
 }
 
@@ -513,8 +520,8 @@ static int cu_count() {
 // rows do not dominate.
 template <class E, bool kBCol>
 static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
-                          int M, int N, int K, float alpha, float beta, hipStream_t s) {
-  if (M <= 64) return launch_gemm<E, 64, 256, 1, 4, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+                          int M, int N, int K, float alpha, float beta, int ldc, hipStream_t s) {
+  if (M <= 64) return launch_gemm<E, 64, 256, 1, 4, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
   const int cus = cu_count();
   auto cost = [&](int bm, int bn, double eff) {
     const long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
@@ -523,10 +530,10 @@ static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* 
   const double c256 = cost(256, 256, 1.0), c384 = cost(128, 384, 0.97), c128x256 = cost(128, 256, 0.95),
                c128 = cost(128, 128, 0.80);
   const double best = std::min(std::min(c256, c384), std::min(c128x256, c128));
-  if (best == c256) return launch_gemm<E, 256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (best == c384) return launch_gemm<E, 128, 384, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  if (best == c128x256) return launch_gemm<E, 128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
-  return launch_gemm<E, 128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, s);
+  if (best == c256) return launch_gemm<E, 256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
+  if (best == c384) return launch_gemm<E, 128, 384, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
+  if (best == c128x256) return launch_gemm<E, 128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
+  return launch_gemm<E, 128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
 }
 
 }  // namespace nf
@@ -550,15 +557,17 @@ static int check_gemm_args(const char* who, const void* A, const void* B, const 
 
 template <class E>
 static int gemm_entry(const char* who, const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
-                      int M, int N, int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
+                      int M, int N, int K, float alpha, float beta, int b_col_major, nf_stream_t stream,
+                      bool c_is_row = false) {
   int rc = check_gemm_args(who, A, B, D, M, N, K);
   if (rc) return rc;
   NF_REQUIRE(beta == 0.f || C, "%s: beta=%g needs C", who, (double)beta);
   NF_REQUIRE(((uintptr_t)C) % 8 == 0, "%s: C must be 8-byte aligned", who);
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
-  return b_col_major ? dispatch_plain<E, true>(A, B, C, D, M, N, K, alpha, beta, s)
-                     : dispatch_plain<E, false>(A, B, C, D, M, N, K, alpha, beta, s);
+  const int ldc = c_is_row ? 0 : N;  // row stride of C: 0 reads the same row for every m
+  return b_col_major ? dispatch_plain<E, true>(A, B, C, D, M, N, K, alpha, beta, ldc, s)
+                     : dispatch_plain<E, false>(A, B, C, D, M, N, K, alpha, beta, ldc, s);
 }
 
 template <class E>
@@ -571,17 +580,17 @@ static int dual_entry(const char* who, const uint16_t* A, const uint16_t* Bgate,
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
   if (M <= 64)
-    return launch_gemm<E, 64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+    return launch_gemm<E, 64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
   const long long t256 = (long long)((M + 255) / 256) * ((N + 127) / 128);
   const int tail = M % 256;  // rows in the last 256-row tile: half-empty tiles go to the 128-row kernel
   if (t256 >= 192 && (tail == 0 || tail > 128)) {
     const int cus = cu_count();
     const int rest = (int)(t256 % cus);  // tiles of the last, partial round
     if (t256 > cus && rest > 0 && rest <= cus / 2)
-      return launch_hybrid<E, 128, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, (int)(t256 - rest), s);
-    return launch_gemm<E, 256, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+      return launch_hybrid<E, 128, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, (int)(t256 - rest), s);
+    return launch_gemm<E, 256, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
   }
-  return launch_gemm<E, 128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, s);
+  return launch_gemm<E, 128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
 }
 
 extern "C" {
@@ -589,6 +598,12 @@ extern "C" {
 int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
   return gemm_entry<F16>("nf_gemm_f16", A, B, C, D, M, N, K, alpha, beta, b_col_major, stream);
+}
+
+int nf_gemm_bias_f16(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M,
+                     int N, int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
+  NF_REQUIRE(bias, "nf_gemm_bias_f16: null bias");
+  return gemm_entry<F16>("nf_gemm_bias_f16", A, B, bias, D, M, N, K, alpha, beta, b_col_major, stream, true);
 }
 
 int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,

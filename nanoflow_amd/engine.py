@@ -73,7 +73,7 @@ class Engine:
         self.dev = torch.device("cuda:0")
         fd, self.cfg_path = tempfile.mkstemp(suffix=".json", prefix="nanoflow_cfg_")
         os.close(fd)
-        n_tags = 4 if pipeline_type == P.PipelineType.NON_OVERLAP_LOCAL else 7
+        n_tags = 4 if pipeline_type.is_sequential else 7
         write_config(self.cfg_path, shape, global_batch=global_batch, nano1=nano1, kqv1=self.kqv1,
                      kqv3=self.kqv3, pipeline_type=pipeline_type, kv_pages=kv_pages,
                      run_layer=run_layer, distinct_layers=distinct_layers, n_tags=n_tags)
@@ -111,6 +111,10 @@ class Engine:
             lw.W_G = _weight(lt["w_gate"], F, H)
             lw.W_D = _weight(lt["w_down"], H, F)
             lw.W_KQV = _weight(lt["w_kqv"], kqv_n, H)
+            if pipeline_type.has_kqv_bias:
+                # biases of real checkpoints (Qwen2) reach tens in a few channels; N(0, 0.5) here
+                lt["b_kqv"] = mk("b_kqv", l, 1, kqv_n, 0.5)
+                lw.B_KQV = _weight(lt["b_kqv"], kqv_n, 1)
             lw.W_LN_Attention = _weight(lt["ln_attn"], H, 1)
             lw.W_LN_FFN = _weight(lt["ln_ffn"], H, 1)
             mw.layer_weight.append(lw)
@@ -178,7 +182,7 @@ class Engine:
         u.setKVLastPageLen(arrs["kv_last"].ctypes.data)
         u.setKeepTokenList(arrs["keep"].ctypes.data)
         u.setGemvBatchSize(synth.gemv_batch_split(nd, self.kqv1, self.nano1, self.kqv3)
-                           if self.pipeline_type != P.PipelineType.NON_OVERLAP_LOCAL else [nd, 0, 0, 0])
+                           if not self.pipeline_type.is_sequential else [nd, 0, 0, 0])
         u.setGemvNumBlocks(list(num_blocks))
         self._hold = (arrs, u)
         P.update([u])

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
 
 SYMBOLS = [
-    "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16",
+    "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16", "nf_gemm_bias_f16",
     "nf_dual_swiglu_f16", "nf_gemm_bf16", "nf_dual_swiglu_bf16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
@@ -44,6 +44,7 @@ def lib() -> C.CDLL:
         l.nf_embedding_f16.argtypes = [vp, vp, vp, i32, i32, vp]
         l.nf_rmsnorm_f16.argtypes = [vp, vp, vp, i32, i32, f32, vp]
         l.nf_gemm_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
+        l.nf_gemm_bias_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
         l.nf_gemm_bf16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_dual_swiglu_bf16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
@@ -109,14 +110,23 @@ def _elem(t, dtype):
     assert t.is_cuda and t.dtype == dtype and t.is_contiguous(), (t.dtype, t.device)
 
 
-def gemm(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None):
-    """fp16 operands run nf_gemm_f16, bfloat16 operands nf_gemm_bf16 (same kernels, other element type)."""
+def gemm(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, bias=None):
+    """fp16 operands run nf_gemm_f16, bfloat16 operands nf_gemm_bf16 (same kernels, other element type).
+    bias [N] (fp16 only, instead of Cmat): beta * bias is added to every row (nf_gemm_bias_f16)."""
     dt = A.dtype
     assert dt in (torch.float16, torch.bfloat16), dt
     _elem(A, dt); _elem(B, dt)
     M, K = A.shape
     N = B.shape[0] if b_col_major else B.shape[1]
     assert tuple(B.shape) == ((N, K) if b_col_major else (K, N)), (A.shape, B.shape)
+    if bias is not None:
+        assert Cmat is None and dt == torch.float16 and bias.numel() == N
+        _elem(bias, dt)
+        out = torch.empty((M, N), dtype=dt, device=A.device) if out is None else out
+        _elem(out, dt)
+        _check(lib().nf_gemm_bias_f16(_p(A), _p(B), _p(bias), _p(out), M, N, K, alpha, beta, int(b_col_major),
+                                      _stream()), "nf_gemm_bias_f16")
+        return out
     if Cmat is not None:
         _elem(Cmat, dt)
         assert tuple(Cmat.shape) == (M, N)

@@ -40,6 +40,17 @@ class PipelineType(enum.IntEnum):
     NON_OVERLAP_LOCAL = 8
     NANOBATCH_LOCAL = 9
 
+    @property
+    def has_kqv_bias(self) -> bool:
+        """The three bias types (pipeline/src/computeBound.cu:234-242) run on this one device as
+        LOCAL / NON_OVERLAP_LOCAL / NANOBATCH_LOCAL with B_KQV added by the QKV GEMMs."""
+        return self in (PipelineType.KQVBIAS, PipelineType.NONOVERLAP_KQVBIAS, PipelineType.NANOBATCH_KQVBIAS)
+
+    @property
+    def is_sequential(self) -> bool:
+        """One stream, no nano-batch split: four GEMM tags, one decode-attention group."""
+        return self in (PipelineType.NON_OVERLAP_LOCAL, PipelineType.NONOVERLAP_KQVBIAS)
+
 
 class VortexWeight(C.Structure):
     _fields_ = [("ptr", C.c_void_p), ("N", C.c_int), ("K", C.c_int)]

@@ -8,7 +8,8 @@ reference's pipeline/utils/serve_8B.py:
   per request; a request of input_len n gets the prompt 0, 1, ..., n-1 as in the reference.
   Rows with input_len -1 (prompt text to tokenize) are rejected: no tokenizer ships here.
 * config: the reference's pipeline JSON (pipeline/config_all/llama3-8B/1024.json schema);
-  ``serve_configs.pipeline_type`` must be LOCAL, NON_OVERLAP_LOCAL or NANOBATCH_LOCAL.
+  ``serve_configs.pipeline_type`` must be LOCAL, NON_OVERLAP_LOCAL or NANOBATCH_LOCAL, or, for models with a
+  bias on the q/k/v projections (Qwen2), KQVBIAS, NONOVERLAP_KQVBIAS or NANOBATCH_KQVBIAS.
 * ``--empty_weight True``: random-init weights on the device, as the reference's own evaluation
   runs (pipeline/eval/eval-fix-offline/run.py:42-50).  Otherwise the weights come from
   ``serve_configs.weight_path``/weight_rank_0.pt (nanoflow_amd/weights.py; serve_8B.py:611-629);
@@ -100,7 +101,7 @@ def main():
             W.convert_hf_checkpoint(hf, wdir)
         print("Loading weights")
         t0 = time.perf_counter()
-        weights = W.load_weight_file(wdir, shape)
+        weights = W.load_weight_file(wdir, shape, kqv_bias=pt.has_kqv_bias)
         print("Time taken to load weights: ", time.perf_counter() - t0)
 
     reqs = read_trace(a.trace_path)

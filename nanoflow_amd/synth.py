@@ -56,9 +56,10 @@ def normal_f16(rng: np.random.Generator, shape, std: float = 1.0, mean: float = 
     return (rng.standard_normal(shape, dtype=np.float32) * std + mean).astype(np.float16)
 
 
-def make_weights(shape: ModelShape, seed: int = 0, layers: int | None = None) -> dict:
+def make_weights(shape: ModelShape, seed: int = 0, layers: int | None = None, kqv_bias: bool = False) -> dict:
     """fp16 N(0, 0.02) weights in the reference's orientation (K x N row-major,
-    KQV columns ordered K | V | Q; pipeline/utils/weightSaver.py:89-149)."""
+    KQV columns ordered K | V | Q; pipeline/utils/weightSaver.py:89-149).  kqv_bias adds the
+    k | v | q bias rows of the bias pipelines, N(0, 0.5), drawn after everything else."""
     rng = np.random.default_rng(seed)
     L = shape.layers if layers is None else layers
     w = {
@@ -75,6 +76,8 @@ def make_weights(shape: ModelShape, seed: int = 0, layers: int | None = None) ->
         w["w_down"].append(normal_f16(rng, (shape.ffn, shape.hidden), 0.02))
         w["ln_attn"].append(normal_f16(rng, (shape.hidden,), 0.02, 1.0))
         w["ln_ffn"].append(normal_f16(rng, (shape.hidden,), 0.02, 1.0))
+    if kqv_bias:
+        w["b_kqv"] = [normal_f16(rng, (shape.kqv_n,), 0.5) for _ in range(L)]
     return w
 
 

@@ -25,9 +25,9 @@ Two steps, as in the reference:
   (with the loader that executes nothing from the file) and returns the dict ``engine.Engine`` takes
   as ``weights=``: fp16 numpy arrays, per-layer entries as lists.
 
-The single-device pipelines have no KQV bias path (the reference's LocalPipeline never reads B_KQV:
-pipeline/src/pipeline_local.cu:862-867); a file with a non-zero BKQV_l is rejected instead of being
-served wrongly.
+BKQV_l is read only for the *_KQVBIAS pipeline types (the reference's LocalPipeline never reads
+B_KQV: pipeline/src/pipeline_local.cu:862-867; its bias pipelines do, pipeline.cu:1048-1058); for
+the other types a file with a non-zero BKQV_l is rejected instead of being served wrongly.
 
     python -m nanoflow_amd.weights --hf_path HF_SNAPSHOT_DIR --weight_path OUT_DIR
 """
@@ -118,9 +118,11 @@ def convert_hf_checkpoint(hf_dir: str, weight_dir: str) -> str:
     return path
 
 
-def load_weight_file(weight_dir: str, shape: synth.ModelShape | None = None) -> dict:
+def load_weight_file(weight_dir: str, shape: synth.ModelShape | None = None, kqv_bias: bool = False) -> dict:
     """``weight_dir/weight_rank_0.pt`` -> the ``weights=`` dict of engine.Engine.  With ``shape`` given,
-    every tensor's shape is checked against it and a mismatch raises ValueError."""
+    every tensor's shape is checked against it and a mismatch raises ValueError.  ``kqv_bias``: the
+    pipeline type adds BKQV_l (one of the *_KQVBIAS types); without it a file whose biases are not
+    all zero is refused, since serving it would silently drop them."""
     path = weight_dir if weight_dir.endswith(".pt") else os.path.join(weight_dir, FILE_NAME)
     sd = torch.load(path, map_location="cpu", weights_only=True)
     layer_ids = [int(m.group(1)) for m in (re.match(r"^D_(\d+)$", k) for k in sd) if m]
@@ -131,8 +133,13 @@ def load_weight_file(weight_dir: str, shape: synth.ModelShape | None = None) -> 
     w = {"embedding": np16(sd["Embed"]), "lm_head": np16(sd["LmHead"]), "model_norm": np16(sd["ModelNorm"]).reshape(-1),
          "w_kqv": [], "w_o": [], "w_gate": [], "w_up": [], "w_down": [], "ln_attn": [], "ln_ffn": []}
     for l in range(L):
-        if f"BKQV_{l}" in sd and bool(torch.any(sd[f"BKQV_{l}"] != 0)):
-            raise ValueError(f"{path}: layer {l} has a non-zero KQV bias; the single-device pipelines have no bias path")
+        if kqv_bias:
+            if f"BKQV_{l}" not in sd:
+                raise ValueError(f"{path}: no BKQV_{l}: the pipeline type adds a KQV bias")
+            w.setdefault("b_kqv", []).append(np16(sd[f"BKQV_{l}"]).reshape(-1))
+        elif f"BKQV_{l}" in sd and bool(torch.any(sd[f"BKQV_{l}"] != 0)):
+            raise ValueError(f"{path}: layer {l} has a non-zero KQV bias; serve this model with KQVBIAS, "
+                             "NONOVERLAP_KQVBIAS or NANOBATCH_KQVBIAS as serve_configs.pipeline_type")
         w["w_kqv"].append(np16(sd[f"KQV_{l}"]))
         w["w_o"].append(np16(sd[f"O1_{l}"]))
         w["w_gate"].append(np16(sd[f"G_{l}"]))
@@ -146,6 +153,8 @@ def load_weight_file(weight_dir: str, shape: synth.ModelShape | None = None) -> 
         per_layer = {"w_kqv": (shape.hidden, shape.kqv_n), "w_o": (shape.Hq * shape.d, shape.hidden),
                      "w_gate": (shape.hidden, shape.ffn), "w_up": (shape.hidden, shape.ffn),
                      "w_down": (shape.ffn, shape.hidden), "ln_attn": (shape.hidden,), "ln_ffn": (shape.hidden,)}
+        if kqv_bias:
+            per_layer["b_kqv"] = (shape.kqv_n,)
         if L < shape.layers:
             raise ValueError(f"{path}: {L} layers, the model configuration asks for {shape.layers}")
         for k, s in want.items():

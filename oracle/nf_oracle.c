@@ -571,6 +571,7 @@ typedef struct {
   const uint16_t* const* ln_attn;  /* [hidden] */
   const uint16_t* const* ln_ffn;   /* [hidden] */
   uint16_t* const* kv_data;        /* per-layer paged pools (read and appended) */
+  const uint16_t* const* b_kqv;    /* NULL, or per layer [(Hq+2Hkv)*d]: bias of the K|V|Q columns */
 } nfo_model;
 
 typedef struct {
@@ -589,6 +590,10 @@ typedef struct {
  *  residual stream x lives in the D output; O adds x (beta 1), D adds the O output
  *  (beta 1); final norm after KeepToken; LOGITS rows padded to 128 are not computed
  *  here because padding rows never reach the sampler].
+ * With b_kqv (the *_KQVBIAS pipeline types) the QKV GEMM gets, as its C operand with beta 1, the
+ * layer's bias row copied into every one of the T rows
+ * [pipeline/src/pipeline.cu:1048-1058 replicateKQVBias, :520-533 setC, :202 init(1);
+ *  pipeline_nonoverlap.cu:163-168,209-211,406].
  * hidden_in (optional, [T,hidden]) replaces the embedding lookup when not NULL.
  * Outputs: hidden_out (optional, [T,hidden]) = residual stream after the last layer;
  * logits (optional, [req,vocab]); sampled [req]. */
@@ -600,6 +605,7 @@ NFO_API void nfo_decoder_forward(const nfo_model* m, const nfo_batch* b, const u
   uint16_t* x = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)T * H);
   uint16_t* xn = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)T * H);
   uint16_t* kqv = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)T * kqv_n);
+  uint16_t* bias_rows = m->b_kqv ? (uint16_t*)malloc(sizeof(uint16_t) * (size_t)T * kqv_n) : NULL;
   uint16_t* qb = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)T * qd);
   uint16_t* ao = (uint16_t*)calloc((size_t)T * qd, sizeof(uint16_t));
   uint16_t* xo = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)T * H);
@@ -610,7 +616,12 @@ NFO_API void nfo_decoder_forward(const nfo_model* m, const nfo_batch* b, const u
     nfo_embedding_f16(b->input_tokens, m->embedding, x, T, H);
   for (int l = 0; l < m->layers; ++l) {
     nfo_rmsnorm_f16(xn, x, m->ln_attn[l], T, H, m->eps);
-    nfo_gemm_f16(xn, m->w_kqv[l], NULL, kqv, T, kqv_n, H, 1.f, 0.f, 0);
+    if (m->b_kqv) {
+      for (int t = 0; t < T; ++t) memcpy(bias_rows + (size_t)t * kqv_n, m->b_kqv[l], sizeof(uint16_t) * kqv_n);
+      nfo_gemm_f16(xn, m->w_kqv[l], bias_rows, kqv, T, kqv_n, H, 1.f, 1.f, 0);
+    } else {
+      nfo_gemm_f16(xn, m->w_kqv[l], NULL, kqv, T, kqv_n, H, 1.f, 0.f, 0);
+    }
     nfo_rope_append_f16(kqv, qb, m->kv_data[l], b->kv_indices, b->kv_indptr, b->rev_input_indptr,
                         b->per_token_offset, T, m->Hq, m->Hkv, m->d, m->page_size, m->rope_scale,
                         m->rope_theta, m->smooth_a, m->smooth_b, NULL, NULL);
@@ -646,6 +657,7 @@ NFO_API void nfo_decoder_forward(const nfo_model* m, const nfo_batch* b, const u
   free(x);
   free(xn);
   free(kqv);
+  free(bias_rows);
   free(qb);
   free(ao);
   free(xo);

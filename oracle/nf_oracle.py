@@ -67,7 +67,7 @@ class NfoModel(C.Structure):
         ("embedding", _u16p), ("lm_head", _u16p), ("model_norm", _u16p),
         ("w_kqv", C.POINTER(_u16p)), ("w_o", C.POINTER(_u16p)), ("w_gate", C.POINTER(_u16p)),
         ("w_up", C.POINTER(_u16p)), ("w_down", C.POINTER(_u16p)), ("ln_attn", C.POINTER(_u16p)),
-        ("ln_ffn", C.POINTER(_u16p)), ("kv_data", C.POINTER(_u16p)),
+        ("ln_ffn", C.POINTER(_u16p)), ("kv_data", C.POINTER(_u16p)), ("b_kqv", C.POINTER(_u16p)),
     ]
 
 
@@ -309,7 +309,7 @@ def decoder_forward(cfg: dict, weights: dict, kv_data: list, batch: dict, hidden
                     want_hidden=True, want_logits=False, want_sampled=True):
     """cfg: hidden,Hq,Hkv,d,ffn,vocab,layers,page_size,eps,rope_theta,rope_scale,smooth_a,smooth_b.
     weights: embedding, lm_head, model_norm and per-layer lists w_kqv,w_o,w_gate,w_up,w_down,
-    ln_attn, ln_ffn.  kv_data: per-layer pools, appended IN PLACE.  batch: the update-data arrays.
+    ln_attn, ln_ffn, and optionally b_kqv (bias rows of the QKV projection).  kv_data: per-layer pools, appended IN PLACE.  batch: the update-data arrays.
     """
     m = NfoModel()
     for k in ("hidden", "Hq", "Hkv", "d", "ffn", "vocab", "layers", "page_size"):
@@ -324,6 +324,10 @@ def decoder_forward(cfg: dict, weights: dict, kv_data: list, batch: dict, hidden
         pa = _ptr_array(weights[k])
         keep.append(pa)
         setattr(m, k, pa)
+    if weights.get("b_kqv") is not None:      # the *_KQVBIAS pipeline types
+        pa = _ptr_array(weights["b_kqv"])
+        keep.append(pa)
+        m.b_kqv = pa
     kva = _ptr_array(kv_data)
     m.kv_data = kva
     b = NfoBatch()

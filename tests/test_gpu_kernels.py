@@ -132,6 +132,24 @@ def test_gemm_column_major_weights(K, oracle):
                      oracle.gemm(A, Bt, b_col_major=True), what="gemm col-major B")
 
 
+@pytest.mark.parametrize("M,N,K_", [(64, 6144, 512), (33, 136, 200), (257, 512, 128), (1408, 6144, 256),
+                                    (2048, 10240, 128), (1930, 5000, 264)])
+def test_gemm_with_bias_row_equals_gemm_with_replicated_bias(K, oracle, M, N, K_):
+    """The QKV projection of the bias pipelines: the reference adds the bias as a C operand holding
+    one copy of it per row (pipeline.cu:1048-1058); reading the one row in the epilogue must give
+    the same bits as that, and agree with the oracle."""
+    rng = np.random.default_rng(7)
+    A = synth.normal_f16(rng, (M, K_))
+    B = synth.normal_f16(rng, (K_, N), 0.02)
+    bias = synth.normal_f16(rng, (N,))
+    rep = np.ascontiguousarray(np.broadcast_to(bias, (M, N)))
+    got = host(K.gemm(dev(A), dev(B), bias=dev(bias), alpha=1.0, beta=1.0))
+    assert np.array_equal(got, host(K.gemm(dev(A), dev(B), dev(rep), alpha=1.0, beta=1.0)))
+    assert_close(got, oracle.gemm(A, B, rep, 1.0, 1.0), what="gemm + bias row")
+    got = host(K.gemm(dev(A), dev(B.T.copy()), bias=dev(bias), alpha=0.5, beta=-1.5, b_col_major=True))
+    assert_close(got, oracle.gemm(A, B, rep, 0.5, -1.5), what="gemm + bias row, col-major B")
+
+
 def test_gemm_identity_is_exact(K):
     rng = np.random.default_rng(6)
     A = synth.normal_f16(rng, (70, 128))

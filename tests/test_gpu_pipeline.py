@@ -139,6 +139,60 @@ def test_update_rejects_inconsistent_batches():
         assert out.shape == (4,) and (out >= 0).all() and (out < shape.vocab).all()
 
 
+@pytest.mark.parametrize("case", ["decode_crosses_border", "prefill_straddles_border"])
+def test_kqv_bias_schedules_match_oracle(oracle, case):
+    """The three bias pipeline types (q/k/v projections with a bias, as Qwen2 has) against the oracle,
+    which adds the bias the way the reference does: a C operand holding one copy per row, beta 1.
+    With an all-zero bias they must reproduce the plain schedules bit for bit."""
+    from nanoflow_amd import engine, pllm_python as P
+    T, nano1, dlens, chunks = CASES[case]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=0)
+    w["b_kqv"] = synth.make_weights(shape, seed=9, kqv_bias=True)["b_kqv"]
+    b1 = synth.make_batch(dlens, chunks, vocab=shape.vocab, seed=21, extra_pages=40)
+    rng = np.random.default_rng(5)
+    pools0 = [synth.make_kv_pool(b1.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok1 = b1.input_tokens.copy()
+    tok1[:b1.decodePrefillBorder] = 1
+    d1 = b1.as_dict()
+    d1["input_tokens"] = tok1
+    pools_ref = [p.copy() for p in pools0]
+    hid, log, samp = oracle.decoder_forward(shape.as_dict(), w, pools_ref, d1, want_logits=True)
+    w_plain = {k: v for k, v in w.items() if k != "b_kqv"}
+    hid_plain, _, _ = oracle.decoder_forward(shape.as_dict(), w_plain, [p.copy() for p in pools0], d1)
+    assert _max_rel(hid_plain, hid) > 10 * E2E_RTOL, "the bias must matter for this test to mean anything"
+    keep = np.ones(b1.decodePrefillBorder, np.int32)
+
+    def run(pt, weights):
+        print(f"case={case} pipeline={pt.name}", flush=True)
+        with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=max(nano1 // 2, 1), kqv3=(T - nano1) // 2,
+                           kv_pages=b1.num_pages, weights=weights, kv_pools=pools0) as e:
+            e.update(b1, keep_token_list=keep)
+            s = e.run()
+            return (s, e.buffer("hidden").cpu().numpy()[:b1.tokens], e.buffer("logits").cpu().numpy()[:b1.req_num],
+                    [p[:b1.num_pages].cpu().numpy() for p in e.kv])
+
+    w_zero = dict(w, b_kqv=[np.zeros_like(b) for b in w["b_kqv"]])
+    pairs = [(P.PipelineType.NONOVERLAP_KQVBIAS, P.PipelineType.NON_OVERLAP_LOCAL),
+             (P.PipelineType.NANOBATCH_KQVBIAS, P.PipelineType.NANOBATCH_LOCAL),
+             (P.PipelineType.KQVBIAS, P.PipelineType.LOCAL)]
+    for bias_pt, plain_pt in pairs:
+        s, h, l, kv = run(bias_pt, w)
+        assert _max_rel(h, hid) < E2E_RTOL, (bias_pt, "hidden", _max_rel(h, hid))
+        assert _max_rel(l, log) < E2E_RTOL, (bias_pt, "logits", _max_rel(l, log))
+        top2 = np.sort(log.astype(np.float32), axis=1)[:, -2:]
+        clear = (top2[:, 1] - top2[:, 0]) > 2 * E2E_RTOL * np.abs(log.astype(np.float32)).max()
+        assert np.array_equal(s[clear], samp[clear]), (bias_pt, "samples")
+        for layer in range(shape.layers):
+            assert np.array_equal((pools_ref[layer] != pools0[layer]).any(axis=(3, 4)),
+                                  (kv[layer] != pools0[layer]).any(axis=(3, 4))), (bias_pt, layer, "KV slots written")
+            assert _max_rel(kv[layer], pools_ref[layer]) < E2E_RTOL, (bias_pt, layer, "KV contents")
+        sz, hz, lz, kvz = run(bias_pt, w_zero)
+        sp, hp, lp, kvp = run(plain_pt, w_plain)
+        assert np.array_equal(sz, sp) and np.array_equal(hz, hp) and np.array_equal(lz, lp), (bias_pt, "zero bias")
+        assert all(np.array_equal(a, b) for a, b in zip(kvz, kvp)), (bias_pt, "zero bias, KV")
+
+
 def test_unsupported_pipeline_types_are_rejected():
     from nanoflow_amd import engine, pllm_python as P
     shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)

@@ -505,6 +505,8 @@ def _numpy_decoder_f64(shape, w, pools, b):
 
     for l in range(shape.layers):
         kqv = norm(x, w["ln_attn"][l]) @ f64(w["w_kqv"][l])
+        if w.get("b_kqv") is not None:        # q/k/v projections with a bias: y = x W + b
+            kqv = kqv + f64(w["b_kqv"][l])[None, :]
         attn = np.zeros((b.tokens, Hq * d))
         qrot = np.zeros((b.tokens, Hq, d))
         for t in range(b.tokens):
@@ -534,10 +536,11 @@ def _numpy_decoder_f64(shape, w, pools, b):
     return x, logits
 
 
-def test_decoder_forward_vs_independent_float64_model(oracle):
+@pytest.mark.parametrize("kqv_bias", [False, True])
+def test_decoder_forward_vs_independent_float64_model(oracle, kqv_bias):
     shape = synth.tiny_shape(layers=2, vocab=512, Hq=4, Hkv=2, ffn=384, hidden=256)
     # larger-than-init weights so the residual stream is not dominated by the embedding
-    w = synth.make_weights(shape, seed=0)
+    w = synth.make_weights(shape, seed=0, kqv_bias=kqv_bias)
     for k in ("w_kqv", "w_o", "w_gate", "w_up", "w_down"):
         w[k] = [(a.astype(np.float32) * 3).astype(np.float16) for a in w[k]]
     w["embedding"] = (w["embedding"].astype(np.float32) * 30).astype(np.float16)
@@ -548,6 +551,9 @@ def test_decoder_forward_vs_independent_float64_model(oracle):
     hidden, logits, sampled = oracle.decoder_forward(shape.as_dict(), w, pools, b.as_dict(),
                                                      want_logits=True)
     ref_x, ref_logits = _numpy_decoder_f64(shape, w, pools_in, b)
+    if kqv_bias:    # dropping the bias must fail the comparison below by a wide margin
+        no_bias, _ = _numpy_decoder_f64(shape, {k: v for k, v in w.items() if k != "b_kqv"}, pools_in, b)
+        assert rel_err(no_bias, ref_x) > 0.1
     assert rel_err(hidden, ref_x) < 4e-3
     assert rel_err(logits, ref_logits) < 6e-3
     # sampled ids agree wherever the float64 top-1/top-2 gap is clear of fp16 noise

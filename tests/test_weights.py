@@ -102,13 +102,20 @@ def test_tied_embeddings_feed_the_lm_head(tmp_path):
     assert np.array_equal(w["lm_head"], _f16(sd["model.embed_tokens.weight"]).T)
 
 
-def test_kqv_bias_is_rejected_not_dropped(tmp_path):
+def test_kqv_bias_is_served_by_the_bias_pipelines_and_never_dropped(tmp_path):
     out_dir = str(tmp_path / "w")
-    W.convert_hf_checkpoint(_write_checkpoint(tmp_path, _hf_state_dict(bias=True)), out_dir)
+    hf = _hf_state_dict(bias=True)
+    W.convert_hf_checkpoint(_write_checkpoint(tmp_path, hf), out_dir)
     sd = torch.load(os.path.join(out_dir, "weight_rank_0.pt"), weights_only=True)
     assert sd["BKQV_0"].shape == (1, 512) and bool(sd["BKQV_0"].any())       # written as K | V | Q like the weights
-    with pytest.raises(ValueError, match="bias"):
+    with pytest.raises(ValueError, match="KQVBIAS"):                          # a plain pipeline type would drop it
         W.load_weight_file(out_dir)
+    shape = W.shape_from_hf_config(CFG)
+    w = W.load_weight_file(out_dir, shape, kqv_bias=True)
+    for l in range(shape.layers):
+        p = f"model.layers.{l}.self_attn."
+        want = np.concatenate([_f16(hf[p + "k_proj.bias"]), _f16(hf[p + "v_proj.bias"]), _f16(hf[p + "q_proj.bias"])])
+        assert w["b_kqv"][l].shape == (shape.kqv_n,) and np.array_equal(w["b_kqv"][l], want)
 
 
 def test_shape_mismatch_and_foreign_files_raise(tmp_path):
