@@ -93,7 +93,23 @@ NF_API int nf_dual_swiglu_bf16(const uint16_t* A, const uint16_t* Bgate, const u
  *   contiguous), fp32 accumulation.  K % 16 == 0, N % 8 == 0.
  * nf_gemm_f8w_f16: fp16 activations against fp8 weights = the two calls above, the quantised
  *   activations and their scales living in `workspace` (nf_gemm_f8w_workspace_bytes(M, K)
- *   bytes, 16-byte aligned). */
+ *   bytes, 16-byte aligned).
+ * nf_quantize_weight_e4m3: a weight in the pipeline's orientation, W fp16 [K,N] row-major, to the
+ *   form the two GEMMs above take: Wq [N,K] e4m3 with col_scale[n] = max_k |W[k][n]| / 448 (1 for
+ *   an all-zero column), Wq[n][k] = e4m3(W[k][n] / col_scale[n]): the row quantiser applied to the
+ *   transpose.  K % 16 == 0, N % 8 == 0.
+ * nf_dual_swiglu_f8_f16: out = half(silu(g) * u) with g = half(a_scale[m] * g_scale[n] * sum_k
+ *   Aq[m][k] * Gq[n][k]) and u likewise from Uq, u_scale: nf_dual_swiglu_f16 on fp8 operands
+ *   (products rounded to fp16 before SiLU-mul, as there).  nf_dual_swiglu_f8w_f16: the same from
+ *   fp16 activations, quantised into `workspace` (nf_gemm_f8w_workspace_bytes(M, K) bytes). */
+NF_API int nf_quantize_weight_e4m3(const uint16_t* W, uint8_t* Wq, float* col_scale, int K, int N,
+                                   nf_stream_t stream);
+NF_API int nf_dual_swiglu_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Gq, const float* g_scale,
+                                 const uint8_t* Uq, const float* u_scale, uint16_t* out, int M, int N, int K,
+                                 nf_stream_t stream);
+NF_API int nf_dual_swiglu_f8w_f16(const uint16_t* A, const uint8_t* Gq, const float* g_scale, const uint8_t* Uq,
+                                  const float* u_scale, uint16_t* out, int M, int N, int K, void* workspace,
+                                  size_t workspace_bytes, nf_stream_t stream);
 NF_API int nf_quantize_rows_e4m3(const uint16_t* X, uint8_t* Xq, float* row_scale, int M, int K,
                                  nf_stream_t stream);
 NF_API int nf_gemm_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, const float* b_scale,

@@ -243,6 +243,24 @@ typedef struct nf_pipeline_timings {
   double gemm_flop;
   int layer_stride;  /* every layer_stride-th layer is timed: totals per iteration = sums * layer_stride */
 } nf_pipeline_timings;
+/* Storage of the five per-layer GEMM weights (W_KQV, W_O1/W_O2, W_G, W_U, W_D) in the init data
+ * the next pllm_init is given; everything else (embedding, norms, B_KQV, LM head) is fp16 in both.
+ * No counterpart in the reference, whose wrappers are half-only
+ * (pipeline/include/cutlassGemmWrapperImpl.cuh:24-27).
+ *   NF_WEIGHTS_F16:  ptr -> fp16 [K][N] row-major, as in the reference (the default).
+ *   NF_WEIGHTS_E4M3: ptr -> N*K OCP e4m3 bytes [N][K] (one row per output channel), followed at byte
+ *     pllm_e4m3_weight_scale_offset(N, K) by N fp32 per-output-channel scales;
+ *     pllm_e4m3_weight_bytes(N, K) bytes in all, 16-byte aligned.  N and K keep their meaning.
+ *     pllm_quantize_weight_e4m3 writes that form from a device-resident fp16 [K][N] weight
+ *     (scale[n] = max_k |w[k][n]| / 448).  The GEMMs then quantise their input rows per launch and
+ *     run on the fp8 matrix cores; the QKV bias pipeline types are not available in this format. */
+enum nf_weight_format { NF_WEIGHTS_F16 = 0, NF_WEIGHTS_E4M3 = 1 };
+NF_PLLM_API int pllm_set_weight_format(int format);
+NF_PLLM_API int pllm_get_weight_format(void);
+NF_PLLM_API size_t pllm_e4m3_weight_bytes(int N, int K);
+NF_PLLM_API size_t pllm_e4m3_weight_scale_offset(int N, int K);
+NF_PLLM_API int pllm_quantize_weight_e4m3(const uint16_t* w_f16, void* out, int N, int K, void* stream);
+
 NF_PLLM_API int pllm_set_profiling(int on);
 /* Time every stride-th launch of each operator (0 = automatic: 4 on schedules of 8 or more layers,
  * else 1).  Takes effect at the next pllm_set_profiling / pllm_init.  pllm_get_timings reports the

@@ -22,6 +22,13 @@ public:
     allocated += n;
     return ret;
   }
+  // bytes of scratch at a 256-byte boundary of the buffer (nullptr for 0 bytes)
+  void* allocBytes(size_t bytes) {
+    if (bytes == 0) return nullptr;
+    const size_t unit = 256 / sizeof(T);
+    alloc((unit - allocated % unit) % unit);
+    return alloc((bytes + sizeof(T) - 1) / sizeof(T));
+  }
   std::span<T> allocSpan(size_t n) { return std::span<T>{alloc(n), n}; }
   pllmTensor<T> allocTensor(int M, int N, PllmLayout layout) {
     if (layout == PllmLayout::ROW_MAJOR) return pllmTensor<T>{alloc((size_t)M * N), M, N, layout};

@@ -20,6 +20,9 @@ static std::unique_ptr<SimpleThreadSync> global_sync;  // workers + the caller's
 static vortexInitData* persistant_input = nullptr;
 static std::vector<int> complete_input_tokens;
 static int g_profiling = 0;
+static WeightFormat g_weight_format = WeightFormat::F16;
+void setWeightFormat(WeightFormat format) { g_weight_format = format; }
+WeightFormat getWeightFormat() { return g_weight_format; }
 static bool g_graph_mode = false;
 
 int buildInputTokens(const int* prev_output, int prev_count, const int32_t* keep_token_list,
@@ -69,6 +72,10 @@ void init(int nranks, int vnranks, std::vector<vortexInitData>& input,
   }
   if (!workers.empty()) {
     std::fprintf(stderr, "init: already initialised; call finalize() first\n");
+    std::exit(EXIT_FAILURE);
+  }
+  if (g_weight_format == WeightFormat::E4M3 && Worker::hasKQVBias(pipeTy)) {
+    std::fprintf(stderr, "init: the QKV bias pipelines take fp16 weights only\n");
     std::exit(EXIT_FAILURE);
   }
   Worker::PipeTy = pipeTy;

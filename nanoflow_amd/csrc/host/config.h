@@ -59,6 +59,9 @@ struct vortexModelConfig {
     // covers when the vocabulary term is large
     k_temp_size = (size_t)max_batch_size * model_hidden_dim * 16 + (size_t)max_batch_size * vocab_size * 2 +
                   (size_t)max_batch_size * model_ff_dim + 65536;
+    // quantised activations of the fp8-weight GEMMs (one byte per element of the QKV, O, gate/up
+    // and down inputs, a scale per row, 256-byte alignment of up to 8 wrappers)
+    k_temp_size += (size_t)max_batch_size * (3 * model_hidden_dim + model_ff_dim + 32) / 2 + 8 * 256;
     if (!rope_3_1) {
       smooth_a = 0;
       smooth_b = 0;

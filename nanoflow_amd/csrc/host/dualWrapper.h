@@ -12,6 +12,17 @@ struct DualWrapper : public OperatorWrapper {
   pllmTensor<half> pllm_tensor_a, pllm_tensor_b1, pllm_tensor_b2, pllm_tensor_c;
   pllmTensor<half> pllm_tensor_d0, pllm_tensor_d1, pllm_tensor_d2;
   bool inited = false;
+  // WeightFormat::E4M3: b1 / b2 point at e4m3 weights with their scales behind them; the rows of A
+  // are quantised into the workspace on every launch (nf_dual_swiglu_f8w_f16)
+  bool e4m3 = false;
+  void* workspace = nullptr;
+  size_t workspace_bytes = 0;
+  void setWeightFormat(WeightFormat f) { e4m3 = f == WeightFormat::E4M3; }
+  size_t workspaceBytes() const { return e4m3 ? nf_gemm_f8w_workspace_bytes(M, K) : 0; }
+  void setWorkspace(void* ptr, size_t bytes) {
+    workspace = ptr;
+    workspace_bytes = bytes;
+  }
 
   void set_shape(int m, int n, int k) {
     M = m;
@@ -20,6 +31,15 @@ struct DualWrapper : public OperatorWrapper {
     NF_LOG_INFO("name:%s M:%d, N:%d, K:%d", name.c_str(), M, N, K);
   }
   void work() override {
+    if (e4m3) {
+      const uint8_t* g = reinterpret_cast<const uint8_t*>(pllm_tensor_b1.ptr);
+      const uint8_t* u = reinterpret_cast<const uint8_t*>(pllm_tensor_b2.ptr);
+      const size_t so = e4m3WeightScaleOffset((size_t)N, (size_t)K);
+      NF_KERNEL_CHECK(nf_dual_swiglu_f8w_f16(pllm_tensor_a.ptr, g, reinterpret_cast<const float*>(g + so), u,
+                                             reinterpret_cast<const float*>(u + so), pllm_tensor_d2.ptr, M, N, K,
+                                             workspace, workspace_bytes, stream));
+      return;
+    }
     NF_KERNEL_CHECK(nf_dual_swiglu_f16(pllm_tensor_a.ptr, pllm_tensor_b1.ptr, pllm_tensor_b2.ptr,
                                        pllm_tensor_d2.ptr, M, N, K, stream));
   }

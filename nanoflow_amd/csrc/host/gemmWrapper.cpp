@@ -28,7 +28,7 @@ bool parseGemmTag(const std::string& tag, GemmTag& out) {
   return true;
 }
 
-BaseGEMMWrapper* generateGEMM(const std::string& tag) {
+BaseGEMMWrapper* generateGEMM(const std::string& tag, WeightFormat format) {
   GemmTag t;
   if (!parseGemmTag(tag, t)) {
     NF_LOG_ERROR("generateGEMM: malformed tag \"%s\"", tag.c_str());
@@ -38,7 +38,21 @@ BaseGEMMWrapper* generateGEMM(const std::string& tag) {
     NF_LOG_ERROR("generateGEMM: tag \"%s\": A and output must be RowMajor in this build", tag.c_str());
     return nullptr;
   }
+  if (format == WeightFormat::E4M3) {
+    if (t.layout_b != PllmLayout::ROW_MAJOR) {
+      NF_LOG_ERROR("generateGEMM: tag \"%s\": e4m3 weights have one layout; the tag must say RowMajor", tag.c_str());
+      return nullptr;
+    }
+    return new HipGEMMWrapperF8W(t);
+  }
   return new HipGEMMWrapper(t);
+}
+
+void HipGEMMWrapperF8W::work() {
+  const uint8_t* bq = reinterpret_cast<const uint8_t*>(pllm_tensor_b.ptr);
+  const float* bs = reinterpret_cast<const float*>(bq + e4m3WeightScaleOffset(N, K));
+  NF_KERNEL_CHECK(nf_gemm_f8w_f16(pllm_tensor_a.ptr, bq, bs, pllm_tensor_c.ptr, pllm_tensor_d.ptr, (int)M,
+                                  (int)N, (int)K, alpha, beta, workspace, workspace_bytes, stream));
 }
 
 void HipGEMMWrapper::work() {
@@ -106,6 +120,43 @@ bool HipGEMMWrapper::checkResult() {
     uint16_t c16 = 0, d16 = 0;
     if (beta != 0.f) {
       HIP_CHECK(hipMemcpy(&c16, pllm_tensor_c.ptr + (c_is_row ? 0 : m * N) + n, 2, hipMemcpyDeviceToHost));
+      ref += beta * half_bits_to_float(c16);
+    }
+    HIP_CHECK(hipMemcpy(&d16, pllm_tensor_d.ptr + m * N + n, 2, hipMemcpyDeviceToHost));
+    double d = half_bits_to_float(d16);
+    if ((std::fabs(d - ref) - 0.01) / std::max(std::fabs(ref), 1e-6) > 0.1) ok = false;
+  }
+  return ok;
+}
+
+static float e4m3_bits_to_float(uint8_t v) {
+  const int e = (v >> 3) & 0xf, m = v & 7;
+  const float f = e == 0 ? std::ldexp((float)m, -9) : std::ldexp((float)(8 + m), e - 10);
+  return (v & 0x80) ? -f : f;
+}
+
+// As HipGEMMWrapper::checkResult, the reference value taken from fp16 activations and the
+// dequantised weight (so the activation quantisation counts as error, within the same pass rule).
+bool HipGEMMWrapperF8W::checkResult() {
+  work();
+  HIP_CHECK(hipStreamSynchronize(stream));
+  const uint8_t* bq = reinterpret_cast<const uint8_t*>(pllm_tensor_b.ptr);
+  const float* bs = reinterpret_cast<const float*>(bq + e4m3WeightScaleOffset(N, K));
+  std::vector<uint16_t> arow(K);
+  std::vector<uint8_t> brow(K);
+  bool ok = true;
+  for (int s = 0; s < 64 && ok; ++s) {
+    size_t m = (size_t)(s * 2654435761u) % M, n = (size_t)(s * 40503u + 7) % N;
+    float scale = 0;
+    HIP_CHECK(hipMemcpy(arow.data(), pllm_tensor_a.ptr + m * K, K * 2, hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpy(brow.data(), bq + n * K, K, hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpy(&scale, bs + n, 4, hipMemcpyDeviceToHost));
+    double ref = 0;
+    for (size_t k = 0; k < K; ++k) ref += (double)half_bits_to_float(arow[k]) * e4m3_bits_to_float(brow[k]);
+    ref *= (double)alpha * scale;
+    uint16_t c16 = 0, d16 = 0;
+    if (beta != 0.f) {
+      HIP_CHECK(hipMemcpy(&c16, pllm_tensor_c.ptr + m * N + n, 2, hipMemcpyDeviceToHost));
       ref += beta * half_bits_to_float(c16);
     }
     HIP_CHECK(hipMemcpy(&d16, pllm_tensor_d.ptr + m * N + n, 2, hipMemcpyDeviceToHost));

@@ -54,6 +54,14 @@ struct BaseGEMMWrapper : public OperatorWrapper {
   // product, read by the kernel's epilogue.  Takes the place of setC() with the bias replicated
   // over max-batch rows (replicateKQVBias, pipeline/src/pipeline.cu:520-533,1048-1058).
   virtual BaseGEMMWrapper& setCRow(pllmTensor<ElementOutput> row) = 0;
+  // Also not in the reference's interface: device scratch a wrapper needs per launch (the
+  // quantised activations of the fp8-weight wrapper), handed out by the pipeline's buffer plan
+  // once the shape is set.  Zero for the fp16 wrapper.
+  virtual size_t workspaceBytes() const { return 0; }
+  virtual void setWorkspace(void* ptr, size_t bytes) {
+    (void)ptr;
+    (void)bytes;
+  }
 };
 
 struct GemmTag {
@@ -134,6 +142,32 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   bool checkResult() override;  // spot-checks D against a host fp64 dot product
 };
 
+// fp16 activations against an e4m3 weight with per-output-channel scales (WeightFormat::E4M3):
+// each launch quantises the rows of A into the workspace (per-row scale) and multiplies on the
+// fp8 matrix cores, D = half(alpha * sa[m] * sb[n] * sum_k Aq.Bq + beta * C).  No counterpart in
+// the reference (its wrappers are half-only, cutlassGemmWrapperImpl.cuh:24-27).
+struct HipGEMMWrapperF8W : public HipGEMMWrapper {
+  void* workspace = nullptr;
+  size_t workspace_bytes = 0;
+  explicit HipGEMMWrapperF8W(const GemmTag& t) : HipGEMMWrapper(t) {}
+  void work() override;
+  void set_weight(half* blob) override {  // see WeightFormat::E4M3
+    pllm_tensor_b = pllmTensor<half>(blob, N, K, PllmLayout::COL_MAJOR);
+  }
+  using HipGEMMWrapper::set_weight;
+  HipGEMMWrapperF8W& setCRow(pllmTensor<half> row) override {
+    (void)row;
+    std::fprintf(stderr, "%s: a bias row is not implemented for e4m3 weights\n", name.c_str());
+    std::exit(EXIT_FAILURE);
+  }
+  size_t workspaceBytes() const override { return nf_gemm_f8w_workspace_bytes((int)M, (int)K); }
+  void setWorkspace(void* ptr, size_t bytes) override {
+    workspace = ptr;
+    workspace_bytes = bytes;
+  }
+  bool checkResult() override;  // against the dequantised weight
+};
+
 // Unknown or unsupported tags are an error here (nullptr + logged message) rather than the
 // reference's null dereference (pipeline/include/gemmFactory.cuh, pipeline_local.cu:850).
-BaseGEMMWrapper* generateGEMM(const std::string& tag);
+BaseGEMMWrapper* generateGEMM(const std::string& tag, WeightFormat format = WeightFormat::F16);

@@ -62,6 +62,7 @@ protected:
   // The *_KQVBIAS pipeline types (models whose q/k/v projections have a bias, Qwen2): the QKV
   // GEMMs add vortexLayerWeight::B_KQV ([1, kqv_n], columns K|V|Q) to every row, beta = 1
   // (pipeline/src/pipeline.cu:520-533, pipeline_nonoverlap.cu:209-211).
+  WeightFormat weight_format = getWeightFormat();  // of the five per-layer GEMM weights
   bool kqv_bias = false;
   bool bindKQVBias(BaseGEMMWrapper* kqv, vortexWeight& bias) {
     if (!kqv_bias) return true;

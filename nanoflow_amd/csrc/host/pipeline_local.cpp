@@ -317,6 +317,11 @@ void LocalPipeline::ScheduleInit() {
   pllmTensor<int> sample_output = {sample_output_alloc, T, 1, ROW};
   const auto maxSampler_maxVals = tmpBufferM.allocTensor(T, 1, ROW);
   maxSampler.init(LOGITS_output, maxSampler_maxVals, sample_output);
+  // scratch of the fp8-weight wrappers (none for fp16 weights)
+  for (int i = 0; i < gemmNum; ++i)
+    gemms[i]->setWorkspace(tmpBufferM.allocBytes(gemms[i]->workspaceBytes()), gemms[i]->workspaceBytes());
+  dual1.setWorkspace(tmpBufferM.allocBytes(dual1.workspaceBytes()), dual1.workspaceBytes());
+  dual2.setWorkspace(tmpBufferM.allocBytes(dual2.workspaceBytes()), dual2.workspaceBytes());
   NF_LOG_INFO("allocated num: %zu", tmpBufferM.getAllocation());
 }
 
@@ -594,7 +599,8 @@ void LocalPipeline::config(vortexConfigData* config_data_) {
   for (int i = 0; i < gemmNum; ++i) {
     const std::string& tag =
         i < (int)config_data.gemm_op_tag.size() ? config_data.gemm_op_tag[i] : std::string(gemmConfig[i]);
-    gemms[i] = generateGEMM(tag);
+    // the LM head stays fp16 in both weight formats
+    gemms[i] = generateGEMM(tag, i == static_cast<int>(GEMM_NAME::LOGITS) ? WeightFormat::F16 : weight_format);
     if (!gemms[i]) {
       std::fprintf(stderr, "LocalPipeline::config: cannot build GEMM %d from tag \"%s\"\n", i, tag.c_str());
       std::exit(EXIT_FAILURE);
@@ -621,6 +627,8 @@ void LocalPipeline::config(vortexConfigData* config_data_) {
   LOGITS->set_shape(globalbatch / nranks, (int)ModelConfig.vocab_size, ModelConfig.model_hidden_dim);
   dual1.set_shape(nano1, ModelConfig.model_ff_dim_gpu, ModelConfig.model_hidden_dim);
   dual2.set_shape(nano2, ModelConfig.model_ff_dim_gpu, ModelConfig.model_hidden_dim);
+  dual1.setWeightFormat(weight_format);
+  dual2.setWeightFormat(weight_format);
 
   setName();
   ScheduleInit();

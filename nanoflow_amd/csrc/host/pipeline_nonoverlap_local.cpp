@@ -125,7 +125,8 @@ void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
   for (int i = 0; i < gemmNum; ++i) {
     const std::string& tag =
         i < (int)config_data.gemm_op_tag.size() ? config_data.gemm_op_tag[i] : std::string(gemmConfig[i]);
-    gemms[i] = generateGEMM(tag);
+    // the LM head stays fp16 in both weight formats
+    gemms[i] = generateGEMM(tag, i == static_cast<int>(GEMM_NAME::LOGITS) ? WeightFormat::F16 : weight_format);
     if (!gemms[i]) {
       std::fprintf(stderr, "NonOverlapLocalPipeline::config: cannot build GEMM %d from tag \"%s\"\n", i,
                    tag.c_str());
@@ -146,6 +147,7 @@ void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
                  ModelConfig.model_hidden_dim);
   LOGITS->set_shape(globalbatch, (int)ModelConfig.vocab_size, ModelConfig.model_hidden_dim);
   dual.set_shape(globalbatch, ModelConfig.model_ff_dim_gpu, ModelConfig.model_hidden_dim);
+  dual.setWeightFormat(weight_format);
   ScheduleInit();
   GEMMOpInit();
   GEMVOpInit();
@@ -224,6 +226,10 @@ void NonOverlapLocalPipeline::ScheduleInit() {
   const auto maxSampler_maxVals = tmpBufferM.allocTensor(T, 1, ROW);
   maxSampler.init(LOGITS_output, maxSampler_maxVals, sample_output);
   genEmbedding.setOutput(D->getD());
+  // scratch of the fp8-weight wrappers (none for fp16 weights)
+  for (int i = 0; i < gemmNum; ++i)
+    gemms[i]->setWorkspace(tmpBufferM.allocBytes(gemms[i]->workspaceBytes()), gemms[i]->workspaceBytes());
+  dual.setWorkspace(tmpBufferM.allocBytes(dual.workspaceBytes()), dual.workspaceBytes());
   NF_LOG_INFO("allocated %zu halfs", tmpBufferM.getAllocation());
 }
 

@@ -96,6 +96,8 @@ int pllm_init(const nf_vortex_init_data* input, int pipeline_type) {
                 "pllm_init: pipeline type %d is a tensor-parallel schedule; LOCAL(7), "
                 "NON_OVERLAP_LOCAL(8), NANOBATCH_LOCAL(9) and, as those with a QKV bias, KQVBIAS(4), "
                 "NONOVERLAP_KQVBIAS(5), NANOBATCH_KQVBIAS(6) are implemented", pipeline_type);
+  if (getWeightFormat() == WeightFormat::E4M3 && Worker::hasKQVBias(ty))
+    return fail(NF_PLLM_ERR_UNSUPPORTED, "pllm_init: the QKV bias pipelines take fp16 weights only");
   if (input->weight.num_layers < ModelConfig.model_layer)
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_init: %d layers of weights, model has %d",
                 input->weight.num_layers, ModelConfig.model_layer);
@@ -326,6 +328,34 @@ int pllm_build_input_tokens(const int32_t* prev_output, int prev_count, const in
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_build_input_tokens: null pointer");
   return buildInputTokens(prev_output, prev_count, keep_token_list, keep_token_list_length, prefill_tokens,
                           prefill_tokens_num, out);
+}
+
+int pllm_set_weight_format(int format) {
+  if (g_inited) return fail(NF_PLLM_ERR_STATE, "pllm_set_weight_format: call it before pllm_init");
+  if (format != NF_WEIGHTS_F16 && format != NF_WEIGHTS_E4M3)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_set_weight_format: unknown format %d", format);
+  setWeightFormat(format == NF_WEIGHTS_E4M3 ? WeightFormat::E4M3 : WeightFormat::F16);
+  return NF_PLLM_OK;
+}
+
+int pllm_get_weight_format(void) { return getWeightFormat() == WeightFormat::E4M3 ? NF_WEIGHTS_E4M3 : NF_WEIGHTS_F16; }
+
+size_t pllm_e4m3_weight_bytes(int N, int K) {
+  return N > 0 && K > 0 ? e4m3WeightBytes((size_t)N, (size_t)K) : 0;
+}
+
+size_t pllm_e4m3_weight_scale_offset(int N, int K) {
+  return N > 0 && K > 0 ? e4m3WeightScaleOffset((size_t)N, (size_t)K) : 0;
+}
+
+int pllm_quantize_weight_e4m3(const uint16_t* w_f16, void* out, int N, int K, void* stream) {
+  if (!w_f16 || !out || N <= 0 || K <= 0)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_quantize_weight_e4m3: bad argument");
+  uint8_t* q = static_cast<uint8_t*>(out);
+  if (nf_quantize_weight_e4m3(w_f16, q, reinterpret_cast<float*>(q + e4m3WeightScaleOffset((size_t)N, (size_t)K)), K, N,
+                              stream) != 0)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_quantize_weight_e4m3: %s", nf_last_error());
+  return NF_PLLM_OK;
 }
 
 int pllm_set_profiling_stride(int stride) {

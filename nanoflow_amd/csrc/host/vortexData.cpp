@@ -42,6 +42,17 @@ static vortexWeight device_weight(int N, int K) {
   HIP_CHECK(hipMemset(w.ptr, 0, w.size() * sizeof(half)));
   return w;
 }
+// One of the five per-layer GEMM weights in the current weight format (zero-filled).
+static vortexWeight device_gemm_weight(int N, int K) {
+  if (getWeightFormat() != WeightFormat::E4M3) return device_weight(N, K);
+  vortexWeight w;
+  w.N = N;
+  w.K = K;
+  const size_t bytes = e4m3WeightBytes((size_t)N, (size_t)K);
+  HIP_CHECK(hipMalloc(&w.ptr, bytes));
+  HIP_CHECK(hipMemset(w.ptr, 0, bytes));
+  return w;
+}
 static vortexWeight host_weight(int N, int K) {
   vortexWeight w;
   w.N = N;
@@ -49,9 +60,17 @@ static vortexWeight host_weight(int N, int K) {
   w.ptr = new half[w.size()]();
   return w;
 }
+static vortexWeight host_gemm_weight(int N, int K) {
+  if (getWeightFormat() != WeightFormat::E4M3) return host_weight(N, K);
+  vortexWeight w;
+  w.N = N;
+  w.K = K;
+  w.ptr = new half[(e4m3WeightBytes((size_t)N, (size_t)K) + 1) / 2]();
+  return w;
+}
 
-template <typename MakeWeight>
-static void fill_model_weight(vortexModelWeight& data, MakeWeight make) {
+template <typename MakeWeight, typename MakeGemmWeight>
+static void fill_model_weight(vortexModelWeight& data, MakeWeight make, MakeGemmWeight make_gemm) {
   const int H = ModelConfig.model_hidden_dim, Hg = ModelConfig.model_hidden_dim_pergpu;
   const int F = ModelConfig.model_ff_dim_gpu;
   const int kqv_n = (2 * ModelConfig.model_kv_heads_gpu + ModelConfig.model_qo_heads_gpu) *
@@ -62,12 +81,12 @@ static void fill_model_weight(vortexModelWeight& data, MakeWeight make) {
   data.model_layernorm = make(H, 1);
   data.layer_weight.resize(ModelConfig.model_layer);
   for (auto& lw : data.layer_weight) {
-    lw.W_O1 = make(Hg, H);
-    lw.W_O2 = make(H, Hg);
-    lw.W_U = make(F, H);
-    lw.W_G = make(F, H);
-    lw.W_D = make(H, F);
-    lw.W_KQV = make(kqv_n, H);
+    lw.W_O1 = make_gemm(Hg, H);
+    lw.W_O2 = make_gemm(H, Hg);
+    lw.W_U = make_gemm(F, H);
+    lw.W_G = make_gemm(F, H);
+    lw.W_D = make_gemm(H, F);
+    lw.W_KQV = make_gemm(kqv_n, H);
     lw.B_KQV = make(1, kqv_n);
     lw.W_LN_Attention = make(H, 1);
     lw.W_LN_FFN = make(H, 1);
@@ -77,18 +96,21 @@ static void fill_model_weight(vortexModelWeight& data, MakeWeight make) {
 
 void createModelWeight(vortexModelWeight& data, int rank) {
   HIP_CHECK(hipSetDevice(rank));
-  fill_model_weight(data, device_weight);
+  fill_model_weight(data, device_weight, device_gemm_weight);
 }
 void createModelWeightCPU(vortexModelWeight& data, int rank) {
   (void)rank;
-  fill_model_weight(data, host_weight);
+  fill_model_weight(data, host_weight, host_gemm_weight);
 }
 
-static vortexWeight upload(const vortexWeight& h) {
+static vortexWeight upload(const vortexWeight& h, bool gemm_weight = false) {
   vortexWeight d = h;
   if (!h.ptr || h.size() == 0) return d;
-  HIP_CHECK(hipMalloc(&d.ptr, h.size() * sizeof(half)));
-  HIP_CHECK(hipMemcpy(d.ptr, h.ptr, h.size() * sizeof(half), hipMemcpyHostToDevice));
+  const size_t bytes = gemm_weight && getWeightFormat() == WeightFormat::E4M3
+                           ? e4m3WeightBytes((size_t)h.N, (size_t)h.K)
+                           : h.size() * sizeof(half);
+  HIP_CHECK(hipMalloc(&d.ptr, bytes));
+  HIP_CHECK(hipMemcpy(d.ptr, h.ptr, bytes, hipMemcpyHostToDevice));
   return d;
 }
 
@@ -102,12 +124,12 @@ vortexModelWeight modelWeightToGPU(vortexModelWeight& hw, int rank) {
   for (size_t i = 0; i < hw.layer_weight.size(); ++i) {
     const auto& s = hw.layer_weight[i];
     auto& t = d.layer_weight[i];
-    t.W_O1 = upload(s.W_O1);
-    t.W_O2 = s.W_O2.ptr == s.W_O1.ptr ? t.W_O1 : upload(s.W_O2);
-    t.W_U = upload(s.W_U);
-    t.W_G = upload(s.W_G);
-    t.W_D = upload(s.W_D);
-    t.W_KQV = upload(s.W_KQV);
+    t.W_O1 = upload(s.W_O1, true);
+    t.W_O2 = s.W_O2.ptr == s.W_O1.ptr ? t.W_O1 : upload(s.W_O2, true);
+    t.W_U = upload(s.W_U, true);
+    t.W_G = upload(s.W_G, true);
+    t.W_D = upload(s.W_D, true);
+    t.W_KQV = upload(s.W_KQV, true);
     t.B_KQV = upload(s.B_KQV);
     t.W_LN_Attention = upload(s.W_LN_Attention);
     t.W_LN_FFN = upload(s.W_LN_FFN);

@@ -15,6 +15,21 @@ struct vortexWeight {
   size_t size() const { return (size_t)N * K; }
 };
 
+// Storage of the five per-layer GEMM weights (W_KQV, W_O1/W_O2, W_G, W_U, W_D); embedding, norms,
+// B_KQV and the LM head are fp16 in both.  The reference knows fp16 only.
+//   F16:  ptr -> fp16 [K][N] row-major (K = input features), as in the reference.
+//   E4M3: ptr -> N*K OCP e4m3 bytes [N][K] (one row per output channel, k contiguous), followed at
+//         byte e4m3WeightScaleOffset(N, K) by N fp32 per-output-channel scales
+//         (w[k][n] ~ scale[n] * e4m3[n][k]); e4m3WeightBytes(N, K) bytes in all, 16-byte aligned.
+//         N and K keep their meaning, so size() still checks the shape.
+enum class WeightFormat { F16 = 0, E4M3 = 1 };
+inline size_t e4m3WeightScaleOffset(size_t N, size_t K) { return (N * K + 255) / 256 * 256; }
+inline size_t e4m3WeightBytes(size_t N, size_t K) { return e4m3WeightScaleOffset(N, K) + N * sizeof(float); }
+
+// The format of the init data the next init() is given (process-wide, F16 unless set).
+void setWeightFormat(WeightFormat format);
+WeightFormat getWeightFormat();
+
 struct vortexLayerWeight {
   vortexWeight W_O1, W_O2, W_U, W_G, W_D, W_KQV, B_KQV, W_LN_Attention, W_LN_FFN, W_ROT;
 };

@@ -25,9 +25,9 @@ constexpr int F8_BK = 128;  // k-bytes per slab = one 128-byte LDS row per matri
 
 typedef int v8i32 __attribute__((ext_vector_type(8)));
 
-template <int BM, int BN>
+template <int BM, int BN, int NB>
 struct F8Smem {
-  static constexpr int stage_bytes = (BM + BN) * 128;
+  static constexpr int stage_bytes = (BM + NB * BN) * 128;
   static constexpr int stages = (144 * 1024) / stage_bytes > 4 ? 4 : (144 * 1024) / stage_bytes;
   static_assert(stages >= 2, "tile too large for two LDS stages");
   static constexpr size_t bytes = (size_t)stages * stage_bytes;
@@ -92,18 +92,84 @@ __global__ __launch_bounds__(256) void quantize_rows_e4m3_kernel(const uint16_t*
   }
 }
 
-template <int BM, int BN, int WM, int WN>
+// Weight quantiser: W fp16 [K][N] (the pipeline's weight orientation) -> Wq e4m3 [N][K] (one row
+// per output channel, k contiguous) with scale[n] = max_k |W[k][n]| / 448 (1 for an all-zero
+// column), Wq[n][k] = e4m3_rne(W[k][n] / scale[n]): the row quantiser applied to the transpose.
+// First the column maxima (64 columns per workgroup, rows read in 128-byte runs) ...
+__global__ __launch_bounds__(256) void weight_col_scale_kernel(const uint16_t* __restrict__ W,
+                                                               float* __restrict__ scale, int K, int N) {
+  __shared__ float red[8][64];
+  const int tid = threadIdx.x, c2 = tid & 31, r = tid >> 5;
+  const int n = blockIdx.x * 64 + 2 * c2;
+  float a0 = 0.f, a1 = 0.f;
+  if (n < N)
+    for (int k = r; k < K; k += 8) {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(W + (size_t)k * N + n);
+      a0 = fmaxf(a0, fabsf(h2f_bits(w & 0xffffu)));
+      a1 = fmaxf(a1, fabsf(h2f_bits(w >> 16)));
+    }
+  red[r][2 * c2] = a0;
+  red[r][2 * c2 + 1] = a1;
+  __syncthreads();
+  if (tid < 64 && blockIdx.x * 64 + tid < N) {
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a = fmaxf(a, red[i][tid]);
+    scale[blockIdx.x * 64 + tid] = a > 0.f ? a / 448.f : 1.f;
+  }
+}
+
+// ... then 64 x 64 tiles are quantised on the way into LDS and written out transposed, 16 bytes
+// of one output channel per thread.
+__global__ __launch_bounds__(256) void weight_quantize_transpose_kernel(const uint16_t* __restrict__ W,
+                                                                        const float* __restrict__ scale,
+                                                                        uint8_t* __restrict__ Wq, int K, int N) {
+  __shared__ __attribute__((aligned(16))) uint8_t tile[64][64 + 16];  // [n][k]
+  const int tid = threadIdx.x, c2 = tid & 31, r = tid >> 5;
+  const int k0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+  const int n = n0 + 2 * c2;
+  float s0 = 1.f, s1 = 1.f;
+  if (n < N) {
+    s0 = scale[n];
+    s1 = scale[n + 1];
+  }
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const int kl = p * 8 + r, k = k0 + kl;
+    uint32_t w = 0;
+    if (n < N && k < K) w = *reinterpret_cast<const uint32_t*>(W + (size_t)k * N + n);
+    tile[2 * c2][kl] = (uint8_t)f32_to_e4m3(h2f_bits(w & 0xffffu) / s0);
+    tile[2 * c2 + 1][kl] = (uint8_t)f32_to_e4m3(h2f_bits(w >> 16) / s1);
+  }
+  __syncthreads();
+  const int nl = tid >> 2, kc = (tid & 3) * 16;
+  if (n0 + nl < N && k0 + kc < K)  // K % 16 == 0: a chunk is inside or outside as a whole
+    *reinterpret_cast<u32x4*>(Wq + (size_t)(n0 + nl) * K + k0 + kc) = *reinterpret_cast<const u32x4*>(&tile[nl][kc]);
+}
+
+// SiLU(g) * u on products already rounded to fp16, as the fp16 dual kernel's epilogue does it.
+__device__ __forceinline__ float swiglu_rounded_f16(float g_acc, float u_acc) {
+  const float g = __half2float(__float2half_rn(g_acc));
+  const float u = __half2float(__float2half_rn(u_acc));
+  return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
+}
+
+// kDual: two weight matrices B (gate) and B1 (up) with scales sb and sb1,
+//   D[m][n] = half(silu(g) * u),  g = half(sa[m] * sb[n] * sum_k Aq.Bq),  u = half(sa[m] * sb1[n] * sum_k Aq.B1q);
+// alpha, beta and C are not used.
+template <int BM, int BN, int WM, int WN, bool kDual>
 __global__ __launch_bounds__(256) void gemm_f8_kernel(
-    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const float* __restrict__ sa,
-    const float* __restrict__ sb, const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha,
-    float beta, int tiles_m, int tiles_n) {
-  using SM = F8Smem<BM, BN>;
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ B1,
+    const float* __restrict__ sa, const float* __restrict__ sb, const float* __restrict__ sb1,
+    const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n) {
+  constexpr int NB = kDual ? 2 : 1;
+  using SM = F8Smem<BM, BN, NB>;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(WM * WN == 4, "four wavefronts");
   constexpr int A_LOADS = BM / 32;  // 1 KB (8 rows) load instructions per wave per slab
-  constexpr int B_LOADS = BN / 32;
+  constexpr int B_LOADS = BN / 32;  // ... per weight matrix
   constexpr int NS = SM::stages;
-  constexpr int LOADS = A_LOADS + B_LOADS;
+  constexpr int LOADS = A_LOADS + NB * B_LOADS;
   // k-steps the loads of one slab are spread over; with two stages they must land within one step
   constexpr int PARTS = NS == 2 ? 1 : 2;
 
@@ -124,13 +190,15 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   const int wm = wave / WN, wn = wave % WN;
   const int l32 = lane & 31, lg = lane >> 5;
 
-  float16_t acc[TM][TN];
+  float16_t acc[NB][TM][TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int b = 0; b < NB; ++b)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[b][i][j][r] = 0.f;
 
   // Both operands are rows of 128 k-bytes; they go from global memory straight into LDS
   // (see gemm.hip): 8 rows per load instruction, row r keeping its logical 16-byte chunk c at
@@ -139,24 +207,26 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   // one lie at or past the end of the buffer and read as zero, which leaves only k >= K inside a
   // row to be masked.
   const rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K);
-  const rsrc_t b_rsrc = make_rsrc(B, (size_t)N * K);
+  const rsrc_t b_rsrc[2] = {make_rsrc(B, (size_t)N * K), make_rsrc(kDual ? B1 : B, (size_t)N * K)};
   const int kc = ((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2))) * 16;  // k-byte of this lane's chunk inside the slab
-  uint32_t a_off[A_LOADS], b_off[B_LOADS];
+  uint32_t a_off[A_LOADS], b_off[NB][B_LOADS];
 #pragma unroll
   for (int t = 0; t < A_LOADS; ++t)
     a_off[t] = (uint32_t)(m_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)K + kc;
 #pragma unroll
-  for (int t = 0; t < B_LOADS; ++t)
-    b_off[t] = (uint32_t)(n_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)K + kc;
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int t = 0; t < B_LOADS; ++t)
+      b_off[b][t] = (uint32_t)(n_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)K + kc;
   auto load_one = [&](auto t_c, uint32_t st, bool k_ok) {
     constexpr int t = decltype(t_c)::value;
     if constexpr (t < A_LOADS) {
       load16_to_lds<t * 4096>(a_rsrc, k_ok ? a_off[t] : kOob, st);
       a_off[t] += F8_BK;
     } else {
-      constexpr int tt = t - A_LOADS;
-      load16_to_lds<BM * 128 + tt * 4096>(b_rsrc, k_ok ? b_off[tt] : kOob, st);
-      b_off[tt] += F8_BK;
+      constexpr int b = (t - A_LOADS) / B_LOADS, tt = (t - A_LOADS) % B_LOADS;
+      load16_to_lds<(BM + b * BN) * 128 + tt * 4096>(b_rsrc[b], k_ok ? b_off[b][tt] : kOob, st);
+      b_off[b][tt] += F8_BK;
     }
   };
   auto load_slab = [&](int stage, int k0) {
@@ -172,23 +242,27 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   uint32_t swz[2];
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) swz[kk] = (uint32_t)(((kk * 4 + lg * 2) ^ ((l32 >> 1) & 7)) << 4);
-  v8i32 af[2][TM], bf[2][TN];
+  v8i32 af[2][TM], bf[2][NB][TN];
   auto read32 = [&](const uint8_t* p, uint32_t pos) {
     const u32x4 lo = *reinterpret_cast<const u32x4*>(p + pos);
     const u32x4 hi = *reinterpret_cast<const u32x4*>(p + (pos ^ 16u));
     return v8i32{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
   };
-  constexpr int READS = TM + TN;
+  constexpr int READS = TM + NB * TN;
   auto read_one = [&](auto q_c, auto kk_c, auto buf_c, const uint8_t* st) {
     constexpr int q = decltype(q_c)::value, kk = decltype(kk_c)::value, buf = decltype(buf_c)::value;
-    if constexpr (q < TM) af[buf][q] = read32(st + a_rd + q * 32 * 128, swz[kk]);
-    else bf[buf][q - TM] = read32(st + b_rd + (q - TM) * 32 * 128, swz[kk]);
+    if constexpr (q < TM) {
+      af[buf][q] = read32(st + a_rd + q * 32 * 128, swz[kk]);
+    } else {
+      constexpr int b = (q - TM) / TN, j = (q - TM) % TN;
+      bf[buf][b][j] = read32(st + b_rd + (b * BN + j * 32) * 128, swz[kk]);
+    }
   };
 
   // One k-step: its MFMAs (64 cycles of the matrix pipe each) with the loads LP, LP + PARTS, ...
   // of the slab being fetched (LP < 0: none) and the fragment reads of k-step RK (RK < 0: none)
   // dealt out between them, order pinned -- the scheme of gemm.hip.
-  constexpr int NM = TN * TM;
+  constexpr int NM = NB * TN * TM;
   auto step = [&](auto kk_c, auto lp_c, auto rk_c, uint32_t ld_st, bool ld_ok, const uint8_t* rd_st) {
     constexpr int kk = decltype(kk_c)::value, LP = decltype(lp_c)::value, RK = decltype(rk_c)::value;
     constexpr int NL = LP < 0 ? 0 : (LOADS - LP + PARTS - 1) / PARTS;
@@ -196,8 +270,8 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
     constexpr int S = NL + NR;
     static_for<NM>([&](auto n_c) {
       constexpr int n = decltype(n_c)::value;
-      constexpr int j = n / TM, i = n % TM;
-      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[kk][j], af[kk][i], acc[i][j], 0, 0, 0, 0, 0, 0);
+      constexpr int b = n / (TN * TM), j = n / TM % TN, i = n % TM;
+      acc[b][i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[kk][b][j], af[kk][i], acc[b][i][j], 0, 0, 0, 0, 0, 0);
       constexpr int lo = n * S / NM, hi = (n + 1) * S / NM;
       static_for<hi - lo>([&](auto d_c) {
         constexpr int q = lo + decltype(d_c)::value;
@@ -268,15 +342,20 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   // time in fp32, and stores (and reads C and the row scales) in whole runs through buffer
   // descriptors that end with the matrix, so a pass has no branches.
   constexpr int CW = BN / WN, ROWP = CW * 4 + 16, CPR = CW / 4, ITER = 32 * CPR / 64;
-  static_assert(4 * 32 * ROWP <= (int)SM::bytes && (32 * CPR) % 64 == 0 && 64 % CPR == 0, "epilogue staging");
+  static_assert(NB * 4 * 32 * ROWP <= (int)SM::bytes && (32 * CPR) % 64 == 0 && 64 % CPR == 0, "epilogue staging");
   typedef unsigned int u32v2_t __attribute__((ext_vector_type(2)));
   __syncthreads();  // every wavefront has read its last fragments
   uint8_t* ep = smem8 + wave * (32 * ROWP);
+  uint8_t* ep1 = smem8 + (4 + wave) * (32 * ROWP);  // kDual: the second product
   const int gn0 = n_base + wn * CW;
   const int gn = gn0 + (lane % CPR) * 4;  // the same 4 columns in every pass: 64 % CPR == 0
-  float4_t cs4 = float4_t{0.f, 0.f, 0.f, 0.f};
+  float4_t cs4 = float4_t{0.f, 0.f, 0.f, 0.f}, cu4 = float4_t{0.f, 0.f, 0.f, 0.f};
   if (gn < N) cs4 = *reinterpret_cast<const float4_t*>(sb + gn);
-  cs4 *= alpha;
+  if constexpr (kDual) {
+    if (gn < N) cu4 = *reinterpret_cast<const float4_t*>(sb1 + gn);
+  } else {
+    cs4 *= alpha;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int gm0 = m_base + wm * (BM / WM) + i * 32;
@@ -295,21 +374,25 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
       rs[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(s_rsrc, r * 4, 0, 0));
     }
     u32v2_t cv[ITER];
-    if (beta != 0.f) {
-      const __amdgpu_buffer_rsrc_t c_rsrc =
-          __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(C) + row0 * N, 0, recs, 0x00020000);
+    if constexpr (!kDual) {
+      if (beta != 0.f) {
+        const __amdgpu_buffer_rsrc_t c_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(C) + row0 * N, 0, recs, 0x00020000);
 #pragma unroll
-      for (int it = 0; it < ITER; ++it) cv[it] = __builtin_amdgcn_raw_buffer_load_b64(c_rsrc, off[it], 0, 0);
+        for (int it = 0; it < ITER; ++it) cv[it] = __builtin_amdgcn_raw_buffer_load_b64(c_rsrc, off[it], 0, 0);
+      }
     }
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        float4_t v;
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][qd * 4 + e];
-        *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
-      }
+        for (int qd = 0; qd < 4; ++qd) {
+          float4_t v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = acc[b][i][j][qd * 4 + e];
+          *reinterpret_cast<float4_t*>((b ? ep1 : ep) + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
+        }
     float4_t a4[ITER];
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {
@@ -319,7 +402,18 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
     auto store_group = [&](int it, float4_t v) {
       __builtin_amdgcn_raw_buffer_store_b64(u32v2_t{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3])}, d_rsrc, off[it], 0, 0);
     };
-    if (beta == 0.f) {
+    if constexpr (kDual) {
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        const int c = it * 64 + lane;
+        const float4_t u4 = *reinterpret_cast<const float4_t*>(ep1 + (c / CPR) * ROWP + (c % CPR) * 16);
+        const float4_t g = a4[it] * cs4 * rs[it], u = u4 * cu4 * rs[it];
+        float4_t v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = swiglu_rounded_f16(g[e], u[e]);
+        store_group(it, v);
+      }
+    } else if (beta == 0.f) {
 #pragma unroll
       for (int it = 0; it < ITER; ++it) store_group(it, a4[it] * cs4 * rs[it]);
     } else {
@@ -336,12 +430,12 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   }
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool kDual = false>
 static int launch_gemm_f8(const uint8_t* A, const uint8_t* B, const float* sa, const float* sb,
                           const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha, float beta,
-                          hipStream_t stream) {
-  using SM = F8Smem<BM, BN>;
-  auto kern = gemm_f8_kernel<BM, BN, WM, WN>;
+                          hipStream_t stream, const uint8_t* B1 = nullptr, const float* sb1 = nullptr) {
+  using SM = F8Smem<BM, BN, kDual ? 2 : 1>;
+  auto kern = gemm_f8_kernel<BM, BN, WM, WN, kDual>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -354,7 +448,7 @@ static int launch_gemm_f8(const uint8_t* A, const uint8_t* B, const float* sa, c
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int grid = ((tiles_m * tiles_n + 7) / 8) * 8;
-  kern<<<grid, 256, SM::bytes, stream>>>(A, B, sa, sb, C, D, M, N, K, alpha, beta, tiles_m, tiles_n);
+  kern<<<grid, 256, SM::bytes, stream>>>(A, B, B1, sa, sb, sb1, C, D, M, N, K, alpha, beta, tiles_m, tiles_n);
   return check_launch("gemm_f8 launch");
 }
 
@@ -395,6 +489,42 @@ int nf_gemm_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, c
   return launch_gemm_f8<128, 128, 2, 2>(Aq, Bq, a_scale, b_scale, C, D, M, N, K, alpha, beta, s);
 }
 
+int nf_quantize_weight_e4m3(const uint16_t* W, uint8_t* Wq, float* col_scale, int K, int N,
+                            nf_stream_t stream) {
+  NF_REQUIRE(K > 0 && N > 0 && K % 16 == 0 && N % 8 == 0,
+             "nf_quantize_weight_e4m3: bad shape K=%d N=%d (K %% 16, N %% 8)", K, N);
+  NF_REQUIRE(W && Wq && col_scale, "nf_quantize_weight_e4m3: null pointer");
+  NF_REQUIRE(((uintptr_t)W | (uintptr_t)Wq) % 16 == 0, "nf_quantize_weight_e4m3: operands must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  weight_col_scale_kernel<<<(N + 63) / 64, 256, 0, s>>>(W, col_scale, K, N);
+  int rc = check_launch("weight_col_scale launch");
+  if (rc) return rc;
+  weight_quantize_transpose_kernel<<<dim3((K + 63) / 64, (N + 63) / 64), 256, 0, s>>>(W, col_scale, Wq, K, N);
+  return check_launch("weight_quantize_transpose launch");
+}
+
+int nf_dual_swiglu_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Gq, const float* g_scale,
+                          const uint8_t* Uq, const float* u_scale, uint16_t* out, int M, int N, int K,
+                          nf_stream_t stream) {
+  NF_REQUIRE(M >= 0 && N > 0 && K > 0, "nf_dual_swiglu_f8_f16: bad shape M=%d N=%d K=%d", M, N, K);
+  NF_REQUIRE(K % 16 == 0 && N % 8 == 0, "nf_dual_swiglu_f8_f16: K=%d must be a multiple of 16 and N=%d of 8", K, N);
+  NF_REQUIRE(M == 0 || (Aq && a_scale && Gq && g_scale && Uq && u_scale && out), "nf_dual_swiglu_f8_f16: null pointer");
+  NF_REQUIRE(((uintptr_t)Aq | (uintptr_t)Gq | (uintptr_t)Uq | (uintptr_t)g_scale | (uintptr_t)u_scale) % 16 == 0 &&
+                 (uintptr_t)out % 8 == 0,
+             "nf_dual_swiglu_f8_f16: Aq, Gq, Uq and the weight scales must be 16-byte, out 8-byte aligned");
+  NF_REQUIRE(((size_t)M + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull && ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull,
+             "nf_dual_swiglu_f8_f16: an operand of %d x %d x %d exceeds the 4 GiB buffer-addressing limit", M, N, K);
+  if (M == 0) return NF_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (M <= 64)
+    return launch_gemm_f8<64, 128, 2, 2, true>(Aq, Gq, a_scale, g_scale, nullptr, out, M, N, K, 1.f, 0.f, s, Uq, u_scale);
+  const long long t256 = (long long)((M + 255) / 256) * ((N + 127) / 128);
+  const int tail = M % 256;  // rows in the last 256-row tile: half-empty tiles go to the 128-row kernel
+  if (t256 >= 192 && (tail == 0 || tail > 128))
+    return launch_gemm_f8<256, 128, 2, 2, true>(Aq, Gq, a_scale, g_scale, nullptr, out, M, N, K, 1.f, 0.f, s, Uq, u_scale);
+  return launch_gemm_f8<128, 128, 2, 2, true>(Aq, Gq, a_scale, g_scale, nullptr, out, M, N, K, 1.f, 0.f, s, Uq, u_scale);
+}
+
 size_t nf_gemm_f8w_workspace_bytes(int M, int K) {
   if (M <= 0 || K <= 0) return 0;
   return ((size_t)M * K + 255) / 256 * 256 + (size_t)M * sizeof(float);
@@ -416,6 +546,24 @@ int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* b_scale, 
   int rc = nf_quantize_rows_e4m3(A, Aq, sa, M, K, stream);
   if (rc) return rc;
   return nf_gemm_f8_f16(Aq, sa, Bq, b_scale, C, D, M, N, K, alpha, beta, stream);
+}
+
+int nf_dual_swiglu_f8w_f16(const uint16_t* A, const uint8_t* Gq, const float* g_scale, const uint8_t* Uq,
+                           const float* u_scale, uint16_t* out, int M, int N, int K, void* workspace,
+                           size_t workspace_bytes, nf_stream_t stream) {
+  NF_REQUIRE(M >= 0 && K > 0, "nf_dual_swiglu_f8w_f16: bad shape M=%d K=%d", M, K);
+  if (M == 0) return NF_OK;
+  const size_t need = nf_gemm_f8w_workspace_bytes(M, K);
+  if (!workspace || workspace_bytes < need) {
+    set_error("nf_dual_swiglu_f8w_f16: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    return NF_ERR_WORKSPACE;
+  }
+  NF_REQUIRE((uintptr_t)workspace % 16 == 0, "nf_dual_swiglu_f8w_f16: workspace must be 16-byte aligned");
+  uint8_t* Aq = static_cast<uint8_t*>(workspace);
+  float* sa = reinterpret_cast<float*>(Aq + ((size_t)M * K + 255) / 256 * 256);
+  int rc = nf_quantize_rows_e4m3(A, Aq, sa, M, K, stream);
+  if (rc) return rc;
+  return nf_dual_swiglu_f8_f16(Aq, sa, Gq, g_scale, Uq, u_scale, out, M, N, K, stream);
 }
 
 }  // extern "C"

@@ -62,9 +62,13 @@ class Engine:
 
     def __init__(self, shape: synth.ModelShape, pipeline_type=P.PipelineType.LOCAL, *, global_batch,
                  nano1, kqv1=None, kqv3=None, kv_pages, weights=None, kv_pools=None, run_layer=None,
-                 distinct_layers=None, seed=0, profiling=False, kv_fill="randn"):
+                 distinct_layers=None, seed=0, profiling=False, kv_fill="randn", weight_format="f16"):
         self.shape = shape
         self.pipeline_type = pipeline_type
+        # "e4m3": the five GEMM weights of every layer are quantised on the device as they are
+        # made (per-output-channel scales) and only the fp8 form is kept
+        self.weight_format = P.WeightFormat[weight_format.upper()]
+        P.setWeightFormat(self.weight_format)
         self.T = global_batch
         self.nano1 = nano1
         self.kqv1 = nano1 if kqv1 is None else kqv1
@@ -98,19 +102,32 @@ class Engine:
         mw.lm_head = _weight(self.t["lm_head"], H, V)
         mw.embedding = _weight(self.t["embedding"], V, H)
         mw.model_layernorm = _weight(self.t["model_norm"], H, 1)
+        e4m3 = self.weight_format == P.WeightFormat.E4M3
+
+        def gemm_weight(key, layer, rows, cols):
+            """(tensor to keep alive, VortexWeight) of a [rows = K, cols = N] GEMM weight."""
+            t = mk(key, layer, rows, cols)
+            if not e4m3:
+                return t, _weight(t, cols, rows)
+            blob = torch.empty((P.e4m3WeightBytes(cols, rows),), dtype=torch.uint8, device=self.dev)
+            P.quantizeWeightE4M3(t.data_ptr(), blob.data_ptr(), cols, rows, torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()              # t is dropped on return
+            w = P.VortexWeight()
+            w.setPtr(blob.data_ptr())
+            w.N, w.K = cols, rows
+            return blob, w
+
         for l in range(self.layers):
-            lt = {"w_kqv": mk("w_kqv", l, H, kqv_n), "w_o": mk("w_o", l, shape.Hq * d, H),
-                  "w_gate": mk("w_gate", l, H, F), "w_up": mk("w_up", l, H, F),
-                  "w_down": mk("w_down", l, F, H), "ln_attn": mk("ln_attn", l, 1, H, 0.02, 1.0),
-                  "ln_ffn": mk("ln_ffn", l, 1, H, 0.02, 1.0)}
+            lt, lw = {}, P.VortexLayerWeight()
+            lt["w_kqv"], lw.W_KQV = gemm_weight("w_kqv", l, H, kqv_n)
+            lt["w_o"], lw.W_O1 = gemm_weight("w_o", l, shape.Hq * d, H)
+            lw.W_O2 = lw.W_O1
+            lt["w_gate"], lw.W_G = gemm_weight("w_gate", l, H, F)
+            lt["w_up"], lw.W_U = gemm_weight("w_up", l, H, F)
+            lt["w_down"], lw.W_D = gemm_weight("w_down", l, F, H)
+            lt["ln_attn"] = mk("ln_attn", l, 1, H, 0.02, 1.0)
+            lt["ln_ffn"] = mk("ln_ffn", l, 1, H, 0.02, 1.0)
             self.t["layers"].append(lt)
-            lw = P.VortexLayerWeight()
-            lw.W_O1 = _weight(lt["w_o"], H, shape.Hq * d)
-            lw.W_O2 = _weight(lt["w_o"], H, shape.Hq * d)
-            lw.W_U = _weight(lt["w_up"], F, H)
-            lw.W_G = _weight(lt["w_gate"], F, H)
-            lw.W_D = _weight(lt["w_down"], H, F)
-            lw.W_KQV = _weight(lt["w_kqv"], kqv_n, H)
             if pipeline_type.has_kqv_bias:
                 # biases of real checkpoints (Qwen2) reach tens in a few channels; N(0, 0.5) here
                 lt["b_kqv"] = mk("b_kqv", l, 1, kqv_n, 0.5)

@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
 SYMBOLS = [
     "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16", "nf_gemm_bias_f16",
     "nf_dual_swiglu_f16", "nf_gemm_bf16", "nf_dual_swiglu_bf16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
+    "nf_quantize_weight_e4m3", "nf_dual_swiglu_f8_f16", "nf_dual_swiglu_f8w_f16",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
 ]
@@ -53,6 +54,9 @@ def lib() -> C.CDLL:
         l.nf_gemm_f8w_workspace_bytes.restype = C.c_size_t
         l.nf_gemm_f8w_workspace_bytes.argtypes = [i32, i32]
         l.nf_gemm_f8w_f16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp, C.c_size_t, vp]
+        l.nf_quantize_weight_e4m3.argtypes = [vp, vp, vp, i32, i32, vp]
+        l.nf_dual_swiglu_f8_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp]
+        l.nf_dual_swiglu_f8w_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, C.c_size_t, vp]
         l.nf_rope_append_f16.argtypes = [vp] * 7 + [i32] * 5 + [f32] * 4 + [vp]
         l.nf_attention_workspace_bytes.restype = sz
         l.nf_attention_workspace_bytes.argtypes = [i32, i32, i32]
@@ -190,6 +194,44 @@ def gemm_f8w(A, Bq_nk, b_scale, Cmat=None, alpha=1.0, beta=0.0, out=None, worksp
     _check(lib().nf_gemm_f8w_f16(_p(A), _p(Bq_nk), _p(b_scale), _p(Cmat), _p(out), M, N, K, alpha, beta,
                                  _p(workspace), workspace.numel() * workspace.element_size(), _stream()),
            "nf_gemm_f8w_f16")
+    return out
+
+
+def quantize_weight_e4m3(W):
+    """W fp16 [K,N] (the pipeline's weight orientation) -> (Wq e4m3 bytes [N,K], col_scale fp32 [N])."""
+    _f16(W)
+    Kd, N = W.shape
+    Wq = torch.empty((N, Kd), dtype=torch.uint8, device=W.device)
+    scale = torch.empty((N,), dtype=torch.float32, device=W.device)
+    _check(lib().nf_quantize_weight_e4m3(_p(W), _p(Wq), _p(scale), Kd, N, _stream()), "nf_quantize_weight_e4m3")
+    return Wq, scale
+
+
+def dual_swiglu_f8(Aq, a_scale, Gq, g_scale, Uq, u_scale, out=None):
+    assert Aq.dtype == torch.uint8 and Gq.dtype == torch.uint8 and Uq.dtype == torch.uint8
+    M, Kd = Aq.shape
+    N = Gq.shape[0]
+    assert tuple(Gq.shape) == (N, Kd) and tuple(Uq.shape) == (N, Kd)
+    assert a_scale.numel() == M and g_scale.numel() == N and u_scale.numel() == N
+    out = torch.empty((M, N), dtype=torch.float16, device=Aq.device) if out is None else out
+    _check(lib().nf_dual_swiglu_f8_f16(_p(Aq), _p(a_scale), _p(Gq), _p(g_scale), _p(Uq), _p(u_scale), _p(out),
+                                       M, N, Kd, _stream()), "nf_dual_swiglu_f8_f16")
+    return out
+
+
+def dual_swiglu_f8w(A, Gq, g_scale, Uq, u_scale, out=None, workspace=None):
+    """fp16 activations [M,K] against e4m3 gate/up weights [N,K] with per-output-channel scales."""
+    _f16(A)
+    M, Kd = A.shape
+    N = Gq.shape[0]
+    assert tuple(Gq.shape) == (N, Kd) and tuple(Uq.shape) == (N, Kd)
+    need = lib().nf_gemm_f8w_workspace_bytes(M, Kd)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
+    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
+    _check(lib().nf_dual_swiglu_f8w_f16(_p(A), _p(Gq), _p(g_scale), _p(Uq), _p(u_scale), _p(out), M, N, Kd,
+                                        _p(workspace), workspace.numel() * workspace.element_size(), _stream()),
+           "nf_dual_swiglu_f8w_f16")
     return out
 
 

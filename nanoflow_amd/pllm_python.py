@@ -193,6 +193,8 @@ SYMBOLS = [
     "pllm_run", "pllm_run_async", "pllm_run_async_wait", "pllm_get_pipeline_output",
     "pllm_finalize", "pllm_build_input_tokens", "pllm_set_profiling", "pllm_set_profiling_stride", "pllm_get_timings",
     "pllm_reset_timings", "pllm_debug_buffer", "pllm_set_graph_mode", "pllm_get_graph_counters",
+    "pllm_set_weight_format", "pllm_get_weight_format", "pllm_e4m3_weight_bytes", "pllm_e4m3_weight_scale_offset",
+    "pllm_quantize_weight_e4m3",
 ]
 
 _lib = None
@@ -223,6 +225,12 @@ def lib() -> C.CDLL:
         l.pllm_get_pipeline_output.argtypes = [C.POINTER(_i32p), C.POINTER(C.c_int)]
         l.pllm_build_input_tokens.argtypes = [_i32p, C.c_int, _i32p, C.c_int, _i32p, C.c_int, _i32p]
         l.pllm_set_profiling.argtypes = [C.c_int]
+        l.pllm_set_weight_format.argtypes = [C.c_int]
+        l.pllm_e4m3_weight_bytes.restype = C.c_size_t
+        l.pllm_e4m3_weight_bytes.argtypes = [C.c_int, C.c_int]
+        l.pllm_e4m3_weight_scale_offset.restype = C.c_size_t
+        l.pllm_e4m3_weight_scale_offset.argtypes = [C.c_int, C.c_int]
+        l.pllm_quantize_weight_e4m3.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         l.pllm_get_timings.argtypes = [C.POINTER(PipelineTimings)]
         l.pllm_debug_buffer.argtypes = [C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_int),
                                         C.POINTER(C.c_int)]
@@ -351,6 +359,35 @@ def buildInputTokens(prev_output, keep_token_list, prefill_tokens) -> np.ndarray
     if n < 0:
         _check(n, "buildInputTokens")
     return out[:n]
+
+
+class WeightFormat(enum.IntEnum):
+    """Storage of the five per-layer GEMM weights in the init data (include/nanoflow_pllm.h)."""
+    F16 = 0
+    E4M3 = 1
+
+
+def setWeightFormat(fmt):
+    """Call before init.  E4M3: VortexWeight.ptr of W_KQV, W_O1/W_O2, W_G, W_U, W_D points at N*K e4m3
+    bytes [N][K] + N fp32 scales (e4m3WeightBytes / quantizeWeightE4M3)."""
+    _check(lib().pllm_set_weight_format(int(fmt)), "setWeightFormat")
+
+
+def getWeightFormat() -> WeightFormat:
+    return WeightFormat(lib().pllm_get_weight_format())
+
+
+def e4m3WeightBytes(N: int, K: int) -> int:
+    return int(lib().pllm_e4m3_weight_bytes(N, K))
+
+
+def e4m3WeightScaleOffset(N: int, K: int) -> int:
+    return int(lib().pllm_e4m3_weight_scale_offset(N, K))
+
+
+def quantizeWeightE4M3(w_f16_ptr: int, out_ptr: int, N: int, K: int, stream: int = 0):
+    """Device fp16 [K][N] weight -> the E4M3 form at out_ptr (e4m3WeightBytes(N, K) bytes)."""
+    _check(lib().pllm_quantize_weight_e4m3(w_f16_ptr, out_ptr, N, K, stream), "quantizeWeightE4M3")
 
 
 def setProfilingStride(stride: int):

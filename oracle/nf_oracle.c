@@ -223,6 +223,18 @@ NFO_API void nfo_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bg, const ui
   }
 }
 
+/* out = half(silu(g) * u) on fp16 inputs, fp32 arithmetic: the tail of the dual epilogue above,
+ * for the fp8 variant of the gate/up pair, whose two products come from nfo_gemm_f8f8_f16 or
+ * nfo_gemm_f8w_f16 already rounded to fp16. */
+NFO_API void nfo_silu_mul_f16(const uint16_t* g16, const uint16_t* u16, uint16_t* out, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; ++i) {
+    float g = h2f(g16[i]), u = h2f(u16[i]);
+    float silu = g / (1.f + expf(-g));
+    out[i] = f2h(silu * u);
+  }
+}
+
 /* fp8 e4m3 (OCP, finite-only, max 448) weight GEMM with per-output-channel fp32 scale:
  * D = half(alpha * scale[n] * sum_k A[m,k]*dequant(Bq[k,n]) + beta*C).  There is no
  * reference implementation of this variant (the reference GEMM wrappers are

@@ -289,6 +289,59 @@ def test_gemm_f8w_within_fp8_tolerance_of_dequantised_reference(K, oracle, M, N,
     assert np.array_equal(two, got)
 
 
+@pytest.mark.parametrize("Kd,N", [(16, 8), (144, 136), (512, 6144), (4096, 1000), (1040, 72)])
+def test_quantize_weight_e4m3_is_bit_exact(K, oracle, Kd, N):
+    rng = np.random.default_rng(Kd + N)
+    W = (rng.normal(0, 0.02, (Kd, N)) * rng.uniform(0.1, 10, (1, N))).astype(np.float16)
+    if N > 3:
+        W[:, 3] = 0                                # all-zero output channel: scale 1, codes 0
+    q_ref, s_ref = oracle.quantize_weight_e4m3(W)
+    q, s = K.quantize_weight_e4m3(dev(W))
+    assert np.array_equal(host(s), s_ref)
+    assert np.array_equal(host(q), q_ref)
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 8, 16), (37, 136, 144), (64, 512, 256), (130, 520, 1040), (300, 264, 4096),
+                                     (256, 24576, 128), (1930, 3200, 272), (2048, 3072, 128)])
+def test_dual_swiglu_f8_matches_oracle(K, oracle, M, N, K_):
+    """The fp8 gate/up pair: products exact, fp32 accumulation, both rounded to fp16 before
+    SiLU-mul.  A product that lands on an fp16 rounding boundary may round the other way than the
+    oracle's double-precision sum, which moves g or u by a whole fp16 step (2^-10 relative) and
+    the output with it: bounded at twice the fp16 GEMM tolerance, as for the bf16 pair."""
+    rng = np.random.default_rng(M + N + K_)
+    fin = np.array([c for c in range(256) if (c & 0x7F) < 0x50], np.uint8)       # magnitudes below 8
+    Aq, Gq, Uq = rng.choice(fin, (M, K_)), rng.choice(fin, (N, K_)), rng.choice(fin, (N, K_))
+    sa = rng.uniform(0.05, 0.2, M).astype(np.float32)
+    sg = (rng.uniform(0.5, 2, N) / np.sqrt(K_)).astype(np.float32)
+    su = (rng.uniform(0.5, 2, N) / np.sqrt(K_)).astype(np.float32)
+    ref = oracle.dual_swiglu_f8f8(Aq, sa, Gq, sg, Uq, su)
+    got = host(K.dual_swiglu_f8(dev(Aq), dev(sa), dev(Gq), dev(sg), dev(Uq), dev(su)))
+    assert_close(got, ref, 2 * RTOL, what=f"dual_swiglu_f8 {M}x{N}x{K_}")
+    # swapping gate and up must change the result (silu is taken of the first)
+    if M * N > 64:
+        assert not np.array_equal(got, host(K.dual_swiglu_f8(dev(Aq), dev(sa), dev(Uq), dev(su), dev(Gq), dev(sg))))
+
+
+def test_dual_swiglu_f8w_is_quantise_then_dual(K, oracle):
+    rng = np.random.default_rng(11)
+    M, N, K_ = 200, 1024, 4096
+    A = rng.normal(0, 1, (M, K_)).astype(np.float16)
+    Wg = rng.normal(0, 0.02, (K_, N)).astype(np.float16)
+    Wu = rng.normal(0, 0.02, (K_, N)).astype(np.float16)
+    Gq, sg = K.quantize_weight_e4m3(dev(Wg))
+    Uq, su = K.quantize_weight_e4m3(dev(Wu))
+    got = host(K.dual_swiglu_f8w(dev(A), Gq, sg, Uq, su))
+    q, s = K.quantize_rows_e4m3(dev(A))
+    assert np.array_equal(got, host(K.dual_swiglu_f8(q, s, Gq, sg, Uq, su)))
+    # against fp16 activations on the dequantised weights: the output is a product of two GEMM
+    # results that are each within the fp8 tolerance, so it is held to twice that
+    g = oracle.gemm_f8w(A, np.ascontiguousarray(host(Gq).T), host(sg))
+    u = oracle.gemm_f8w(A, np.ascontiguousarray(host(Uq).T), host(su))
+    ref = oracle.silu_mul(g, u)
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    assert err.max() <= 2 * F8_RTOL * np.abs(ref).max(), (err.max(), np.abs(ref).max())
+
+
 def test_gemm_f8w_rejects_short_workspace(K):
     from nanoflow_amd import kernels
     A = torch.zeros((8, 64), dtype=torch.float16, device="cuda")

@@ -193,6 +193,87 @@ def test_kqv_bias_schedules_match_oracle(oracle, case):
         assert all(np.array_equal(a, b) for a, b in zip(kvz, kvp)), (bias_pt, "zero bias, KV")
 
 
+@pytest.mark.parametrize("case", ["decode_crosses_border", "prefill_straddles_border"])
+def test_fp8_weight_pipelines_match_oracle(oracle, case):
+    """The three schedules with the five per-layer GEMM weights in e4m3 (quantised on the device from
+    the same fp16 weights, per-output-channel scales), against the oracle's forward with the same
+    arithmetic (input rows re-quantised per GEMM, fp8 x fp8 products) and against fp16 activations
+    on the dequantised weights, the definition the fp8 tolerance of 3e-2 per GEMM is stated for.
+
+    Re-quantising activations makes the forward discontinuous: a one-ulp fp16 difference upstream
+    flips e4m3 codes (steps of 6-12 %) downstream.  Nudging the oracle's own norm weights by one
+    ulp moves its output by 1.3 % rms / 2.4 % of the largest magnitude on this model, so agreement
+    between two correct implementations is bounded here at 3e-2 rms and 8e-2 of the largest
+    magnitude (1e-1 against fp16 activations); every operator is held to its tight bound on
+    identical inputs in tests/test_gpu_kernels.py.  The weights are N(0, 0.02) unscaled: the x3
+    weights of the fp16 tests make attention so peaked that fp8 noise on q and k alone moves the
+    output by 10 %."""
+    from nanoflow_amd import engine, pllm_python as P
+    T, nano1, dlens, chunks = CASES[case]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = synth.make_weights(shape, seed=0)
+    w["embedding"] = (w["embedding"].astype(np.float32) * 30).astype(np.float16)
+
+    def rms_rel(got, ref):
+        g, r = got.astype(np.float64), ref.astype(np.float64)
+        return np.sqrt(((g - r) ** 2).mean() / (r ** 2).mean())
+    wq = oracle.quantize_model_weights(w)
+    b1 = synth.make_batch(dlens, chunks, vocab=shape.vocab, seed=21, extra_pages=40)
+    rng = np.random.default_rng(5)
+    pools0 = [synth.make_kv_pool(b1.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok1 = b1.input_tokens.copy()
+    tok1[:b1.decodePrefillBorder] = 1
+    d1 = b1.as_dict()
+    d1["input_tokens"] = tok1
+    pools_ref = [p.copy() for p in pools0]
+    hid, log, samp = oracle.decoder_forward_f8(shape.as_dict(), w, wq, pools_ref, d1, "e4m3", want_logits=True)
+    hid16, _, _ = oracle.decoder_forward_f8(shape.as_dict(), w, wq, [p.copy() for p in pools0], d1, "f16")
+    keep = np.ones(b1.decodePrefillBorder, np.int32)
+    results = {}
+    try:
+        for pt in (P.PipelineType.NON_OVERLAP_LOCAL, P.PipelineType.NANOBATCH_LOCAL, P.PipelineType.LOCAL):
+            print(f"case={case} pipeline={pt.name} weights=e4m3", flush=True)
+            with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=max(nano1 // 2, 1), kqv3=(T - nano1) // 2,
+                               kv_pages=b1.num_pages, weights=w, kv_pools=pools0, weight_format="e4m3") as e:
+                e.update(b1, keep_token_list=keep)
+                s = e.run()
+                h = e.buffer("hidden").cpu().numpy()[:b1.tokens]
+                l = e.buffer("logits").cpu().numpy()[:b1.req_num]
+                kv = [p[:b1.num_pages].cpu().numpy() for p in e.kv]
+            results[pt] = (s, h)
+            print(f"  hidden: rms {rms_rel(h, hid):.4f} max {_max_rel(h, hid):.4f}; vs fp16 activations "
+                  f"{_max_rel(h, hid16):.4f}; logits rms {rms_rel(l, log):.4f}", flush=True)
+            assert rms_rel(h, hid) < 3e-2 and _max_rel(h, hid) < 8e-2, (pt, "hidden", rms_rel(h, hid), _max_rel(h, hid))
+            assert rms_rel(l, log) < 3e-2 and _max_rel(l, log) < 8e-2, (pt, "logits", rms_rel(l, log), _max_rel(l, log))
+            assert _max_rel(h, hid16) < 1e-1, (pt, "hidden vs fp16 activations", _max_rel(h, hid16))
+            top2 = np.sort(log.astype(np.float32), axis=1)[:, -2:]
+            clear = (top2[:, 1] - top2[:, 0]) > 2 * 8e-2 * np.abs(log.astype(np.float32)).max()
+            assert np.array_equal(s[clear], samp[clear]), (pt, "samples")
+            for layer in range(shape.layers):
+                assert np.array_equal((pools_ref[layer] != pools0[layer]).any(axis=(3, 4)),
+                                      (kv[layer] != pools0[layer]).any(axis=(3, 4))), (pt, layer, "KV slots written")
+                assert _max_rel(kv[layer], pools_ref[layer]) < 8e-2, (pt, layer, "KV contents")
+    finally:
+        P.setWeightFormat(P.WeightFormat.F16)
+    base = results[P.PipelineType.NON_OVERLAP_LOCAL]
+    for pt in (P.PipelineType.NANOBATCH_LOCAL, P.PipelineType.LOCAL):
+        # per-row activation scales and a fixed k order: splitting the rows differently changes no
+        # bit of a row, which is what keeps the schedules comparable despite the discontinuity
+        assert np.array_equal(results[pt][0], base[0]), (pt, "samples differ between schedules")
+        assert np.array_equal(results[pt][1], base[1]), (pt, "hidden differs between schedules")
+
+
+def test_fp8_weights_and_kqv_bias_do_not_combine():
+    from nanoflow_amd import engine, pllm_python as P
+    shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)
+    try:
+        with pytest.raises(P.NanoflowPipelineError, match="fp16 weights only"):
+            engine.Engine(shape, P.PipelineType.KQVBIAS, global_batch=32, nano1=16, kv_pages=64, weight_format="e4m3")
+    finally:
+        P.finalize()
+        P.setWeightFormat(P.WeightFormat.F16)
+
+
 def test_unsupported_pipeline_types_are_rejected():
     from nanoflow_amd import engine, pllm_python as P
     shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)

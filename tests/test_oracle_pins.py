@@ -223,6 +223,77 @@ def test_gemm_f8f8_matches_float64(oracle):
     assert np.array_equal(g1, g2.T)
 
 
+def test_silu_mul_and_fp8_dual_closed_form(oracle):
+    rng = np.random.default_rng(4)
+    g = rng.normal(0, 3, 4096).astype(np.float16)
+    u = rng.normal(0, 3, 4096).astype(np.float16)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    ref = g64 / (1 + np.exp(-g64)) * u64
+    got = oracle.silu_mul(g, u).astype(np.float64)
+    assert np.abs(got - ref).max() <= 1e-3 * np.abs(ref).max()
+    assert np.array_equal(oracle.silu_mul(np.zeros(8, np.float16), u[:8]), np.zeros(8, np.float16))   # silu(0) = 0
+    # the order of the operands matters: silu is taken of the first
+    assert not np.array_equal(oracle.silu_mul(g, u), oracle.silu_mul(u, g))
+    # the fp8 gate/up pair = the two fp8 products, rounded to fp16, through that function; against
+    # float64 on the dequantised operands
+    M, N, K = 7, 24, 96
+    fin = np.array(_finite_codes(), np.uint8)
+    small = fin[(fin & 0x7F) < 0x50]                       # magnitudes below 8: keeps products in fp16 range
+    Aq, Gq, Uq = rng.choice(small, (M, K)), rng.choice(small, (N, K)), rng.choice(small, (N, K))
+    sa = rng.uniform(0.05, 0.2, M).astype(np.float32)
+    sg, su = rng.uniform(0.01, 0.05, N).astype(np.float32), rng.uniform(0.01, 0.05, N).astype(np.float32)
+    lut = np.array([oracle.e4m3_to_float(c) if (c & 0x7F) != 0x7F else 0.0 for c in range(256)])
+    g64 = (sa[:, None] * sg[None, :]).astype(np.float64) * (lut[Aq] @ lut[Gq].T)
+    u64 = (sa[:, None] * su[None, :]).astype(np.float64) * (lut[Aq] @ lut[Uq].T)
+    ref = g64 / (1 + np.exp(-g64)) * u64
+    got = oracle.dual_swiglu_f8f8(Aq, sa, Gq, sg, Uq, su).astype(np.float64)
+    assert np.abs(got - ref).max() <= 3e-3 * np.abs(ref).max()
+
+
+def test_quantize_weight_is_the_row_quantiser_on_the_transpose(oracle):
+    rng = np.random.default_rng(5)
+    W = rng.normal(0, 0.02, (48, 24)).astype(np.float16)         # [K, N]
+    W[:, 3] = 0                                                   # an all-zero output channel
+    Wq, sc = oracle.quantize_weight_e4m3(W)
+    assert Wq.shape == (24, 48) and sc.shape == (24,)
+    amax = np.abs(W.astype(np.float32)).max(axis=0)
+    assert sc[3] == 1.0 and not Wq[3].any()
+    live = np.arange(24) != 3
+    assert np.array_equal(sc[live], (amax / np.float32(448.0))[live])
+    assert np.array_equal((Wq[live] & 0x7F).max(axis=1), np.full(23, 0x7E))    # each channel's max maps to 448
+    deq = np.vectorize(oracle.e4m3_to_float)(Wq) * sc[:, None]                  # [N, K]
+    assert np.abs(deq.T - W.astype(np.float32)).max() <= amax.max() * 2.0 ** -4
+
+
+def test_decoder_forward_f8_vs_float64_model_on_dequantised_weights(oracle):
+    """Both activation modes of the fp8 forward against the independent float64 model run on the
+    dequantised weights: fp16 activations within the fp16 pipeline's own error; fp8 activations
+    (each GEMM input re-quantised per row, 3 mantissa bits) within 3e-2 per GEMM, which chained
+    through the 8 fp8 GEMMs of two layers is bounded here at 1e-1 of the largest magnitude."""
+    shape = synth.tiny_shape(layers=2, vocab=512, Hq=4, Hkv=2, ffn=384, hidden=256)
+    w = synth.make_weights(shape, seed=0)
+    for k in ("w_kqv", "w_o", "w_gate", "w_up", "w_down"):
+        w[k] = [(a.astype(np.float32) * 3).astype(np.float16) for a in w[k]]
+    w["embedding"] = (w["embedding"].astype(np.float32) * 30).astype(np.float16)
+    wq = oracle.quantize_model_weights(w)
+    lut = np.array([oracle.e4m3_to_float(c) for c in range(256)], np.float64)
+    w_deq = dict(w)
+    for k in oracle.FP8_LAYER_WEIGHTS:
+        w_deq[k] = [(lut[q] * s[:, None].astype(np.float64)).T for q, s in wq[k]]      # float64 [K, N]
+    b = synth.make_batch([17, 40, 3], [(0, 21), (16, 10)], vocab=shape.vocab, seed=7, extra_pages=2)
+    rng = np.random.default_rng(1)
+    pools = [synth.make_kv_pool(b.num_pages, shape, rng) for _ in range(shape.layers)]
+    ref_x, ref_logits = _numpy_decoder_f64(shape, w_deq, [p.copy() for p in pools], b)
+    cfg = shape.as_dict()
+    h16, l16, _ = oracle.decoder_forward_f8(cfg, w, wq, [p.copy() for p in pools], b.as_dict(), "f16", want_logits=True)
+    assert rel_err(h16, ref_x) < 4e-3 and rel_err(l16, ref_logits) < 6e-3
+    h8, l8, s8 = oracle.decoder_forward_f8(cfg, w, wq, [p.copy() for p in pools], b.as_dict(), "e4m3", want_logits=True)
+    assert 1e-2 < rel_err(h8, ref_x) < 1e-1 and rel_err(l8, ref_logits) < 1e-1
+    # the quantisation is visible: the fp16-weight forward differs from both by more than fp16 noise
+    h_plain, _, _ = oracle.decoder_forward(cfg, w, [p.copy() for p in pools], b.as_dict())
+    assert rel_err(h_plain, ref_x) > 6e-3
+
+
 def test_rmsnorm_closed_form(oracle):
     rng = np.random.default_rng(5)
     x = synth.normal_f16(rng, (11, 256), 3.0)
