@@ -35,6 +35,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0       # dense fp16
+MFMA_FP8_PEAK_TFLOPS = 5000.0   # dense fp8
 A100_PUBLISHED_TOKENS_PER_S = 12756.0   # reference, 1x A100 80GB, same offline workload
 # HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
 # by what the same counter reads for a 1 GiB device copy), as a ratio to the algorithmic bytes of
@@ -122,30 +123,38 @@ def _attention_roofline(tm, bytes_per_launch, name="roofline"):
 GEMM_TRAFFIC_RATIO = 2.66
 
 
-def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows):
-    """fp16 operands once plus outputs (and the residual operand of O and down) of one cycle's dense
-    GEMMs, averaged over its launches (4 per layer + the LM head)."""
+def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows, weight_bytes=2):
+    """Operands once plus outputs (and the residual operand of O and down) of one cycle's dense
+    GEMMs, averaged over its launches (4 per layer + the LM head).  Activations are fp16; the
+    per-layer weights take weight_bytes per element (1 for e4m3), the LM head 2."""
     H, F, V = shape.hidden, shape.ffn, shape.vocab
     hq = shape.Hq * shape.d
-    per_layer = (rows * H + H * shape.kqv_n + rows * shape.kqv_n            # QKV
-                 + rows * hq + hq * H + 2 * rows * H                         # O (+ C)
-                 + rows * H + 2 * H * F + rows * F                           # gate/up
-                 + rows * F + F * H + 2 * rows * H)                          # down (+ C)
+    act = (rows * H + rows * shape.kqv_n            # QKV
+           + rows * hq + 2 * rows * H               # O (+ C)
+           + rows * H + rows * F                    # gate/up
+           + rows * F + 2 * rows * H)               # down (+ C)
+    wts = H * shape.kqv_n + hq * H + 2 * H * F + F * H
     m_lm = (sampled_rows + 127) // 128 * 128
-    total = 2 * (shape.layers * per_layer + m_lm * H + H * V + m_lm * V)
+    total = shape.layers * (2 * act + weight_bytes * wts) + 2 * (m_lm * H + H * V + m_lm * V)
     return total / (4 * shape.layers + 1)
 
 
-def _gemm_roofline(tm, alg_bytes_per_launch=None):
+def _gemm_roofline(tm, alg_bytes_per_launch=None, fp8_share=0.0):
+    """fp8_share: the fraction of the timed GEMM flops that runs on the fp8 matrix cores (the
+    per-layer GEMMs with e4m3 weights; the LM head stays fp16).  The peak the launches are priced
+    against is then the flop-weighted blend of the two published peaks."""
     n = max(tm.gemm_launches, 1)
     avg_ms = tm.gemm_ms / n
     flop_per_launch = tm.gemm_flop / n
     achieved = flop_per_launch / (avg_ms * 1e-3) / 1e12 if avg_ms > 0 else 0.0
+    peak = 1.0 / (fp8_share / MFMA_FP8_PEAK_TFLOPS + (1.0 - fp8_share) / MFMA_PEAK_TFLOPS)
     return {
-        "kernel": "gemm_f16_kernel / dual_swiglu_f16_kernel (all dense GEMM launches of the iteration)",
-        "bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-        "frac": achieved / MFMA_PEAK_TFLOPS,
-        "traffic": None if alg_bytes_per_launch is None else alg_bytes_per_launch * GEMM_TRAFFIC_RATIO,
+        "kernel": ("gemm_f16_kernel / dual_swiglu_f16_kernel (all dense GEMM launches of the iteration)" if not fp8_share
+                   else "gemm_f8_kernel incl. the fused gate/up variant (e4m3 weights, activations quantised per "
+                        "launch; the quantiser's time is not in these launches) + the fp16 LM head"),
+        "bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+        "frac": achieved / peak,
+        "traffic": None if alg_bytes_per_launch is None or fp8_share else alg_bytes_per_launch * GEMM_TRAFFIC_RATIO,
         "algorithmic_bytes_per_launch": alg_bytes_per_launch,
         "algorithmic_flop_per_launch": flop_per_launch, "avg_launch_ms": avg_ms,
         "launches_timed": int(tm.gemm_launches),
@@ -156,11 +165,13 @@ def run_iteration(args):
     import torch
     from nanoflow_amd import engine, synth, pllm_python as P
     assert torch.cuda.is_available(), "bench.py needs the MI355X (no CPU path)"
-    shape = synth.LLAMA3_8B
+    shape = synth.LLAMA3_70B if args.shape == "70b" else synth.LLAMA3_8B
+    wb = 1 if args.weights == "e4m3" else 2                    # bytes per element of the per-layer GEMM weights
+    shape_name = "Llama-3-70B" if args.shape == "70b" else "Llama-3-8B"
     T = 2048
     steps = args.steps or 5
     warmup = 2 if args.warmup is None else args.warmup
-    batch = synth.config2_batch(seed=args.seed)
+    batch = synth.config2_batch(seed=args.seed, vocab=shape.vocab)
     assert batch.tokens == T
     pages = batch.num_pages
 
@@ -168,14 +179,15 @@ def run_iteration(args):
     # modulo `distinct` (the reference's own run_layer > model_layer device).
     free_b, total_b = torch.cuda.mem_get_info()
     per_layer = pages * 2 * 16 * shape.Hkv * shape.d * 2 + \
-        2 * (shape.hidden * (shape.kqv_n + shape.Hq * shape.d + 2 * shape.ffn) + shape.ffn * shape.hidden)
+        wb * (shape.hidden * (shape.kqv_n + shape.Hq * shape.d + 2 * shape.ffn) + shape.ffn * shape.hidden)
     fixed = 2 * (2 * shape.vocab * shape.hidden) + 2 * (T * shape.hidden * 16 + T * shape.vocab * 2) + (4 << 30)
     distinct = args.distinct_layers or int(max(1, min(shape.layers, (free_b * 0.92 - fixed) // per_layer)))
 
     t_setup = time.perf_counter()
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, run_layer=shape.layers,
-                        distinct_layers=distinct, seed=args.seed, profiling=args.profile_level)
+                        distinct_layers=distinct, seed=args.seed, profiling=args.profile_level,
+                        weight_format=args.weights)
     P.setGraphMode(args.graph)
     eng.update(batch)
     torch.cuda.synchronize()
@@ -204,17 +216,21 @@ def run_iteration(args):
     nd = batch.decodePrefillBorder
     groups = synth.gemv_batch_split(nd, args.kqv1, args.nano1, args.kqv3) if args.pipeline != "NON_OVERLAP_LOCAL" else [nd]
     launches_per_layer = sum(1 for g in groups if g > 0)
-    bytes_per_layer = decode_attention_bytes(batch.kv_len[:nd])
-    flops = gemm_flops_per_iteration(shape, T, min((batch.req_num + 127) // 128 * 128, T), shape.layers)
+    bytes_per_layer = decode_attention_bytes(batch.kv_len[:nd], shape.Hq, shape.Hkv, shape.d)
+    lm_rows = min((batch.req_num + 127) // 128 * 128, T)
+    flops = gemm_flops_per_iteration(shape, T, lm_rows, shape.layers)
+    fp8_share = 1.0 - 2.0 * lm_rows * shape.hidden * shape.vocab / flops if wb == 1 else 0.0
 
     rec = {
         "metric": "tokens/s/GPU", "value": T / (ms_per_step * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if wb == 2 else "f8e4m3 weights and GEMM inputs, f16 activations and KV",
         "data": "synthetic",
         "config": {
-            "workload": ("Llama-3-8B shape, one dense 2048-token iteration: 1792 decode tokens "
+            "workload": (f"{shape_name} shape, one dense 2048-token iteration: 1792 decode tokens "
                          "(KV U[1024,1536], page 16, permuted page table) + one 256-token prefill chunk"),
+            "weights": args.weights,
             "pipeline": args.pipeline, "global_batch": T, "nanobatch_1_size": args.nano1,
             "kqv1_size": args.kqv1, "kqv3_size": args.kqv3, "layers_executed": shape.layers,
             "distinct_layers_in_hbm": distinct, "kv_pages_per_layer": int(pages),
@@ -226,12 +242,13 @@ def run_iteration(args):
             "decode_attention_ms_per_step": tm.decode_attn_ms * tm.layer_stride / steps,
             "prefill_attention_ms_per_step": tm.prefill_attn_ms * tm.layer_stride / steps,
             "gemm_tflop_per_step": flops / 1e12,
-            "gemm_mfma_frac_if_serial": (flops / 1e12) / (max(ms_per_step, 1e-9) * 1e-3) / MFMA_PEAK_TFLOPS,
+            "gemm_mfma_frac_if_serial": (flops / 1e12) / (max(ms_per_step, 1e-9) * 1e-3) /
+            (MFMA_PEAK_TFLOPS if wb == 2 else 1.0 / (fp8_share / MFMA_FP8_PEAK_TFLOPS + (1 - fp8_share) / MFMA_PEAK_TFLOPS)),
             "setup_s": t_setup, "sampled_tokens": int(out.shape[0]),
         },
     }
     if tm.gemm_launches:
-        rec["roofline_gemm"] = _gemm_roofline(tm)
+        rec["roofline_gemm"] = _gemm_roofline(tm, fp8_share=fp8_share)
         rec["iteration"]["gemm_ms_per_step"] = tm.gemm_ms * tm.layer_stride / steps
     eng.close()
     if args.cpu_sample > 0:
@@ -243,7 +260,9 @@ def run_offline(args):
     import torch
     from nanoflow_amd import engine, synth, pllm_python as P
     assert torch.cuda.is_available(), "bench.py needs the MI355X (no CPU path)"
-    shape = synth.LLAMA3_8B
+    shape = synth.LLAMA3_70B if args.shape == "70b" else synth.LLAMA3_8B
+    wb = 1 if args.weights == "e4m3" else 2                    # bytes per element of the per-layer GEMM weights
+    shape_name = "Llama-3-70B" if args.shape == "70b" else "Llama-3-8B"
     T, n_req, in_len, out_len = 2048, args.requests, 1024, 512
     steps = args.steps or 256
     warmup = 8 if args.warmup is None else args.warmup
@@ -251,8 +270,8 @@ def run_offline(args):
     # KV pool: every layer distinct; 2 MiB per page over the 32 layers.  The trace peaks near
     # 66k pages in flight; the pool is sized to HBM with headroom, capped at 128 Ki pages.
     free_b, _ = torch.cuda.mem_get_info()
-    weight_b = 2 * (shape.layers * (shape.hidden * (shape.kqv_n + shape.Hq * shape.d + 2 * shape.ffn)
-                                    + shape.ffn * shape.hidden) + 2 * shape.vocab * shape.hidden)
+    weight_b = wb * shape.layers * (shape.hidden * (shape.kqv_n + shape.Hq * shape.d + 2 * shape.ffn)
+                                    + shape.ffn * shape.hidden) + 2 * 2 * shape.vocab * shape.hidden
     page_b = shape.layers * 2 * 16 * shape.Hkv * shape.d * 2
     pages = args.kv_pages or int(min(131072, (free_b * 0.90 - weight_b - (6 << 30)) // page_b))
     pages = pages // 64 * 64
@@ -264,7 +283,7 @@ def run_offline(args):
     P.setProfilingStride(16 if steps >= 64 else 0)
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, seed=args.seed,
-                        profiling=args.profile_level, kv_fill="zeros")
+                        profiling=args.profile_level, kv_fill="zeros", weight_format=args.weights)
     P.setGraphMode(args.graph)
     former = P.BatchFormer(pages, shape.page_size, T, args.nano1, args.kqv1, args.kqv3, in_len, out_len)
     rng = np.random.default_rng(args.seed)
@@ -297,7 +316,11 @@ def run_offline(args):
     kv_len = ((np.diff(nxt["kv_indptr"]) - 1) * shape.page_size + nxt["kv_last_page_len"])[:nd]
     groups = [g for g in nxt["gemv_batch_size"].tolist() if g > 0] if args.pipeline != "NON_OVERLAP_LOCAL" else [nd]
     launches_per_layer = max(len(groups), 1)
-    bytes_per_layer = decode_attention_bytes(kv_len) if nd else 0
+    bytes_per_layer = decode_attention_bytes(kv_len, shape.Hq, shape.Hkv, shape.d) if nd else 0
+    rows_next, reqs_next = nd + int(nxt["prefillTokensNum"]), nd + int(nxt["prefillNum"])
+    flops_next = gemm_flops_per_iteration(shape, rows_next, (reqs_next + 127) // 128 * 128, shape.layers)
+    fp8_share = (1.0 - 2.0 * ((reqs_next + 127) // 128 * 128) * shape.hidden * shape.vocab / flops_next
+                 if wb == 1 and flops_next else 0.0)
     prefill_chunks = [(int(nxt["per_token_offset"][nxt["input_indptr"][nd + j]]),
                        int(nxt["input_indptr"][nd + j + 1] - nxt["input_indptr"][nd + j]))
                       for j in range(nxt["prefillNum"])]
@@ -306,9 +329,11 @@ def run_offline(args):
         "metric": "tokens/s/GPU", "value": value, "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": st.cycle_ms,
         "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": value / A100_PUBLISHED_TOKENS_PER_S, "dtype": "f16", "data": "synthetic",
+        "vs_baseline": value / A100_PUBLISHED_TOKENS_PER_S if args.shape == "8b" and wb == 2 else None,
+        "dtype": "f16" if wb == 2 else "f8e4m3 weights and GEMM inputs, f16 activations and KV", "data": "synthetic",
         "config": {
-            "workload": (f"Llama-3-8B shape, offline throughput: {n_req} requests, constant {in_len}-token "
+            "weights": args.weights,
+            "workload": (f"{shape_name} shape, offline throughput: {n_req} requests, constant {in_len}-token "
                          f"prompts (ids uniform over the vocab) / {out_len} output tokens, greedy, EOS "
                          f"ignored, <= {T} tokens per iteration with chunked prefill; "
                          + ("whole job timed" if args.full_run else
@@ -320,10 +345,12 @@ def run_offline(args):
             "kv_pool_gib": pages * page_b / 2**30,
             "value_formula": ("retired_requests * 1536 / wall_s" if use_retired else
                               "dense_rows_processed / 1535 * 1536 / wall_s (fewer than 200 retirements in the window)"),
-            "baseline": "12756 tokens/s/GPU published by the reference for this workload on 1x A100 80GB",
+            "baseline": ("12756 tokens/s/GPU published by the reference for this workload on 1x A100 80GB"
+                         if args.shape == "8b" and wb == 2 else
+                         "none: the reference publishes no single-GPU figure for this shape / weight format"),
         },
-        "roofline": _gemm_roofline(tm, _gemm_algorithmic_bytes_per_launch(
-            shape, nd + int(nxt["prefillTokensNum"]), nd + int(nxt["prefillNum"]))) if tm.gemm_launches else _attention_roofline(
+        "roofline": _gemm_roofline(tm, _gemm_algorithmic_bytes_per_launch(shape, rows_next, reqs_next, wb),
+                                   fp8_share) if tm.gemm_launches else _attention_roofline(
             tm, bytes_per_layer / launches_per_layer),
         "serving": {
             "cycles": st.cycles, "retired_requests": st.retired, "wall_s": st.wall_s,
@@ -362,6 +389,11 @@ def main():
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default: offline 256, iteration 5)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps (default: offline 8, iteration 2)")
     ap.add_argument("--workload", default="offline", choices=["offline", "iteration"])
+    ap.add_argument("--shape", default="8b", choices=["8b", "70b"],
+                    help="8b: the Llama-3-8B shape the headline metric is quoted on; 70b: the Llama-3-70B shape\n"
+                         "(80 layers, hidden 8192, 64 Q / 8 KV heads, FFN 28672) resident on the one GPU")
+    ap.add_argument("--weights", default="f16", choices=["f16", "e4m3"],
+                    help="e4m3: the five per-layer GEMM weights in fp8 with per-output-channel scales")
     ap.add_argument("--pipeline", default="auto", choices=["auto", "LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL"],
                     help="auto = the fastest schedule measured on MI355X for both workloads: NON_OVERLAP_LOCAL\n"
                          "(one stream); LOCAL measures the two-stream overlapped schedule")

@@ -14,6 +14,9 @@ struct DualWrapper : public OperatorWrapper {
   bool inited = false;
   // WeightFormat::E4M3: b1 / b2 point at e4m3 weights with their scales behind them; the rows of A
   // are quantised into the workspace on every launch (nf_dual_swiglu_f8w_f16)
+  int live_rows = -1;  // rows of A that hold tokens in this iteration (see BaseGEMMWrapper::live_rows)
+  void set_live_rows(int r) { live_rows = r; }
+  int rows() const { return live_rows >= 0 && live_rows < M ? live_rows : M; }
   bool e4m3 = false;
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
@@ -36,12 +39,12 @@ struct DualWrapper : public OperatorWrapper {
       const uint8_t* u = reinterpret_cast<const uint8_t*>(pllm_tensor_b2.ptr);
       const size_t so = e4m3WeightScaleOffset((size_t)N, (size_t)K);
       NF_KERNEL_CHECK(nf_dual_swiglu_f8w_f16(pllm_tensor_a.ptr, g, reinterpret_cast<const float*>(g + so), u,
-                                             reinterpret_cast<const float*>(u + so), pllm_tensor_d2.ptr, M, N, K,
+                                             reinterpret_cast<const float*>(u + so), pllm_tensor_d2.ptr, rows(), N, K,
                                              workspace, workspace_bytes, stream));
       return;
     }
     NF_KERNEL_CHECK(nf_dual_swiglu_f16(pllm_tensor_a.ptr, pllm_tensor_b1.ptr, pllm_tensor_b2.ptr,
-                                       pllm_tensor_d2.ptr, M, N, K, stream));
+                                       pllm_tensor_d2.ptr, rows(), N, K, stream));
   }
   DualWrapper& setA(pllmTensor<half> a) {
     assert(a.layout == PllmLayout::ROW_MAJOR && (int)a.dim1 == M && (int)a.dim2 == K);
@@ -73,5 +76,5 @@ struct DualWrapper : public OperatorWrapper {
     pllm_tensor_b2 = pllmTensor<half>(weight2.ptr, K, N, PllmLayout::ROW_MAJOR);
     return true;
   }
-  double totalCompute() { return 4.0 * (double)M * (double)N * (double)K; }
+  double totalCompute() { return 4.0 * (double)rows() * (double)N * (double)K; }
 };

@@ -51,19 +51,19 @@ BaseGEMMWrapper* generateGEMM(const std::string& tag, WeightFormat format) {
 void HipGEMMWrapperF8W::work() {
   const uint8_t* bq = reinterpret_cast<const uint8_t*>(pllm_tensor_b.ptr);
   const float* bs = reinterpret_cast<const float*>(bq + e4m3WeightScaleOffset(N, K));
-  NF_KERNEL_CHECK(nf_gemm_f8w_f16(pllm_tensor_a.ptr, bq, bs, pllm_tensor_c.ptr, pllm_tensor_d.ptr, (int)M,
+  NF_KERNEL_CHECK(nf_gemm_f8w_f16(pllm_tensor_a.ptr, bq, bs, pllm_tensor_c.ptr, pllm_tensor_d.ptr, (int)rows(),
                                   (int)N, (int)K, alpha, beta, workspace, workspace_bytes, stream));
 }
 
 void HipGEMMWrapper::work() {
   if (c_is_row) {
     NF_KERNEL_CHECK(nf_gemm_bias_f16(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
-                                     pllm_tensor_d.ptr, (int)M, (int)N, (int)K, alpha, beta,
+                                     pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
                                      tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, stream));
     return;
   }
   NF_KERNEL_CHECK(nf_gemm_f16(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
-                              pllm_tensor_d.ptr, (int)M, (int)N, (int)K, alpha, beta,
+                              pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
                               tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, stream));
 }
 
@@ -110,7 +110,7 @@ bool HipGEMMWrapper::checkResult() {
   std::vector<uint16_t> arow(K), bcolv(K);
   bool ok = true;
   for (int s = 0; s < 64 && ok; ++s) {
-    size_t m = (size_t)(s * 2654435761u) % M, n = (size_t)(s * 40503u + 7) % N;
+    size_t m = (size_t)(s * 2654435761u) % std::max<size_t>(rows(), 1), n = (size_t)(s * 40503u + 7) % N;
     HIP_CHECK(hipMemcpy(arow.data(), pllm_tensor_a.ptr + m * K, K * 2, hipMemcpyDeviceToHost));
     if (bcol) HIP_CHECK(hipMemcpy(bcolv.data(), pllm_tensor_b.ptr + n * K, K * 2, hipMemcpyDeviceToHost));
     else HIP_CHECK(hipMemcpy2D(bcolv.data(), 2, pllm_tensor_b.ptr + n, N * 2, 2, K, hipMemcpyDeviceToHost));
@@ -146,7 +146,7 @@ bool HipGEMMWrapperF8W::checkResult() {
   std::vector<uint8_t> brow(K);
   bool ok = true;
   for (int s = 0; s < 64 && ok; ++s) {
-    size_t m = (size_t)(s * 2654435761u) % M, n = (size_t)(s * 40503u + 7) % N;
+    size_t m = (size_t)(s * 2654435761u) % std::max<size_t>(rows(), 1), n = (size_t)(s * 40503u + 7) % N;
     float scale = 0;
     HIP_CHECK(hipMemcpy(arow.data(), pllm_tensor_a.ptr + m * K, K * 2, hipMemcpyDeviceToHost));
     HIP_CHECK(hipMemcpy(brow.data(), bq + n * K, K, hipMemcpyDeviceToHost));

@@ -27,6 +27,13 @@ struct BaseGEMMWrapper : public OperatorWrapper {
     K = k;
     NF_LOG_INFO("name:%s M:%zu, N:%zu, K:%zu", name.c_str(), M, N, K);
   }
+  // Rows of A that hold tokens in this iteration; the launch and the flop count cover only
+  // those.  The reference's GEMMs always run their configured M (a dense batch is assumed full);
+  // when admission is limited by KV memory the batch is not, and the padding rows would cost as
+  // much as live ones.  Not in the reference's interface.
+  size_t live_rows = (size_t)-1;
+  void set_live_rows(size_t r) { live_rows = r; }
+  size_t rows() const { return live_rows < M ? live_rows : M; }
   size_t mk() const { return M * K; }
   size_t kn() const { return K * N; }
   size_t mn() const { return M * N; }
@@ -136,7 +143,7 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   void set_alpha(float a) override { alpha = a; }
   void set_beta(float b) override { beta = b; }
 
-  double totalCompute() override { return 2.0 * (double)M * (double)N * (double)K; }
+  double totalCompute() override { return 2.0 * (double)rows() * (double)N * (double)K; }
   float gflops(double runtime_ms) override { return float(totalCompute() / 1e9 / (runtime_ms / 1e3)); }
   void profile() override;      // times 100 launches on the op's stream, logs GFLOP/s
   bool checkResult() override;  // spot-checks D against a host fp64 dot product

@@ -570,6 +570,11 @@ void LocalPipeline::update(vortexUpdateData* update_data_) {
   genEmbedding2.setInput(input_span.subtensor(nano1, T - nano1));
 
   update_token_num = update_data.decodePrefillBorder + update_data.prefillTokensNum;
+  const int live1 = std::min(update_token_num, nano1), live2 = std::max(update_token_num - nano1, 0);
+  for (BaseGEMMWrapper* g : {O1, D1, KQV1}) g->set_live_rows((size_t)live1);
+  for (BaseGEMMWrapper* g : {O2, D2, KQV2}) g->set_live_rows((size_t)live2);
+  dual1.set_live_rows(live1);
+  dual2.set_live_rows(live2);
   const int req_num = update_data.decodePrefillBorder + update_data.prefillNum;
   maxSampler.set_batch_size(req_num);
   keepToken.update(req_num, update_data.input_indptr);

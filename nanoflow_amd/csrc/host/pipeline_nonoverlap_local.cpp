@@ -109,6 +109,8 @@ void NonOverlapLocalPipeline::update(vortexUpdateData* update_data_) {
   genEmbedding.setInput(pllmTensor<int>(update_data.input_tokens, T, 1, PllmLayout::ROW_MAJOR));
   const int req_num = update_data.decodePrefillBorder + update_data.prefillNum;
   update_token_num = update_data.decodePrefillBorder + update_data.prefillTokensNum;
+  for (BaseGEMMWrapper* g : {O, D, KQV}) g->set_live_rows((size_t)update_token_num);
+  dual.set_live_rows(update_token_num);
   maxSampler.set_batch_size(req_num / nranks);
   keepToken.update(req_num, update_data.input_indptr);
   LOGITS->set_shape(std::min((req_num / nranks + 127) / 128 * 128, T), (int)ModelConfig.vocab_size,

@@ -41,6 +41,14 @@
  *                           by what the format fixes: the OCP e4m3 decode table against
  *                           torch's, encode by round trip over all codes, ties at every
  *                           midpoint, saturation, and float64 closed forms for the GEMMs.
+ *   nfo_silu_mul_f16; (oracle/nf_oracle.py) quantize_weight_e4m3, dual_swiglu_f8f8,
+ *   decoder_forward_f8      PARITY UNPINNED against the reference for the same reason.  Pinned by
+ *                           float64 closed forms (the pair on dequantised operands; the weight
+ *                           quantiser as the row quantiser on the transpose; the forward against
+ *                           the independent float64 model on the dequantised weights).
+ *   the b_kqv path of nfo_decoder_forward   follows pipeline/src/pipeline.cu:520-533,1048-1058
+ *                           (bias replicated per row, C operand, beta 1); pinned by the float64
+ *                           model with y = xW + b.
  *   (oracle/nf_oracle.py) gemm_bf16, dual_swiglu_bf16
  *                           PARITY UNPINNED against the reference (no bf16 path there);
  *                           float64 closed forms, conversions checked against torch's.
