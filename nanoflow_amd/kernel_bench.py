@@ -60,6 +60,7 @@ def main():
     ap.add_argument("--num-blocks", type=int, default=0, help="attn: cap on resident workgroups (0 = none)")
     ap.add_argument("--mib", type=int, default=1024, help="copy: MiB moved")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"], help="gemm, dual: element type")
+    ap.add_argument("--b-col-major", action="store_true", help="gemm: weights stored [N][K] (k contiguous)")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warm", type=int, default=3)
     a = ap.parse_args()
@@ -75,8 +76,9 @@ def main():
                 continue
             out = torch.empty(M, N, dtype=edt if a.op == "gemm" else torch.float16, device=DEV)
             if a.op == "gemm":
-                A, B = rnd(M, Kd).to(edt), rnd(Kd, N, std=0.02).to(edt)
-                fn = lambda: K.gemm(A, B, out=out)
+                A = rnd(M, Kd).to(edt)
+                B = (rnd(N, Kd, std=0.02) if a.b_col_major else rnd(Kd, N, std=0.02)).to(edt)
+                fn = lambda: K.gemm(A, B, out=out, b_col_major=a.b_col_major)
             else:
                 Aq = torch.randint(0, 120, (M, Kd), dtype=torch.uint8, device=DEV)
                 Bq = torch.randint(0, 120, (N, Kd), dtype=torch.uint8, device=DEV)

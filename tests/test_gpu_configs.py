@@ -6,7 +6,8 @@
   tolerance;
 * the one-iteration workload (1792 decode + 256 prefill tokens) at full width through the three
   schedules: size-independent properties (schedule independence, page-permutation invariance);
-* fp8 GEMM at the 70B FFN shape.
+* fp8 GEMM at the 70B FFN shape, and one 70B-shaped layer with e4m3 weights through the pipeline
+  (the shape and weight format of the fp8 benchmark configuration).
 """
 import numpy as np
 import pytest
@@ -24,7 +25,7 @@ def _max_rel(got, ref):
     return np.abs(got.astype(np.float64) - ref).max() / np.abs(ref).max()
 
 
-def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines):
+def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines, weight_format="f16"):
     """Iteration 0 prefills the last prompt token of every request (so that the decode iteration
     is fed distinct tokens: the samples of iteration 0); iteration 1 is the decode step under test."""
     from nanoflow_amd import engine, pllm_python as P
@@ -57,7 +58,7 @@ def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines):
         print(f"shape hidden={shape.hidden} pipeline={pt.name}", flush=True)
         T = max(64, (n + 63) // 64 * 64)
         with engine.Engine(shape, pt, global_batch=T, nano1=T // 2, kqv1=T // 4, kqv3=T // 4,
-                           kv_pages=b0.num_pages, weights=w, kv_pools=pools0) as e:
+                           kv_pages=b0.num_pages, weights=w, kv_pools=pools0, weight_format=weight_format) as e:
             e.update(b0, keep_token_list=np.zeros(0, np.int32))
             s0 = e.run()
             kv_after0 = [p[:b0.num_pages].cpu().numpy() for p in e.kv]
@@ -68,17 +69,34 @@ def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines):
             kv = [p[:b0.num_pages].cpu().numpy() for p in e.kv]
         # the oracle runs the decode iteration from the GPU's state after iteration 0
         pools_ref = [p.copy() for p in kv_after0]
-        hid_ref, _, _ = oracle.decoder_forward(shape.as_dict(), w, pools_ref, b1.as_dict(), want_logits=False)
-        err = _max_rel(hid, hid_ref)
-        print(f"  residual stream max-norm relative error {err:.2e}", flush=True)
-        assert err < LAYER_RTOL, (pt, err)
+        if weight_format == "e4m3":
+            # same arithmetic in the oracle (rows re-quantised per GEMM); re-quantisation makes the
+            # layer discontinuous, so two correct implementations agree statistically, not to fp16
+            # rounding (tests/test_gpu_pipeline.py::test_fp8_weight_pipelines_match_oracle).  At
+            # this width the layer's own output dominates the residual stream (rms 7.3 against an
+            # input of 1), so nothing damps that noise: nudging the oracle's norm weights by one
+            # fp16 ulp moves its output by 5.3 % rms here; the bound is 8 % rms
+            P.setWeightFormat(P.WeightFormat.F16)
+            hid_ref, _, _ = oracle.decoder_forward_f8(shape.as_dict(), w, oracle.quantize_model_weights(w), pools_ref,
+                                                      b1.as_dict(), "e4m3")
+            d = hid.astype(np.float64) - hid_ref.astype(np.float64)
+            rms = np.sqrt((d ** 2).mean() / (hid_ref.astype(np.float64) ** 2).mean())
+            print(f"  residual stream rms relative error {rms:.2e}, max-norm {_max_rel(hid, hid_ref):.2e}", flush=True)
+            assert rms < 8e-2 and _max_rel(hid, hid_ref) < 2.5e-1, (pt, rms)
+            kv_tol = 8e-2
+        else:
+            hid_ref, _, _ = oracle.decoder_forward(shape.as_dict(), w, pools_ref, b1.as_dict(), want_logits=False)
+            err = _max_rel(hid, hid_ref)
+            print(f"  residual stream max-norm relative error {err:.2e}", flush=True)
+            assert err < LAYER_RTOL, (pt, err)
+            kv_tol = 2e-3
         assert len(set(s0.tolist())) > n // 2          # the decode rows really were fed distinct tokens
         for l in range(shape.layers):
             wrote_ref = (pools_ref[l] != kv_after0[l]).any(axis=(3, 4))       # [page, k/v, entry]
             wrote_got = (kv[l] != kv_after0[l]).any(axis=(3, 4))
             assert np.array_equal(wrote_ref, wrote_got), (pt, l, "KV slots written")
             assert wrote_got.sum() == 2 * n
-            assert _max_rel(kv[l][wrote_got], pools_ref[l][wrote_ref]) < 2e-3, (pt, l, "appended K/V rows")
+            assert _max_rel(kv[l][wrote_got], pools_ref[l][wrote_ref]) < kv_tol, (pt, l, "appended K/V rows")
 
 
 def test_llama3_8b_layer_64_decode_tokens(oracle):
@@ -94,6 +112,17 @@ def test_llama3_70b_shaped_layer(oracle):
     shape = synth.ModelShape(hidden=8192, Hq=64, Hkv=8, ffn=28672, vocab=2048, layers=1)
     kv_lens = np.random.default_rng(3).integers(200, 400, size=16)
     _decode_layer_case(oracle, shape, kv_lens, seed=1, pipelines=(P.PipelineType.NON_OVERLAP_LOCAL,))
+
+
+def test_llama3_70b_shaped_layer_with_e4m3_weights(oracle):
+    from nanoflow_amd import pllm_python as P
+    shape = synth.ModelShape(hidden=8192, Hq=64, Hkv=8, ffn=28672, vocab=2048, layers=1)
+    kv_lens = np.random.default_rng(4).integers(200, 400, size=16)
+    try:
+        _decode_layer_case(oracle, shape, kv_lens, seed=2, pipelines=(P.PipelineType.NON_OVERLAP_LOCAL,),
+                           weight_format="e4m3")
+    finally:
+        P.setWeightFormat(P.WeightFormat.F16)
 
 
 def test_one_iteration_workload_is_schedule_independent_at_full_width():
