@@ -98,6 +98,7 @@ GEMM_SHAPES = [
     (1408, 6144, 512),    # 256x256 tiles with an M tail, XCD-remapped grid
     (2048, 6144, 256),    # one round of 128x384 tiles (the QKV projection of a full batch)
     (1930, 5000, 264),    # 128x384 tiles with M, N and K tails
+    (267, 1160, 520),     # a few hundred rows (the KV-bound 70B serving regime), N and K tails
 ]
 
 
@@ -159,7 +160,8 @@ def test_gemm_identity_is_exact(K):
 
 @pytest.mark.parametrize("M,N,K_", [(64, 14336, 4096), (5, 136, 72), (200, 512, 256), (640, 2048, 512),
                                     (2048, 14336, 128),    # 3.5 rounds of 256-row tiles: two tile heights in one launch
-                                    (1992, 14328, 200)])   # the same with M, N and K tails
+                                    (1992, 14328, 200),    # the same with M, N and K tails
+                                    (267, 1160, 264)])     # a few hundred rows, N and K tails
 def test_dual_swiglu(K, oracle, M, N, K_):
     rng = np.random.default_rng(7)
     A = synth.normal_f16(rng, (M, K_))
