@@ -43,6 +43,17 @@ NF_API const char* nf_last_error(void);
 NF_API int nf_embedding_f16(const int32_t* tokens, const uint16_t* table, uint16_t* out, int n_tokens,
                      int hidden, nf_stream_t stream);
 
+/* Moves the KV pages of the listed requests between one layer's pool and a staging buffer laid
+ * out like kv_indices: for every r = req_idx[i], i < req_num, and every
+ * j in [kv_indptr[r], kv_indptr[r+1]): staging page j <- pool page kv_indices[j] (to_pool == 0,
+ * offloading) or pool page kv_indices[j] <- staging page j (to_pool != 0, loading back).  A page
+ * is page_bytes bytes (K and V halves together: vortexModelConfig::page_mem_size), a multiple
+ * of 16.  All pointers are device (or device-accessible pinned) memory.
+ * Replaces moveKVcacheKernel (pipeline/src/offloadKernel.cu:17-34) behind PageAggregator /
+ * PageDispatcher (pipeline/include/otherWrapper.cuh:413-472). */
+NF_API int nf_move_kv_pages(int req_num, const int32_t* req_idx, const int32_t* kv_indptr, const int32_t* kv_indices,
+                            uint16_t* staging, uint16_t* kv_data, size_t page_bytes, int to_pool, nf_stream_t stream);
+
 /* out = half(x * rsqrt(mean(x^2) + eps) * weight), fp32 math; hidden % 8 == 0.
  * Replaces rms_norm() (pipeline/include/rms_norm.cuh:48-127,210-233) called by
  * LayerNorm::work (pipeline/include/otherWrapper.cuh:94-102). */

@@ -179,3 +179,55 @@ public:
     return *this;
   }
 };
+
+// KV offload operators (pipeline/include/otherWrapper.cuh:413-472).  PageAggregator gathers the
+// pages of the listed (finished) requests from one layer's pool into a staging buffer laid out
+// like kv_indices, ready for one contiguous copy to host memory; PageDispatcher scatters a staging
+// buffer loaded from host memory back into the pages the requests now own.  The reference wires
+// them only into its tensor-parallel offload pipeline, with fixed request lists as a cost model
+// (pipeline/src/pipeline.cu:37-59,701-726,915-931); here they are free-standing operators.
+class PageAggregator : public OtherWrapper {
+public:
+  int finished_req_num = 0;
+  int32_t* finished_idx = nullptr;
+  int32_t* kv_indptr = nullptr;
+  int32_t* kv_indices = nullptr;
+  half* output = nullptr;
+  half* kv_data = nullptr;
+
+  void init(int finished_req_num, int32_t* finished_idx, int32_t* kv_indptr, int32_t* kv_indices, half* output) {
+    this->finished_req_num = finished_req_num;
+    this->finished_idx = finished_idx;
+    this->kv_indptr = kv_indptr;
+    this->kv_indices = kv_indices;
+    this->output = output;
+  }
+  void setKVData(half* kv_data) { this->kv_data = kv_data; }
+  void work() override {
+    NF_KERNEL_CHECK(nf_move_kv_pages(finished_req_num, finished_idx, kv_indptr, kv_indices, output, kv_data,
+                                     ModelConfig.page_mem_size, 0, stream));
+  }
+};
+
+class PageDispatcher : public OtherWrapper {
+public:
+  int load_req_num = 0;
+  int32_t* load_idx = nullptr;
+  int32_t* kv_indptr = nullptr;
+  int32_t* kv_indices = nullptr;
+  half* host_input = nullptr;  // the staging buffer the host copy was loaded into (device memory)
+  half* kv_data = nullptr;
+
+  void init(int load_req_num, int32_t* load_idx, int32_t* kv_indptr, int32_t* kv_indices, half* host_input) {
+    this->load_req_num = load_req_num;
+    this->load_idx = load_idx;
+    this->kv_indptr = kv_indptr;
+    this->kv_indices = kv_indices;
+    this->host_input = host_input;
+  }
+  void setKVData(half* kv_data) { this->kv_data = kv_data; }
+  void work() override {
+    NF_KERNEL_CHECK(nf_move_kv_pages(load_req_num, load_idx, kv_indptr, kv_indices, host_input, kv_data,
+                                     ModelConfig.page_mem_size, 1, stream));
+  }
+};

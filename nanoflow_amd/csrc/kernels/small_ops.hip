@@ -210,6 +210,27 @@ __global__ __launch_bounds__(256) void rope_append_kernel(
   }
 }
 
+// Pages of the listed requests between a layer's pool and a staging buffer indexed like
+// kv_indices: staging page j <-> pool page kv_indices[j] for j in [kv_indptr[r], kv_indptr[r+1])
+// of every listed request r.  grid.y walks the requests, grid.x strides over a request's pages;
+// a workgroup moves one page (K and V: page_chunks 16-byte chunks) at a time.
+template <bool kToPool>
+__global__ __launch_bounds__(256) void move_kv_pages_kernel(const int32_t* __restrict__ req_idx,
+                                                            const int32_t* __restrict__ kv_indptr,
+                                                            const int32_t* __restrict__ kv_indices,
+                                                            u32x4* staging, u32x4* pool, int page_chunks) {
+  const int r = req_idx[blockIdx.y];
+  const int begin = kv_indptr[r], end = kv_indptr[r + 1];
+  for (int j = begin + blockIdx.x; j < end; j += gridDim.x) {
+    u32x4* s = staging + (size_t)j * page_chunks;
+    u32x4* p = pool + (size_t)kv_indices[j] * page_chunks;
+    for (int c = threadIdx.x; c < page_chunks; c += 256) {
+      if constexpr (kToPool) p[c] = s[c];
+      else s[c] = p[c];
+    }
+  }
+}
+
 }  // namespace nf
 
 using namespace nf;
@@ -241,6 +262,26 @@ int nf_keep_token_f16(const uint16_t* in, uint16_t* out, const int32_t* input_in
   gather_rows_kernel<true><<<req_num, 256, 0, (hipStream_t)stream>>>(
       input_indptr, reinterpret_cast<const u32x4*>(in), reinterpret_cast<u32x4*>(out), hidden / 8);
   return check_launch("nf_keep_token_f16");
+}
+
+int nf_move_kv_pages(int req_num, const int32_t* req_idx, const int32_t* kv_indptr, const int32_t* kv_indices,
+                     uint16_t* staging, uint16_t* kv_data, size_t page_bytes, int to_pool, nf_stream_t stream) {
+  NF_REQUIRE(req_num >= 0 && page_bytes > 0 && page_bytes % 16 == 0 && page_bytes < ((size_t)1 << 31),
+             "nf_move_kv_pages: page_bytes=%zu must be a positive multiple of 16 (req_num=%d)", page_bytes, req_num);
+  if (req_num == 0) return NF_OK;
+  NF_REQUIRE(req_num <= 65535, "nf_move_kv_pages: at most 65535 requests per call (%d)", req_num);
+  NF_REQUIRE(req_idx && kv_indptr && kv_indices && staging && kv_data, "nf_move_kv_pages: null pointer");
+  NF_REQUIRE(((uintptr_t)staging | (uintptr_t)kv_data) % 16 == 0, "nf_move_kv_pages: buffers must be 16-byte aligned");
+  // 64 workgroups per request stride over its pages (a 1024-token request has 64 of them)
+  const dim3 grid(64, (unsigned)req_num);
+  const int chunks = (int)(page_bytes / 16);
+  if (to_pool)
+    move_kv_pages_kernel<true><<<grid, 256, 0, (hipStream_t)stream>>>(
+        req_idx, kv_indptr, kv_indices, reinterpret_cast<u32x4*>(staging), reinterpret_cast<u32x4*>(kv_data), chunks);
+  else
+    move_kv_pages_kernel<false><<<grid, 256, 0, (hipStream_t)stream>>>(
+        req_idx, kv_indptr, kv_indices, reinterpret_cast<u32x4*>(staging), reinterpret_cast<u32x4*>(kv_data), chunks);
+  return check_launch("nf_move_kv_pages");
 }
 
 int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* weight, int rows, int hidden,

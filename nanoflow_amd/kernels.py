@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
 SYMBOLS = [
     "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16", "nf_gemm_bias_f16",
     "nf_dual_swiglu_f16", "nf_gemm_bf16", "nf_dual_swiglu_bf16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
-    "nf_quantize_weight_e4m3", "nf_dual_swiglu_f8_f16", "nf_dual_swiglu_f8w_f16",
+    "nf_quantize_weight_e4m3", "nf_dual_swiglu_f8_f16", "nf_dual_swiglu_f8w_f16", "nf_move_kv_pages",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
 ]
@@ -57,6 +57,7 @@ def lib() -> C.CDLL:
         l.nf_quantize_weight_e4m3.argtypes = [vp, vp, vp, i32, i32, vp]
         l.nf_dual_swiglu_f8_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp]
         l.nf_dual_swiglu_f8w_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, C.c_size_t, vp]
+        l.nf_move_kv_pages.argtypes = [i32, vp, vp, vp, vp, vp, sz, i32, vp]
         l.nf_rope_append_f16.argtypes = [vp] * 7 + [i32] * 5 + [f32] * 4 + [vp]
         l.nf_attention_workspace_bytes.restype = sz
         l.nf_attention_workspace_bytes.argtypes = [i32, i32, i32]
@@ -271,6 +272,18 @@ def attention_paged(q, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_l
                                         _p(workspace), workspace.numel(), _stream()),
            "nf_attention_paged_f16")
     return out
+
+
+def move_kv_pages(req_idx, kv_indptr, kv_indices, staging, kv_data, to_pool: bool):
+    """Pages of the requests in req_idx between one layer's pool kv_data [pages, 2, page, Hkv, d] and
+    staging [len(kv_indices), 2, page, Hkv, d] (page j of staging <-> pool page kv_indices[j])."""
+    for t in (req_idx, kv_indptr, kv_indices):
+        _i32(t)
+    _f16(staging); _f16(kv_data)
+    page_bytes = kv_data[0].numel() * 2
+    assert staging[0].numel() * 2 == page_bytes and staging.shape[0] >= kv_indices.numel()
+    _check(lib().nf_move_kv_pages(req_idx.numel(), _p(req_idx), _p(kv_indptr), _p(kv_indices), _p(staging),
+                                  _p(kv_data), page_bytes, int(bool(to_pool)), _stream()), "nf_move_kv_pages")
 
 
 def keep_token(x, input_indptr, req_num, out=None):

@@ -312,6 +312,18 @@ def decoder_forward_f8(cfg: dict, weights: dict, wq: dict, kv_data: list, batch:
     return x, (logits if want_logits else None), sampled
 
 
+def move_kv_pages(req_idx, kv_indptr, kv_indices, staging, kv_data, to_pool: bool):
+    """Pages of the listed requests between a layer's pool [pages, ...] and a staging buffer indexed
+    like kv_indices, IN PLACE (pipeline/src/offloadKernel.cu:17-34: for each listed request, for j in
+    [kv_indptr[r], kv_indptr[r+1]): host page j <-> pool page kv_indices[j]).  Plain loops."""
+    for r in np.asarray(req_idx).tolist():
+        for j in range(int(kv_indptr[r]), int(kv_indptr[r + 1])):
+            if to_pool:
+                kv_data[int(kv_indices[j])] = staging[j]
+            else:
+                staging[j] = kv_data[int(kv_indices[j])]
+
+
 def rmsnorm(x, w, eps=1e-5):
     rows, H = x.shape
     out = np.empty_like(x)

@@ -229,6 +229,37 @@ def test_dual_swiglu_bf16(K, oracle, M, N, K_):
                  "dual swiglu bf16")
 
 
+# ---------------------------------------------------------------- KV pages to and from a staging buffer
+
+def test_move_kv_pages_is_bit_exact_and_round_trips(K, oracle):
+    rng = np.random.default_rng(17)
+    shape = synth.LLAMA3_8B                                     # 64 KB pages (K and V of 16 tokens, 8 heads)
+    b = synth.make_batch([1023, 17, 300, 64, 1], [(0, 33)], vocab=10, seed=4, extra_pages=7)
+    pool = synth.make_kv_pool(b.num_pages, shape, rng)
+    n_idx = b.kv_indices.shape[0]
+    listed = np.array([4, 0, 5, 2], np.int32)                   # out of order, not all requests
+    staging_ref = np.zeros((n_idx,) + pool.shape[1:], np.float16)
+    oracle.move_kv_pages(listed, b.kv_indptr, b.kv_indices, staging_ref, pool, to_pool=False)
+    staging = torch.zeros(staging_ref.shape, dtype=torch.float16, device="cuda")
+    d_idx, d_indptr, d_indices, d_pool = dev(listed), dev(b.kv_indptr), dev(b.kv_indices), dev(pool)
+    K.move_kv_pages(d_idx, d_indptr, d_indices, staging, d_pool, to_pool=False)
+    assert np.array_equal(host(staging), staging_ref)
+    assert np.array_equal(host(d_pool), pool)                   # the pool is only read
+    # back into a pool whose page table has been re-drawn (the requests own other pages now)
+    perm = rng.permutation(b.num_pages).astype(np.int32)
+    indices2 = perm[b.kv_indices]
+    pool2_ref = np.zeros_like(pool)
+    oracle.move_kv_pages(listed, b.kv_indptr, indices2, staging_ref, pool2_ref, to_pool=True)
+    d_pool2 = torch.zeros_like(d_pool)
+    K.move_kv_pages(d_idx, d_indptr, dev(indices2), staging, d_pool2, to_pool=True)
+    assert np.array_equal(host(d_pool2), pool2_ref)
+    for r in listed:                                            # every listed request got its pages back
+        for j in range(b.kv_indptr[r], b.kv_indptr[r + 1]):
+            assert np.array_equal(pool2_ref[indices2[j]], pool[b.kv_indices[j]])
+    # an empty list is a no-op
+    K.move_kv_pages(dev(np.zeros(0, np.int32)), d_indptr, d_indices, staging, d_pool, to_pool=True)
+
+
 # ---------------------------------------------------------------- RoPE + paged append
 
 F8_RTOL = 3e-2   # fp8 path: activations rounded to e4m3 (3 mantissa bits) on the way in

@@ -294,6 +294,21 @@ def test_decoder_forward_f8_vs_float64_model_on_dequantised_weights(oracle):
     assert rel_err(h_plain, ref_x) > 6e-3
 
 
+def test_move_kv_pages_hand_case(oracle):
+    # 3 requests owning pages [4, 1], [0], [3, 2, 5]; requests 2 and 0 are listed
+    indptr = np.array([0, 2, 3, 6], np.int32)
+    indices = np.array([4, 1, 0, 3, 2, 5], np.int32)
+    pool = np.arange(6 * 4, dtype=np.float16).reshape(6, 4)
+    staging = np.full((6, 4), -1, np.float16)
+    oracle.move_kv_pages([2, 0], indptr, indices, staging, pool, to_pool=False)
+    want = np.full((6, 4), -1, np.float16)
+    want[0], want[1], want[3], want[4], want[5] = pool[4], pool[1], pool[3], pool[2], pool[5]   # slot 2 (request 1) untouched
+    assert np.array_equal(staging, want)
+    pool2 = np.zeros_like(pool)
+    oracle.move_kv_pages([2, 0], indptr, indices, staging, pool2, to_pool=True)
+    assert np.array_equal(pool2[[1, 2, 3, 4, 5]], pool[[1, 2, 3, 4, 5]]) and not pool2[0].any()   # page 0 is request 1's
+
+
 def test_rmsnorm_closed_form(oracle):
     rng = np.random.default_rng(5)
     x = synth.normal_f16(rng, (11, 256), 3.0)
