@@ -377,8 +377,9 @@ def test_serve_skip_cycles_reach_steady_state_without_gpu_work():
     assert stats.gpu_iter_ms > 0 and stats.cycle_ms > 0
 
 
-@pytest.mark.parametrize("pt_name", ["LOCAL", "NON_OVERLAP_LOCAL"])
-def test_graph_replay_is_identical_to_eager(pt_name):
+@pytest.mark.parametrize("pt_name,weight_format", [("LOCAL", "f16"), ("NON_OVERLAP_LOCAL", "f16"),
+                                                    ("NON_OVERLAP_LOCAL", "e4m3"), ("KQVBIAS", "f16")])
+def test_graph_replay_is_identical_to_eager(pt_name, weight_format):
     """The same sequence of iterations, eagerly and with hipGraph replay (two launch signatures,
     several replays each, with other device work and synchronisations in between): sampled ids
     and the residual stream must be identical step by step."""
@@ -386,6 +387,8 @@ def test_graph_replay_is_identical_to_eager(pt_name):
     pt = P.PipelineType[pt_name]
     shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
     w = _scaled_weights(shape, seed=4)
+    if pt.has_kqv_bias:
+        w["b_kqv"] = synth.make_weights(shape, seed=5, kqv_bias=True)["b_kqv"]
     T, nano1 = 96, 40
     b1 = synth.make_batch([5, 17, 33, 64, 20, 9], [(0, 50)], vocab=shape.vocab, seed=31, extra_pages=8)
     b2 = synth.make_batch([7, 12, 40, 3, 28], [(16, 30), (0, 21)], vocab=shape.vocab, seed=32, extra_pages=8)
@@ -399,7 +402,7 @@ def test_graph_replay_is_identical_to_eager(pt_name):
     def run_sequence(graph):
         outs = []
         with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=20, kqv3=28, kv_pages=pages,
-                           weights=w, kv_pools=pools0) as e:
+                           weights=w, kv_pools=pools0, weight_format=weight_format) as e:
             P.setGraphMode(graph)
             scratch = torch.zeros(1 << 16, device="cuda")
             for i, b in enumerate(order):
@@ -414,8 +417,11 @@ def test_graph_replay_is_identical_to_eager(pt_name):
             P.setGraphMode(False)
         return outs, counters
 
-    eager, c0 = run_sequence(False)
-    replay, c1 = run_sequence(True)
+    try:
+        eager, c0 = run_sequence(False)
+        replay, c1 = run_sequence(True)
+    finally:
+        P.setWeightFormat(P.WeightFormat.F16)
     assert c0["captured"] == 0 and c0["replayed"] == 0 and c0["eager"] == len(order)
     assert c1["captured"] == 2 and c1["eager"] == 2 and c1["replayed"] == len(order) - 2, c1
     for i, ((s0, h0), (s1, h1)) in enumerate(zip(eager, replay)):
