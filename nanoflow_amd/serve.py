@@ -16,6 +16,9 @@ reference's pipeline/utils/serve_8B.py:
   when that file is missing it is first converted from the Hugging Face checkpoint directory
   ``serve_configs.hf_path``.  Nothing is downloaded.  (The flag is parsed as a truth value here;
   the reference's ``type=bool`` turns every non-empty string, "False" included, into True.)
+* ``serve_configs.weight_format`` (optional, not in the reference's schema): "f16" (default) or "e4m3" --
+  the five GEMM weights of every layer are quantised on the device as they are loaded or made
+  (per-output-channel scales) and served from the fp8 form.
 * KV pool = ``1024 * allocate_kv_data_batch // 16`` pages per layer (serve_8B.py:643).
 * writes PREFIX.stat, PREFIX.stat.csv (same columns as serve_8B.py:792-793), PREFIX.req_time and
   PREFIX.req_tokens (prompt + generated ids of every retired request, one Python list per line,
@@ -108,7 +111,8 @@ def main():
     avg_in = sum(r[1] for r in reqs) // len(reqs)
     avg_out = sum(r[2] for r in reqs) // len(reqs)
     eng = engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=kqv1, kqv3=kqv3, kv_pages=pages,
-                        run_layer=mc.get("run_layer", shape.layers), kv_fill="zeros", weights=weights)
+                        run_layer=mc.get("run_layer", shape.layers), kv_fill="zeros", weights=weights,
+                        weight_format=sc.get("weight_format", "f16"))
     former = P.BatchFormer(pages, shape.page_size, T, nano1, kqv1, kqv3, avg_in, avg_out)
 
     pending = list(reqs)                  # not yet released, in arrival order

@@ -488,8 +488,9 @@ def test_weights_loaded_from_a_checkpoint_run_like_the_oracle(oracle, tmp_path):
     assert np.array_equal(got[:len(samp)], samp)
 
 
-@pytest.mark.parametrize("online,from_file", [(False, False), (True, False), (False, True)])
-def test_serve_command_line_writes_the_reference_result_files(tmp_path, online, from_file):
+@pytest.mark.parametrize("online,from_file,weight_format", [(False, False, "f16"), (True, False, "f16"),
+                                                            (False, True, "f16"), (False, True, "e4m3")])
+def test_serve_command_line_writes_the_reference_result_files(tmp_path, online, from_file, weight_format):
     """nanoflow_amd.serve with the reference's flags on a tiny model: offline trace (whole loop in
     the library) and a trace with arrival times (loop driven per phase)."""
     import subprocess, sys, os, csv
@@ -507,7 +508,8 @@ def test_serve_command_line_writes_the_reference_result_files(tmp_path, online, 
         import json
         _write_hf_checkpoint(str(tmp_path / "hf"), _scaled_weights(shape, seed=4), shape)
         c = json.load(open(cfg))
-        c["serve_configs"].update({"weight_path": str(tmp_path / "w"), "hf_path": str(tmp_path / "hf")})
+        c["serve_configs"].update({"weight_path": str(tmp_path / "w"), "hf_path": str(tmp_path / "hf"),
+                                   "weight_format": weight_format})
         json.dump(c, open(cfg, "w"))
     prefix = tmp_path / "out"
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
