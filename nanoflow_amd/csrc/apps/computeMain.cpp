@@ -4,6 +4,8 @@
 // pools) -> config data -> synthetic update data for an average prompt of 1024 and an average
 // output of 512 tokens -> init, config, update, run x N, finalize.  Prints the wall time of each
 // run and the number of sampled tokens, and exits non-zero when anything fails.
+// An optional serve_configs.weight_format of "e4m3" in the config (not in the reference's schema)
+// makes the weights and the pipeline use the fp8 form of the per-layer GEMM weights.
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -49,6 +51,13 @@ int main(int argc, char** argv) {
     vnranks = j.at("model_configs").value<int>("gpu_num", 1);
     global_batch_size = j.at("pipeline_configs").value<int>("global_batch_size", 0);
     pipe_name = j.at("serve_configs").at("pipeline_type").str;
+    const auto& sc = j.at("serve_configs");
+    const std::string fmt = sc.contains("weight_format") ? sc.at("weight_format").str : std::string("f16");
+    if (fmt != "f16" && fmt != "e4m3") {
+      std::fprintf(stderr, "unknown weight_format %s\n", fmt.c_str());
+      return 2;
+    }
+    setWeightFormat(fmt == "e4m3" ? WeightFormat::E4M3 : WeightFormat::F16);
   } catch (const std::exception& e) {
     std::fprintf(stderr, "%s: %s\n", config_path.c_str(), e.what());
     return 2;
@@ -59,8 +68,8 @@ int main(int argc, char** argv) {
     return 2;
   }
   if (nranks != 1 || vnranks != 1 || !Worker::isSupported(pipe)) {
-    std::fprintf(stderr, "this build runs LOCAL, NON_OVERLAP_LOCAL and NANOBATCH_LOCAL on one GPU "
-                         "(got %s, %d ranks, gpu_num %d)\n", pipe_name.c_str(), nranks, vnranks);
+    std::fprintf(stderr, "this build runs LOCAL, NON_OVERLAP_LOCAL, NANOBATCH_LOCAL and the three *_KQVBIAS "
+                         "types on one GPU (got %s, %d ranks, gpu_num %d)\n", pipe_name.c_str(), nranks, vnranks);
     return 2;
   }
 

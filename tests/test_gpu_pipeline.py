@@ -573,7 +573,7 @@ def test_autosearch_writes_a_tuned_pipeline_config(tmp_path):
     assert t["model"] == json.load(open(cfg))["model"]
 
 
-@pytest.mark.parametrize("pt_name", ["LOCAL", "NON_OVERLAP_LOCAL"])
+@pytest.mark.parametrize("pt_name", ["LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_KQVBIAS"])
 def test_cpp_end_to_end_program_runs_the_reference_sequence(tmp_path, pt_name):
     """nanoflow_amd/test_compute (C++ API only: createModelWeight, createInitData, readConfigData,
     createUpdateData, init, config, update, run x N, finalize) on a 2-layer model."""
@@ -586,6 +586,11 @@ def test_cpp_end_to_end_program_runs_the_reference_sequence(tmp_path, pt_name):
     cfg = tmp_path / "tiny.json"
     engine.write_config(str(cfg), shape, global_batch=256, nano1=128, kqv1=64, kqv3=64,
                         pipeline_type=P.PipelineType[pt_name], kv_pages=16384)
+    if pt_name == "NON_OVERLAP_LOCAL":      # this schedule also with the fp8 form of the weights, the bias type without
+        import json
+        c = json.load(open(cfg))
+        c["serve_configs"]["weight_format"] = "e4m3"
+        json.dump(c, open(cfg, "w"))
     r = subprocess.run([exe, str(cfg), "3"], capture_output=True, text=True, timeout=110)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     head = re.search(r"(\d+) tokens per iteration \((\d+) decode requests, (\d+) prefill requests with (\d+) tokens\)", r.stdout)
