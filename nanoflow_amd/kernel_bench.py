@@ -3,7 +3,8 @@
 
     python -m nanoflow_amd.kernel_bench --op gemm --m 2048            # KQV, O, down, LM head
     python -m nanoflow_amd.kernel_bench --op dual --m 1024
-    python -m nanoflow_amd.kernel_bench --op gemm_f8 --m 2048
+    python -m nanoflow_amd.kernel_bench --op gemm_f8 --m 2048 --model 70b
+    python -m nanoflow_amd.kernel_bench --op dual_f8 --m 2048 --model 70b     # fused fp8 gate/up pair
     python -m nanoflow_amd.kernel_bench --op attn --requests 1792 --kv-lo 1024 --kv-hi 1536
     python -m nanoflow_amd.kernel_bench --op prefill --chunks 755:269,0:1024,0:74
     python -m nanoflow_amd.kernel_bench --op copy                     # counter-calibration kernel
@@ -48,7 +49,7 @@ def layer_shapes(shape: synth.ModelShape, M: int):
 
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--op", required=True, choices=["gemm", "dual", "gemm_f8", "attn", "prefill", "copy"])
+    ap.add_argument("--op", required=True, choices=["gemm", "dual", "gemm_f8", "dual_f8", "attn", "prefill", "copy"])
     ap.add_argument("--chunks", default="755:269,0:1024,0:74",
                     help="prefill: prev_len:chunk_len per request (default: a steady-state offline iteration)")
     ap.add_argument("--model", default="8b", choices=["8b", "70b"])
@@ -93,6 +94,15 @@ def main():
         ms = timeit(lambda: K.dual_swiglu(A, Bg, Bu, out=out), a.iters, a.warm)
         print(f"dual gate/up {a.m}x{shape.ffn}x{shape.hidden}: {ms * 1e3:9.1f} us  "
               f"{4.0 * a.m * shape.ffn * shape.hidden / ms / 1e9:8.1f} TFLOP/s", flush=True)
+    elif a.op == "dual_f8":
+        M, N, Kd = a.m, shape.ffn, shape.hidden
+        Aq = torch.randint(0, 120, (M, Kd), dtype=torch.uint8, device=DEV)
+        Gq = torch.randint(0, 120, (N, Kd), dtype=torch.uint8, device=DEV)
+        Uq = torch.randint(0, 120, (N, Kd), dtype=torch.uint8, device=DEV)
+        sa, sg, su = torch.ones(M, device=DEV), torch.full((N,), 1e-4, device=DEV), torch.full((N,), 1e-4, device=DEV)
+        out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+        ms = timeit(lambda: K.dual_swiglu_f8(Aq, sa, Gq, sg, Uq, su, out=out), a.iters, a.warm)
+        print(f"dual_f8 gate/up {M}x{N}x{Kd}: {ms * 1e3:9.1f} us  {4.0 * M * N * Kd / ms / 1e9:8.1f} TFLOP/s", flush=True)
     elif a.op == "attn":
         b = synth.config2_batch(seed=0, n_decode=a.requests, lo=a.kv_lo, hi=a.kv_hi, prefill_chunk=16)
         nd = b.decodePrefillBorder
