@@ -69,6 +69,25 @@ NF_API int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* wei
 NF_API int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
 
+/* nf_gemm_f16 with scratch: a GEMM of at most 256 rows whose output tiles would leave most of the
+ * chip idle (few rows against a narrow N: the QKV, O and down projections of a small decode batch)
+ * is split over K into shares that fill it, summed in fp32 through `workspace`
+ * (nf_gemm_workspace_bytes(M, N, K) bytes, 16-byte aligned; 0 = this shape is not split).  With a
+ * null or short workspace, or a shape that does not profit, it is nf_gemm_f16.  The sum over k is
+ * then taken share by share, so results differ from nf_gemm_f16 in fp32 rounding only.
+ * nf_gemm_workspace_bytes_upto(max_M, N, K): the largest requirement over 1..max_M rows.
+ * No counterpart in the reference (its serial split-K is a tag field of the CUTLASS kernel,
+ * pipeline/include/gemmShape.cuh:5-6). */
+NF_API size_t nf_gemm_workspace_bytes(int M, int N, int K);
+NF_API size_t nf_gemm_workspace_bytes_upto(int max_M, int N, int K);
+NF_API int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
+                          float alpha, float beta, int b_col_major, void* workspace, size_t workspace_bytes,
+                          nf_stream_t stream);
+/* the same for nf_gemm_bias_f16 (declared below) */
+NF_API int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M, int N,
+                               int K, float alpha, float beta, int b_col_major, void* workspace,
+                               size_t workspace_bytes, nf_stream_t stream);
+
 /* D = half(alpha * A.B + beta * bias[n]): nf_gemm_f16 with one row, bias [N], added to every row
  * of the product, read in the epilogue instead of from an [M,N] copy of it.
  * Replaces the QKV GEMM of the *_KQVBIAS pipelines, whose C operand is the bias replicated over

@@ -5,6 +5,7 @@
 // (allocate_kv_data_batch requests x 1024 tokens), not a figure derived from a fixed
 // 64 GiB as at config.h:97-99, so it scales with the 288 GB of an MI355X.
 #pragma once
+#include <algorithm>
 #include <cmath>
 #include <cstddef>
 #include <string>
@@ -62,6 +63,9 @@ struct vortexModelConfig {
     // quantised activations of the fp8-weight GEMMs (one byte per element of the QKV, O, gate/up
     // and down inputs, a scale per row, 256-byte alignment of up to 8 wrappers)
     k_temp_size += (size_t)max_batch_size * (3 * model_hidden_dim + model_ff_dim + 32) / 2 + 8 * 256;
+    // fp32 partial sums of GEMM launches split over K: shares x M x N is at most CUs x one tile
+    // (256 x 128 x 128 elements = 16.8 MB) per wrapper, up to 7 wrappers, 256-byte alignment
+    k_temp_size += (size_t)7 * (256 * 16384 * 2 + 128);
     if (!rope_3_1) {
       smooth_a = 0;
       smooth_b = 0;

@@ -57,14 +57,16 @@ void HipGEMMWrapperF8W::work() {
 
 void HipGEMMWrapper::work() {
   if (c_is_row) {
-    NF_KERNEL_CHECK(nf_gemm_bias_f16(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
-                                     pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
-                                     tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, stream));
+    NF_KERNEL_CHECK(nf_gemm_bias_f16_ws(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
+                                        pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
+                                        tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, splitk_workspace,
+                                        splitk_workspace_bytes, stream));
     return;
   }
-  NF_KERNEL_CHECK(nf_gemm_f16(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
-                              pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
-                              tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, stream));
+  NF_KERNEL_CHECK(nf_gemm_f16_ws(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
+                                 pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
+                                 tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, splitk_workspace,
+                                 splitk_workspace_bytes, stream));
 }
 
 void HipGEMMWrapper::profile() {

@@ -84,6 +84,15 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   pllmTensor<half> pllm_tensor_a, pllm_tensor_b, pllm_tensor_c, pllm_tensor_d;
   float alpha = 1.f, beta = 0.f;
   bool inited = false;
+  // scratch for the fp32 partial sums of launches that are split over K (few live rows against a
+  // narrow N would otherwise leave most of the chip idle); sized for the worst case up to M rows
+  void* splitk_workspace = nullptr;
+  size_t splitk_workspace_bytes = 0;
+  size_t workspaceBytes() const override { return nf_gemm_workspace_bytes_upto((int)M, (int)N, (int)K); }
+  void setWorkspace(void* ptr, size_t bytes) override {
+    splitk_workspace = ptr;
+    splitk_workspace_bytes = bytes;
+  }
   bool c_is_row = false;  // pllm_tensor_c is a [1, N] row added to every row
 
   explicit HipGEMMWrapper(const GemmTag& t) : tag(t) {}

@@ -89,11 +89,16 @@ __device__ __forceinline__ float swiglu_rounded(float g_acc, float u_acc) {
 
 // kDual: two weight matrices, SwiGLU epilogue.  kBCol: weights stored [N][K].
 // One BM x BN output tile at (m_base, n_base), computed by the whole workgroup.
-template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
+// K is the extent of the contraction and lda the row stride (elements) of the k-contiguous
+// operands (A, and [N][K] weights): equal for a whole GEMM, K < lda for one share of a GEMM split
+// over K, whose operand pointers already point at the share's first k.
+// kPartial: the fp32 sums are stored as they are to D taken as float [M][N] (no alpha, beta, C).
+template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol, bool kPartial = false>
 __device__ __forceinline__ void gemm_tile(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
-    int M, int N, int K, float alpha, float beta, const int ldc, const int m_base, const int n_base) {
+    int M, int N, int K, float alpha, float beta, const int ldc, const int m_base, const int n_base,
+    const int lda) {
   constexpr int NB = kDual ? 2 : 1;
   using SM = GemmSmem<BM, BN, NB>;
   constexpr int TM = BM / WM / 32;  // MFMA tiles per wave along M
@@ -124,10 +129,11 @@ __device__ __forceinline__ void gemm_tile(
         for (int r = 0; r < 16; ++r) acc[b][i][j][r] = 0.f;
 
   // ---- global -> LDS: per-lane byte offsets of the chunks this lane fetches
-  const rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K * 2);
+  const rsrc_t a_rsrc = make_rsrc(A, ((size_t)(M - 1) * lda + K) * 2);
   rsrc_t b_rsrc[NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) b_rsrc[b] = make_rsrc(b ? B1 : B0, (size_t)N * K * 2);
+  for (int b = 0; b < NB; ++b)
+    b_rsrc[b] = make_rsrc(b ? B1 : B0, kBCol ? ((size_t)(N - 1) * lda + K) * 2 : (size_t)N * K * 2);
   // A-style rows: lane -> (row lane/8 of the instruction's 8 rows, position lane%8), fetching
   // logical chunk position ^ ((row >> 1) & 7); bit 3 of the row number is the wave's parity.
   const int a_kc = ((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2))) * 8;
@@ -140,7 +146,7 @@ __device__ __forceinline__ void gemm_tile(
 #pragma unroll
   for (int t = 0; t < A_LOADS; ++t) {
     const int gm = m_base + (t * 4 + wave) * 8 + (lane >> 3);
-    a_off[t] = ((uint32_t)gm * (uint32_t)K + a_kc) * 2u;
+    a_off[t] = ((uint32_t)gm * (uint32_t)lda + a_kc) * 2u;
   }
   uint32_t b_off[NB][B_LOADS];
   const uint32_t b_slab = (uint32_t)BK * (uint32_t)N * 2u;
@@ -149,7 +155,7 @@ __device__ __forceinline__ void gemm_tile(
     uint32_t off;
     if constexpr (kBCol) {
       const int gn = n_base + (t * 4 + wave) * 8 + (lane >> 3);
-      off = ((uint32_t)gn * (uint32_t)K + a_kc) * 2u;
+      off = ((uint32_t)gn * (uint32_t)lda + a_kc) * 2u;
     } else {
       const int g = (t * 4 + wave) * 64 + lane;  // 16-byte slot of the slab's LDS image
       const int row = g / B_CPR;
@@ -386,6 +392,16 @@ __device__ __forceinline__ void gemm_tile(
       const int c = it * 64 + lane;
       a4[it] = *reinterpret_cast<const float4_t*>(ep + (c / CPR) * ROWP + (c % CPR) * 16);
     }
+    if constexpr (kPartial) {
+      typedef unsigned int u32v4_t __attribute__((ext_vector_type(4)));
+      const __amdgpu_buffer_rsrc_t p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          reinterpret_cast<float*>(D) + row0, 0, rows > 0 ? rows * N * 4 : 0, 0x00020000);
+#pragma unroll
+      for (int it = 0; it < ITER; ++it)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32v4_t, a4[it]), p_rsrc,
+                                               off[it] == kOob ? kOob : off[it] * 2u, 0, 0);
+      continue;
+    }
     auto store_group = [&](int it, float4_t v) {
       __builtin_amdgcn_raw_buffer_store_b64(u32v2_t{E::pack2(v[0], v[1]), E::pack2(v[2], v[3])}, d_rsrc, off[it], 0, 0);
     };
@@ -423,7 +439,7 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(
   const int logical = xcd_order(blockIdx.x, tiles_m * tiles_n);
   if (logical >= tiles_m * tiles_n) return;
   gemm_tile<E, BM, BN, WM, WN, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc,
-                                              (logical % tiles_m) * BM, (logical / tiles_m) * BN);
+                                              (logical % tiles_m) * BM, (logical / tiles_m) * BN, K);
 }
 
 // Two tile heights in one launch, for shapes whose 256-row tiles fill the 256 CUs a whole number
@@ -440,7 +456,7 @@ __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
     const int t = xcd_order(blockIdx.x, n_big);
     if (t >= n_big) return;
     gemm_tile<E, 256, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc,
-                                            (t % tiles_m) * 256, (t / tiles_m) * BN);
+                                            (t % tiles_m) * 256, (t / tiles_m) * BN, K);
   } else {
     const int n_small = 2 * (tiles_m * tiles_n - n_big);
     const int u = xcd_order(blockIdx.x - big_grid, n_small);
@@ -449,8 +465,76 @@ __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
     const int m_base = (t % tiles_m) * 256 + (u & 1) * 128;
     if (m_base >= M) return;
     gemm_tile<E, 128, BN, 2, 2, kDual, kBCol>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc, m_base,
-                                            (t / tiles_m) * BN);
+                                            (t / tiles_m) * BN, K);
   }
+}
+
+// A GEMM with too few output tiles to fill the chip (few rows against a narrow N), split over K:
+// workgroup (tile, share) computes the tile's sums over k in [share * k_per, ...) and stores them
+// as fp32 to P[share][M][N]; splitk_reduce_kernel adds the shares and applies alpha, beta and C.
+template <class E, int BM, int BN, int WM, int WN, bool kBCol>
+__global__ __launch_bounds__(256) void gemm_f16_splitk_kernel(
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, float* __restrict__ P,
+    int M, int N, int K, int shares, int k_per, int tiles_m, int tiles_n) {
+  const int total = tiles_m * tiles_n * shares;
+  const int logical = xcd_order(blockIdx.x, total);
+  if (logical >= total) return;
+  const int share = logical % shares, tile = logical / shares;
+  const int k0 = share * k_per;
+  const int k_len = K - k0 < k_per ? K - k0 : k_per;
+  gemm_tile<E, BM, BN, WM, WN, false, kBCol, true>(
+      A + k0, kBCol ? B + k0 : B + (size_t)k0 * N, nullptr, nullptr,
+      reinterpret_cast<uint16_t*>(P + (size_t)share * M * N), M, N, k_len, 1.f, 0.f, N,
+      (tile % tiles_m) * BM, (tile / tiles_m) * BN, K);
+}
+
+// D[m][n..n+3] = round(alpha * sum_s P[s][m][n..] + beta * C[m][n..]); C has row stride ldc.
+template <class E>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ P, int shares,
+                                                            const uint16_t* C, int ldc, uint16_t* D,
+                                                            int M, int N, float alpha, float beta) {
+  const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
+  for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
+    float4_t v = *reinterpret_cast<const float4_t*>(P + g * 4);
+    for (int s = 1; s < shares; ++s) v += *reinterpret_cast<const float4_t*>(P + s * mn + g * 4);
+    v *= alpha;
+    if (beta != 0.f) {
+      const size_t m = g * 4 / N, n = g * 4 % N;
+      const u32x2 c = *reinterpret_cast<const u32x2*>(C + m * ldc + n);
+      v[0] += beta * E::widen(c.x & 0xffffu);
+      v[1] += beta * E::widen(c.x >> 16);
+      v[2] += beta * E::widen(c.y & 0xffffu);
+      v[3] += beta * E::widen(c.y >> 16);
+    }
+    *reinterpret_cast<u32x2*>(D + g * 4) = u32x2{E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+  }
+}
+
+template <class E, int BM, int BN, int WM, int WN, bool kBCol>
+static int launch_splitk(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
+                         int K, float alpha, float beta, int ldc, int shares, int k_per, float* P,
+                         hipStream_t stream) {
+  using SM = GemmSmem<BM, BN, 1>;
+  auto kern = gemm_f16_splitk_kernel<E, BM, BN, WM, WN, kBCol>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)SM::bytes);
+    if (e != hipSuccess) {
+      set_error("gemm: cannot reserve %zu bytes of LDS: %s", SM::bytes, hipGetErrorString(e));
+      return NF_ERR_RUNTIME;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int grid = ((tiles_m * tiles_n * shares + 7) / 8) * 8;
+  kern<<<grid, 256, SM::bytes, stream>>>(A, B, P, M, N, K, shares, k_per, tiles_m, tiles_n);
+  int rc = check_launch("gemm split-K launch");
+  if (rc) return rc;
+  const size_t groups = (size_t)M * N / 4;
+  const int rgrid = (int)std::min<size_t>((groups + 255) / 256, 2048);
+  splitk_reduce_kernel<E><<<rgrid, 256, 0, stream>>>(P, shares, C, ldc, D, M, N, alpha, beta);
+  return check_launch("gemm split-K reduction launch");
 }
 
 template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
@@ -513,6 +597,20 @@ static int cu_count() {
   return n;
 }
 
+// Split over K: for at most 256 rows whose tiles (64 x 256 up to 64 rows, else 128 x 128) would
+// leave more than half of the CUs idle, as many shares as fill them, each at least 512 deep.
+// Returns the number of shares (1 = no split) and their depth.
+static int splitk_plan(int M, int N, int K, int* k_per) {
+  if (M > 256 || K < 1024) return 1;
+  const int bm = M <= 64 ? 64 : 128, bn = M <= 64 ? 256 : 128;
+  const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+  const int cus = cu_count();
+  int shares = std::min(std::min(cus / tiles, K / 512), 16);
+  if (shares < 2) return 1;
+  *k_per = ((K + shares - 1) / shares + BK - 1) / BK * BK;
+  return (K + *k_per - 1) / *k_per;  // shares that are not empty
+}
+
 // Tile choice.  A launch takes ceil(tiles / CUs) rounds of one tile each, a round costing the
 // tile's area over its relative efficiency (bigger tiles re-read less through LDS); the cheapest
 // candidate wins.  So 192 tiles of 256x256 beat 1.5 rounds of 128x256, and 2048 x 6144 takes
@@ -570,6 +668,28 @@ static int gemm_entry(const char* who, const uint16_t* A, const uint16_t* B, con
                      : dispatch_plain<E, false>(A, B, C, D, M, N, K, alpha, beta, ldc, s);
 }
 
+// gemm_entry with a workspace: shapes that profit are split over K through it.
+template <class E>
+static int gemm_ws_entry(const char* who, const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                         int M, int N, int K, float alpha, float beta, int b_col_major, void* workspace,
+                         size_t workspace_bytes, nf_stream_t stream, bool c_is_row = false) {
+  int k_per = 0;
+  const int shares = M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0 ? splitk_plan(M, N, K, &k_per) : 1;
+  if (shares < 2 || !workspace || workspace_bytes < (size_t)shares * M * N * sizeof(float))
+    return gemm_entry<E>(who, A, B, C, D, M, N, K, alpha, beta, b_col_major, stream, c_is_row);
+  int rc = check_gemm_args(who, A, B, D, M, N, K);
+  if (rc) return rc;
+  NF_REQUIRE(beta == 0.f || C, "%s: beta=%g needs C", who, (double)beta);
+  NF_REQUIRE(((uintptr_t)C) % 8 == 0 && (uintptr_t)workspace % 16 == 0, "%s: C must be 8-byte and the workspace 16-byte aligned", who);
+  hipStream_t s = (hipStream_t)stream;
+  float* P = static_cast<float*>(workspace);
+  if (M <= 64)
+    return b_col_major ? launch_splitk<E, 64, 256, 1, 4, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
+                       : launch_splitk<E, 64, 256, 1, 4, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
+  return b_col_major ? launch_splitk<E, 128, 128, 2, 2, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
+                     : launch_splitk<E, 128, 128, 2, 2, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
+}
+
 template <class E>
 static int dual_entry(const char* who, const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup,
                       uint16_t* out, int M, int N, int K, nf_stream_t stream) {
@@ -598,6 +718,34 @@ extern "C" {
 int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream) {
   return gemm_entry<F16>("nf_gemm_f16", A, B, C, D, M, N, K, alpha, beta, b_col_major, stream);
+}
+
+size_t nf_gemm_workspace_bytes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int k_per = 0;
+  const int shares = splitk_plan(M, N, K, &k_per);
+  return shares < 2 ? 0 : (size_t)shares * M * N * sizeof(float);
+}
+
+size_t nf_gemm_workspace_bytes_upto(int max_M, int N, int K) {
+  size_t need = 0;
+  for (int m = 1; m <= max_M && m <= 256; ++m) need = std::max(need, nf_gemm_workspace_bytes(m, N, K));
+  return need;
+}
+
+int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
+                   float alpha, float beta, int b_col_major, void* workspace, size_t workspace_bytes,
+                   nf_stream_t stream) {
+  return gemm_ws_entry<F16>("nf_gemm_f16_ws", A, B, C, D, M, N, K, alpha, beta, b_col_major, workspace,
+                            workspace_bytes, stream);
+}
+
+int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M, int N,
+                        int K, float alpha, float beta, int b_col_major, void* workspace, size_t workspace_bytes,
+                        nf_stream_t stream) {
+  NF_REQUIRE(bias, "nf_gemm_bias_f16_ws: null bias");
+  return gemm_ws_entry<F16>("nf_gemm_bias_f16_ws", A, B, bias, D, M, N, K, alpha, beta, b_col_major, workspace,
+                            workspace_bytes, stream, true);
 }
 
 int nf_gemm_bias_f16(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M,

@@ -62,6 +62,7 @@ def main():
     ap.add_argument("--mib", type=int, default=1024, help="copy: MiB moved")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"], help="gemm, dual: element type")
     ap.add_argument("--b-col-major", action="store_true", help="gemm: weights stored [N][K] (k contiguous)")
+    ap.add_argument("--ws", action="store_true", help="gemm: the entry point with a workspace (split over K where it pays)")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warm", type=int, default=3)
     a = ap.parse_args()
@@ -79,7 +80,11 @@ def main():
             if a.op == "gemm":
                 A = rnd(M, Kd).to(edt)
                 B = (rnd(N, Kd, std=0.02) if a.b_col_major else rnd(Kd, N, std=0.02)).to(edt)
-                fn = lambda: K.gemm(A, B, out=out, b_col_major=a.b_col_major)
+                if a.ws:
+                    ws = torch.empty((max(K.lib().nf_gemm_workspace_bytes(M, N, Kd), 16),), dtype=torch.uint8, device=DEV)
+                    fn = lambda: K.gemm_ws(A, B, out=out, b_col_major=a.b_col_major, workspace=ws)
+                else:
+                    fn = lambda: K.gemm(A, B, out=out, b_col_major=a.b_col_major)
             else:
                 Aq = torch.randint(0, 120, (M, Kd), dtype=torch.uint8, device=DEV)
                 Bq = torch.randint(0, 120, (N, Kd), dtype=torch.uint8, device=DEV)

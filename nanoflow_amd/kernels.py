@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
 
 SYMBOLS = [
     "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16", "nf_gemm_bias_f16",
+    "nf_gemm_workspace_bytes", "nf_gemm_workspace_bytes_upto", "nf_gemm_f16_ws", "nf_gemm_bias_f16_ws",
     "nf_dual_swiglu_f16", "nf_gemm_bf16", "nf_dual_swiglu_bf16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
     "nf_quantize_weight_e4m3", "nf_dual_swiglu_f8_f16", "nf_dual_swiglu_f8w_f16", "nf_move_kv_pages",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
@@ -45,6 +46,12 @@ def lib() -> C.CDLL:
         l.nf_embedding_f16.argtypes = [vp, vp, vp, i32, i32, vp]
         l.nf_rmsnorm_f16.argtypes = [vp, vp, vp, i32, i32, f32, vp]
         l.nf_gemm_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
+        l.nf_gemm_workspace_bytes.restype = sz
+        l.nf_gemm_workspace_bytes.argtypes = [i32, i32, i32]
+        l.nf_gemm_workspace_bytes_upto.restype = sz
+        l.nf_gemm_workspace_bytes_upto.argtypes = [i32, i32, i32]
+        l.nf_gemm_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp, sz, vp]
+        l.nf_gemm_bias_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp, sz, vp]
         l.nf_gemm_bias_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
         l.nf_gemm_bf16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
@@ -65,7 +72,8 @@ def lib() -> C.CDLL:
         l.nf_keep_token_f16.argtypes = [vp, vp, vp, i32, i32, vp]
         l.nf_argmax_f16.argtypes = [vp, vp, vp, i32, i32, vp]
         for name in SYMBOLS:
-            if name not in ("nf_last_error", "nf_attention_workspace_bytes"):
+            if name not in ("nf_last_error", "nf_attention_workspace_bytes", "nf_gemm_workspace_bytes",
+                            "nf_gemm_workspace_bytes_upto", "nf_gemm_f8w_workspace_bytes"):
                 getattr(l, name).restype = i32
         _lib = l
     return _lib
@@ -140,6 +148,28 @@ def gemm(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, bias
     fn, name = (lib().nf_gemm_f16, "nf_gemm_f16") if dt == torch.float16 else (lib().nf_gemm_bf16, "nf_gemm_bf16")
     _check(fn(_p(A), _p(B), _p(Cmat), _p(out), M, N, K, alpha, beta, int(b_col_major), _stream()), name)
     return out
+
+
+def gemm_ws(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, workspace=None, bias=None):
+    """nf_gemm_f16_ws: fp16 GEMM that is split over K through a workspace when few rows against a narrow
+    N would leave most of the chip idle.  Returns (out, shares_bytes) where shares_bytes is the
+    workspace the shape asked for (0: not split)."""
+    _f16(A); _f16(B)
+    M, K = A.shape
+    N = B.shape[0] if b_col_major else B.shape[1]
+    need = lib().nf_gemm_workspace_bytes(M, N, K)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
+    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
+    if bias is not None:          # one row [N] added (times beta) to every row: nf_gemm_bias_f16_ws
+        assert Cmat is None and bias.numel() == N
+        _f16(bias)
+        _check(lib().nf_gemm_bias_f16_ws(_p(A), _p(B), _p(bias), _p(out), M, N, K, alpha, beta, int(b_col_major),
+                                         _p(workspace), workspace.numel(), _stream()), "nf_gemm_bias_f16_ws")
+        return out, need
+    _check(lib().nf_gemm_f16_ws(_p(A), _p(B), _p(Cmat), _p(out), M, N, K, alpha, beta, int(b_col_major),
+                                _p(workspace), workspace.numel(), _stream()), "nf_gemm_f16_ws")
+    return out, need
 
 
 def dual_swiglu(A, Bg, Bu, out=None):

@@ -151,6 +151,47 @@ def test_gemm_with_bias_row_equals_gemm_with_replicated_bias(K, oracle, M, N, K_
     assert_close(got, oracle.gemm(A, B, rep, 0.5, -1.5), what="gemm + bias row, col-major B")
 
 
+@pytest.mark.parametrize("M,N,K_", [(16, 6144, 4096), (64, 4096, 14336), (128, 4096, 4096), (200, 6144, 4096),
+                                    (64, 1160, 2056), (1, 1024, 1024), (256, 2048, 8200)])
+def test_gemm_split_over_k_matches_oracle(K, oracle, M, N, K_):
+    """Few rows against a narrow N: the launch is split over K into shares whose fp32 sums meet in a
+    workspace.  Same tolerance as the unsplit kernel; residual operand, column-major weights and
+    the no-workspace fallback included."""
+    from nanoflow_amd import kernels
+    rng = np.random.default_rng(M + N)
+    A = synth.normal_f16(rng, (M, K_))
+    B = synth.normal_f16(rng, (K_, N), 0.02)
+    Cm = synth.normal_f16(rng, (M, N))
+    got, need = K.gemm_ws(dev(A), dev(B))
+    assert need > 0 and need % (M * N * 4) == 0 and need // (M * N * 4) >= 2, "this shape is meant to be split"
+    assert_close(host(got), oracle.gemm(A, B), what="split-K gemm beta=0")
+    got, _ = K.gemm_ws(dev(A), dev(B), dev(Cm), alpha=0.5, beta=1.0)
+    assert_close(host(got), oracle.gemm(A, B, Cm, 0.5, 1.0), what="split-K gemm beta=1")
+    d = dev(Cm)
+    K.gemm_ws(dev(A), dev(B), d, alpha=1.0, beta=1.0, out=d)            # C aliases D (the residual stream)
+    assert_close(host(d), oracle.gemm(A, B, Cm, 1.0, 1.0), what="split-K gemm in place")
+    got, _ = K.gemm_ws(dev(A), dev(np.ascontiguousarray(B.T)), b_col_major=True)
+    assert_close(host(got), oracle.gemm(A, B), what="split-K gemm col-major B")
+    bias = synth.normal_f16(rng, (N,))
+    rep = np.ascontiguousarray(np.broadcast_to(bias, (M, N)))
+    got, _ = K.gemm_ws(dev(A), dev(B), bias=dev(bias), alpha=1.0, beta=1.0)
+    assert np.array_equal(host(got), host(K.gemm_ws(dev(A), dev(B), dev(rep), alpha=1.0, beta=1.0)[0]))   # bias row = replicated C
+    # a workspace that is too small: the unsplit kernel, bit for bit
+    short, _ = K.gemm_ws(dev(A), dev(B), workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+    assert np.array_equal(host(short), host(K.gemm(dev(A), dev(B))))
+
+
+def test_gemm_with_workspace_is_the_plain_kernel_for_large_shapes(K):
+    from nanoflow_amd import kernels
+    rng = np.random.default_rng(8)
+    for M, N, K_ in [(2048, 6144, 256), (300, 4096, 512), (64, 14336, 512), (64, 4096, 512)]:
+        A = synth.normal_f16(rng, (M, K_))
+        B = synth.normal_f16(rng, (K_, N), 0.02)
+        got, need = K.gemm_ws(dev(A), dev(B))
+        assert need == 0, (M, N, K_)
+        assert np.array_equal(host(got), host(K.gemm(dev(A), dev(B))))
+
+
 def test_gemm_identity_is_exact(K):
     rng = np.random.default_rng(6)
     A = synth.normal_f16(rng, (70, 128))
