@@ -52,10 +52,13 @@ public:
     pllm_tensor_weight = pllmTensor<half>(w.ptr, size_t(1), w.size(), PllmLayout::ROW_MAJOR);
     return true;
   }
+  // rows that hold tokens in this iteration (-1: all rows of the input); the rest is left as it was
+  int live_rows = -1;
+  void set_live_rows(int r) { live_rows = r; }
   void work() override {
     assert(pllm_tensor_input.dim2 == (size_t)ModelConfig.model_hidden_dim);
-    NF_KERNEL_CHECK(nf_rmsnorm_f16(output, input, weight,
-                                   (int)(input_size / ModelConfig.model_hidden_dim),
+    const int all = (int)(input_size / ModelConfig.model_hidden_dim);
+    NF_KERNEL_CHECK(nf_rmsnorm_f16(output, input, weight, live_rows >= 0 && live_rows < all ? live_rows : all,
                                    ModelConfig.model_hidden_dim, ModelConfig.rms_norm_eps, stream));
   }
 };

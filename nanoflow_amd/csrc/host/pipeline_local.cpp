@@ -575,6 +575,10 @@ void LocalPipeline::update(vortexUpdateData* update_data_) {
   for (BaseGEMMWrapper* g : {O2, D2, KQV2}) g->set_live_rows((size_t)live2);
   dual1.set_live_rows(live1);
   dual2.set_live_rows(live2);
+  layerNormAttention1.set_live_rows(live1);
+  layerNormFFN1.set_live_rows(live1);
+  layerNormAttention2.set_live_rows(live2);
+  layerNormFFN2.set_live_rows(live2);
   const int req_num = update_data.decodePrefillBorder + update_data.prefillNum;
   maxSampler.set_batch_size(req_num);
   keepToken.update(req_num, update_data.input_indptr);
@@ -583,6 +587,7 @@ void LocalPipeline::update(vortexUpdateData* update_data_) {
   LOGITS->set_shape(std::min((req_num + 127) / 128 * 128, T), (int)ModelConfig.vocab_size,
                     ModelConfig.model_hidden_dim);
   LOGITS->init();
+  layerNormModel.set_live_rows((int)LOGITS->M);  // the rows the LM head reads (sampled rows padded to 128)
   output_data.sampled_tokens = req_num;
   GEMVOpUpdate();
   NF_LOG_INFO("prefill: %d, decode: %d; Batch size: %d, %d, %d, %d", update_data.prefillNum,

@@ -111,11 +111,14 @@ void NonOverlapLocalPipeline::update(vortexUpdateData* update_data_) {
   update_token_num = update_data.decodePrefillBorder + update_data.prefillTokensNum;
   for (BaseGEMMWrapper* g : {O, D, KQV}) g->set_live_rows((size_t)update_token_num);
   dual.set_live_rows(update_token_num);
+  layerNormAttention.set_live_rows(update_token_num);
+  layerNormFFN.set_live_rows(update_token_num);
   maxSampler.set_batch_size(req_num / nranks);
   keepToken.update(req_num, update_data.input_indptr);
   LOGITS->set_shape(std::min((req_num / nranks + 127) / 128 * 128, T), (int)ModelConfig.vocab_size,
                     ModelConfig.model_hidden_dim);
   LOGITS->init();
+  layerNormModel.set_live_rows((int)LOGITS->M);  // the rows the LM head reads (sampled rows padded to 128)
   output_data.sampled_tokens = req_num;
   GEMVOpUpdate();
 }
