@@ -83,6 +83,12 @@ NF_API size_t nf_gemm_workspace_bytes_upto(int max_M, int N, int K);
 NF_API int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
                           float alpha, float beta, int b_col_major, void* workspace, size_t workspace_bytes,
                           nf_stream_t stream);
+/* the same for the fused gate/up pair: both products are split, their fp32 sums rounded to fp16 and
+ * put through SiLU-mul by the reduction (workspace: nf_dual_swiglu_workspace_bytes(M, N, K)) */
+NF_API size_t nf_dual_swiglu_workspace_bytes(int M, int N, int K);
+NF_API size_t nf_dual_swiglu_workspace_bytes_upto(int max_M, int N, int K);
+NF_API int nf_dual_swiglu_f16_ws(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
+                                 int M, int N, int K, void* workspace, size_t workspace_bytes, nf_stream_t stream);
 /* the same for nf_gemm_bias_f16 (declared below) */
 NF_API int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M, int N,
                                int K, float alpha, float beta, int b_col_major, void* workspace,

@@ -65,7 +65,8 @@ struct vortexModelConfig {
     k_temp_size += (size_t)max_batch_size * (3 * model_hidden_dim + model_ff_dim + 32) / 2 + 8 * 256;
     // fp32 partial sums of GEMM launches split over K: shares x M x N is at most CUs x one tile
     // (256 x 128 x 128 elements = 16.8 MB) per wrapper, up to 7 wrappers, 256-byte alignment
-    k_temp_size += (size_t)7 * (256 * 16384 * 2 + 128);
+    // (the fused gate/up pair keeps two sets of sums: 2 x that for up to 2 of its wrappers)
+    k_temp_size += (size_t)(7 + 4) * (256 * 16384 * 2 + 128);
     if (!rope_3_1) {
       smooth_a = 0;
       smooth_b = 0;

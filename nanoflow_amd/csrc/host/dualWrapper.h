@@ -21,7 +21,10 @@ struct DualWrapper : public OperatorWrapper {
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
   void setWeightFormat(WeightFormat f) { e4m3 = f == WeightFormat::E4M3; }
-  size_t workspaceBytes() const { return e4m3 ? nf_gemm_f8w_workspace_bytes(M, K) : 0; }
+  // fp16 weights: scratch for launches of few rows that are split over K (nf_dual_swiglu_f16_ws)
+  size_t workspaceBytes() const {
+    return e4m3 ? nf_gemm_f8w_workspace_bytes(M, K) : nf_dual_swiglu_workspace_bytes_upto(M, N, K);
+  }
   void setWorkspace(void* ptr, size_t bytes) {
     workspace = ptr;
     workspace_bytes = bytes;
@@ -43,8 +46,8 @@ struct DualWrapper : public OperatorWrapper {
                                              workspace, workspace_bytes, stream));
       return;
     }
-    NF_KERNEL_CHECK(nf_dual_swiglu_f16(pllm_tensor_a.ptr, pllm_tensor_b1.ptr, pllm_tensor_b2.ptr,
-                                       pllm_tensor_d2.ptr, rows(), N, K, stream));
+    NF_KERNEL_CHECK(nf_dual_swiglu_f16_ws(pllm_tensor_a.ptr, pllm_tensor_b1.ptr, pllm_tensor_b2.ptr,
+                                          pllm_tensor_d2.ptr, rows(), N, K, workspace, workspace_bytes, stream));
   }
   DualWrapper& setA(pllmTensor<half> a) {
     assert(a.layout == PllmLayout::ROW_MAJOR && (int)a.dim1 == M && (int)a.dim2 == K);

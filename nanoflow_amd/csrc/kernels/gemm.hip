@@ -359,7 +359,7 @@ __device__ __forceinline__ void gemm_tile(
       off[it] = gn < N ? (uint32_t)((c / CPR) * N + gn) * 2u : kOob;
     }
     u32v2_t cv[ITER];
-    if constexpr (!kDual) {
+    if constexpr (!kDual && !kPartial) {
       if (beta != 0.f) {  // issued first: the longest latency of the pass
         // C has row stride ldc (N, or 0 when one row is added to every row of the product):
         // the D offset less the row's share of the difference
@@ -373,6 +373,34 @@ __device__ __forceinline__ void gemm_tile(
           cv[it] = __builtin_amdgcn_raw_buffer_load_b64(c_rsrc, off[it] == kOob ? kOob : off[it] - r * c_skip, 0, 0);
         }
       }
+    }
+    if constexpr (kPartial) {
+      // the fp32 sums as they are, one product after the other through the staging area; the
+      // gate sums go to D, the up sums of the dual form to C (both float [M][N] here)
+      typedef unsigned int u32v4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int qd = 0; qd < 4; ++qd) {
+            float4_t v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[b][i][j][qd * 4 + e];
+            *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
+          }
+        float* dst = b == 0 ? reinterpret_cast<float*>(D) : reinterpret_cast<float*>(const_cast<uint16_t*>(C));
+        const __amdgpu_buffer_rsrc_t p_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(dst + row0, 0, rows > 0 ? rows * N * 4 : 0, 0x00020000);
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+          const int c = it * 64 + lane;
+          const float4_t p4 = *reinterpret_cast<const float4_t*>(ep + (c / CPR) * ROWP + (c % CPR) * 16);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32v4_t, p4), p_rsrc,
+                                                 off[it] == kOob ? kOob : off[it] * 2u, 0, 0);
+        }
+      }
+      continue;
     }
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -391,16 +419,6 @@ __device__ __forceinline__ void gemm_tile(
     for (int it = 0; it < ITER; ++it) {
       const int c = it * 64 + lane;
       a4[it] = *reinterpret_cast<const float4_t*>(ep + (c / CPR) * ROWP + (c % CPR) * 16);
-    }
-    if constexpr (kPartial) {
-      typedef unsigned int u32v4_t __attribute__((ext_vector_type(4)));
-      const __amdgpu_buffer_rsrc_t p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-          reinterpret_cast<float*>(D) + row0, 0, rows > 0 ? rows * N * 4 : 0, 0x00020000);
-#pragma unroll
-      for (int it = 0; it < ITER; ++it)
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32v4_t, a4[it]), p_rsrc,
-                                               off[it] == kOob ? kOob : off[it] * 2u, 0, 0);
-      continue;
     }
     auto store_group = [&](int it, float4_t v) {
       __builtin_amdgcn_raw_buffer_store_b64(u32v2_t{E::pack2(v[0], v[1]), E::pack2(v[2], v[3])}, d_rsrc, off[it], 0, 0);
@@ -472,20 +490,43 @@ __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
 // A GEMM with too few output tiles to fill the chip (few rows against a narrow N), split over K:
 // workgroup (tile, share) computes the tile's sums over k in [share * k_per, ...) and stores them
 // as fp32 to P[share][M][N]; splitk_reduce_kernel adds the shares and applies alpha, beta and C.
-template <class E, int BM, int BN, int WM, int WN, bool kBCol>
+// kDual: two weight matrices; the sums of the second go to P1[share][M][N].
+template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
 __global__ __launch_bounds__(256) void gemm_f16_splitk_kernel(
-    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, float* __restrict__ P,
-    int M, int N, int K, int shares, int k_per, int tiles_m, int tiles_n) {
+    const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, const uint16_t* __restrict__ B1,
+    float* __restrict__ P, float* __restrict__ P1, int M, int N, int K, int shares, int k_per, int tiles_m,
+    int tiles_n) {
   const int total = tiles_m * tiles_n * shares;
   const int logical = xcd_order(blockIdx.x, total);
   if (logical >= total) return;
   const int share = logical % shares, tile = logical / shares;
   const int k0 = share * k_per;
   const int k_len = K - k0 < k_per ? K - k0 : k_per;
-  gemm_tile<E, BM, BN, WM, WN, false, kBCol, true>(
-      A + k0, kBCol ? B + k0 : B + (size_t)k0 * N, nullptr, nullptr,
-      reinterpret_cast<uint16_t*>(P + (size_t)share * M * N), M, N, k_len, 1.f, 0.f, N,
-      (tile % tiles_m) * BM, (tile / tiles_m) * BN, K);
+  const size_t b_off = kBCol ? (size_t)k0 : (size_t)k0 * N, p_off = (size_t)share * M * N;
+  gemm_tile<E, BM, BN, WM, WN, kDual, kBCol, true>(
+      A + k0, B + b_off, kDual ? B1 + b_off : nullptr,
+      kDual ? reinterpret_cast<const uint16_t*>(P1 + p_off) : nullptr, reinterpret_cast<uint16_t*>(P + p_off), M, N,
+      k_len, 1.f, 0.f, N, (tile % tiles_m) * BM, (tile / tiles_m) * BN, K);
+}
+
+// out[m][n..n+3] = round(silu(g) * u) with g = round(sum_s P0[s][m][n..]), u likewise from P1: the
+// epilogue of the fused gate/up pair on the summed shares.
+template <class E>
+__global__ __launch_bounds__(256) void splitk_reduce_dual_kernel(const float* __restrict__ P0,
+                                                                 const float* __restrict__ P1, int shares,
+                                                                 uint16_t* out, int M, int N) {
+  const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
+  for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
+    float4_t a = *reinterpret_cast<const float4_t*>(P0 + g * 4), b = *reinterpret_cast<const float4_t*>(P1 + g * 4);
+    for (int s = 1; s < shares; ++s) {
+      a += *reinterpret_cast<const float4_t*>(P0 + s * mn + g * 4);
+      b += *reinterpret_cast<const float4_t*>(P1 + s * mn + g * 4);
+    }
+    float4_t v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = swiglu_rounded<E>(a[e], b[e]);
+    *reinterpret_cast<u32x2*>(out + g * 4) = u32x2{E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+  }
 }
 
 // D[m][n..n+3] = round(alpha * sum_s P[s][m][n..] + beta * C[m][n..]); C has row stride ldc.
@@ -510,12 +551,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
-template <class E, int BM, int BN, int WM, int WN, bool kBCol>
+// kDual: B1 is the second weight matrix, C is not used, D = the SwiGLU output.
+template <class E, int BM, int BN, int WM, int WN, bool kBCol, bool kDual = false>
 static int launch_splitk(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
                          int K, float alpha, float beta, int ldc, int shares, int k_per, float* P,
-                         hipStream_t stream) {
-  using SM = GemmSmem<BM, BN, 1>;
-  auto kern = gemm_f16_splitk_kernel<E, BM, BN, WM, WN, kBCol>;
+                         hipStream_t stream, const uint16_t* B1 = nullptr) {
+  using SM = GemmSmem<BM, BN, kDual ? 2 : 1>;
+  auto kern = gemm_f16_splitk_kernel<E, BM, BN, WM, WN, kDual, kBCol>;
+  float* P1 = kDual ? P + (size_t)shares * M * N : nullptr;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -528,12 +571,13 @@ static int launch_splitk(const uint16_t* A, const uint16_t* B, const uint16_t* C
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int grid = ((tiles_m * tiles_n * shares + 7) / 8) * 8;
-  kern<<<grid, 256, SM::bytes, stream>>>(A, B, P, M, N, K, shares, k_per, tiles_m, tiles_n);
+  kern<<<grid, 256, SM::bytes, stream>>>(A, B, B1, P, P1, M, N, K, shares, k_per, tiles_m, tiles_n);
   int rc = check_launch("gemm split-K launch");
   if (rc) return rc;
   const size_t groups = (size_t)M * N / 4;
   const int rgrid = (int)std::min<size_t>((groups + 255) / 256, 2048);
-  splitk_reduce_kernel<E><<<rgrid, 256, 0, stream>>>(P, shares, C, ldc, D, M, N, alpha, beta);
+  if constexpr (kDual) splitk_reduce_dual_kernel<E><<<rgrid, 256, 0, stream>>>(P, P1, shares, D, M, N);
+  else splitk_reduce_kernel<E><<<rgrid, 256, 0, stream>>>(P, shares, C, ldc, D, M, N, alpha, beta);
   return check_launch("gemm split-K reduction launch");
 }
 
@@ -609,6 +653,17 @@ static int splitk_plan(int M, int N, int K, int* k_per) {
   if (shares < 2) return 1;
   *k_per = ((K + shares - 1) / shares + BK - 1) / BK * BK;
   return (K + *k_per - 1) / *k_per;  // shares that are not empty
+}
+
+// The same for the fused gate/up pair (tiles of 64 x 128 up to 64 rows, else 128 x 128).
+static int splitk_plan_dual(int M, int N, int K, int* k_per) {
+  if (M > 256 || K < 1024) return 1;
+  const int bm = M <= 64 ? 64 : 128;
+  const int tiles = ((M + bm - 1) / bm) * ((N + 127) / 128);
+  const int shares = std::min(std::min(cu_count() / tiles, K / 512), 16);
+  if (shares < 2) return 1;
+  *k_per = ((K + shares - 1) / shares + BK - 1) / BK * BK;
+  return (K + *k_per - 1) / *k_per;
 }
 
 // Tile choice.  A launch takes ceil(tiles / CUs) rounds of one tile each, a round costing the
@@ -713,6 +768,24 @@ static int dual_entry(const char* who, const uint16_t* A, const uint16_t* Bgate,
   return launch_gemm<E, 128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
 }
 
+template <class E>
+static int dual_ws_entry(const char* who, const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup,
+                         uint16_t* out, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                         nf_stream_t stream) {
+  int k_per = 0;
+  const int shares = M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0 ? splitk_plan_dual(M, N, K, &k_per) : 1;
+  if (shares < 2 || !workspace || workspace_bytes < (size_t)2 * shares * M * N * sizeof(float))
+    return dual_entry<E>(who, A, Bgate, Bup, out, M, N, K, stream);
+  int rc = check_gemm_args(who, A, Bgate, out, M, N, K);
+  if (rc) return rc;
+  NF_REQUIRE(Bup && ((uintptr_t)Bup | (uintptr_t)workspace) % 16 == 0, "%s: Bup and the workspace must be 16-byte aligned", who);
+  hipStream_t s = (hipStream_t)stream;
+  float* P = static_cast<float*>(workspace);
+  if (M <= 64)
+    return launch_splitk<E, 64, 128, 2, 2, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
+  return launch_splitk<E, 128, 128, 2, 2, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
+}
+
 extern "C" {
 
 int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
@@ -731,6 +804,24 @@ size_t nf_gemm_workspace_bytes_upto(int max_M, int N, int K) {
   size_t need = 0;
   for (int m = 1; m <= max_M && m <= 256; ++m) need = std::max(need, nf_gemm_workspace_bytes(m, N, K));
   return need;
+}
+
+size_t nf_dual_swiglu_workspace_bytes(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int k_per = 0;
+  const int shares = splitk_plan_dual(M, N, K, &k_per);
+  return shares < 2 ? 0 : (size_t)2 * shares * M * N * sizeof(float);
+}
+
+size_t nf_dual_swiglu_workspace_bytes_upto(int max_M, int N, int K) {
+  size_t need = 0;
+  for (int m = 1; m <= max_M && m <= 256; ++m) need = std::max(need, nf_dual_swiglu_workspace_bytes(m, N, K));
+  return need;
+}
+
+int nf_dual_swiglu_f16_ws(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out, int M,
+                          int N, int K, void* workspace, size_t workspace_bytes, nf_stream_t stream) {
+  return dual_ws_entry<F16>("nf_dual_swiglu_f16_ws", A, Bgate, Bup, out, M, N, K, workspace, workspace_bytes, stream);
 }
 
 int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,

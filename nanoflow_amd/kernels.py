@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libnf_kernels.so")
 SYMBOLS = [
     "nf_abi_version", "nf_last_error", "nf_embedding_f16", "nf_rmsnorm_f16", "nf_gemm_f16", "nf_gemm_bias_f16",
     "nf_gemm_workspace_bytes", "nf_gemm_workspace_bytes_upto", "nf_gemm_f16_ws", "nf_gemm_bias_f16_ws",
+    "nf_dual_swiglu_workspace_bytes", "nf_dual_swiglu_workspace_bytes_upto", "nf_dual_swiglu_f16_ws",
     "nf_dual_swiglu_f16", "nf_gemm_bf16", "nf_dual_swiglu_bf16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
     "nf_quantize_weight_e4m3", "nf_dual_swiglu_f8_f16", "nf_dual_swiglu_f8w_f16", "nf_move_kv_pages",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
@@ -51,6 +52,11 @@ def lib() -> C.CDLL:
         l.nf_gemm_workspace_bytes_upto.restype = sz
         l.nf_gemm_workspace_bytes_upto.argtypes = [i32, i32, i32]
         l.nf_gemm_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp, sz, vp]
+        l.nf_dual_swiglu_workspace_bytes.restype = sz
+        l.nf_dual_swiglu_workspace_bytes.argtypes = [i32, i32, i32]
+        l.nf_dual_swiglu_workspace_bytes_upto.restype = sz
+        l.nf_dual_swiglu_workspace_bytes_upto.argtypes = [i32, i32, i32]
+        l.nf_dual_swiglu_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp, sz, vp]
         l.nf_gemm_bias_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp, sz, vp]
         l.nf_gemm_bias_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
@@ -73,7 +79,8 @@ def lib() -> C.CDLL:
         l.nf_argmax_f16.argtypes = [vp, vp, vp, i32, i32, vp]
         for name in SYMBOLS:
             if name not in ("nf_last_error", "nf_attention_workspace_bytes", "nf_gemm_workspace_bytes",
-                            "nf_gemm_workspace_bytes_upto", "nf_gemm_f8w_workspace_bytes"):
+                            "nf_gemm_workspace_bytes_upto", "nf_gemm_f8w_workspace_bytes",
+                            "nf_dual_swiglu_workspace_bytes", "nf_dual_swiglu_workspace_bytes_upto"):
                 getattr(l, name).restype = i32
         _lib = l
     return _lib
@@ -157,6 +164,10 @@ def gemm_ws(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, w
     _f16(A); _f16(B)
     M, K = A.shape
     N = B.shape[0] if b_col_major else B.shape[1]
+    assert tuple(B.shape) == ((N, K) if b_col_major else (K, N)), (A.shape, B.shape)
+    if Cmat is not None:
+        _f16(Cmat)
+        assert tuple(Cmat.shape) == (M, N)
     need = lib().nf_gemm_workspace_bytes(M, N, K)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
@@ -169,6 +180,21 @@ def gemm_ws(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, w
         return out, need
     _check(lib().nf_gemm_f16_ws(_p(A), _p(B), _p(Cmat), _p(out), M, N, K, alpha, beta, int(b_col_major),
                                 _p(workspace), workspace.numel(), _stream()), "nf_gemm_f16_ws")
+    return out, need
+
+
+def dual_swiglu_ws(A, Bg, Bu, out=None, workspace=None):
+    """nf_dual_swiglu_f16_ws; returns (out, bytes of workspace the shape asks for: 0 = not split)."""
+    _f16(A); _f16(Bg); _f16(Bu)
+    M, K = A.shape
+    N = Bg.shape[1]
+    assert tuple(Bg.shape) == (K, N) and tuple(Bu.shape) == (K, N)
+    need = lib().nf_dual_swiglu_workspace_bytes(M, N, K)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
+    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
+    _check(lib().nf_dual_swiglu_f16_ws(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, _p(workspace), workspace.numel(),
+                                       _stream()), "nf_dual_swiglu_f16_ws")
     return out, need
 
 

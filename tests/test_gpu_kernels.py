@@ -212,6 +212,25 @@ def test_dual_swiglu(K, oracle, M, N, K_):
                  what="dual swiglu")
 
 
+@pytest.mark.parametrize("M,N,K_", [(16, 14336, 4096), (64, 1160, 2056), (128, 14336, 1024), (200, 2048, 4096)])
+def test_dual_swiglu_split_over_k_matches_oracle(K, oracle, M, N, K_):
+    """Few rows: both products of the gate/up pair are split over K, summed in fp32, rounded to fp16 and
+    put through SiLU-mul by the reduction.  Twice the fp16 tolerance, as for the bf16 and fp8 pairs: a
+    product on an fp16 rounding boundary may round the other way than in the oracle."""
+    rng = np.random.default_rng(M + N)
+    A = synth.normal_f16(rng, (M, K_))
+    Bg = synth.normal_f16(rng, (K_, N), 0.02)
+    Bu = synth.normal_f16(rng, (K_, N), 0.02)
+    got, need = K.dual_swiglu_ws(dev(A), dev(Bg), dev(Bu))
+    assert need > 0 and need % (2 * M * N * 4) == 0 and need // (2 * M * N * 4) >= 2, "this shape is meant to be split"
+    assert_close(host(got), oracle.dual_swiglu(A, Bg, Bu), 2 * RTOL, what="split-K dual swiglu")
+    assert not np.array_equal(host(got), host(K.dual_swiglu_ws(dev(A), dev(Bu), dev(Bg))[0]))     # gate is the first
+    short, _ = K.dual_swiglu_ws(dev(A), dev(Bg), dev(Bu), workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+    assert np.array_equal(host(short), host(K.dual_swiglu(dev(A), dev(Bg), dev(Bu))))
+    _, need = K.dual_swiglu_ws(dev(A[:, :512]), dev(Bg[:512]), dev(Bu[:512]))                     # K < 1024: not split
+    assert need == 0
+
+
 def test_dual_known_answer_inputs(K, oracle):
     # inputs of the reference's dual-GEMM test program (all operands (j+k)/2560, 128^3)
     j, k = np.meshgrid(np.arange(128), np.arange(128), indexing="ij")
