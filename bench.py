@@ -14,6 +14,8 @@ layers, vocab 128256, fp16 random-init weights, paged KV with page 16).
 --workload iteration: ONE dense 2048-token iteration = 1792 decode tokens (KV length uniform
   in [1024, 1536], permuted page table) + one 256-token prefill chunk, update data staged once
   before the timed region; a step is one ``run()`` = embedding ... sampler.
+  --decode-requests / --prefill-chunk give other mixes, e.g. 64 and 0: the decode-only iteration
+  of a lightly loaded server.
 
 Prints one JSON line: tokens/s, the roofline record of the dominant kernel (offline: the dense
 MFMA GEMMs; iteration: paged decode attention, HBM-bound -- durations from HIP events recorded
@@ -171,8 +173,17 @@ def run_iteration(args):
     T = 2048
     steps = args.steps or 5
     warmup = 2 if args.warmup is None else args.warmup
-    batch = synth.config2_batch(seed=args.seed, vocab=shape.vocab)
-    assert batch.tokens == T
+    # the default mix fills the iteration; --decode-requests / --prefill-chunk give others
+    # (e.g. 64 and 0: the decode-only iteration of a lightly loaded server)
+    n_dec, n_pre = args.decode_requests, args.prefill_chunk
+    if n_dec < 1 or n_pre < 0 or n_dec + n_pre > T:
+        raise SystemExit(f"--decode-requests must be at least 1 and, with --prefill-chunk, at most {T}")
+    if n_pre > 0:
+        batch = synth.config2_batch(seed=args.seed, n_decode=n_dec, prefill_chunk=n_pre, vocab=shape.vocab)
+    else:
+        lens = np.random.default_rng(args.seed + 2).integers(1024, 1537, size=n_dec)
+        batch = synth.make_batch(lens, [], shape.vocab, seed=args.seed)
+    assert batch.tokens == n_dec + n_pre
     pages = batch.num_pages
 
     # Distinct layers held: 32 layers of this KV (9.5 GB each) exceed 288 GB, so layers alias
@@ -218,18 +229,19 @@ def run_iteration(args):
     launches_per_layer = sum(1 for g in groups if g > 0)
     bytes_per_layer = decode_attention_bytes(batch.kv_len[:nd], shape.Hq, shape.Hkv, shape.d)
     lm_rows = min((batch.req_num + 127) // 128 * 128, T)
-    flops = gemm_flops_per_iteration(shape, T, lm_rows, shape.layers)
+    flops = gemm_flops_per_iteration(shape, batch.tokens, lm_rows, shape.layers)
     fp8_share = 1.0 - 2.0 * lm_rows * shape.hidden * shape.vocab / flops if wb == 1 else 0.0
 
     rec = {
-        "metric": "tokens/s/GPU", "value": T / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "metric": "tokens/s/GPU", "value": batch.tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16" if wb == 2 else "f8e4m3 weights and GEMM inputs, f16 activations and KV",
         "data": "synthetic",
         "config": {
-            "workload": (f"{shape_name} shape, one dense 2048-token iteration: 1792 decode tokens "
-                         "(KV U[1024,1536], page 16, permuted page table) + one 256-token prefill chunk"),
+            "workload": (f"{shape_name} shape, one " + ("dense 2048-token " if n_dec + n_pre == T else "")
+                         + f"iteration: {n_dec} decode tokens (KV U[1024,1536], page 16, permuted page table)"
+                         + (f" + one {n_pre}-token prefill chunk" if n_pre else "")),
             "weights": args.weights,
             "pipeline": args.pipeline, "global_batch": T, "nanobatch_1_size": args.nano1,
             "kqv1_size": args.kqv1, "kqv3_size": args.kqv3, "layers_executed": shape.layers,
@@ -400,6 +412,8 @@ def main():
     ap.add_argument("--nano1", type=int, default=1024, help="rows of nano-batch 1")
     ap.add_argument("--kqv1", type=int, default=512)
     ap.add_argument("--kqv3", type=int, default=512)
+    ap.add_argument("--decode-requests", type=int, default=1792, help="iteration workload: decode requests (one token each)")
+    ap.add_argument("--prefill-chunk", type=int, default=256, help="iteration workload: tokens of the one prefill chunk (0 = none)")
     ap.add_argument("--distinct-layers", type=int, default=0,
                     help="iteration workload: distinct weight/KV layers held in HBM (0 = as many of the 32 as fit)")
     ap.add_argument("--requests", type=int, default=4096, help="offline workload: requests in the trace")
