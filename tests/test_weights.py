@@ -118,6 +118,20 @@ def test_kqv_bias_is_served_by_the_bias_pipelines_and_never_dropped(tmp_path):
         assert w["b_kqv"][l].shape == (shape.kqv_n,) and np.array_equal(w["b_kqv"][l], want)
 
 
+def test_trace_generator_writes_what_the_serving_command_reads(tmp_path):
+    from nanoflow_amd import gen_req, serve
+    p = gen_req.write_trace(str(tmp_path / "t.csv"), 50, "200:700", "512", rate=10.0, poisson=True, seed=3)
+    reqs = serve.read_trace(p)
+    assert len(reqs) == 50 and [r[0] for r in reqs] == list(range(50))
+    assert all(200 <= r[1] <= 700 and r[2] == 512 for r in reqs)
+    arr = [r[3] for r in reqs]
+    assert arr == sorted(arr) and 2.0 < arr[-1] < 12.0            # 50 requests at 10 per second
+    p = gen_req.write_trace(str(tmp_path / "c.csv"), 8, rate=4.0)
+    assert [r[3] for r in serve.read_trace(p)] == [i / 4.0 for i in range(8)]
+    p = gen_req.write_trace(str(tmp_path / "o.csv"), 3)
+    assert serve.read_trace(p) == [(0, 1024, 512, 0.0), (1, 1024, 512, 0.0), (2, 1024, 512, 0.0)]
+
+
 def test_shape_mismatch_and_foreign_files_raise(tmp_path):
     out_dir = str(tmp_path / "w")
     W.convert_hf_checkpoint(_write_checkpoint(tmp_path, _hf_state_dict()), out_dir)
