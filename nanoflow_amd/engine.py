@@ -30,7 +30,7 @@ def write_config(path, shape: synth.ModelShape, *, global_batch, nano1, kqv1, kq
             "hidden_size": shape.hidden, "intermediate_size": shape.ffn,
             "num_attention_heads": shape.Hq, "num_key_value_heads": shape.Hkv,
             "num_hidden_layers": layers, "rms_norm_eps": shape.eps, "rope_theta": shape.rope_theta,
-            "rope_scaling": None, "vocab_size": shape.vocab,
+            "rope_scaling": shape.rope_scaling, "vocab_size": shape.vocab,
         },
         "model_configs": {
             "gpu_num": 1, "run_layer": shape.layers if run_layer is None else run_layer,

@@ -84,7 +84,8 @@ def main():
     shape = synth.ModelShape(hidden=m["hidden_size"], Hq=m["num_attention_heads"], Hkv=m["num_key_value_heads"],
                              d=m["hidden_size"] // m["num_attention_heads"], ffn=m["intermediate_size"],
                              vocab=m["vocab_size"], layers=m["num_hidden_layers"], page_size=mc.get("frame_page_size", 16),
-                             eps=m.get("rms_norm_eps", 1e-5), rope_theta=m.get("rope_theta", 1e4))
+                             eps=m.get("rms_norm_eps", 1e-5), rope_theta=m.get("rope_theta", 1e4),
+                             rope_scaling=m.get("rope_scaling") or None)   # Llama-3.1 (config_all/llama3.1-8B)
     pt = P.PipelineType[sc["pipeline_type"]]
     T, nano1, kqv1, kqv3 = pc["global_batch_size"], pc["nanobatch_1_size"], pc["kqv1_size"], pc["kqv3_size"]
     pages = 1024 * mc["allocate_kv_data_batch"] // 16

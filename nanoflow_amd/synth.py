@@ -31,6 +31,18 @@ class ModelShape:
     rope_scale: float = 1.0
     smooth_a: float = 0.0
     smooth_b: float = 0.0
+    # the Llama-3.1 "rope_scaling" block of a model config (factor, low_freq_factor, high_freq_factor,
+    # original_max_position_embeddings); when given, rope_scale / smooth_a / smooth_b are derived from
+    # it as the pipeline's configuration does (pipeline/include/config.h:101-110)
+    rope_scaling: dict | None = None
+
+    def __post_init__(self):
+        rs = self.rope_scaling
+        if rs:
+            lo, hi = float(rs["low_freq_factor"]), float(rs["high_freq_factor"])
+            self.rope_scale = float(rs["factor"])
+            self.smooth_a = float(rs["original_max_position_embeddings"]) / (2 * np.pi * hi - 2 * np.pi * lo)
+            self.smooth_b = -1.0 / (hi / lo - 1.0)
 
     @property
     def kqv_n(self) -> int:

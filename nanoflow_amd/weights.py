@@ -70,7 +70,8 @@ def shape_from_hf_config(cfg: dict, page_size: int = 16) -> synth.ModelShape:
     return synth.ModelShape(hidden=cfg["hidden_size"], Hq=hq, Hkv=cfg.get("num_key_value_heads", hq),
                             d=cfg.get("head_dim") or cfg["hidden_size"] // hq, ffn=cfg["intermediate_size"],
                             vocab=cfg["vocab_size"], layers=cfg["num_hidden_layers"], page_size=page_size,
-                            eps=cfg.get("rms_norm_eps", 1e-5), rope_theta=cfg.get("rope_theta", 1e4))
+                            eps=cfg.get("rms_norm_eps", 1e-5), rope_theta=cfg.get("rope_theta", 1e4),
+                            rope_scaling=cfg.get("rope_scaling") or None)
 
 
 def _read_safetensors_dir(hf_dir: str) -> dict:

@@ -274,6 +274,38 @@ def test_fp8_weights_and_kqv_bias_do_not_combine():
         P.setWeightFormat(P.WeightFormat.F16)
 
 
+def test_llama31_rope_scaling_reaches_the_kernel_through_the_config(oracle):
+    """A model config with a "rope_scaling" block (Llama-3.1): the pipeline derives the frequency rule
+    from the JSON (factor, smoothing constants) and must agree with the oracle given the same
+    constants -- and differ from the unscaled rule, so that a dropped block cannot pass."""
+    from nanoflow_amd import engine, pllm_python as P
+    T, nano1, dlens, chunks = CASES["decode_crosses_border"]
+    rs = {"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 64,
+          "rope_type": "llama3"}            # a short original context, so that positions below 60 already feel it
+    base = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    shape = synth.ModelShape(**{**base.as_dict(), "rope_scaling": rs, "rope_theta": 1e4})
+    plain = synth.ModelShape(**{**base.as_dict(), "rope_theta": 1e4})
+    assert shape.rope_scale == 8.0 and shape.smooth_a > 0 and shape.smooth_b < 0
+    w = _scaled_weights(shape, seed=0)
+    b1 = synth.make_batch(dlens, chunks, vocab=shape.vocab, seed=21, extra_pages=40)
+    rng = np.random.default_rng(5)
+    pools0 = [synth.make_kv_pool(b1.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok1 = b1.input_tokens.copy()
+    tok1[:b1.decodePrefillBorder] = 1
+    d1 = b1.as_dict()
+    d1["input_tokens"] = tok1
+    hid, _, _ = oracle.decoder_forward(shape.as_dict(), w, [p.copy() for p in pools0], d1)
+    hid_plain, _, _ = oracle.decoder_forward(plain.as_dict(), w, [p.copy() for p in pools0], d1)
+    assert _max_rel(hid_plain, hid) > 10 * E2E_RTOL, "the scaling must matter for this test to mean anything"
+    for pt in (P.PipelineType.NON_OVERLAP_LOCAL, P.PipelineType.LOCAL):
+        with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=max(nano1 // 2, 1), kqv3=(T - nano1) // 2,
+                           kv_pages=b1.num_pages, weights=w, kv_pools=pools0) as e:
+            e.update(b1, keep_token_list=np.ones(b1.decodePrefillBorder, np.int32))
+            e.run()
+            h = e.buffer("hidden").cpu().numpy()[:b1.tokens]
+        assert _max_rel(h, hid) < E2E_RTOL, (pt, _max_rel(h, hid))
+
+
 def test_unsupported_pipeline_types_are_rejected():
     from nanoflow_amd import engine, pllm_python as P
     shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)
