@@ -138,6 +138,15 @@ NF_API int nf_dual_swiglu_bf16(const uint16_t* A, const uint16_t* Bgate, const u
  *   Aq[m][k] * Gq[n][k]) and u likewise from Uq, u_scale: nf_dual_swiglu_f16 on fp8 operands
  *   (products rounded to fp16 before SiLU-mul, as there).  nf_dual_swiglu_f8w_f16: the same from
  *   fp16 activations, quantised into `workspace` (nf_gemm_f8w_workspace_bytes(M, K) bytes). */
+/* nf_gemm_f8w_f16 and nf_dual_swiglu_f8w_f16 split launches of at most 256 rows over K, like
+ * nf_gemm_f16_ws, when the workspace also has room for the fp32 sums behind the quantised rows:
+ * nf_gemm_f8w_split_workspace_bytes(M, N, K) / nf_dual_swiglu_f8w_split_workspace_bytes(M, N, K)
+ * bytes (equal to nf_gemm_f8w_workspace_bytes(M, K) for shapes that are not split); *_upto: the
+ * largest requirement over 1..max_M rows. */
+NF_API size_t nf_gemm_f8w_split_workspace_bytes(int M, int N, int K);
+NF_API size_t nf_gemm_f8w_split_workspace_bytes_upto(int max_M, int N, int K);
+NF_API size_t nf_dual_swiglu_f8w_split_workspace_bytes(int M, int N, int K);
+NF_API size_t nf_dual_swiglu_f8w_split_workspace_bytes_upto(int max_M, int N, int K);
 NF_API int nf_quantize_weight_e4m3(const uint16_t* W, uint8_t* Wq, float* col_scale, int K, int N,
                                    nf_stream_t stream);
 NF_API int nf_dual_swiglu_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Gq, const float* g_scale,

@@ -23,7 +23,7 @@ struct DualWrapper : public OperatorWrapper {
   void setWeightFormat(WeightFormat f) { e4m3 = f == WeightFormat::E4M3; }
   // fp16 weights: scratch for launches of few rows that are split over K (nf_dual_swiglu_f16_ws)
   size_t workspaceBytes() const {
-    return e4m3 ? nf_gemm_f8w_workspace_bytes(M, K) : nf_dual_swiglu_workspace_bytes_upto(M, N, K);
+    return e4m3 ? nf_dual_swiglu_f8w_split_workspace_bytes_upto(M, N, K) : nf_dual_swiglu_workspace_bytes_upto(M, N, K);
   }
   void setWorkspace(void* ptr, size_t bytes) {
     workspace = ptr;

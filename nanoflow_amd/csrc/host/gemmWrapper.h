@@ -176,7 +176,8 @@ struct HipGEMMWrapperF8W : public HipGEMMWrapper {
     std::fprintf(stderr, "%s: a bias row is not implemented for e4m3 weights\n", name.c_str());
     std::exit(EXIT_FAILURE);
   }
-  size_t workspaceBytes() const override { return nf_gemm_f8w_workspace_bytes((int)M, (int)K); }
+  // quantised input rows, and the fp32 sums of launches of few rows that are split over K
+  size_t workspaceBytes() const override { return nf_gemm_f8w_split_workspace_bytes_upto((int)M, (int)N, (int)K); }
   void setWorkspace(void* ptr, size_t bytes) override {
     workspace = ptr;
     workspace_bytes = bytes;

@@ -15,6 +15,7 @@
 //
 // A dot product does not depend on which k a lane slot holds as long as both operands use the
 // same assignment; lane (l32, lg) slot s of k-step kk holds k = kk*64 + lg*32 + s for both.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -157,11 +158,16 @@ __device__ __forceinline__ float swiglu_rounded_f16(float g_acc, float u_acc) {
 // kDual: two weight matrices B (gate) and B1 (up) with scales sb and sb1,
 //   D[m][n] = half(silu(g) * u),  g = half(sa[m] * sb[n] * sum_k Aq.Bq),  u = half(sa[m] * sb1[n] * sum_k Aq.B1q);
 // alpha, beta and C are not used.
-template <int BM, int BN, int WM, int WN, bool kDual>
+// kPartial: one share of a GEMM split over K (see gemm.hip).  Workgroup (tile, share) sums over
+// k in [share * k_per, ...) and stores the fp32 sums, unscaled, to D taken as float
+// [shares][M][N] (kDual: the sums of the second product to C taken the same way); Kt is then the
+// whole contraction (the row stride of both operands), shares and k_per describe the split.
+template <int BM, int BN, int WM, int WN, bool kDual, bool kPartial = false>
 __global__ __launch_bounds__(256) void gemm_f8_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, const uint8_t* __restrict__ B1,
     const float* __restrict__ sa, const float* __restrict__ sb, const float* __restrict__ sb1,
-    const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha, float beta, int tiles_m, int tiles_n) {
+    const uint16_t* C, uint16_t* D, int M, int N, int Kt, float alpha, float beta, int tiles_m, int tiles_n,
+    int shares, int k_per) {
   constexpr int NB = kDual ? 2 : 1;
   using SM = F8Smem<BM, BN, NB>;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -178,10 +184,23 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
 
   // XCD-aware tile order (workgroup ids round-robin over 8 XCDs): each XCD walks one
   // contiguous range of tiles, M fastest, so a weight panel stays in that XCD's L2.
-  const int ntiles = tiles_m * tiles_n;
+  const int ntiles = tiles_m * tiles_n * (kPartial ? shares : 1);
   const int per_xcd = (ntiles + 7) / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (logical >= ntiles) return;
+  int K = Kt;                       // extent of this workgroup's contraction
+  const int lda = Kt;               // row stride of both operands (k contiguous)
+  size_t p_off = 0;                 // this share's slice of the partial sums
+  if constexpr (kPartial) {
+    const int share = logical % shares;
+    logical /= shares;
+    const int k0 = share * k_per;
+    K = Kt - k0 < k_per ? Kt - k0 : k_per;
+    A += k0;
+    B += k0;
+    if constexpr (kDual) B1 += k0;
+    p_off = (size_t)share * M * N;
+  }
   const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
   const int m_base = tile_m * BM, n_base = tile_n * BN;
 
@@ -206,18 +225,18 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   // offset per load instruction, advanced by a slab after each use; rows past the operand's last
   // one lie at or past the end of the buffer and read as zero, which leaves only k >= K inside a
   // row to be masked.
-  const rsrc_t a_rsrc = make_rsrc(A, (size_t)M * K);
-  const rsrc_t b_rsrc[2] = {make_rsrc(B, (size_t)N * K), make_rsrc(kDual ? B1 : B, (size_t)N * K)};
+  const rsrc_t a_rsrc = make_rsrc(A, (size_t)(M - 1) * lda + K);
+  const rsrc_t b_rsrc[2] = {make_rsrc(B, (size_t)(N - 1) * lda + K), make_rsrc(kDual ? B1 : B, (size_t)(N - 1) * lda + K)};
   const int kc = ((lane & 7) ^ (((lane >> 4) & 3) | ((wave & 1) << 2))) * 16;  // k-byte of this lane's chunk inside the slab
   uint32_t a_off[A_LOADS], b_off[NB][B_LOADS];
 #pragma unroll
   for (int t = 0; t < A_LOADS; ++t)
-    a_off[t] = (uint32_t)(m_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)K + kc;
+    a_off[t] = (uint32_t)(m_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)lda + kc;
 #pragma unroll
   for (int b = 0; b < NB; ++b)
 #pragma unroll
     for (int t = 0; t < B_LOADS; ++t)
-      b_off[b][t] = (uint32_t)(n_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)K + kc;
+      b_off[b][t] = (uint32_t)(n_base + (t * 4 + wave) * 8 + (lane >> 3)) * (uint32_t)lda + kc;
   auto load_one = [&](auto t_c, uint32_t st, bool k_ok) {
     constexpr int t = decltype(t_c)::value;
     if constexpr (t < A_LOADS) {
@@ -350,11 +369,13 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
   const int gn0 = n_base + wn * CW;
   const int gn = gn0 + (lane % CPR) * 4;  // the same 4 columns in every pass: 64 % CPR == 0
   float4_t cs4 = float4_t{0.f, 0.f, 0.f, 0.f}, cu4 = float4_t{0.f, 0.f, 0.f, 0.f};
-  if (gn < N) cs4 = *reinterpret_cast<const float4_t*>(sb + gn);
-  if constexpr (kDual) {
-    if (gn < N) cu4 = *reinterpret_cast<const float4_t*>(sb1 + gn);
-  } else {
-    cs4 *= alpha;
+  if constexpr (!kPartial) {
+    if (gn < N) cs4 = *reinterpret_cast<const float4_t*>(sb + gn);
+    if constexpr (kDual) {
+      if (gn < N) cu4 = *reinterpret_cast<const float4_t*>(sb1 + gn);
+    } else {
+      cs4 *= alpha;
+    }
   }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -362,6 +383,34 @@ __global__ __launch_bounds__(256) void gemm_f8_kernel(
     const int rows = M - gm0 < 32 ? M - gm0 : 32;
     const int recs = rows > 0 ? rows * N * 2 : 0;
     const size_t row0 = (size_t)(rows > 0 ? gm0 : 0);
+    if constexpr (kPartial) {
+      // the fp32 sums as they are (scales, alpha, beta and C belong to the reduction), one product
+      // after the other through the first staging area
+      typedef unsigned int u32v4_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int qd = 0; qd < 4; ++qd) {
+            float4_t v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[b][i][j][qd * 4 + e];
+            *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
+          }
+        float* dst = (b == 0 ? reinterpret_cast<float*>(D) : reinterpret_cast<float*>(const_cast<uint16_t*>(C))) + p_off;
+        const __amdgpu_buffer_rsrc_t p_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(dst + row0 * N, 0, rows > 0 ? rows * N * 4 : 0, 0x00020000);
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+          const int c = it * 64 + lane;
+          const float4_t p4 = *reinterpret_cast<const float4_t*>(ep + (c / CPR) * ROWP + (c % CPR) * 16);
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32v4_t, p4), p_rsrc,
+                                                 gn < N ? (uint32_t)((c / CPR) * N + gn) * 4u : kOob, 0, 0);
+        }
+      }
+      continue;
+    }
     const __amdgpu_buffer_rsrc_t d_rsrc = __builtin_amdgcn_make_buffer_rsrc(D + row0 * N, 0, recs, 0x00020000);
     const __amdgpu_buffer_rsrc_t s_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(sa) + row0, 0, rows > 0 ? rows * 4 : 0, 0x00020000);
@@ -448,8 +497,100 @@ static int launch_gemm_f8(const uint8_t* A, const uint8_t* B, const float* sa, c
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int grid = ((tiles_m * tiles_n + 7) / 8) * 8;
-  kern<<<grid, 256, SM::bytes, stream>>>(A, B, B1, sa, sb, sb1, C, D, M, N, K, alpha, beta, tiles_m, tiles_n);
+  kern<<<grid, 256, SM::bytes, stream>>>(A, B, B1, sa, sb, sb1, C, D, M, N, K, alpha, beta, tiles_m, tiles_n, 1, K);
   return check_launch("gemm_f8 launch");
+}
+
+// D[m][n..n+3] = half(alpha * sa[m] * sb[n..] * sum_s P[s][m][n..] + beta * C[m][n..])
+__global__ __launch_bounds__(256) void splitk_reduce_f8_kernel(const float* __restrict__ P, int shares,
+                                                               const float* __restrict__ sa,
+                                                               const float* __restrict__ sb, const uint16_t* C,
+                                                               uint16_t* D, int M, int N, float alpha, float beta) {
+  const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
+  for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
+    float4_t v = *reinterpret_cast<const float4_t*>(P + g * 4);
+    for (int s = 1; s < shares; ++s) v += *reinterpret_cast<const float4_t*>(P + s * mn + g * 4);
+    const size_t m = g * 4 / N, n = g * 4 % N;
+    v = v * (*reinterpret_cast<const float4_t*>(sb + n) * alpha) * sa[m];
+    if (beta != 0.f) {
+      const u32x2 c = *reinterpret_cast<const u32x2*>(C + g * 4);
+      v[0] += beta * h2f_bits(c.x & 0xffffu);
+      v[1] += beta * h2f_bits(c.x >> 16);
+      v[2] += beta * h2f_bits(c.y & 0xffffu);
+      v[3] += beta * h2f_bits(c.y >> 16);
+    }
+    *reinterpret_cast<u32x2*>(D + g * 4) = u32x2{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3])};
+  }
+}
+
+// the gate/up pair: both sums scaled, rounded to fp16, then SiLU-mul
+__global__ __launch_bounds__(256) void splitk_reduce_dual_f8_kernel(const float* __restrict__ P0,
+                                                                    const float* __restrict__ P1, int shares,
+                                                                    const float* __restrict__ sa,
+                                                                    const float* __restrict__ sg,
+                                                                    const float* __restrict__ su, uint16_t* out,
+                                                                    int M, int N) {
+  const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
+  for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
+    float4_t a = *reinterpret_cast<const float4_t*>(P0 + g * 4), b = *reinterpret_cast<const float4_t*>(P1 + g * 4);
+    for (int s = 1; s < shares; ++s) {
+      a += *reinterpret_cast<const float4_t*>(P0 + s * mn + g * 4);
+      b += *reinterpret_cast<const float4_t*>(P1 + s * mn + g * 4);
+    }
+    const size_t m = g * 4 / N, n = g * 4 % N;
+    a = a * *reinterpret_cast<const float4_t*>(sg + n) * sa[m];
+    b = b * *reinterpret_cast<const float4_t*>(su + n) * sa[m];
+    float4_t v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = swiglu_rounded_f16(a[e], b[e]);
+    *reinterpret_cast<u32x2*>(out + g * 4) = u32x2{pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3])};
+  }
+}
+
+// Shares of a split over K (see gemm.hip): at most 256 rows, tiles of 64 x 256 (the pair: 64 x 128)
+// up to 64 rows, else 128 x 128, as many shares as fill the CUs, each at least 1024 k deep (8 slabs).
+static int splitk_plan_f8(int M, int N, int K, bool dual, int* k_per) {
+  if (M > 256 || K < 2048) return 1;
+  const int bm = M <= 64 ? 64 : 128, bn = M <= 64 && !dual ? 256 : 128;
+  const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+  int cus = 256, dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  const int shares = std::min(std::min(cus / tiles, K / 1024), 16);
+  if (shares < 2) return 1;
+  *k_per = ((K + shares - 1) / shares + F8_BK - 1) / F8_BK * F8_BK;
+  return (K + *k_per - 1) / *k_per;
+}
+
+template <int BM, int BN, int WM, int WN, bool kDual>
+static int launch_splitk_f8(const uint8_t* A, const uint8_t* B, const uint8_t* B1, const float* sa,
+                            const float* sb, const float* sb1, const uint16_t* C, uint16_t* D, int M, int N,
+                            int K, float alpha, float beta, int shares, int k_per, float* P, hipStream_t stream) {
+  using SM = F8Smem<BM, BN, kDual ? 2 : 1>;
+  auto kern = gemm_f8_kernel<BM, BN, WM, WN, kDual, true>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)SM::bytes);
+    if (e != hipSuccess) {
+      set_error("gemm_f8: cannot reserve %zu bytes of LDS: %s", SM::bytes, hipGetErrorString(e));
+      return NF_ERR_RUNTIME;
+    }
+    attr_set = true;
+  }
+  float* P1 = kDual ? P + (size_t)shares * M * N : nullptr;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int grid = ((tiles_m * tiles_n * shares + 7) / 8) * 8;
+  kern<<<grid, 256, SM::bytes, stream>>>(A, B, B1, nullptr, nullptr, nullptr, reinterpret_cast<const uint16_t*>(P1),
+                                         reinterpret_cast<uint16_t*>(P), M, N, K, 1.f, 0.f, tiles_m, tiles_n,
+                                         shares, k_per);
+  int rc = check_launch("gemm_f8 split-K launch");
+  if (rc) return rc;
+  const int rgrid = (int)std::min<size_t>(((size_t)M * N / 4 + 255) / 256, 2048);
+  if constexpr (kDual) splitk_reduce_dual_f8_kernel<<<rgrid, 256, 0, stream>>>(P, P1, shares, sa, sb, sb1, D, M, N);
+  else splitk_reduce_f8_kernel<<<rgrid, 256, 0, stream>>>(P, shares, sa, sb, C, D, M, N, alpha, beta);
+  return check_launch("gemm_f8 split-K reduction launch");
 }
 
 }  // namespace nf
@@ -545,7 +686,48 @@ int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* b_scale, 
   float* sa = reinterpret_cast<float*>(Aq + ((size_t)M * K + 255) / 256 * 256);
   int rc = nf_quantize_rows_e4m3(A, Aq, sa, M, K, stream);
   if (rc) return rc;
+  // few rows against a narrow N: split over K when the workspace also holds the partial sums
+  int k_per = 0;
+  const int shares = N > 0 && N % 8 == 0 && K % 16 == 0 ? splitk_plan_f8(M, N, K, false, &k_per) : 1;
+  const size_t p_at = (need + 255) / 256 * 256;
+  if (shares >= 2 && workspace_bytes >= p_at + (size_t)shares * M * N * sizeof(float) && Bq && b_scale && D &&
+      ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull &&
+      (beta == 0.f || C) && ((uintptr_t)Bq | (uintptr_t)b_scale) % 16 == 0 && ((uintptr_t)D | (uintptr_t)C) % 8 == 0) {
+    float* P = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p_at);
+    hipStream_t s = (hipStream_t)stream;
+    if (M <= 64)
+      return launch_splitk_f8<64, 256, 1, 4, false>(Aq, Bq, nullptr, sa, b_scale, nullptr, C, D, M, N, K, alpha, beta, shares, k_per, P, s);
+    return launch_splitk_f8<128, 128, 2, 2, false>(Aq, Bq, nullptr, sa, b_scale, nullptr, C, D, M, N, K, alpha, beta, shares, k_per, P, s);
+  }
   return nf_gemm_f8_f16(Aq, sa, Bq, b_scale, C, D, M, N, K, alpha, beta, stream);
+}
+
+size_t nf_gemm_f8w_split_workspace_bytes(int M, int N, int K) {
+  const size_t need = nf_gemm_f8w_workspace_bytes(M, K);
+  if (M <= 0 || N <= 0 || K <= 0) return need;
+  int k_per = 0;
+  const int shares = splitk_plan_f8(M, N, K, false, &k_per);
+  return shares < 2 ? need : (need + 255) / 256 * 256 + (size_t)shares * M * N * sizeof(float);
+}
+
+size_t nf_gemm_f8w_split_workspace_bytes_upto(int max_M, int N, int K) {
+  size_t need = nf_gemm_f8w_workspace_bytes(max_M, K);
+  for (int m = 1; m <= max_M && m <= 256; ++m) need = std::max(need, nf_gemm_f8w_split_workspace_bytes(m, N, K));
+  return need;
+}
+
+size_t nf_dual_swiglu_f8w_split_workspace_bytes(int M, int N, int K) {
+  const size_t need = nf_gemm_f8w_workspace_bytes(M, K);
+  if (M <= 0 || N <= 0 || K <= 0) return need;
+  int k_per = 0;
+  const int shares = splitk_plan_f8(M, N, K, true, &k_per);
+  return shares < 2 ? need : (need + 255) / 256 * 256 + (size_t)2 * shares * M * N * sizeof(float);
+}
+
+size_t nf_dual_swiglu_f8w_split_workspace_bytes_upto(int max_M, int N, int K) {
+  size_t need = nf_gemm_f8w_workspace_bytes(max_M, K);
+  for (int m = 1; m <= max_M && m <= 256; ++m) need = std::max(need, nf_dual_swiglu_f8w_split_workspace_bytes(m, N, K));
+  return need;
 }
 
 int nf_dual_swiglu_f8w_f16(const uint16_t* A, const uint8_t* Gq, const float* g_scale, const uint8_t* Uq,
@@ -563,6 +745,19 @@ int nf_dual_swiglu_f8w_f16(const uint16_t* A, const uint8_t* Gq, const float* g_
   float* sa = reinterpret_cast<float*>(Aq + ((size_t)M * K + 255) / 256 * 256);
   int rc = nf_quantize_rows_e4m3(A, Aq, sa, M, K, stream);
   if (rc) return rc;
+  int k_per = 0;
+  const int shares = N > 0 && N % 8 == 0 && K % 16 == 0 ? splitk_plan_f8(M, N, K, true, &k_per) : 1;
+  const size_t p_at = (need + 255) / 256 * 256;
+  if (shares >= 2 && workspace_bytes >= p_at + (size_t)2 * shares * M * N * sizeof(float) && Gq && g_scale && Uq &&
+      ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull &&
+      u_scale && out &&
+      ((uintptr_t)Gq | (uintptr_t)Uq | (uintptr_t)g_scale | (uintptr_t)u_scale) % 16 == 0 && (uintptr_t)out % 8 == 0) {
+    float* P = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p_at);
+    hipStream_t s = (hipStream_t)stream;
+    if (M <= 64)
+      return launch_splitk_f8<64, 128, 2, 2, true>(Aq, Gq, Uq, sa, g_scale, u_scale, nullptr, out, M, N, K, 1.f, 0.f, shares, k_per, P, s);
+    return launch_splitk_f8<128, 128, 2, 2, true>(Aq, Gq, Uq, sa, g_scale, u_scale, nullptr, out, M, N, K, 1.f, 0.f, shares, k_per, P, s);
+  }
   return nf_dual_swiglu_f8_f16(Aq, sa, Gq, g_scale, Uq, u_scale, out, M, N, K, stream);
 }
 

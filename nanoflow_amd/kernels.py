@@ -20,6 +20,8 @@ SYMBOLS = [
     "nf_dual_swiglu_workspace_bytes", "nf_dual_swiglu_workspace_bytes_upto", "nf_dual_swiglu_f16_ws",
     "nf_dual_swiglu_f16", "nf_gemm_bf16", "nf_dual_swiglu_bf16", "nf_quantize_rows_e4m3", "nf_gemm_f8_f16", "nf_gemm_f8w_workspace_bytes",
     "nf_quantize_weight_e4m3", "nf_dual_swiglu_f8_f16", "nf_dual_swiglu_f8w_f16", "nf_move_kv_pages",
+    "nf_gemm_f8w_split_workspace_bytes", "nf_gemm_f8w_split_workspace_bytes_upto",
+    "nf_dual_swiglu_f8w_split_workspace_bytes", "nf_dual_swiglu_f8w_split_workspace_bytes_upto",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
 ]
@@ -67,6 +69,10 @@ def lib() -> C.CDLL:
         l.nf_gemm_f8w_workspace_bytes.restype = C.c_size_t
         l.nf_gemm_f8w_workspace_bytes.argtypes = [i32, i32]
         l.nf_gemm_f8w_f16.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp, C.c_size_t, vp]
+        for name in ("nf_gemm_f8w_split_workspace_bytes", "nf_gemm_f8w_split_workspace_bytes_upto",
+                     "nf_dual_swiglu_f8w_split_workspace_bytes", "nf_dual_swiglu_f8w_split_workspace_bytes_upto"):
+            getattr(l, name).restype = sz
+            getattr(l, name).argtypes = [i32, i32, i32]
         l.nf_quantize_weight_e4m3.argtypes = [vp, vp, vp, i32, i32, vp]
         l.nf_dual_swiglu_f8_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp]
         l.nf_dual_swiglu_f8w_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, C.c_size_t, vp]
@@ -80,7 +86,9 @@ def lib() -> C.CDLL:
         for name in SYMBOLS:
             if name not in ("nf_last_error", "nf_attention_workspace_bytes", "nf_gemm_workspace_bytes",
                             "nf_gemm_workspace_bytes_upto", "nf_gemm_f8w_workspace_bytes",
-                            "nf_dual_swiglu_workspace_bytes", "nf_dual_swiglu_workspace_bytes_upto"):
+                            "nf_dual_swiglu_workspace_bytes", "nf_dual_swiglu_workspace_bytes_upto",
+                            "nf_gemm_f8w_split_workspace_bytes", "nf_gemm_f8w_split_workspace_bytes_upto",
+                            "nf_dual_swiglu_f8w_split_workspace_bytes", "nf_dual_swiglu_f8w_split_workspace_bytes_upto"):
                 getattr(l, name).restype = i32
         _lib = l
     return _lib
@@ -244,7 +252,7 @@ def gemm_f8w(A, Bq_nk, b_scale, Cmat=None, alpha=1.0, beta=0.0, out=None, worksp
     M, K = A.shape
     N = Bq_nk.shape[0]
     assert tuple(Bq_nk.shape) == (N, K) and b_scale.numel() == N
-    need = lib().nf_gemm_f8w_workspace_bytes(M, K)
+    need = lib().nf_gemm_f8w_split_workspace_bytes(M, N, K)      # quantised rows (+ the sums of a split over K)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
     out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
@@ -282,7 +290,7 @@ def dual_swiglu_f8w(A, Gq, g_scale, Uq, u_scale, out=None, workspace=None):
     M, Kd = A.shape
     N = Gq.shape[0]
     assert tuple(Gq.shape) == (N, Kd) and tuple(Uq.shape) == (N, Kd)
-    need = lib().nf_gemm_f8w_workspace_bytes(M, Kd)
+    need = lib().nf_dual_swiglu_f8w_split_workspace_bytes(M, N, Kd)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
     out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out

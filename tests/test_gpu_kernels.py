@@ -435,6 +435,48 @@ def test_dual_swiglu_f8w_is_quantise_then_dual(K, oracle):
     assert err.max() <= 2 * F8_RTOL * np.abs(ref).max(), (err.max(), np.abs(ref).max())
 
 
+@pytest.mark.parametrize("M,N,K_", [(16, 6144, 4096), (64, 4096, 14336), (128, 4096, 4096), (200, 1160, 4112)])
+def test_gemm_f8w_split_over_k_matches_the_unsplit_kernel_and_the_oracle(K, oracle, M, N, K_):
+    """Few rows: nf_gemm_f8w_f16 splits the contraction when its workspace has room for the sums.
+    Same quantised operands as the unsplit path (the row quantiser is bit-exact), fp32 sums taken
+    share by share: the fp16 tolerance against the oracle's double-precision sum."""
+    from nanoflow_amd import kernels
+    rng = np.random.default_rng(M + N)
+    A = rng.normal(0, 1, (M, K_)).astype(np.float16)
+    W = rng.normal(0, 0.02, (K_, N)).astype(np.float16)
+    Cm = rng.normal(0, 1, (M, N)).astype(np.float16)
+    Wq, sc = K.quantize_weight_e4m3(dev(W))
+    l = kernels.lib()
+    assert l.nf_gemm_f8w_split_workspace_bytes(M, N, K_) > l.nf_gemm_f8w_workspace_bytes(M, K_), "meant to be split"
+    got = host(K.gemm_f8w(dev(A), Wq, sc, dev(Cm), alpha=0.5, beta=1.0))
+    q, s = oracle.quantize_rows_e4m3(A)
+    ref = oracle.gemm_f8f8(q, s, host(Wq), host(sc), Cm, alpha=0.5, beta=1.0)
+    assert_close(got, ref, what="split-K fp8 gemm")
+    small = torch.empty(l.nf_gemm_f8w_workspace_bytes(M, K_), dtype=torch.uint8, device="cuda")   # no room: unsplit
+    unsplit = host(K.gemm_f8w(dev(A), Wq, sc, dev(Cm), alpha=0.5, beta=1.0, workspace=small))
+    assert_close(unsplit, ref, what="unsplit fp8 gemm")
+    assert_close(got, unsplit, what="split vs unsplit")
+
+
+@pytest.mark.parametrize("M,N,K_", [(16, 14336, 4096), (64, 1160, 4112), (128, 14336, 2048)])
+def test_dual_swiglu_f8w_split_over_k_matches_oracle(K, oracle, M, N, K_):
+    from nanoflow_amd import kernels
+    rng = np.random.default_rng(M + N + 1)
+    A = rng.normal(0, 1, (M, K_)).astype(np.float16)
+    Wg = rng.normal(0, 0.02, (K_, N)).astype(np.float16)
+    Wu = rng.normal(0, 0.02, (K_, N)).astype(np.float16)
+    Gq, sg = K.quantize_weight_e4m3(dev(Wg))
+    Uq, su = K.quantize_weight_e4m3(dev(Wu))
+    l = kernels.lib()
+    assert l.nf_dual_swiglu_f8w_split_workspace_bytes(M, N, K_) > l.nf_gemm_f8w_workspace_bytes(M, K_), "meant to be split"
+    got = host(K.dual_swiglu_f8w(dev(A), Gq, sg, Uq, su))
+    q, s = oracle.quantize_rows_e4m3(A)
+    ref = oracle.dual_swiglu_f8f8(q, s, host(Gq), host(sg), host(Uq), host(su))
+    assert_close(got, ref, 2 * RTOL, what="split-K fp8 gate/up pair")       # two fp16 roundings before SiLU-mul
+    small = torch.empty(l.nf_gemm_f8w_workspace_bytes(M, K_), dtype=torch.uint8, device="cuda")
+    assert_close(host(K.dual_swiglu_f8w(dev(A), Gq, sg, Uq, su, workspace=small)), ref, 2 * RTOL, what="unsplit pair")
+
+
 def test_gemm_f8w_rejects_short_workspace(K):
     from nanoflow_amd import kernels
     A = torch.zeros((8, 64), dtype=torch.float16, device="cuda")
