@@ -641,12 +641,18 @@ static int cu_count() {
   return n;
 }
 
-// Split over K: for at most 256 rows whose tiles (64 x 256 up to 64 rows, else 128 x 128) would
-// leave more than half of the CUs idle, as many shares as fill them, each at least 512 deep.
+// Split over K: for at most 512 rows whose tiles (64 x 256 up to 64 rows, 128 x 128 up to 256,
+// else 256 x 256) would leave more than half of the CUs idle, as many shares as fill them, each
+// at least 512 deep.  Between 257 and 512 rows the unsplit launch already fills the chip with
+// 128 x 128 tiles, but those pass four times the weight bytes through LDS; two 256-row tiles per
+// column panel, split over K, pass half of that.  Measured, that pays for a long contraction only
+// (the down projection: 95 -> 56 us at 267 x 4096 x 14336, 250 -> 210 us at 267 x 8192 x 28672;
+// at K = 4096 it loses 10-20 %), so above 256 rows the split needs K >= 12288.
 // Returns the number of shares (1 = no split) and their depth.
+constexpr int kSplitMaxRows = 512;
 static int splitk_plan(int M, int N, int K, int* k_per) {
-  if (M > 256 || K < 1024) return 1;
-  const int bm = M <= 64 ? 64 : 128, bn = M <= 64 ? 256 : 128;
+  if (M > kSplitMaxRows || K < 1024 || (M > 256 && K < 12288)) return 1;
+  const int bm = M <= 64 ? 64 : M <= 256 ? 128 : 256, bn = M <= 64 || M > 256 ? 256 : 128;
   const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
   const int cus = cu_count();
   int shares = std::min(std::min(cus / tiles, K / 512), 16);
@@ -741,6 +747,9 @@ static int gemm_ws_entry(const char* who, const uint16_t* A, const uint16_t* B, 
   if (M <= 64)
     return b_col_major ? launch_splitk<E, 64, 256, 1, 4, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
                        : launch_splitk<E, 64, 256, 1, 4, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
+  if (M > 256)
+    return b_col_major ? launch_splitk<E, 256, 256, 2, 2, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
+                       : launch_splitk<E, 256, 256, 2, 2, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
   return b_col_major ? launch_splitk<E, 128, 128, 2, 2, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
                      : launch_splitk<E, 128, 128, 2, 2, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
 }
@@ -802,7 +811,7 @@ size_t nf_gemm_workspace_bytes(int M, int N, int K) {
 
 size_t nf_gemm_workspace_bytes_upto(int max_M, int N, int K) {
   size_t need = 0;
-  for (int m = 1; m <= max_M && m <= 256; ++m) need = std::max(need, nf_gemm_workspace_bytes(m, N, K));
+  for (int m = 1; m <= max_M && m <= kSplitMaxRows; ++m) need = std::max(need, nf_gemm_workspace_bytes(m, N, K));
   return need;
 }
 

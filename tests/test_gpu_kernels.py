@@ -152,7 +152,8 @@ def test_gemm_with_bias_row_equals_gemm_with_replicated_bias(K, oracle, M, N, K_
 
 
 @pytest.mark.parametrize("M,N,K_", [(16, 6144, 4096), (64, 4096, 14336), (128, 4096, 4096), (200, 6144, 4096),
-                                    (64, 1160, 2056), (1, 1024, 1024), (256, 2048, 8200)])
+                                    (64, 1160, 2056), (1, 1024, 1024), (256, 2048, 8200),
+                                    (267, 4096, 12288), (421, 1160, 12304), (512, 2048, 14336)])   # 256-row tiles
 def test_gemm_split_over_k_matches_oracle(K, oracle, M, N, K_):
     """Few rows against a narrow N: the launch is split over K into shares whose fp32 sums meet in a
     workspace.  Same tolerance as the unsplit kernel; residual operand, column-major weights and
@@ -184,7 +185,7 @@ def test_gemm_split_over_k_matches_oracle(K, oracle, M, N, K_):
 def test_gemm_with_workspace_is_the_plain_kernel_for_large_shapes(K):
     from nanoflow_amd import kernels
     rng = np.random.default_rng(8)
-    for M, N, K_ in [(2048, 6144, 256), (300, 4096, 512), (64, 14336, 512), (64, 4096, 512)]:
+    for M, N, K_ in [(2048, 6144, 256), (300, 4096, 512), (64, 14336, 512), (64, 4096, 512), (520, 4096, 2048)]:
         A = synth.normal_f16(rng, (M, K_))
         B = synth.normal_f16(rng, (K_, N), 0.02)
         got, need = K.gemm_ws(dev(A), dev(B))
