@@ -565,22 +565,29 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
   if (bound < 1) bound = 1;
   if (decode_mode) {
     // wavefronts per (request, kv head) workgroup: with 2 (64 KB of LDS) two workgroups share a
-    // CU, and one streams while the other starts or merges -- a few percent faster than 4 or 1
-    constexpr int kWaves = 2;
-    constexpr int kDecodeLds = kWaves * 32768;
-    auto kern = attn_decode_kernel<GROUP, kWaves>;
-    static bool attr_set = false;  // benign race: the call is idempotent
-    if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLds);
-      if (e != hipSuccess) {
-        set_error("attention: cannot reserve %d bytes of LDS: %s", kDecodeLds, hipGetErrorString(e));
-        return NF_ERR_RUNTIME;
+    // CU, and one streams while the other starts or merges -- a few percent faster than 4 or 1.
+    // A batch so small that its workgroups leave CUs empty (at most one per CU) runs with 4
+    // wavefronts per workgroup instead: twice the loads in flight per request.
+    auto launch = [&](auto waves_c) -> int {
+      constexpr int kWaves = decltype(waves_c)::value;
+      constexpr int kDecodeLds = kWaves * 32768;
+      auto kern = attn_decode_kernel<GROUP, kWaves>;
+      static bool attr_set = false;  // benign race: the call is idempotent
+      if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLds);
+        if (e != hipSuccess) {
+          set_error("attention: cannot reserve %d bytes of LDS: %s", kDecodeLds, hipGetErrorString(e));
+          return NF_ERR_RUNTIME;
+        }
+        attr_set = true;
       }
-      attr_set = true;
-    }
-    kern<<<(int)bound, kWaves * 64, kDecodeLds, stream>>>(q, o, qo_indptr, kv_data, kv_indptr, kv_indices,
-                                                  kv_last_page_len, batch, Hq, Hkv, causal, scale_log2);
+      kern<<<(int)bound, kWaves * 64, kDecodeLds, stream>>>(q, o, qo_indptr, kv_data, kv_indptr, kv_indices,
+                                                            kv_last_page_len, batch, Hq, Hkv, causal, scale_log2);
+      return NF_OK;
+    };
+    int rc = (long long)batch * Hkv <= 256 ? launch(ic<4>{}) : launch(ic<2>{});
+    if (rc) return rc;
   } else
     attn_prefill_kernel<GROUP, NQB_PREFILL><<<(int)bound, 256, 2 * 16384, stream>>>(
         q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, batch, Hq,
