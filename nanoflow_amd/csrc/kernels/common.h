@@ -54,6 +54,22 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Sum over the shares of a GEMM split over K, for 4 neighbouring outputs: P[s * mn + at .. +3],
+// s = 0 .. shares-1 (at most kMaxShares), added in that order.  Every load is issued before the
+// first addition, so the lane waits for one memory round trip instead of one per share.
+constexpr int kMaxShares = 16;
+__device__ __forceinline__ float4_t sum_shares(const float* __restrict__ P, size_t mn, size_t at, int shares) {
+  float4_t p[kMaxShares];
+#pragma unroll
+  for (int s = 0; s < kMaxShares; ++s)
+    if (s < shares) p[s] = *reinterpret_cast<const float4_t*>(P + s * mn + at);
+  float4_t v = p[0];
+#pragma unroll
+  for (int s = 1; s < kMaxShares; ++s)
+    if (s < shares) v += p[s];
+  return v;
+}
+
 __device__ __forceinline__ float h2f_bits(uint32_t bits16) {
   return __half2float(__ushort_as_half((unsigned short)bits16));
 }

@@ -517,11 +517,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_dual_kernel(const float* __
                                                                  uint16_t* out, int M, int N) {
   const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
   for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
-    float4_t a = *reinterpret_cast<const float4_t*>(P0 + g * 4), b = *reinterpret_cast<const float4_t*>(P1 + g * 4);
-    for (int s = 1; s < shares; ++s) {
-      a += *reinterpret_cast<const float4_t*>(P0 + s * mn + g * 4);
-      b += *reinterpret_cast<const float4_t*>(P1 + s * mn + g * 4);
-    }
+    const float4_t a = sum_shares(P0, mn, g * 4, shares), b = sum_shares(P1, mn, g * 4, shares);
     float4_t v;
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = swiglu_rounded<E>(a[e], b[e]);
@@ -536,9 +532,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
                                                             int M, int N, float alpha, float beta) {
   const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
   for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
-    float4_t v = *reinterpret_cast<const float4_t*>(P + g * 4);
-    for (int s = 1; s < shares; ++s) v += *reinterpret_cast<const float4_t*>(P + s * mn + g * 4);
-    v *= alpha;
+    float4_t v = sum_shares(P, mn, g * 4, shares) * alpha;
     if (beta != 0.f) {
       const size_t m = g * 4 / N, n = g * 4 % N;
       const u32x2 c = *reinterpret_cast<const u32x2*>(C + m * ldc + n);
@@ -655,7 +649,7 @@ static int splitk_plan(int M, int N, int K, int* k_per) {
   const int bm = M <= 64 ? 64 : M <= 256 ? 128 : 256, bn = M <= 64 || M > 256 ? 256 : 128;
   const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
   const int cus = cu_count();
-  int shares = std::min(std::min(cus / tiles, K / 512), 16);
+  int shares = std::min(std::min(cus / tiles, K / 512), kMaxShares);
   if (shares < 2) return 1;
   *k_per = ((K + shares - 1) / shares + BK - 1) / BK * BK;
   return (K + *k_per - 1) / *k_per;  // shares that are not empty
@@ -666,7 +660,7 @@ static int splitk_plan_dual(int M, int N, int K, int* k_per) {
   if (M > 256 || K < 1024) return 1;
   const int bm = M <= 64 ? 64 : 128;
   const int tiles = ((M + bm - 1) / bm) * ((N + 127) / 128);
-  const int shares = std::min(std::min(cu_count() / tiles, K / 512), 16);
+  const int shares = std::min(std::min(cu_count() / tiles, K / 512), kMaxShares);
   if (shares < 2) return 1;
   *k_per = ((K + shares - 1) / shares + BK - 1) / BK * BK;
   return (K + *k_per - 1) / *k_per;

@@ -508,8 +508,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_f8_kernel(const float* __re
                                                                uint16_t* D, int M, int N, float alpha, float beta) {
   const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
   for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
-    float4_t v = *reinterpret_cast<const float4_t*>(P + g * 4);
-    for (int s = 1; s < shares; ++s) v += *reinterpret_cast<const float4_t*>(P + s * mn + g * 4);
+    float4_t v = sum_shares(P, mn, g * 4, shares);
     const size_t m = g * 4 / N, n = g * 4 % N;
     v = v * (*reinterpret_cast<const float4_t*>(sb + n) * alpha) * sa[m];
     if (beta != 0.f) {
@@ -532,11 +531,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_dual_f8_kernel(const float*
                                                                     int M, int N) {
   const size_t groups = (size_t)M * N / 4, mn = (size_t)M * N;
   for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
-    float4_t a = *reinterpret_cast<const float4_t*>(P0 + g * 4), b = *reinterpret_cast<const float4_t*>(P1 + g * 4);
-    for (int s = 1; s < shares; ++s) {
-      a += *reinterpret_cast<const float4_t*>(P0 + s * mn + g * 4);
-      b += *reinterpret_cast<const float4_t*>(P1 + s * mn + g * 4);
-    }
+    float4_t a = sum_shares(P0, mn, g * 4, shares), b = sum_shares(P1, mn, g * 4, shares);
     const size_t m = g * 4 / N, n = g * 4 % N;
     a = a * *reinterpret_cast<const float4_t*>(sg + n) * sa[m];
     b = b * *reinterpret_cast<const float4_t*>(su + n) * sa[m];
@@ -557,7 +552,7 @@ static int splitk_plan_f8(int M, int N, int K, bool dual, int* k_per) {
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
     cus = 256;
-  const int shares = std::min(std::min(cus / tiles, K / 1024), 16);
+  const int shares = std::min(std::min(cus / tiles, K / 1024), kMaxShares);
   if (shares < 2) return 1;
   *k_per = ((K + shares - 1) / shares + F8_BK - 1) / F8_BK * F8_BK;
   return (K + *k_per - 1) / *k_per;
