@@ -63,10 +63,11 @@ struct vortexModelConfig {
     // quantised activations of the fp8-weight GEMMs (one byte per element of the QKV, O, gate/up
     // and down inputs, a scale per row, 256-byte alignment of up to 8 wrappers)
     k_temp_size += (size_t)max_batch_size * (3 * model_hidden_dim + model_ff_dim + 32) / 2 + 8 * 256;
-    // fp32 partial sums of GEMM launches split over K: shares x M x N is at most CUs x one tile
-    // (256 x 128 x 128 elements = 16.8 MB) per wrapper, up to 7 wrappers, 256-byte alignment
-    // (the fused gate/up pair keeps two sets of sums: 2 x that for up to 2 of its wrappers)
-    k_temp_size += (size_t)(7 + 4) * (256 * 16384 * 2 + 128);
+    // fp32 partial sums of GEMM launches split over K: shares x M x N is at most CUs x the largest
+    // split tile (256 x 256 x 256 elements = 67 MB) per wrapper, up to 7 wrappers, 256-byte
+    // alignment (the fused gate/up pair keeps two sets of sums of 128 x 128 tiles, 34 MB together,
+    // for up to 2 of its wrappers)
+    k_temp_size += (size_t)(7 + 2) * ((size_t)256 * 65536 * 2 + 128);
     if (!rope_3_1) {
       smooth_a = 0;
       smooth_b = 0;

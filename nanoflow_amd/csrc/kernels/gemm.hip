@@ -636,17 +636,21 @@ static int cu_count() {
 }
 
 // Split over K: for at most 512 rows whose tiles (64 x 256 up to 64 rows, 128 x 128 up to 256,
-// else 256 x 256) would leave more than half of the CUs idle, as many shares as fill them, each
-// at least 512 deep.  Between 257 and 512 rows the unsplit launch already fills the chip with
-// 128 x 128 tiles, but those pass four times the weight bytes through LDS; two 256-row tiles per
-// column panel, split over K, pass half of that.  Measured, that pays for a long contraction only
-// (the down projection: 95 -> 56 us at 267 x 4096 x 14336, 250 -> 210 us at 267 x 8192 x 28672;
-// at K = 4096 it loses 10-20 %), so above 256 rows the split needs K >= 12288.
+// 320 x 128 up to 320, else 256 x 256) would leave more than half of the CUs idle, as many shares
+// as fill them, each at least 512 deep.  Above 256 rows the unsplit launch already fills the chip
+// with 128 x 128 tiles, but those pass the weight bytes through LDS once per 128 rows.  From 257
+// to 320 rows one 320-row tile per column panel passes them once (267 x 10240 x 8192: 72 -> 63 us,
+// 267 x 8192 x 28672: 209 -> 188 us, 267 x 4096 x 4096: 32 -> 28 us).  From 321 to 512 rows two
+// 256-row tiles per panel pass them twice instead of four times, but half of the second tile's
+// MFMAs are padding: measured, that pays for a long contraction only (the down projection), so
+// there the split needs K >= 12288.
 // Returns the number of shares (1 = no split) and their depth.
 constexpr int kSplitMaxRows = 512;
+constexpr int kTallRows = 320;  // 257 .. 320 rows: one 320 x 128 tile per column panel
 static int splitk_plan(int M, int N, int K, int* k_per) {
-  if (M > kSplitMaxRows || K < 1024 || (M > 256 && K < 12288)) return 1;
-  const int bm = M <= 64 ? 64 : M <= 256 ? 128 : 256, bn = M <= 64 || M > 256 ? 256 : 128;
+  if (M > kSplitMaxRows || K < 1024 || (M > kTallRows && K < 12288)) return 1;
+  const int bm = M <= 64 ? 64 : M <= 256 ? 128 : M <= kTallRows ? 320 : 256;
+  const int bn = M <= 64 || M > kTallRows ? 256 : 128;
   const int tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
   const int cus = cu_count();
   int shares = std::min(std::min(cus / tiles, K / 512), kMaxShares);
@@ -655,7 +659,8 @@ static int splitk_plan(int M, int N, int K, int* k_per) {
   return (K + *k_per - 1) / *k_per;  // shares that are not empty
 }
 
-// The same for the fused gate/up pair (tiles of 64 x 128 up to 64 rows, else 128 x 128).
+// The same for the fused gate/up pair (tiles of 64 x 128 up to 64 rows, else 128 x 128; a
+// 320 x 128 pair of accumulators does not fit the register file).
 static int splitk_plan_dual(int M, int N, int K, int* k_per) {
   if (M > 256 || K < 1024) return 1;
   const int bm = M <= 64 ? 64 : 128;
@@ -741,6 +746,9 @@ static int gemm_ws_entry(const char* who, const uint16_t* A, const uint16_t* B, 
   if (M <= 64)
     return b_col_major ? launch_splitk<E, 64, 256, 1, 4, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
                        : launch_splitk<E, 64, 256, 1, 4, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
+  if (M > 256 && M <= kTallRows)
+    return b_col_major ? launch_splitk<E, 320, 128, 2, 2, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
+                       : launch_splitk<E, 320, 128, 2, 2, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
   if (M > 256)
     return b_col_major ? launch_splitk<E, 256, 256, 2, 2, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
                        : launch_splitk<E, 256, 256, 2, 2, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);

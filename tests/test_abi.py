@@ -53,7 +53,8 @@ def test_argument_errors_are_reported_without_a_gpu():
 def test_split_over_k_plan_without_a_gpu():
     """Which GEMM launches are split over K, and into how many shares, is host arithmetic (the CU count
     defaults to the MI355X's 256 without a device): at most 512 rows, at least 1024 deep, as many
-    shares as fill the chip (tiles of 64 x 256 up to 64 rows, 128 x 128 up to 256, else 256 x 256),
+    shares as fill the chip (tiles of 64 x 256 up to 64 rows, 128 x 128 up to 256, 320 x 128 up to 320, else
+    256 x 256),
     each at least 512 deep, at most 16."""
     from nanoflow_amd import kernels
     l = kernels.lib()
@@ -62,9 +63,10 @@ def test_split_over_k_plan_without_a_gpu():
     assert shares(64, 4096, 14336) == 16          # 16 tiles, capped at 16 shares
     assert shares(128, 4096, 4096) == 8           # 32 tiles of 128 x 128
     assert shares(200, 6144, 4096) == 2           # 96 tiles
-    assert shares(257, 4096, 4096) == 0           # above 256 rows only long contractions are split
-    assert shares(267, 8192, 28672) == 4          # the down projection in the KV-bound 70B regime
-    assert shares(300, 4096, 14336) == 8          # two 256-row tiles per 256 columns: 32 tiles
+    assert shares(257, 4096, 4096) == 8           # 257 .. 320 rows: one 320-row tile per 128 columns, 32 tiles
+    assert shares(267, 8192, 28672) == 4          # the down projection in the KV-bound 70B regime: 64 tiles
+    assert shares(321, 4096, 4096) == 0           # above 320 rows only long contractions are split
+    assert shares(400, 4096, 14336) == 8          # two 256-row tiles per 256 columns: 32 tiles
     assert shares(513, 4096, 4096) == 0           # more than 512 rows
     assert shares(64, 128256, 4096) == 0          # the LM head has tiles enough
     assert shares(64, 4096, 512) == 0             # too shallow

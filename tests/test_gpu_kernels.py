@@ -153,7 +153,8 @@ def test_gemm_with_bias_row_equals_gemm_with_replicated_bias(K, oracle, M, N, K_
 
 @pytest.mark.parametrize("M,N,K_", [(16, 6144, 4096), (64, 4096, 14336), (128, 4096, 4096), (200, 6144, 4096),
                                     (64, 1160, 2056), (1, 1024, 1024), (256, 2048, 8200),
-                                    (267, 4096, 12288), (421, 1160, 12304), (512, 2048, 14336)])   # 256-row tiles
+                                    (267, 4096, 12288), (300, 1160, 4112), (320, 6144, 4096),   # one 320-row tile
+                                    (421, 1160, 12304), (512, 2048, 14336)])                    # 256-row tiles
 def test_gemm_split_over_k_matches_oracle(K, oracle, M, N, K_):
     """Few rows against a narrow N: the launch is split over K into shares whose fp32 sums meet in a
     workspace.  Same tolerance as the unsplit kernel; residual operand, column-major weights and
