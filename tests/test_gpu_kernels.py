@@ -556,11 +556,13 @@ def test_attention_decode(K, oracle, Hq, Hkv):
     _attn_case(K, oracle, Hq, Hkv, lens, [], seed=11)
 
 
-def test_attention_decode_many_requests(K, oracle):
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (64, 8), (8, 4), (4, 4)])
+def test_attention_decode_many_requests(K, oracle, Hq, Hkv):
     # more (request, kv head) pairs than CUs: the launch with two wavefronts per workgroup
     # (smaller batches, as above, run with four)
     lens = [int(x) for x in np.random.default_rng(16).integers(1, 260, size=72)]
-    _attn_case(K, oracle, 32, 8, lens, [], seed=16)
+    assert len(lens) * Hkv > 256
+    _attn_case(K, oracle, Hq, Hkv, lens, [], seed=16)
 
 
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (64, 8), (8, 4), (4, 4)])
