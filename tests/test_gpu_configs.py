@@ -176,6 +176,21 @@ def test_decode_attention_page_permutation_invariance_at_full_size():
     o2 = run(pool2, perm.numpy()[b.kv_indices].astype(np.int32))
     assert torch.equal(o1, o2)
     assert torch.isfinite(o1).all() and o1.abs().max() > 0
+    # a sample of requests (the pool spans more than 4 GiB; the highest page ids included) against
+    # fp32 softmax attention in plain PyTorch on the gathered pages
+    assert pool.numel() * 2 > (4 << 30)
+    top = int(np.argmax([b.kv_indices[b.kv_indptr[r]:b.kv_indptr[r + 1]].max() for r in range(nd)]))
+    group = shape.Hq // shape.Hkv
+    for r in sorted({0, nd // 3, nd - 1, top}):
+        pages = t(b.kv_indices[b.kv_indptr[r]:b.kv_indptr[r + 1]].astype(np.int64))
+        kv_len = (len(pages) - 1) * 16 + int(b.kv_last_page_len[r])
+        k = pool[pages, 0].reshape(-1, shape.Hkv, shape.d)[:kv_len].float()          # [keys, Hkv, d]
+        v = pool[pages, 1].reshape(-1, shape.Hkv, shape.d)[:kv_len].float()
+        qr = q[r].view(shape.Hkv, group, shape.d).float()                               # q head = kv head * group + g
+        p_ = torch.softmax(torch.einsum("hgd,khd->hgk", qr, k) / np.sqrt(shape.d), dim=-1)
+        ref = torch.einsum("hgk,khd->hgd", p_, v).reshape(-1)
+        err = (o1[r].float() - ref).abs().max().item()
+        assert err <= 2e-3 * ref.abs().max().item() + 1e-6, (r, err)
 
 
 def test_fp8_gemm_at_70b_ffn_shape(oracle):
