@@ -6,7 +6,10 @@ reference's pipeline/utils/serve_8B.py:
 
 * trace (pipeline/utils/frontend.py:23-58): a header line, then ``idx,input_len,output_len,arrival``
   per request; a request of input_len n gets the prompt 0, 1, ..., n-1 as in the reference.
-  Rows with input_len -1 (prompt text to tokenize) are rejected: no tokenizer ships here.
+  A row with input_len -1 carries its prompt as text after the fourth comma and is tokenized with the
+  tokenizer found in the directory ``serve_configs.model`` (the reference's key, serve_8B.py:639-640;
+  a hub name is not fetched: there is no network) or else ``serve_configs.hf_path``; without a
+  tokenizer such rows are rejected.
 * config: the reference's pipeline JSON (pipeline/config_all/llama3-8B/1024.json schema);
   ``serve_configs.pipeline_type`` must be LOCAL, NON_OVERLAP_LOCAL or NANOBATCH_LOCAL, or, for models with a
   bias on the q/k/v projections (Qwen2), KQVBIAS, NONOVERLAP_KQVBIAS or NANOBATCH_KQVBIAS.
@@ -20,9 +23,12 @@ reference's pipeline/utils/serve_8B.py:
   the five GEMM weights of every layer are quantised on the device as they are loaded or made
   (per-output-channel scales) and served from the fp8 form.
 * KV pool = ``1024 * allocate_kv_data_batch // 16`` pages per layer (serve_8B.py:643).
-* writes PREFIX.stat, PREFIX.stat.csv (same columns as serve_8B.py:792-793), PREFIX.req_time and
+* writes PREFIX.stat, PREFIX.stat.csv (same columns as serve_8B.py:792-793), PREFIX.req_time,
   PREFIX.req_tokens (prompt + generated ids of every retired request, one Python list per line,
-  by request index: serve_8B.py:718-721).
+  by request index: serve_8B.py:718-722), PREFIX.req_tokens.uniq (its distinct lines with their
+  counts, serve_8B.py:731) and, when a tokenizer was found, PREFIX.req_words (the same sequences
+  decoded without special tokens, preceded by ``Req k:`` lines under ``--output_idx``:
+  serve_8B.py:723-728).
 
 Skip cycles advance the scheduler without GPU work and release requests by the estimated cycle
 time; run cycles form batch i+1 on the CPU while the GPU runs batch i.  When every request has
@@ -42,7 +48,21 @@ import numpy as np
 sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
 
-def read_trace(path):
+def load_tokenizer(serve_configs):
+    """The tokenizer of the first of serve_configs.model / serve_configs.hf_path that is a local
+    directory holding one, or None.  Nothing is fetched."""
+    for key in ("model", "hf_path"):
+        d = serve_configs.get(key)
+        if d and os.path.isdir(d) and any(os.path.isfile(os.path.join(d, f))
+                                          for f in ("tokenizer.json", "tokenizer.model", "tokenizer_config.json")):
+            os.environ.setdefault("HF_HUB_OFFLINE", "1")
+            from transformers import AutoTokenizer
+            return AutoTokenizer.from_pretrained(d, local_files_only=True)
+    return None
+
+
+def read_trace(path, tokenizer=None):
+    """[(request index, prompt ids as int32 array, output_len, arrival)] (frontend.py:23-58)."""
     reqs = []
     with open(path) as f:
         next(f, None)                                   # header
@@ -51,10 +71,19 @@ def read_trace(path):
                 continue
             p = line.split(",")
             n_in, n_out, arrival = int(p[1]), int(p[2]), float(p[3])
-            if n_in < 0:
-                raise SystemExit(f"{path}: request {p[0]} carries prompt text (input_len -1); only token-length "
-                                 "traces are supported here")
-            reqs.append((len(reqs), n_in, n_out, arrival))
+            if n_in == -1:
+                if tokenizer is None:
+                    raise SystemExit(f"{path}: request {p[0]} carries prompt text (input_len -1) and neither "
+                                     "serve_configs.model nor serve_configs.hf_path is a directory with a tokenizer")
+                text = line.split(",", 4)[4]            # everything after the fourth comma, commas included
+                if text.endswith("\n"):
+                    text = text[:-1]
+                prompt = np.asarray(tokenizer(text)["input_ids"], dtype=np.int32)
+            elif n_in < 0:
+                raise SystemExit(f"{path}: request {p[0]} has input_len {n_in}")
+            else:
+                prompt = np.arange(n_in, dtype=np.int32)
+            reqs.append((len(reqs), prompt, n_out, arrival))
     if not reqs:
         raise SystemExit(f"{path}: empty trace")
     return reqs
@@ -70,6 +99,7 @@ def main():
     ap.add_argument("-o", "--output_prefix", default="")
     ap.add_argument("--allocate_page_num", type=int, default=740, help="accepted and unused, as in the reference")
     ap.add_argument("--empty_weight", default="True")
+    ap.add_argument("--output_idx", default="False", help="precede every line of PREFIX.req_words by 'Req k:'")
     a = ap.parse_args()
     empty_weight = str(a.empty_weight).lower() in ("true", "1", "yes")
     prefix = a.output_prefix or a.trace_path[:-4]
@@ -108,8 +138,12 @@ def main():
         weights = W.load_weight_file(wdir, shape, kqv_bias=pt.has_kqv_bias)
         print("Time taken to load weights: ", time.perf_counter() - t0)
 
-    reqs = read_trace(a.trace_path)
-    avg_in = sum(r[1] for r in reqs) // len(reqs)
+    tokenizer = load_tokenizer(sc)
+    reqs = read_trace(a.trace_path, tokenizer)
+    too_big = [r[0] for r in reqs if len(r[1]) and int(r[1].max()) >= shape.vocab]
+    if too_big:
+        raise SystemExit(f"{a.trace_path}: request {too_big[0]} has a token id beyond the model's vocabulary of {shape.vocab}")
+    avg_in = sum(len(r[1]) for r in reqs) // len(reqs)
     avg_out = sum(r[2] for r in reqs) // len(reqs)
     eng = engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=kqv1, kqv3=kqv3, kv_pages=pages,
                         run_layer=mc.get("run_layer", shape.layers), kv_fill="zeros", weights=weights,
@@ -121,8 +155,8 @@ def main():
 
     def release(now_clock):
         while pending and pending[0][3] < passed:
-            idx, n_in, n_out, _ = pending.pop(0)
-            former.add_request(idx, np.arange(n_in, dtype=np.int32), n_out, now_clock)
+            idx, prompt, n_out, _ = pending.pop(0)
+            former.add_request(idx, prompt, n_out, now_clock)
 
     def busy():
         st = former.state()
@@ -191,13 +225,26 @@ def main():
     infos = [former.retired_info(k) for k in range(n_retired)]
     outputs = dict(former.retired_output(k) for k in range(n_retired))
     eng.close()
-    prompt_len = {r[0]: r[1] for r in reqs}
+    prompts = {r[0]: r[1] for r in reqs}
+    lines = []
+    for idx in sorted(outputs):
+        gen = [int(t) for t in outputs[idx]]
+        if gen and gen[-1] == -1:           # the placeholder of a sample that was never harvested
+            gen.pop()
+        lines.append([int(t) for t in prompts[idx]] + gen)
     with open(prefix + ".req_tokens", "w") as fq:
-        for idx in sorted(outputs):
-            gen = [int(t) for t in outputs[idx]]
-            if gen and gen[-1] == -1:       # the placeholder of a sample that was never harvested
-                gen.pop()
-            fq.write(f"{list(range(prompt_len[idx])) + gen}\n")
+        for l in lines:
+            fq.write(f"{l}\n")
+    with open(prefix + ".req_tokens.uniq", "w") as fu:      # what `sort | uniq -c` prints
+        import collections
+        for text, n in sorted(collections.Counter(str(l) for l in lines).items()):
+            fu.write(f"{n:7d} {text}\n")
+    if tokenizer is not None:
+        with open(prefix + ".req_words", "w") as fw:
+            for k, l in enumerate(lines):
+                if str(a.output_idx).lower() in ("true", "1", "yes"):
+                    fw.write(f"Req {k}:\n")
+                fw.write(f"{tokenizer.decode(l, skip_special_tokens=True)}\n")
     with open(prefix + ".stat", "w") as fs, open(prefix + ".stat.csv", "w") as fc, open(prefix + ".req_time", "w") as ft:
         def out(s):
             print(s)

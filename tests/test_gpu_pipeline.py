@@ -572,6 +572,55 @@ def test_serve_command_line_writes_the_reference_result_files(tmp_path, online, 
             assert len(l) - n_in in (n_out - 1, n_out) and all(0 <= t < shape.vocab for t in l[n_in:]), (k, l[n_in:])
     if from_file:
         assert os.path.isfile(str(tmp_path / "w" / "weight_rank_0.pt")) and "Loading weights" in r.stdout
+    assert not os.path.exists(str(prefix) + ".req_words")          # no tokenizer in these configurations
+    uniq = [l.split(None, 1) for l in open(str(prefix) + ".req_tokens.uniq")]
+    assert sum(int(n) for n, _ in uniq) == len(lines) and sorted(t.strip() for _, t in uniq) == sorted({str(l) for l in lines})
+
+
+def test_serve_command_line_tokenizes_prompt_text_and_writes_the_words_file(tmp_path):
+    """Trace rows with input_len -1 carry prompt text (pipeline/utils/frontend.py:41-47); the tokenizer
+    comes from the directory serve_configs.model, and PREFIX.req_words holds prompt + output decoded
+    (pipeline/utils/serve_8B.py:723-728)."""
+    import subprocess, sys, os, json, ast
+    from nanoflow_amd import engine, pllm_python as P
+    from test_weights import write_word_tokenizer
+    words = ["the", "quick", "brown", "fox", ",", "jumps", "over", "lazy", "dog"]
+    vocab = write_word_tokenizer(str(tmp_path / "tok"), words)
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    cfg = tmp_path / "tiny.json"
+    engine.write_config(str(cfg), shape, global_batch=96, nano1=40, kqv1=20, kqv3=28,
+                        pipeline_type=P.PipelineType.NON_OVERLAP_LOCAL, kv_pages=256)
+    c = json.load(open(cfg))
+    c["serve_configs"]["model"] = str(tmp_path / "tok")
+    json.dump(c, open(cfg, "w"))
+    prompts = ["the quick brown fox jumps over the lazy dog", "the lazy dog, the quick fox", "fox"]
+    trace = tmp_path / "trace.csv"
+    with open(trace, "w") as f:
+        f.write("idx,input_len,output_len,arrival,prompt\n")
+        for i, text in enumerate(prompts):
+            f.write(f"{i},-1,{3 + i},0,{text}\n")
+        f.write("3,12,4,0\n")
+    prefix = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, "-m", "nanoflow_amd.serve", "-t", str(trace), "-c", str(cfg), "-r", "100", "--empty_weight", "True",
+           "--output_idx", "True", "-o", str(prefix)]
+    print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    lines = [ast.literal_eval(l) for l in open(str(prefix) + ".req_tokens")]
+    assert len(lines) == 4
+    from transformers import AutoTokenizer
+    tok = AutoTokenizer.from_pretrained(str(tmp_path / "tok"), local_files_only=True)
+    for i, text in enumerate(prompts):
+        ids = tok(text)["input_ids"]
+        assert ids[0] == vocab["<s>"] and lines[i][:len(ids)] == ids and len(lines[i]) - len(ids) in (2 + i, 3 + i)
+    assert lines[3][:12] == list(range(12))
+    out = open(str(prefix) + ".req_words").read().split("\n")
+    assert out[0] == "Req 0:" and out[2] == "Req 1:" and out[6] == "Req 3:"
+    assert out[1].startswith("the quick brown fox jumps over the lazy dog")
+    assert out[3].startswith("the lazy dog , the quick fox") and out[5].startswith("fox")
+    times = {int(t["req_idx"]): int(t["input_len"]) for t in __import__("csv").DictReader(open(str(prefix) + ".req_time"))}
+    assert times == {0: 10, 1: 8, 2: 2, 3: 12}          # tokens, <s> included
 
 
 def test_autosearch_writes_a_tuned_pipeline_config(tmp_path):

@@ -123,13 +123,54 @@ def test_trace_generator_writes_what_the_serving_command_reads(tmp_path):
     p = gen_req.write_trace(str(tmp_path / "t.csv"), 50, "200:700", "512", rate=10.0, poisson=True, seed=3)
     reqs = serve.read_trace(p)
     assert len(reqs) == 50 and [r[0] for r in reqs] == list(range(50))
-    assert all(200 <= r[1] <= 700 and r[2] == 512 for r in reqs)
+    assert all(200 <= len(r[1]) <= 700 and r[2] == 512 for r in reqs)
+    assert all(np.array_equal(r[1], np.arange(len(r[1]))) and r[1].dtype == np.int32 for r in reqs)   # prompt 0, 1, ..., n-1
     arr = [r[3] for r in reqs]
     assert arr == sorted(arr) and 2.0 < arr[-1] < 12.0            # 50 requests at 10 per second
     p = gen_req.write_trace(str(tmp_path / "c.csv"), 8, rate=4.0)
     assert [r[3] for r in serve.read_trace(p)] == [i / 4.0 for i in range(8)]
     p = gen_req.write_trace(str(tmp_path / "o.csv"), 3)
-    assert serve.read_trace(p) == [(0, 1024, 512, 0.0), (1, 1024, 512, 0.0), (2, 1024, 512, 0.0)]
+    assert [(r[0], len(r[1]), r[2], r[3]) for r in serve.read_trace(p)] == [(0, 1024, 512, 0.0), (1, 1024, 512, 0.0),
+                                                                               (2, 1024, 512, 0.0)]
+
+
+def write_word_tokenizer(directory, words):
+    """A word-level tokenizer directory that transformers' AutoTokenizer loads offline: ids 0.. are
+    <unk>, <s>, then the words; every encoded text starts with <s>."""
+    import json, os
+    from tokenizers import Tokenizer, models, pre_tokenizers, processors
+    vocab = {"<unk>": 0, "<s>": 1, **{w: i + 2 for i, w in enumerate(words)}}
+    tok = Tokenizer(models.WordLevel(vocab, unk_token="<unk>"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.post_processor = processors.TemplateProcessing(single="<s> $A", special_tokens=[("<s>", 1)])
+    os.makedirs(directory, exist_ok=True)
+    tok.save(os.path.join(directory, "tokenizer.json"))
+    json.dump({"tokenizer_class": "PreTrainedTokenizerFast", "unk_token": "<unk>", "bos_token": "<s>"},
+              open(os.path.join(directory, "tokenizer_config.json"), "w"))
+    return vocab
+
+
+def test_prompt_text_rows_are_tokenized_as_the_reference_front_end_does(tmp_path):
+    """pipeline/utils/frontend.py:41-47: input_len -1 = the prompt is the text after the fourth comma
+    (commas of the text included, the line's newline dropped), tokenized with the model's tokenizer."""
+    from nanoflow_amd import serve
+    vocab = write_word_tokenizer(str(tmp_path / "tok"), ["the", "quick", "brown", "fox", ",", "jumps", "over", "lazy", "dog"])
+    tok = serve.load_tokenizer({"model": str(tmp_path / "tok")})
+    assert tok is not None and serve.load_tokenizer({"model": "meta-llama/Meta-Llama-3-8B"}) is None   # a hub name: not fetched
+    assert serve.load_tokenizer({"hf_path": str(tmp_path / "tok")}) is not None
+    p = tmp_path / "t.csv"
+    p.write_text("idx,input_len,output_len,arrival,prompt\n"
+                 "0,-1,5,0.0,the quick brown fox, the lazy dog\n"
+                 "1,4,6,0.5\n"
+                 "2,-1,7,1.0,zebra jumps over\n")
+    reqs = serve.read_trace(str(p), tok)
+    v = vocab
+    assert reqs[0][1].tolist() == [1, v["the"], v["quick"], v["brown"], v["fox"], v[","], v["the"], v["lazy"], v["dog"]]
+    assert reqs[1][1].tolist() == [0, 1, 2, 3] and reqs[1][2:] == (6, 0.5)
+    assert reqs[2][1].tolist() == [1, 0, v["jumps"], v["over"]] and reqs[2][2:] == (7, 1.0)      # unknown word -> <unk>
+    assert tok.decode(reqs[0][1].tolist(), skip_special_tokens=True) == "the quick brown fox , the lazy dog"
+    with pytest.raises(SystemExit, match="tokenizer"):
+        serve.read_trace(str(p))
 
 
 def test_shape_mismatch_and_foreign_files_raise(tmp_path):
