@@ -65,8 +65,8 @@ void init(int nranks, int vnranks, std::vector<vortexInitData>& input,
   }
   if (!Worker::isSupported(pipeTy)) {
     std::fprintf(stderr,
-                 "init: pipeline type %d is a tensor-parallel schedule; this build implements LOCAL, "
-                 "NON_OVERLAP_LOCAL, NANOBATCH_LOCAL and, as those with a QKV bias, the three *_KQVBIAS types\n",
+                 "init: pipeline type %d is the offload pipeline, whose host and SSD tiers this build does not "
+                 "have; every other type runs (the tensor-parallel ones as their one-device schedules)\n",
                  static_cast<int>(pipeTy));
     std::exit(EXIT_FAILURE);
   }
@@ -162,10 +162,11 @@ void Worker::init() {
   // The *_KQVBIAS types name the tensor-parallel pipelines with a QKV bias
   // (pipeline/src/computeBound.cu:234-242); on one device, with no exchange steps left, they are
   // the local schedules with the bias switched on.
-  if (PipeTy == PipelineType::LOCAL || PipeTy == PipelineType::NANOBATCH_LOCAL)
-    pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks,
-                                               PipeTy == PipelineType::NANOBATCH_LOCAL);
-  else if (PipeTy == PipelineType::NON_OVERLAP_LOCAL)
+  // So are PLLM, NANOBATCH and NONOVERLAP without the bias.
+  const bool nanobatch_only = PipeTy == PipelineType::NANOBATCH_LOCAL || PipeTy == PipelineType::NANOBATCH;
+  if (PipeTy == PipelineType::LOCAL || PipeTy == PipelineType::PLLM || nanobatch_only)
+    pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks, nanobatch_only);
+  else if (PipeTy == PipelineType::NON_OVERLAP_LOCAL || PipeTy == PipelineType::NONOVERLAP)
     pipeline = std::make_unique<NonOverlapLocalPipeline>(input, rank, nranks, vnranks);
   else if ((PipeTy == PipelineType::KQVBIAS || PipeTy == PipelineType::NANOBATCH_KQVBIAS) && nranks == 1)
     pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks,

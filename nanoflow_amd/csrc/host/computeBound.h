@@ -59,17 +59,19 @@ public:
     NANOBATCH_LOCAL,
   };
   static PipelineType PipeTy;
-  static bool isSupported(PipelineType t) {
-    return t == PipelineType::LOCAL || t == PipelineType::NON_OVERLAP_LOCAL ||
-           t == PipelineType::NANOBATCH_LOCAL || hasKQVBias(t);
-  }
+  // Everything but the offload pipeline.  PLLM, NONOVERLAP and NANOBATCH name the tensor-parallel
+  // schedules (pipeline/src/computeBound.cu:225-233); on the one rank of this build their exchange
+  // steps move nothing, and they run as LOCAL, NON_OVERLAP_LOCAL and NANOBATCH_LOCAL, so that the
+  // reference's multi-GPU pipeline files serve here once their gpu_num is 1.
+  static bool isSupported(PipelineType t) { return t != PipelineType::PLLMOFFLOAD; }
   // the three bias types run as the local schedules with the QKV bias switched on
   static bool hasKQVBias(PipelineType t) {
     return t == PipelineType::KQVBIAS || t == PipelineType::NONOVERLAP_KQVBIAS ||
            t == PipelineType::NANOBATCH_KQVBIAS;
   }
   static bool isSequential(PipelineType t) {
-    return t == PipelineType::NON_OVERLAP_LOCAL || t == PipelineType::NONOVERLAP_KQVBIAS;
+    return t == PipelineType::NON_OVERLAP_LOCAL || t == PipelineType::NONOVERLAP_KQVBIAS ||
+           t == PipelineType::NONOVERLAP;
   }
 
 private:

@@ -93,9 +93,10 @@ int pllm_init(const nf_vortex_init_data* input, int pipeline_type) {
   auto ty = static_cast<Worker::PipelineType>(pipeline_type);
   if (!Worker::isSupported(ty))
     return fail(NF_PLLM_ERR_UNSUPPORTED,
-                "pllm_init: pipeline type %d is a tensor-parallel schedule; LOCAL(7), "
-                "NON_OVERLAP_LOCAL(8), NANOBATCH_LOCAL(9) and, as those with a QKV bias, KQVBIAS(4), "
-                "NONOVERLAP_KQVBIAS(5), NANOBATCH_KQVBIAS(6) are implemented", pipeline_type);
+                "pllm_init: pipeline type %d is the offload pipeline, whose host and SSD tiers are not "
+                "built; every other type runs (PLLM(0), NONOVERLAP(1), NANOBATCH(2) as LOCAL(7), "
+                "NON_OVERLAP_LOCAL(8), NANOBATCH_LOCAL(9); the *_KQVBIAS types as those with a QKV bias)",
+                pipeline_type);
   if (getWeightFormat() == WeightFormat::E4M3 && Worker::hasKQVBias(ty))
     return fail(NF_PLLM_ERR_UNSUPPORTED, "pllm_init: the QKV bias pipelines take fp16 weights only");
   if (input->weight.num_layers < ModelConfig.model_layer)

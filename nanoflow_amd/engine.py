@@ -41,7 +41,7 @@ def write_config(path, shape: synth.ModelShape, *, global_batch, nano1, kqv1, kq
             "gemm_op_tag": [DEFAULT_TAG] * n_tags, "global_batch_size": global_batch,
             "nanobatch_1_size": nano1, "kqv1_size": kqv1, "kqv3_size": kqv3,
         },
-        "serve_configs": {"actual_gpu_num": 1, "pipeline_type": pipeline_type.name},
+        "serve_configs": {"actual_gpu_num": 1, "pipeline_type": {v: k for k, v in P.pipeline_map.items()}[pipeline_type]},
     }
     with open(path, "w") as f:
         json.dump(cfg, f, indent=1)

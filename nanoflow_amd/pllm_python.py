@@ -49,7 +49,24 @@ class PipelineType(enum.IntEnum):
     @property
     def is_sequential(self) -> bool:
         """One stream, no nano-batch split: four GEMM tags, one decode-attention group."""
-        return self in (PipelineType.NON_OVERLAP_LOCAL, PipelineType.NONOVERLAP_KQVBIAS)
+        return self in (PipelineType.NON_OVERLAP_LOCAL, PipelineType.NONOVERLAP_KQVBIAS, PipelineType.NONOVERLAP)
+
+
+# serve_configs.pipeline_type of the reference's pipeline files (pipeline/utils/serve_8B.py:48-59).
+# PLLM, NON_OVERLAP and NANOBATCH, the tensor-parallel schedules, run on this one device as LOCAL,
+# NON_OVERLAP_LOCAL and NANOBATCH_LOCAL; PLLM_OFFLOAD is refused by init.
+pipeline_map = {
+    "LOCAL": PipelineType.LOCAL,
+    "PLLM": PipelineType.PLLM,
+    "NON_OVERLAP": PipelineType.NONOVERLAP,
+    "NANOBATCH": PipelineType.NANOBATCH,
+    "PLLM_OFFLOAD": PipelineType.PLLMOFFLOAD,
+    "NON_OVERLAP_LOCAL": PipelineType.NON_OVERLAP_LOCAL,
+    "NANOBATCH_LOCAL": PipelineType.NANOBATCH_LOCAL,
+    "KQVBIAS": PipelineType.KQVBIAS,
+    "NANOBATCH_KQVBIAS": PipelineType.NANOBATCH_KQVBIAS,
+    "NONOVERLAP_KQVBIAS": PipelineType.NONOVERLAP_KQVBIAS,
+}
 
 
 class VortexWeight(C.Structure):

@@ -11,8 +11,10 @@ reference's pipeline/utils/serve_8B.py:
   a hub name is not fetched: there is no network) or else ``serve_configs.hf_path``; without a
   tokenizer such rows are rejected.
 * config: the reference's pipeline JSON (pipeline/config_all/llama3-8B/1024.json schema);
-  ``serve_configs.pipeline_type`` must be LOCAL, NON_OVERLAP_LOCAL or NANOBATCH_LOCAL, or, for models with a
-  bias on the q/k/v projections (Qwen2), KQVBIAS, NONOVERLAP_KQVBIAS or NANOBATCH_KQVBIAS.
+  ``serve_configs.pipeline_type`` is one of the reference's names (serve_8B.py:48-59): LOCAL,
+  NON_OVERLAP_LOCAL, NANOBATCH_LOCAL; PLLM, NON_OVERLAP, NANOBATCH (the tensor-parallel schedules, which
+  on this one device run as the three above); for models with a bias on the q/k/v projections (Qwen2)
+  KQVBIAS, NONOVERLAP_KQVBIAS, NANOBATCH_KQVBIAS.  PLLM_OFFLOAD is refused.
 * ``--empty_weight True``: random-init weights on the device, as the reference's own evaluation
   runs (pipeline/eval/eval-fix-offline/run.py:42-50).  Otherwise the weights come from
   ``serve_configs.weight_path``/weight_rank_0.pt (nanoflow_amd/weights.py; serve_8B.py:611-629);
@@ -116,7 +118,9 @@ def main():
                              vocab=m["vocab_size"], layers=m["num_hidden_layers"], page_size=mc.get("frame_page_size", 16),
                              eps=m.get("rms_norm_eps", 1e-5), rope_theta=m.get("rope_theta", 1e4),
                              rope_scaling=m.get("rope_scaling") or None)   # Llama-3.1 (config_all/llama3.1-8B)
-    pt = P.PipelineType[sc["pipeline_type"]]
+    if sc["pipeline_type"] not in P.pipeline_map:
+        raise SystemExit(f"serve_configs.pipeline_type {sc['pipeline_type']!r}: one of {', '.join(P.pipeline_map)}")
+    pt = P.pipeline_map[sc["pipeline_type"]]
     T, nano1, kqv1, kqv3 = pc["global_batch_size"], pc["nanobatch_1_size"], pc["kqv1_size"], pc["kqv3_size"]
     pages = 1024 * mc["allocate_kv_data_batch"] // 16
 

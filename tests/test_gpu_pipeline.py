@@ -306,12 +306,37 @@ def test_llama31_rope_scaling_reaches_the_kernel_through_the_config(oracle):
         assert _max_rel(h, hid) < E2E_RTOL, (pt, _max_rel(h, hid))
 
 
-def test_unsupported_pipeline_types_are_rejected():
+def test_the_offload_pipeline_type_is_rejected():
     from nanoflow_amd import engine, pllm_python as P
     shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)
-    with pytest.raises(P.NanoflowPipelineError, match="tensor-parallel"):
-        engine.Engine(shape, P.PipelineType.PLLM, global_batch=32, nano1=16, kv_pages=64)
+    with pytest.raises(P.NanoflowPipelineError, match="offload"):
+        engine.Engine(shape, P.PipelineType.PLLMOFFLOAD, global_batch=32, nano1=16, kv_pages=64)
     P.finalize()
+
+
+def test_tensor_parallel_schedule_types_run_as_their_one_device_schedules():
+    """PLLM, NONOVERLAP and NANOBATCH (pipeline/src/computeBound.cu:225-233) on one rank: no exchange step
+    moves anything, so they are LOCAL, NON_OVERLAP_LOCAL and NANOBATCH_LOCAL, bit for bit."""
+    from nanoflow_amd import engine, pllm_python as P
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    b = synth.make_batch(list(range(5, 25)), [(7, 30), (0, 46)], vocab=shape.vocab, seed=31, extra_pages=40)
+    rng = np.random.default_rng(6)
+    pools = [synth.make_kv_pool(b.num_pages, shape, rng) for _ in range(shape.layers)]
+    w = synth.make_weights(shape, seed=9)
+
+    def run(pt):
+        with engine.Engine(shape, pt, global_batch=96, nano1=40, kqv1=20, kqv3=28, kv_pages=b.num_pages,
+                           weights=w, kv_pools=pools) as e:
+            e.update(b)
+            ids = e.run().copy()
+            return ids, e.buffer("hidden").cpu().numpy()[:b.tokens], [p.cpu().numpy() for p in e.kv]
+    for tp, local in ((P.PipelineType.PLLM, P.PipelineType.LOCAL), (P.PipelineType.NONOVERLAP, P.PipelineType.NON_OVERLAP_LOCAL),
+                      (P.PipelineType.NANOBATCH, P.PipelineType.NANOBATCH_LOCAL)):
+        print("pipeline type", tp.name, flush=True)
+        assert tp.is_sequential == local.is_sequential
+        a, b_ = run(tp), run(local)
+        assert np.array_equal(a[0], b_[0]) and np.array_equal(a[1], b_[1])
+        assert all(np.array_equal(x, y) for x, y in zip(a[2], b_[2]))
 
 
 def _serve_requests(n=14, seed=3):
@@ -589,8 +614,9 @@ def test_serve_command_line_tokenizes_prompt_text_and_writes_the_words_file(tmp_
     shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
     cfg = tmp_path / "tiny.json"
     engine.write_config(str(cfg), shape, global_batch=96, nano1=40, kqv1=20, kqv3=28,
-                        pipeline_type=P.PipelineType.NON_OVERLAP_LOCAL, kv_pages=256)
+                        pipeline_type=P.PipelineType.NONOVERLAP, kv_pages=256)
     c = json.load(open(cfg))
+    assert c["serve_configs"]["pipeline_type"] == "NON_OVERLAP"      # the reference's name of the tensor-parallel type
     c["serve_configs"]["model"] = str(tmp_path / "tok")
     json.dump(c, open(cfg, "w"))
     prompts = ["the quick brown fox jumps over the lazy dog", "the lazy dog, the quick fox", "fox"]
