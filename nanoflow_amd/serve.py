@@ -100,7 +100,8 @@ def main():
     ap.add_argument("--est_cycle_time", type=float, default=0.175)
     ap.add_argument("-o", "--output_prefix", default="")
     ap.add_argument("--allocate_page_num", type=int, default=740, help="accepted and unused, as in the reference")
-    ap.add_argument("--empty_weight", default="True")
+    ap.add_argument("--empty_weight", default="False", help="random-init weights on the device instead of weight_path")
+    ap.add_argument("--profile_mode", default="False", help="accepted and unused, as in the reference")
     ap.add_argument("--output_idx", default="False", help="precede every line of PREFIX.req_words by 'Req k:'")
     a = ap.parse_args()
     empty_weight = str(a.empty_weight).lower() in ("true", "1", "yes")
