@@ -91,6 +91,24 @@ def read_trace(path, tokenizer=None):
     return reqs
 
 
+def parse_config(cfg):
+    """(model shape, pipeline type, (global batch, nano-batch 1, kqv1, kqv3), KV pages per layer) of a
+    pipeline JSON in the reference's schema."""
+    from nanoflow_amd import synth, pllm_python as P
+    m, mc, pc, sc = cfg["model"], cfg["model_configs"], cfg["pipeline_configs"], cfg["serve_configs"]
+    if mc.get("gpu_num", 1) != 1 or sc.get("actual_gpu_num", 1) != 1:
+        raise SystemExit("this build serves on one GPU (gpu_num and actual_gpu_num must be 1)")
+    shape = synth.ModelShape(hidden=m["hidden_size"], Hq=m["num_attention_heads"], Hkv=m["num_key_value_heads"],
+                             d=m["hidden_size"] // m["num_attention_heads"], ffn=m["intermediate_size"],
+                             vocab=m["vocab_size"], layers=m["num_hidden_layers"], page_size=mc.get("frame_page_size", 16),
+                             eps=m.get("rms_norm_eps", 1e-5), rope_theta=m.get("rope_theta", 1e4),
+                             rope_scaling=m.get("rope_scaling") or None)   # Llama-3.1 (config_all/llama3.1-8B)
+    if sc["pipeline_type"] not in P.pipeline_map:
+        raise SystemExit(f"serve_configs.pipeline_type {sc['pipeline_type']!r}: one of {', '.join(P.pipeline_map)}")
+    sizes = (pc["global_batch_size"], pc["nanobatch_1_size"], pc["kqv1_size"], pc["kqv3_size"])
+    return shape, P.pipeline_map[sc["pipeline_type"]], sizes, 1024 * mc["allocate_kv_data_batch"] // 16   # serve_8B.py:643
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("-t", "--trace_path", required=True)
@@ -111,19 +129,8 @@ def main():
     from nanoflow_amd import engine, synth, pllm_python as P
     assert torch.cuda.is_available(), "needs the MI355X"
     cfg = json.load(open(a.config_path))
-    m, mc, pc, sc = cfg["model"], cfg["model_configs"], cfg["pipeline_configs"], cfg["serve_configs"]
-    if mc.get("gpu_num", 1) != 1 or sc.get("actual_gpu_num", 1) != 1:
-        raise SystemExit("this build serves on one GPU (gpu_num must be 1)")
-    shape = synth.ModelShape(hidden=m["hidden_size"], Hq=m["num_attention_heads"], Hkv=m["num_key_value_heads"],
-                             d=m["hidden_size"] // m["num_attention_heads"], ffn=m["intermediate_size"],
-                             vocab=m["vocab_size"], layers=m["num_hidden_layers"], page_size=mc.get("frame_page_size", 16),
-                             eps=m.get("rms_norm_eps", 1e-5), rope_theta=m.get("rope_theta", 1e4),
-                             rope_scaling=m.get("rope_scaling") or None)   # Llama-3.1 (config_all/llama3.1-8B)
-    if sc["pipeline_type"] not in P.pipeline_map:
-        raise SystemExit(f"serve_configs.pipeline_type {sc['pipeline_type']!r}: one of {', '.join(P.pipeline_map)}")
-    pt = P.pipeline_map[sc["pipeline_type"]]
-    T, nano1, kqv1, kqv3 = pc["global_batch_size"], pc["nanobatch_1_size"], pc["kqv1_size"], pc["kqv3_size"]
-    pages = 1024 * mc["allocate_kv_data_batch"] // 16
+    mc, sc = cfg["model_configs"], cfg["serve_configs"]
+    shape, pt, (T, nano1, kqv1, kqv3), pages = parse_config(cfg)
 
     weights = None
     if not empty_weight:

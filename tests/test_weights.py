@@ -210,3 +210,28 @@ def test_converted_file_is_the_reference_converters_file(tmp_path, case, bias):
     assert sorted(got) == sorted(want[case])
     for name in want[case]:
         assert got[name] == want[case][name], name        # shape, dtype and every byte
+
+
+def test_shipped_pipeline_files_parse_and_fit_one_mi355x():
+    """nanoflow_amd/config_all/*.json: the reference's schema with gpu_num 1, sized so that weights, KV
+    pool and scratch stay below 90 % of the 288 GiB of one MI355X."""
+    import glob, json, os
+    from nanoflow_amd import serve, pllm_python as P
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "nanoflow_amd", "config_all")
+    files = sorted(glob.glob(os.path.join(root, "*.json")))
+    assert len(files) >= 7
+    for f in files:
+        cfg = json.load(open(f))
+        shape, pt, (T, nano1, kqv1, kqv3), pages = serve.parse_config(cfg)
+        assert T == 2048 and 0 < nano1 < T and pages % 64 == 0, f
+        assert pt.has_kqv_bias == ("qwen2" in f), f
+        kqv_n = shape.hidden + 2 * shape.Hkv * shape.d
+        per_layer = shape.hidden * kqv_n + shape.hidden * shape.hidden + 3 * shape.hidden * shape.ffn
+        fp8 = cfg["serve_configs"].get("weight_format") == "e4m3"
+        weights = shape.layers * per_layer * (1 if fp8 else 2) + 2 * shape.vocab * shape.hidden * 2
+        kv = shape.layers * pages * (2 * shape.page_size * shape.Hkv * shape.d * 2)
+        scratch = 2 * (T * shape.hidden * 16 + T * shape.vocab * 2 + T * shape.ffn) + (1 << 30)
+        assert weights + kv + scratch < 0.90 * (288 << 30), (f, weights / 1e9, kv / 1e9)
+        assert kv > 0.25 * (288 << 30), (f, kv / 1e9)                      # and the pool is not a token gesture
+        if "3.1" in f:
+            assert shape.rope_scaling and shape.rope_scaling["factor"] == 8.0
