@@ -97,6 +97,23 @@ def cpu_baseline(shape, decode_lens_after, prefill_chunks, total_decode, seed: i
     }
 
 
+def calibrate(fp8: bool):
+    """Ceilings measured on this device in this run, before the model is resident: a register-only
+    MFMA loop (zero operands: the highest clock the part holds; pseudo-random operands: the
+    switching activity a GEMM on N(0,1) data feeds the matrix pipe) and an 8 GiB read stream."""
+    from nanoflow_amd import kernels as K
+    K.lib()
+    K.calibrate_mfma(fp8, True, 4000)                      # power state settles
+    tf_rand, mhz_rand = K.calibrate_mfma(fp8, True, 40000)
+    tf_zero, mhz_zero = K.calibrate_mfma(fp8, False, 40000)
+    hbm = K.calibrate_hbm_read(8.0, 4)
+    return {"mfma_tflops_random_operands": tf_rand, "mfma_clock_mhz_random_operands": mhz_rand,
+            "mfma_tflops_zero_operands": tf_zero, "mfma_clock_mhz_zero_operands": mhz_zero,
+            "mfma_dtype": "f8e4m3" if fp8 else "f16", "hbm_read_stream_gbps": hbm,
+            "how": "nf_calibrate_mfma: 1024 workgroups x 4 wavefronts x 40000 x 16 independent 32x32 MFMAs, "
+                   "registers only; nf_calibrate_hbm_read: 2048 workgroups stream 8 GiB 4 times"}
+
+
 def _check_single_gpu(args):
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the single-device pipeline on ONE GPU; --gpus N>1 is not "
@@ -104,11 +121,18 @@ def _check_single_gpu(args):
         sys.exit(2)
 
 
-def _attention_roofline(tm, bytes_per_launch, name="roofline"):
+def _attention_roofline(tm, bytes_per_launch, name="roofline", calib=None):
     n_launch = max(tm.decode_attn_launches, 1)
     avg_launch_ms = tm.decode_attn_ms / n_launch
     achieved = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9 if avg_launch_ms > 0 else 0.0
+    extra = {}
+    if calib:
+        extra = {"measured_peak": calib["hbm_read_stream_gbps"],
+                 "frac_of_measured_peak": achieved / calib["hbm_read_stream_gbps"]}
+        if "paged_read_no_arithmetic_gbps" in calib:
+            extra["paged_read_no_arithmetic_gbps"] = calib["paged_read_no_arithmetic_gbps"]
     return {
+        **extra,
         "kernel": "attn_decode_kernel (paged decode attention)", "bound": "hbm",
         "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
         "traffic": (None if DECODE_ATTN_TRAFFIC_RATIO is None
@@ -141,7 +165,7 @@ def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows, weight_bytes=2
     return total / (4 * shape.layers + 1)
 
 
-def _gemm_roofline(tm, alg_bytes_per_launch=None, fp8_share=0.0):
+def _gemm_roofline(tm, alg_bytes_per_launch=None, fp8_share=0.0, calib=None):
     """fp8_share: the fraction of the timed GEMM flops that runs on the fp8 matrix cores (the
     per-layer GEMMs with e4m3 weights; the LM head stays fp16).  The peak the launches are priced
     against is then the flop-weighted blend of the two published peaks."""
@@ -150,7 +174,15 @@ def _gemm_roofline(tm, alg_bytes_per_launch=None, fp8_share=0.0):
     flop_per_launch = tm.gemm_flop / n
     achieved = flop_per_launch / (avg_ms * 1e-3) / 1e12 if avg_ms > 0 else 0.0
     peak = 1.0 / (fp8_share / MFMA_FP8_PEAK_TFLOPS + (1.0 - fp8_share) / MFMA_PEAK_TFLOPS)
+    extra = {}
+    if calib and not fp8_share:
+        # the register-only MFMA loop on pseudo-random operands: what the matrix pipe sustains on
+        # this device at the clock it holds under that load
+        extra = {"measured_peak": calib["mfma_tflops_random_operands"],
+                 "frac_of_measured_peak": achieved / calib["mfma_tflops_random_operands"],
+                 "measured_peak_zero_operands": calib["mfma_tflops_zero_operands"]}
     return {
+        **extra,
         "kernel": ("gemm_f16_kernel / dual_swiglu_f16_kernel (all dense GEMM launches of the iteration)" if not fp8_share
                    else "gemm_f8_kernel incl. the fused gate/up variant (e4m3 weights, activations quantised per "
                         "launch; the quantiser's time is not in these launches) + the fp16 LM head"),
@@ -194,6 +226,7 @@ def run_iteration(args):
     fixed = 2 * (2 * shape.vocab * shape.hidden) + 2 * (T * shape.hidden * 16 + T * shape.vocab * 2) + (4 << 30)
     distinct = args.distinct_layers or int(max(1, min(shape.layers, (free_b * 0.92 - fixed) // per_layer)))
 
+    calib = calibrate(wb == 1) if args.calibrate else None
     t_setup = time.perf_counter()
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, run_layer=shape.layers,
@@ -248,7 +281,7 @@ def run_iteration(args):
             "distinct_layers_in_hbm": distinct, "kv_pages_per_layer": int(pages),
             "decode_attention_launches_per_layer": launches_per_layer,
         },
-        "roofline": _attention_roofline(tm, bytes_per_layer / launches_per_layer),
+        "roofline": _attention_roofline(tm, bytes_per_layer / launches_per_layer, calib=calib),
         "iteration": {
             "device_ms_last": tm.iter_ms, "ms_per_step_with_update": ms_with_update,
             "decode_attention_ms_per_step": tm.decode_attn_ms * tm.layer_stride / steps,
@@ -260,8 +293,16 @@ def run_iteration(args):
         },
     }
     if tm.gemm_launches:
-        rec["roofline_gemm"] = _gemm_roofline(tm, fp8_share=fp8_share)
+        rec["roofline_gemm"] = _gemm_roofline(tm, fp8_share=fp8_share, calib=calib)
         rec["iteration"]["gemm_ms_per_step"] = tm.gemm_ms * tm.layer_stride / steps
+    if calib:
+        from nanoflow_amd import kernels as K
+        dv = lambda a_: torch.from_numpy(np.ascontiguousarray(a_, np.int32)).cuda()
+        calib["paged_read_no_arithmetic_gbps"] = K.calibrate_paged_read(
+            eng.kv[0], dv(batch.kv_indptr[:nd + 1]), dv(batch.kv_indices), dv(batch.kv_last_page_len[:nd]),
+            nd, shape.Hkv, int(2 * batch.kv_len[:nd].astype(np.int64).sum() * shape.Hkv * shape.d * 2), 10)
+        rec["roofline"]["paged_read_no_arithmetic_gbps"] = calib["paged_read_no_arithmetic_gbps"]
+        rec["calibration"] = calib
     eng.close()
     if args.cpu_sample > 0:
         rec["cpu_baseline"] = cpu_baseline(shape, batch.kv_len[:args.cpu_sample], [], nd, args.seed)
@@ -289,14 +330,14 @@ def run_offline(args):
     pages = pages // 64 * 64
     assert pages >= 4096, f"not enough free HBM for the KV pool ({free_b / 2**30:.0f} GiB free)"
 
+    calib = calibrate(False) if args.calibrate else None
+
     t_setup = time.perf_counter()
-    # hundreds of timed cycles: two timed layers per cycle are plenty, and the event records and
-    # their collection stay below 0.1 ms of a cycle
-    P.setProfilingStride(16 if steps >= 64 else 0)
+    # Random KV contents (N(0,1), as the weights and activations are random): the pool the decode
+    # rows read must not be a run of zeros.
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, seed=args.seed,
-                        profiling=args.profile_level, kv_fill="zeros", weight_format=args.weights)
-    P.setGraphMode(args.graph)
+                        profiling=0, kv_fill=args.kv_fill, weight_format=args.weights)
     former = P.BatchFormer(pages, shape.page_size, T, args.nano1, args.kqv1, args.kqv3, in_len, out_len)
     rng = np.random.default_rng(args.seed)
     for i in range(n_req):
@@ -304,14 +345,40 @@ def run_offline(args):
     torch.cuda.synchronize()
     t_setup = time.perf_counter() - t_setup
 
+    # ---- pass 1, the one `value` comes from: iterations replayed from captured hipGraphs, no
+    # per-launch events.  Part of the set-up (like the simulated cycles): `prime` serving cycles in
+    # which the steady state's launch signatures are seen and captured.
+    graph = not args.no_graph and not args.full_run
+    P.setGraphMode(graph)
+    prime = 0
     if args.full_run:
         skip, warmup, steps = 0, 0, 1 << 30
     else:
         skip = args.skip_cycles
+        prime = args.prime_cycles if graph else 0
+        if prime:
+            former.serve(skip, prime, warmup_cycles=0)
+            skip = 0
     st = former.serve(skip, steps, warmup_cycles=warmup)
+    counters = P.getGraphCounters()
+    P.setGraphMode(False)
+
+    # ---- pass 2, the one the roofline records come from: the next cycles of the same job run
+    # eagerly with HIP events around every launch of every 16th layer (attention and dense GEMMs),
+    # on the streams the kernels run on
     tm = P.getTimings()
+    prof_cycles = 0
+    if args.profile_level and not args.full_run:
+        prof_cycles = min(st.cycles, args.profile_cycles)
+        P.setProfilingStride(16 if prof_cycles >= 32 else 4)
+        P.setProfiling(args.profile_level)
+        st_prof = former.serve(0, prof_cycles, warmup_cycles=2)
+        tm = P.getTimings()
+        prof_cycles = st_prof.cycles
+        P.setProfiling(0)
     state = former.state()
     steps = st.cycles
+    n_prof = max(prof_cycles if prof_cycles else st.cycles, 1)   # cycles the per-launch timings cover
     rows_per_req = in_len + out_len - 1          # dense-batch rows a request occupies in its life
     by_retired = st.retired * (in_len + out_len) / st.wall_s
     by_rows = st.tokens_processed / rows_per_req * (in_len + out_len) / st.wall_s
@@ -349,8 +416,11 @@ def run_offline(args):
                          f"prompts (ids uniform over the vocab) / {out_len} output tokens, greedy, EOS "
                          f"ignored, <= {T} tokens per iteration with chunked prefill; "
                          + ("whole job timed" if args.full_run else
-                            f"{skip} simulated scheduler cycles to steady state, then {warmup} warm-up and "
-                            f"{steps} timed serving cycles")),
+                            f"{args.skip_cycles} simulated scheduler cycles to steady state, {prime} untimed cycles "
+                            f"that capture the hipGraphs, then {warmup} warm-up and {steps} timed serving cycles "
+                            f"replayed from hipGraphs; the roofline records come from the {prof_cycles} eager, "
+                            f"per-launch-timed cycles that follow")),
+            "kv_contents": args.kv_fill,
             "pipeline": args.pipeline, "global_batch": T, "nanobatch_1_size": args.nano1,
             "kqv1_size": args.kqv1, "kqv3_size": args.kqv3, "layers_executed": shape.layers,
             "distinct_layers_in_hbm": shape.layers, "kv_pages_per_layer": int(pages),
@@ -362,8 +432,8 @@ def run_offline(args):
                          "none: the reference publishes no single-GPU figure for this shape / weight format"),
         },
         "roofline": _gemm_roofline(tm, _gemm_algorithmic_bytes_per_launch(shape, rows_next, reqs_next, wb),
-                                   fp8_share) if tm.gemm_launches else _attention_roofline(
-            tm, bytes_per_layer / launches_per_layer),
+                                   fp8_share, calib) if tm.gemm_launches else _attention_roofline(
+            tm, bytes_per_layer / launches_per_layer, calib=calib),
         "serving": {
             "cycles": st.cycles, "retired_requests": st.retired, "wall_s": st.wall_s,
             "tokens_per_s_by_retired_requests": by_retired, "tokens_per_s_by_rows": by_rows,
@@ -376,17 +446,29 @@ def run_offline(args):
             "cpu_form_hidden_fraction": (1.0 - min(1.0, max(0.0, st.cycle_ms - st.gpu_iter_ms - st.update_ms)
                                                    / st.form_ms) if st.form_ms > 0 else None),
             "steady_state_decode_rows": int(nd), "steady_state_prefill_rows": int(nxt["prefillTokensNum"]),
-            "decode_attention_ms_per_cycle": tm.decode_attn_ms * tm.layer_stride / max(st.cycles, 1),
-            "prefill_attention_ms_per_cycle": tm.prefill_attn_ms * tm.layer_stride / max(st.cycles, 1),
-            "gemm_ms_per_cycle": tm.gemm_ms * tm.layer_stride / max(st.cycles, 1),   # LM head: timed 1 iteration in layer_stride
-            "timed_layer_stride": tm.layer_stride,
-            "graph_counters": P.getGraphCounters(),
+            "decode_attention_ms_per_cycle": tm.decode_attn_ms * tm.layer_stride / n_prof,
+            "prefill_attention_ms_per_cycle": tm.prefill_attn_ms * tm.layer_stride / n_prof,
+            "gemm_ms_per_cycle": tm.gemm_ms * tm.layer_stride / n_prof,   # LM head: timed 1 iteration in layer_stride
+            "timed_layer_stride": tm.layer_stride, "per_launch_timed_cycles": prof_cycles,
+            "per_launch_timed_cycle_ms": st_prof.cycle_ms if prof_cycles else None,
+            "graph_counters": counters,
             "requests_left": state["queued"] + state["decoding"] + state["prefilling"],
             "setup_s": t_setup,
         },
     }
+    if calib and nd:
+        # the decode rows' own page table through the load pattern of the attention kernel with the
+        # arithmetic removed: the ceiling of that access pattern on this device
+        dv = lambda a_: torch.from_numpy(np.ascontiguousarray(a_, np.int32)).cuda()
+        from nanoflow_amd import kernels as K
+        calib["paged_read_no_arithmetic_gbps"] = K.calibrate_paged_read(
+            eng.kv[0], dv(nxt["kv_indptr"][:nd + 1]), dv(nxt["kv_indices"]), dv(nxt["kv_last_page_len"][:nd]),
+            nd, shape.Hkv, int(2 * kv_len.astype(np.int64).sum() * shape.Hkv * shape.d * 2), 10)
+        rec["calibration"] = calib
+        if rec["roofline"]["bound"] == "hbm":
+            rec["roofline"]["paged_read_no_arithmetic_gbps"] = calib["paged_read_no_arithmetic_gbps"]
     if tm.gemm_launches and tm.decode_attn_launches and nd:
-        rec["roofline_decode_attention"] = _attention_roofline(tm, bytes_per_layer / launches_per_layer)
+        rec["roofline_decode_attention"] = _attention_roofline(tm, bytes_per_layer / launches_per_layer, calib=calib)
     eng.close()
     if args.cpu_sample > 0 and nd:
         n = min(args.cpu_sample, nd)
@@ -424,14 +506,22 @@ def main():
     ap.add_argument("--profile-level", type=int, default=2, choices=[0, 1, 2],
                     help="per-launch events: 1 attention, 2 attention and GEMMs")
     ap.add_argument("--graph", action="store_true",
-                    help="replay iterations from captured hipGraphs (disables per-launch profiling)")
+                    help="iteration workload: replay from captured hipGraphs (disables per-launch profiling)")
+    ap.add_argument("--no-graph", action="store_true", help="offline workload: run the timed cycles eagerly")
+    ap.add_argument("--prime-cycles", type=int, default=48,
+                    help="offline workload: untimed serving cycles before the warm-up in which the hipGraphs are captured")
+    ap.add_argument("--profile-cycles", type=int, default=64,
+                    help="offline workload: eager cycles with per-launch events after the timed ones (roofline records)")
+    ap.add_argument("--kv-fill", default="randn", choices=["randn", "zeros"], help="offline workload: KV pool contents")
+    ap.add_argument("--no-calibrate", dest="calibrate", action="store_false",
+                    help="skip the in-run MFMA / HBM calibration micro-benchmarks")
     ap.add_argument("--cpu-sample", type=int, default=96, help="decode requests in the CPU baseline (0 = skip)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     _check_single_gpu(args)
     if args.pipeline == "auto":
         args.pipeline = "NON_OVERLAP_LOCAL"
-    if args.graph:
+    if args.graph and args.workload == "iteration":
         args.profile_level = 0
     rec = run_offline(args) if args.workload == "offline" else run_iteration(args)
     print(json.dumps(rec))

@@ -69,9 +69,10 @@ NF_API int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* wei
 NF_API int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
                 int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
 
-/* nf_gemm_f16 with scratch: a GEMM of at most 256 rows whose output tiles would leave most of the
- * chip idle (few rows against a narrow N: the QKV, O and down projections of a small decode batch)
- * is split over K into shares that fill it, summed in fp32 through `workspace`
+/* nf_gemm_f16 with scratch: a GEMM of at most 512 rows whose output tiles would leave most of the
+ * chip idle (few rows against a narrow N: the QKV, O and down projections of a small decode batch;
+ * up to 320 rows any contraction of 1024 or more, from 321 to 512 rows contractions of 12288 or
+ * more) is split over K into shares that fill it, summed in fp32 through `workspace`
  * (nf_gemm_workspace_bytes(M, N, K) bytes, 16-byte aligned; 0 = this shape is not split).  With a
  * null or short workspace, or a shape that does not profit, it is nf_gemm_f16.  The sum over k is
  * then taken share by share, so results differ from nf_gemm_f16 in fp32 rounding only.
@@ -219,6 +220,28 @@ NF_API int nf_keep_token_f16(const uint16_t* in, uint16_t* out, const int32_t* i
  * MaxSampling::work (pipeline/include/otherWrapper.cuh:489-491). */
 NF_API int nf_argmax_f16(const uint16_t* logits, uint16_t* max_vals, int32_t* argmax, int rows, int cols,
                   nf_stream_t stream);
+
+/* Calibration micro-benchmarks: ceilings measured on the device the library runs on, beside which
+ * the kernels' rates are reported.  Each call launches, waits for and times its own kernels (HIP
+ * events on `stream`); `scratch` is at least 8192 bytes of device memory the kernels may write.
+ * nf_calibrate_mfma: a register-only loop of independent 32x32 MFMA instructions (fp8 == 0:
+ *   v_mfma_f32_32x32x16_f16; else the 32x32x64 fp8 form), one wavefront per SIMD, `iters` x 16
+ *   instructions per wavefront, on zero operands (random_operands == 0) or pseudo-random ones;
+ *   *tflops = the rate, *clock_mhz = shader clock the wavefronts saw while running.
+ * nf_calibrate_hbm_read: all CUs stream `bytes` of `buf` (16-byte aligned, much larger than the
+ *   last-level cache) `reps` times; *gbps = the read rate.
+ * nf_calibrate_paged_read: the access pattern of paged decode attention (arguments as
+ *   nf_attention_paged_f16's: page size 16, head_dim 128) without its arithmetic;
+ *   *gbps = kv_bytes_per_launch x reps / time.
+ * No counterpart in the reference, whose benchmarks divide by vendor peaks. */
+NF_API int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, size_t scratch_bytes,
+                             double* tflops, double* clock_mhz, nf_stream_t stream);
+NF_API int nf_calibrate_hbm_read(const void* buf, size_t bytes, int reps, void* scratch, size_t scratch_bytes,
+                                 double* gbps, nf_stream_t stream);
+NF_API int nf_calibrate_paged_read(const uint16_t* kv_data, const int32_t* kv_indptr, const int32_t* kv_indices,
+                                   const int32_t* kv_last_page_len, int batch, int num_kv_heads,
+                                   size_t kv_bytes_per_launch, int reps, void* scratch, size_t scratch_bytes,
+                                   double* gbps, nf_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -278,7 +278,9 @@ NF_PLLM_API int pllm_get_graph_counters(long counters[3]);
 NF_PLLM_API int pllm_reset_timings(void);
 /* Device address of an intermediate of the current pipeline, for parity checks:
  * name in {"hidden" (residual stream after the last layer, [T, hidden]),
- *          "logits" ([T, vocab])}. */
+ *          "logits" ([T, vocab])}; for the non-overlap pipeline also the last layer's operator
+ *          inputs and outputs: "ln_attn" (QKV input), "kqv", "attn_out" (O input), "o_out",
+ *          "ln_ffn" (gate/up input), "act" (down input). */
 NF_PLLM_API int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols);
 
 #ifdef __cplusplus

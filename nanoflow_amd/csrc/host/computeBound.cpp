@@ -99,14 +99,23 @@ void init(int nranks, int vnranks, std::vector<vortexInitData>& input,
 void update(int nranks, std::vector<vortexUpdateData>& updateData) {
   assert((int)updateData.size() == nranks);
   auto& update_d = updateData[0];
-  complete_input_tokens.resize(update_d.decodePrefillBorder + update_d.prefillTokensNum + 1);
-  [[maybe_unused]] int n = buildInputTokens(aggregated_output.data(), (int)aggregated_output.size(),
-                                            update_d.keep_token_list, update_d.keepTokenListLength,
-                                            update_d.input_tokens, update_d.prefillTokensNum,
-                                            complete_input_tokens.data());
-  if (n != update_d.decodePrefillBorder + update_d.prefillTokensNum)
-    NF_LOG_WARN("update: %d kept + prefill tokens but the batch has %d rows", n,
-                update_d.decodePrefillBorder + update_d.prefillTokensNum);
+  // Checked before anything is written: the kept slots are the decode rows, and every kept slot
+  // must have an output of the previous iteration to take its token from.
+  int kept = 0;
+  for (int i = 0; i < update_d.keepTokenListLength; ++i) kept += update_d.keep_token_list[i] == 1;
+  const bool first = aggregated_output.empty();
+  if (kept != update_d.decodePrefillBorder || update_d.prefillTokensNum < 0 ||
+      (!first && update_d.keepTokenListLength > (int)aggregated_output.size())) {
+    std::fprintf(stderr,
+                 "update: keep list of %d entries keeps %d slots, the batch has %d decode rows and the previous "
+                 "iteration produced %zu outputs\n",
+                 update_d.keepTokenListLength, kept, update_d.decodePrefillBorder, aggregated_output.size());
+    std::exit(EXIT_FAILURE);
+  }
+  complete_input_tokens.resize((size_t)kept + update_d.prefillTokensNum + 1);
+  buildInputTokens(aggregated_output.data(), (int)aggregated_output.size(), update_d.keep_token_list,
+                   update_d.keepTokenListLength, update_d.input_tokens, update_d.prefillTokensNum,
+                   complete_input_tokens.data());
   for (int i = 0; i < nranks; ++i) updateData[i].input_tokens = complete_input_tokens.data();
   shared_state.op = WorkerOp::UPDATE;
   shared_state.updates_ptr = &updateData;

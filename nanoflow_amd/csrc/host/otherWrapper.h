@@ -90,9 +90,14 @@ public:
     pllm_tensor_output = o;
     if (input_size) assert(input_size * ModelConfig.model_hidden_dim == output_size);
   }
+  // rows that hold tokens in this iteration (-1: all); ids beyond them are not uploaded, so
+  // their rows are left as they were
+  int live_rows = -1;
+  void set_live_rows(int r) { live_rows = r; }
   void work() override {
-    NF_KERNEL_CHECK(nf_embedding_f16(tokens, weight, output, input_size,
-                                     ModelConfig.model_hidden_dim, stream));
+    const int rows = live_rows >= 0 && live_rows < input_size ? live_rows : input_size;
+    if (rows == 0) return;
+    NF_KERNEL_CHECK(nf_embedding_f16(tokens, weight, output, rows, ModelConfig.model_hidden_dim, stream));
   }
 };
 

@@ -85,6 +85,7 @@ protected:
   std::set<std::vector<int>> graph_seen;
   long graph_replays = 0, graph_captures = 0, graph_eager = 0;
   static constexpr size_t kMaxGraphs = 64;
+  static constexpr size_t kMaxSeen = 4096;
 
   template <class F>
   void runIteration(hipStream_t origin, const std::vector<int>& sig, F&& enqueue) {
@@ -96,6 +97,7 @@ protected:
     auto it = graph_execs.find(sig);
     if (it == graph_execs.end()) {
       if (!graph_seen.count(sig) || graph_execs.size() >= kMaxGraphs) {
+        if (graph_seen.size() >= kMaxSeen) graph_seen.clear();  // bounded: forgetting only delays a capture
         graph_seen.insert(sig);
         ++graph_eager;
         enqueue();
@@ -208,6 +210,7 @@ public:
   hipStream_t stream_gemv = nullptr;
   hipStream_t stream_other = nullptr;
   int update_token_num = 0;
+  int border_request = -1;  // the prefill request cut by the nano-batch border in this iteration (-1: none)
   vortexUpdateData prefill1_update;   // device copies patched for a prefill request that
   vortexUpdateData prefill1_staging;  // straddles the nano-batch border (+ pinned staging)
   bool nanobatch_only = false;

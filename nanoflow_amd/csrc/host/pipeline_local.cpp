@@ -394,7 +394,13 @@ void LocalPipeline::enqueueIteration() {
 vortexOutputData LocalPipeline::run() {
   setWeight(0);
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_START], stream_gemm));
-  runIteration(stream_gemm, baseSignature(), [this] { enqueueIteration(); });
+  // The attention slices also depend on which request straddles the nano-batch border (a
+  // function of the individual prefill lengths, not of their total): it is part of the signature.
+  std::vector<int> sig = baseSignature();
+  sig.push_back(border_request);
+  sig.push_back((int)prefill1.batch_size);
+  sig.push_back((int)prefill2.batch_size);
+  runIteration(stream_gemm, sig, [this] { enqueueIteration(); });
   // the sampler (stream_gemm) depends on every attention launch through O1/O2
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_END], stream_gemm));
   HIP_CHECK(hipMemcpyAsync(output_data.sampled_token_array, maxSampler.d_argMax.ptr,
@@ -434,6 +440,7 @@ void LocalPipeline::GEMVOpUpdate() {
   const int nano1 = config_data.nanobatch_1_size;
   const int dpb = update_data.decodePrefillBorder;
   bool need_overlap = true;  // a prefill request straddles the nano-batch border
+  border_request = -1;
   if (nano1 >= update_token_num) need_overlap = false;
   else if (dpb >= nano1) need_overlap = false;
 
@@ -494,6 +501,7 @@ void LocalPipeline::GEMVOpUpdate() {
     // (patched copies of input_indptr / kv_indptr / kv_last_page_len), prefill2 sees it whole.
     const vortexUpdateData& h = host_update_data;
     const int border_prefill_request = h.rev_input_indptr[nano1 - 1];
+    border_request = border_prefill_request;
     assert(border_prefill_request - dpb >= 0);
     assert(update_data.prefillNum + dpb - border_prefill_request >= 0);
     uint32_t arr[] = {uint32_t(gb[0]), uint32_t(gb[1]), uint32_t(border_prefill_request - dpb),
@@ -575,6 +583,8 @@ void LocalPipeline::update(vortexUpdateData* update_data_) {
   for (BaseGEMMWrapper* g : {O2, D2, KQV2}) g->set_live_rows((size_t)live2);
   dual1.set_live_rows(live1);
   dual2.set_live_rows(live2);
+  genEmbedding1.set_live_rows(live1);
+  genEmbedding2.set_live_rows(live2);
   layerNormAttention1.set_live_rows(live1);
   layerNormFFN1.set_live_rows(live1);
   layerNormAttention2.set_live_rows(live2);

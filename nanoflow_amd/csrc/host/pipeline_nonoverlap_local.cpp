@@ -111,6 +111,7 @@ void NonOverlapLocalPipeline::update(vortexUpdateData* update_data_) {
   update_token_num = update_data.decodePrefillBorder + update_data.prefillTokensNum;
   for (BaseGEMMWrapper* g : {O, D, KQV}) g->set_live_rows((size_t)update_token_num);
   dual.set_live_rows(update_token_num);
+  genEmbedding.set_live_rows(update_token_num);
   layerNormAttention.set_live_rows(update_token_num);
   layerNormFFN.set_live_rows(update_token_num);
   maxSampler.set_batch_size(req_num / nranks);

@@ -415,8 +415,15 @@ int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols) {
     if (!std::strcmp(name, "hidden")) t = lp->keepToken.input;
     else if (!std::strcmp(name, "logits")) t = lp->maxSampler.d_matrix;
   } else if (auto* np = dynamic_cast<NonOverlapLocalPipeline*>(p)) {
+    // the intermediates hold the LAST layer's values once an iteration has run
     if (!std::strcmp(name, "hidden")) t = np->keepToken.input;
     else if (!std::strcmp(name, "logits")) t = np->maxSampler.d_matrix;
+    else if (!std::strcmp(name, "ln_attn")) t = np->KQV->getA();
+    else if (!std::strcmp(name, "kqv")) t = np->KQV->getD();
+    else if (!std::strcmp(name, "attn_out")) t = np->O->getA();
+    else if (!std::strcmp(name, "o_out")) t = np->O->getD();
+    else if (!std::strcmp(name, "ln_ffn")) t = np->dual.getA();
+    else if (!std::strcmp(name, "act")) t = np->D->getA();
   }
   if (!t.ptr) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_debug_buffer: unknown buffer \"%s\"", name);
   *ptr = t.ptr;

@@ -49,9 +49,17 @@ struct pllmTensor {
   size_t size() const { return dim1 * dim2; }
   size_t bytes() const { return size() * sizeof(T); }
 
+  // Rows [first, first + count) as a view of the same layout; an empty range is the
+  // reference's empty tensor (one "row" of zero columns) so that size() == 0.
+  pllmTensor rowsView(size_t first, size_t count) const {
+    if (count == 0) return pllmTensor(ptr + first * dim2, size_t(1), size_t(0), layout);
+    return pllmTensor(ptr + first * dim2, count, dim2, layout);
+  }
+
   pllmTensor subtensor(size_t startDim1, size_t dim1Count) const {
-    if (startDim1 >= dim1) throw std::out_of_range("Invalid start position for subtensor.");
-    if (startDim1 + dim1Count > dim1) throw std::out_of_range("Invalid row count for subtensor.");
+    if (startDim1 >= dim1 || dim1Count > dim1 - startDim1)
+      throw std::out_of_range("subtensor: rows " + std::to_string(startDim1) + "+" + std::to_string(dim1Count) +
+                              " of a tensor " + shapeString());
     return pllmTensor(ptr + startDim1 * dim2, dim1Count, dim2, layout);
   }
   pllmTensor subtensor(size_t startDim1) const {
@@ -59,86 +67,72 @@ struct pllmTensor {
   }
 
   bool checkShape(const pllmTensor<T>& other) const {
-    return dim1 == other.dim1 && dim2 == other.dim2 && layout == other.layout;
+    return layout == other.layout && dim1 == other.dim1 && dim2 == other.dim2;
   }
   bool assertShape(const pllmTensor<T>& other) const {
-    bool ret = checkShape(other);
-    if (!ret)
-      NF_LOG_ERROR("Shape mismatch: %s vs %s", shapeString().c_str(), other.shapeString().c_str());
-    return ret;
+    if (checkShape(other)) return true;
+    NF_LOG_ERROR("Shape mismatch: %s vs %s", shapeString().c_str(), other.shapeString().c_str());
+    return false;
   }
   std::string shapeString() const {
-    return "[" + std::to_string(dim1) + "x" + std::to_string(dim2) + " " + toString(layout) + "]";
+    std::ostringstream os;
+    os << '[' << dim1 << 'x' << dim2 << ' ' << toString(layout) << ']';
+    return os.str();
   }
+  // a row-major tensor is split along ROW, a column-major one along COLUMN: the enumerators pair up
   bool sameDirection(PllmDimension dim) const {
-    return static_cast<int>(dim) == static_cast<int>(layout);
+    return (dim == PllmDimension::ROW) == (layout == PllmLayout::ROW_MAJOR);
   }
 
-  // rank-th of nranks equal row chunks (the last takes the remainder)
+  // The share of rank `rank` when dim1 is dealt out in nranks equal runs; what does not divide
+  // goes to the last rank.
   pllmTensor<T> getSubTensor(int rank, int nranks, PllmDimension dim) const {
     assert(sameDirection(dim));
-    size_t chunk = dim1 / nranks;
-    size_t final_chunk = chunk + (rank == nranks - 1 ? dim1 % nranks : 0);
-    return pllmTensor<T>{ptr + rank * chunk * dim2, final_chunk, dim2, layout};
+    const size_t each = dim1 / nranks, first = each * rank;
+    return pllmTensor<T>{ptr + first * dim2, rank + 1 == nranks ? dim1 - first : each, dim2, layout};
   }
 
-  // Split along rows into consecutive pieces of the given lengths.  A zero length yields
-  // the empty tensor {ptr, 1, 0}.
+  // Consecutive pieces of the given lengths along dim1, which they must add up to.
   template <std::integral... Lens>
   std::array<pllmTensor<T>, sizeof...(Lens)> splitTensor(PllmDimension dim, Lens... lens) const {
     assert(sameDirection(dim));
-    [[maybe_unused]] size_t total = (size_t(0) + ... + size_t(lens));
-    assert(dim1 == total && "Subtensor length sum mismatches with the input tensor");
-    size_t i = 0, offset = 0;
-    std::array<pllmTensor<T>, sizeof...(Lens)> ret;
-    ((ret[i++] = (static_cast<size_t>(lens) == 0
-                      ? pllmTensor<T>{ptr + offset, size_t(1), size_t(0), layout}
-                      : pllmTensor<T>{ptr + offset, static_cast<size_t>(lens), dim2, layout}),
-      offset += lens * dim2),
-     ...);
-    return ret;
+    constexpr size_t N = sizeof...(Lens);
+    const size_t want[N] = {static_cast<size_t>(lens)...};
+    std::array<pllmTensor<T>, N> pieces;
+    size_t first = 0;
+    for (size_t i = 0; i < N; first += want[i++]) pieces[i] = rowsView(first, want[i]);
+    assert(first == dim1 && "the lengths of the pieces must add up to the tensor's length");
+    return pieces;
   }
 
-  // Split with an overlapping suffix: piece i is lens[i] + suffix rows long and piece i+1
-  // starts lens[i] rows later (used for indptr arrays: n requests need n+1 entries).
+  // Overlapping pieces: piece i starts where the lengths before it end and is lens[i] + suffix
+  // long (n requests own n + 1 entries of an indptr array, the last shared with the next piece).
   template <size_t N, std::unsigned_integral TLen>
   std::array<pllmTensor<T>, N> splitTensor(PllmDimension dim, const std::span<TLen, N>& lens,
                                            TLen suffix = 0) const {
     assert(sameDirection(dim));
-    assert(size() == std::accumulate(lens.begin(), lens.end(), size_t(0)) + suffix &&
-           "Subspan length sum mismatches with the input span");
-    size_t offset = 0;
-    std::array<pllmTensor<T>, N> ret;
-    for (size_t i = 0; i < N; ++i) {
-      size_t l = lens[i];
-      ret[i] = (l + suffix == 0) ? pllmTensor<T>{ptr + offset, size_t(1), size_t(0), layout}
-                                 : pllmTensor<T>{ptr + offset, l + suffix, dim2, layout};
-      offset += l * dim2;
-    }
-    return ret;
+    std::array<pllmTensor<T>, N> pieces;
+    size_t first = 0;
+    for (size_t i = 0; i < N; first += lens[i++]) pieces[i] = rowsView(first, size_t(lens[i]) + suffix);
+    assert((first + suffix) * dim2 == size() && "lengths plus the suffix must cover the tensor");
+    return pieces;
   }
 
-  // Per-piece suffix lengths.
+  // The same with a suffix of its own for every piece.
   template <size_t N, std::unsigned_integral TLen>
   std::array<pllmTensor<T>, N> splitTensor(PllmDimension dim, const std::span<TLen, N>& lens,
                                            const std::span<TLen, N>& suffix) const {
     assert(sameDirection(dim));
-    assert(size() == std::accumulate(lens.begin(), lens.end(), size_t(0)) + suffix[N - 1] &&
-           "Subspan length sum mismatches with the input span");
-    size_t offset = 0;
-    std::array<pllmTensor<T>, N> ret;
-    for (size_t i = 0; i < N; ++i) {
-      size_t l = lens[i];
-      ret[i] = (l + suffix[i] == 0) ? pllmTensor<T>{ptr + offset, size_t(1), size_t(0), layout}
-                                    : pllmTensor<T>{ptr + offset, l + suffix[i], dim2, layout};
-      offset += l * dim2;
-    }
-    return ret;
+    std::array<pllmTensor<T>, N> pieces;
+    size_t first = 0;
+    for (size_t i = 0; i < N; first += lens[i++]) pieces[i] = rowsView(first, size_t(lens[i]) + suffix[i]);
+    assert((first + suffix[N - 1]) * dim2 == size() && "lengths plus the last suffix must cover the tensor");
+    return pieces;
   }
 
   pllmTensor<T> slice(PllmDimension dim, size_t start, size_t end) const {
     assert(sameDirection(dim));
-    assert(end <= dim1 && start < end);
+    assert(start < end && end <= dim1);
     return pllmTensor<T>{ptr + start * dim2, end - start, dim2, layout};
   }
 };
@@ -152,18 +146,19 @@ inline pllmTensor<Tdst> tensor_cast(pllmTensor<Tsrc> src) {
 // Fields of a GEMM tag "ctaM_ctaN_ctaK_warpM_warpN_warpK_splitK_stages_{Row|Column}Major x3"
 // (pipeline/include/gemmShape.cuh:5-6).  idx 0/1/2 = layout of A / B / output.
 inline PllmLayout getMajorType(const std::string& input, int idx) {
-  std::stringstream ss(input);
-  std::string token;
-  std::vector<std::string> parts;
-  while (std::getline(ss, token, '_')) parts.push_back(token);
-  auto it = std::find_if(parts.begin(), parts.end(), [](const std::string& s) {
-    return s == "RowMajor" || s == "ColumnMajor";
-  });
-  if (it == parts.end()) throw std::invalid_argument("No major types found");
-  size_t start = std::distance(parts.begin(), it);
-  if (idx < 0 || start + idx >= parts.size()) throw std::out_of_range("Index is out of range");
-  const std::string& major = parts[start + idx];
-  if (major == "RowMajor") return PllmLayout::ROW_MAJOR;
-  if (major == "ColumnMajor") return PllmLayout::COL_MAJOR;
-  throw std::invalid_argument("Invalid major type");
+  // the three layouts are the tag's last three '_'-separated fields
+  std::array<std::string, 3> last;
+  size_t end = input.size();
+  for (int f = 2; f >= 0; --f) {
+    const size_t us = end == 0 ? std::string::npos : input.rfind('_', end - 1);
+    if (us == std::string::npos && f > 0)
+      throw std::invalid_argument("GEMM tag \"" + input + "\" does not end in three layout fields");
+    const size_t from = us == std::string::npos ? 0 : us + 1;
+    last[f] = input.substr(from, end - from);
+    end = us == std::string::npos ? 0 : us;
+  }
+  if (idx < 0 || idx > 2) throw std::out_of_range("GEMM tag layout index " + std::to_string(idx) + " (0..2)");
+  if (last[idx] == "RowMajor") return PllmLayout::ROW_MAJOR;
+  if (last[idx] == "ColumnMajor") return PllmLayout::COL_MAJOR;
+  throw std::invalid_argument("GEMM tag \"" + input + "\": \"" + last[idx] + "\" is not a layout");
 }

@@ -24,7 +24,9 @@ class TensorManager {
   template <typename T>
   static void alloc_pair(T*& dev, T*& host, size_t n) {
     HIP_CHECK(hipMalloc(&dev, n * sizeof(T)));
+    HIP_CHECK(hipMemset(dev, 0, n * sizeof(T)));  // entries past an iteration's live ones stay valid indices
     HIP_CHECK(hipHostMalloc(&host, n * sizeof(T), hipHostMallocDefault));
+    std::memset(host, 0, n * sizeof(T));
   }
   template <typename T>
   static void stage(T* host_stage, T* dev, const T* src, size_t n, hipStream_t s) {

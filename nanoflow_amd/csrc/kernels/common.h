@@ -99,16 +99,18 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
 // builtin form the compiler makes every later LDS read wait for ALL outstanding loads
 // (vmcnt(0)), because it cannot tell the stage being filled from the stage being read, and
 // that serialises the loads with the MFMAs.  The kernel waits itself (wait_loads below).
-// M0 carries the LDS address; nothing else in these kernels uses M0.
+// M0 carries the LDS address and is declared clobbered (the compiler warns that M0 is a reserved
+// register; the clobber still tells its M0-initialisation merging that the value changed, so the
+// warning is switched off in the build flags).
 __device__ __forceinline__ void load16_to_lds(rsrc_t r, uint32_t byte_off, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :: "s"(lds_addr), "v"(byte_off), "s"(r) : "memory");
+               :: "s"(lds_addr), "v"(byte_off), "s"(r) : "memory", "m0");
 }
 // The same with the LDS address given as a wavefront-uniform base plus a compile-time constant.
 template <int kLdsOffset>
 __device__ __forceinline__ void load16_to_lds(rsrc_t r, uint32_t byte_off, uint32_t lds_base) {
   asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :: "s"(lds_base), "v"(byte_off), "s"(r), "n"(kLdsOffset) : "memory", "scc");
+               :: "s"(lds_base), "v"(byte_off), "s"(r), "n"(kLdsOffset) : "memory", "scc", "m0");
 }
 __device__ __forceinline__ short4_t lds_read_tr16(const uint8_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p);

@@ -24,6 +24,7 @@ SYMBOLS = [
     "nf_dual_swiglu_f8w_split_workspace_bytes", "nf_dual_swiglu_f8w_split_workspace_bytes_upto",
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
+    "nf_calibrate_mfma", "nf_calibrate_hbm_read", "nf_calibrate_paged_read",
 ]
 
 
@@ -78,6 +79,10 @@ def lib() -> C.CDLL:
         l.nf_dual_swiglu_f8w_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, C.c_size_t, vp]
         l.nf_move_kv_pages.argtypes = [i32, vp, vp, vp, vp, vp, sz, i32, vp]
         l.nf_rope_append_f16.argtypes = [vp] * 7 + [i32] * 5 + [f32] * 4 + [vp]
+        dp = C.POINTER(C.c_double)
+        l.nf_calibrate_mfma.argtypes = [i32, i32, i32, vp, sz, dp, dp, vp]
+        l.nf_calibrate_hbm_read.argtypes = [vp, sz, i32, vp, sz, dp, vp]
+        l.nf_calibrate_paged_read.argtypes = [vp, vp, vp, vp, i32, i32, sz, i32, vp, sz, dp, vp]
         l.nf_attention_workspace_bytes.restype = sz
         l.nf_attention_workspace_bytes.argtypes = [i32, i32, i32]
         l.nf_attention_paged_f16.argtypes = [vp] * 7 + [i32] * 8 + [vp, sz, vp]
@@ -367,3 +372,39 @@ def argmax(logits, rows=None):
     arg = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     _check(lib().nf_argmax_f16(_p(logits), _p(mv), _p(arg), rows, cols, _stream()), "nf_argmax_f16")
     return arg, mv
+
+
+# ---------------------------------------------------------------- calibration micro-benchmarks
+
+def calibrate_mfma(fp8: bool = False, random_operands: bool = True, iters: int = 20000):
+    """(TFLOP/s, shader clock in MHz) of a register-only MFMA loop on this device."""
+    scratch = torch.zeros(8192, dtype=torch.uint8, device="cuda")
+    tf, mhz = C.c_double(), C.c_double()
+    _check(lib().nf_calibrate_mfma(int(fp8), int(random_operands), iters, scratch.data_ptr(), scratch.numel(),
+                                   C.byref(tf), C.byref(mhz), _stream()), "nf_calibrate_mfma")
+    return tf.value, mhz.value
+
+
+def calibrate_hbm_read(gib: float = 8.0, reps: int = 4) -> float:
+    """GB/s of all CUs streaming a buffer of `gib` GiB (freed again before returning)."""
+    n = int(gib * (1 << 30)) // 16 * 16
+    buf = torch.empty(n, dtype=torch.uint8, device="cuda")
+    buf.random_()   # touched: every page is backed
+    scratch = torch.zeros(8192, dtype=torch.uint8, device="cuda")
+    g = C.c_double()
+    _check(lib().nf_calibrate_hbm_read(buf.data_ptr(), n, reps, scratch.data_ptr(), scratch.numel(), C.byref(g), _stream()),
+           "nf_calibrate_hbm_read")
+    del buf
+    torch.cuda.empty_cache()
+    return g.value
+
+
+def calibrate_paged_read(pool, kv_indptr, kv_indices, kv_last_page_len, batch: int, num_kv_heads: int,
+                         kv_bytes: int, reps: int = 10) -> float:
+    """GB/s of paged decode attention's load pattern with the arithmetic removed."""
+    scratch = torch.zeros(8192, dtype=torch.uint8, device="cuda")
+    g = C.c_double()
+    _check(lib().nf_calibrate_paged_read(pool.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),
+                                         kv_last_page_len.data_ptr(), batch, num_kv_heads, kv_bytes, reps,
+                                         scratch.data_ptr(), scratch.numel(), C.byref(g), _stream()), "nf_calibrate_paged_read")
+    return g.value

@@ -113,6 +113,35 @@ def test_gemm_plain_and_residual(K, oracle, M, N, K_):
                  oracle.gemm(A, B, Cm, 1.0, 1.0), what="gemm beta=1")
 
 
+@pytest.mark.parametrize("M", [128, 768])
+def test_gemm_at_the_lm_head_shape(K, oracle, M):
+    """The LM head as the pipelines launch it (pipeline_local.cu:305-307,819-820): sampled rows padded
+    to 128 against the [4096, 128256] transposed lm_head, beta = 0.  1.05 GB of weights, 501 column
+    tiles of 256 (the last one 64 columns wide), 32-bit buffer offsets up to 1.05e9.  128 rows are
+    checked against the oracle in full; 768 rows against the oracle on column bands at the start, in
+    the middle and over the ragged last tile, and in full against fp32 PyTorch on the device."""
+    N, K_ = 128256, 4096
+    rng = np.random.default_rng(9)
+    A = synth.normal_f16(rng, (M, K_))
+    g = torch.Generator(device="cuda").manual_seed(10)
+    Bd = torch.empty((K_, N), dtype=torch.float16, device="cuda").normal_(0, 0.02, generator=g)
+    print(f"LM head GEMM M={M}", flush=True)
+    got_d = K.gemm(dev(A), Bd)
+    got = host(got_d)
+    assert got.shape == (M, N)
+    if M <= 128:
+        B = host(Bd)
+        assert_close(got, oracle.gemm(A, B), what="LM head gemm")
+    else:
+        for lo, hi in ((0, 512), (64000, 64512), (127744, N)):
+            Bb = np.ascontiguousarray(host(Bd[:, lo:hi]))
+            assert_close(got[:, lo:hi], oracle.gemm(A, Bb), what=f"LM head gemm columns {lo}:{hi}")
+    ref32 = dev(A).float() @ Bd.float()
+    err = (got_d.float() - ref32).abs().max().item()
+    assert err <= RTOL * ref32.abs().max().item() * 2, err
+    del ref32
+
+
 def test_gemm_alpha_beta_and_in_place_residual(K, oracle):
     rng = np.random.default_rng(4)
     A = synth.normal_f16(rng, (96, 256))

@@ -122,6 +122,61 @@ def test_three_schedules_match_oracle(oracle, case):
         assert _max_rel(r[1], base[1]) < 2e-3, (pt, "hidden differs between schedules")
 
 
+@pytest.mark.parametrize("gemm_cus,gemv_cus", [(128, 128), (160, 96)])
+def test_local_pipeline_on_cu_masked_streams_matches_unmasked_and_oracle(oracle, gemm_cus, gemv_cus):
+    """LocalPipeline with its two streams restricted to disjoint sets of whole XCDs
+    (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS -> hipExtStreamCreateWithCUMask): where a workgroup runs
+    must not change a bit of the result, and the result must be the oracle's."""
+    import os
+    from nanoflow_amd import engine, pllm_python as P
+    T, nano1, dlens, chunks = CASES["prefill_straddles_border"]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=0)
+    b = synth.make_batch(dlens, chunks, vocab=shape.vocab, seed=21, extra_pages=40)
+    rng = np.random.default_rng(5)
+    pools0 = [synth.make_kv_pool(b.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok = b.input_tokens.copy()
+    tok[:b.decodePrefillBorder] = 1
+    d = b.as_dict()
+    d["input_tokens"] = tok
+    pools_ref = [p.copy() for p in pools0]
+    hid_ref, log_ref, samp_ref = oracle.decoder_forward(shape.as_dict(), w, pools_ref, d, want_logits=True)
+
+    def run(env):
+        old = {k: os.environ.get(k) for k in ("NANOFLOW_GEMM_CUS", "NANOFLOW_GEMV_CUS")}
+        os.environ.update(env)
+        for k in old:
+            if k not in env:
+                os.environ.pop(k, None)
+        try:
+            print(f"LOCAL with {env or 'no CU masks'}", flush=True)
+            with engine.Engine(shape, P.PipelineType.LOCAL, global_batch=T, nano1=nano1, kqv1=nano1 // 2,
+                               kqv3=(T - nano1) // 2, kv_pages=b.num_pages, weights=w, kv_pools=pools0) as e:
+                e.update(b, keep_token_list=np.ones(b.decodePrefillBorder, np.int32))
+                ids = e.run().copy()
+                hid = e.buffer("hidden").cpu().numpy()[:b.tokens]
+                kv = [p[:b.num_pages].cpu().numpy() for p in e.kv]
+            return ids, hid, kv
+        finally:
+            for k, v in old.items():
+                if v is None:
+                    os.environ.pop(k, None)
+                else:
+                    os.environ[k] = v
+
+    ids0, hid0, kv0 = run({})
+    ids1, hid1, kv1 = run({"NANOFLOW_GEMM_CUS": str(gemm_cus), "NANOFLOW_GEMV_CUS": str(gemv_cus)})
+    assert np.array_equal(ids0, ids1) and np.array_equal(hid0, hid1)
+    for a, c in zip(kv0, kv1):
+        assert np.array_equal(a, c)
+    assert _max_rel(hid1, hid_ref) < E2E_RTOL
+    top2 = np.sort(log_ref.astype(np.float32), axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 2 * E2E_RTOL * np.abs(log_ref.astype(np.float32)).max()
+    assert np.array_equal(ids1[clear], samp_ref[clear])
+    for l in range(shape.layers):
+        assert np.array_equal((pools_ref[l] != pools0[l]).any(axis=(3, 4)), (kv1[l] != pools0[l]).any(axis=(3, 4)))
+
+
 def test_update_rejects_inconsistent_batches():
     from nanoflow_amd import engine, pllm_python as P
     shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)
@@ -481,6 +536,48 @@ def test_graph_replay_is_identical_to_eager(pt_name, weight_format):
         P.setWeightFormat(P.WeightFormat.F16)
     assert c0["captured"] == 0 and c0["replayed"] == 0 and c0["eager"] == len(order)
     assert c1["captured"] == 2 and c1["eager"] == 2 and c1["replayed"] == len(order) - 2, c1
+    for i, ((s0, h0), (s1, h1)) in enumerate(zip(eager, replay)):
+        assert np.array_equal(s0, s1), (i, "sampled ids")
+        assert np.array_equal(h0, h1), (i, "residual stream")
+
+
+def test_graph_replay_tells_apart_batches_that_differ_only_in_the_border_request():
+    """Two iterations with equal decode rows, prefill requests and prefill tokens, whose prefill
+    lengths differ so that a different request straddles the nano-batch border: the attention
+    slices differ, so a graph captured for one must not be replayed for the other."""
+    from nanoflow_amd import engine, pllm_python as P
+    pt = P.PipelineType.LOCAL
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=4)
+    T, nano1 = 96, 40
+    dl = [5, 17, 33, 64, 20]
+    ba = synth.make_batch(dl, [(0, 30), (0, 21)], vocab=shape.vocab, seed=41, extra_pages=8)   # row 39 belongs to request 6
+    bb = synth.make_batch(dl, [(0, 40), (0, 11)], vocab=shape.vocab, seed=41, extra_pages=8)   # row 39 belongs to request 5
+    assert (ba.decodePrefillBorder, ba.prefillNum, ba.prefillTokensNum) == (bb.decodePrefillBorder, bb.prefillNum, bb.prefillTokensNum)
+    assert ba.rev_input_indptr[nano1 - 1] != bb.rev_input_indptr[nano1 - 1]
+    pages = max(ba.num_pages, bb.num_pages)
+    rng = np.random.default_rng(9)
+    pools0 = [synth.make_kv_pool(pages, shape, rng) for _ in range(shape.layers)]
+    order = [ba, ba, ba, bb, bb, bb, ba, bb]
+
+    def run_sequence(graph):
+        outs = []
+        with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=20, kqv3=28, kv_pages=pages,
+                           weights=w, kv_pools=pools0) as e:
+            P.setGraphMode(graph)
+            for i, b in enumerate(order):
+                print(f"border-request graph={graph} step={i}", flush=True)
+                e.update(b, keep_token_list=np.ones(b.decodePrefillBorder, np.int32) if i == 0
+                         else np.array([1] * 5 + [0, 0], np.int32))
+                s = e.run()
+                outs.append((s.copy(), e.buffer("hidden").cpu().numpy()[:b.tokens]))
+            counters = P.getGraphCounters()
+            P.setGraphMode(False)
+        return outs, counters
+
+    eager, _ = run_sequence(False)
+    replay, c1 = run_sequence(True)
+    assert c1["captured"] == 2 and c1["eager"] == 2 and c1["replayed"] == len(order) - 4, c1
     for i, ((s0, h0), (s1, h1)) in enumerate(zip(eager, replay)):
         assert np.array_equal(s0, s1), (i, "sampled ids")
         assert np.array_equal(h0, h1), (i, "residual stream")
