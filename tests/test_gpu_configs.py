@@ -95,8 +95,11 @@ def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines, weight_format="f
                         continue                       # the residual operand of a deeper model is gone by now
                     got = hid if name == "hidden" else inter[name]
                     err = _max_rel(got, ref)
-                    print(f"  teacher-forced {name}: max-norm relative error {err:.2e} (bound {tol:.0e})", flush=True)
-                    assert err < tol, (pt, name, err, tol)
+                    # the gate/up pair's output is the product of two GEMM outputs (silu(g) * u), each
+                    # within the fp8 bound of its definition: the bound of the product is twice that
+                    bound = 2 * tol if name == "act" and tol > 2e-3 else tol
+                    print(f"  teacher-forced {name}: max-norm relative error {err:.2e} (bound {bound:.0e})", flush=True)
+                    assert err < bound, (pt, name, err, bound)
             # (2) free-running: the same arithmetic in the oracle end to end (rows re-quantised per
             # GEMM).  Re-quantisation makes the layer discontinuous, so two correct implementations
             # agree statistically here, not to fp16 rounding: nudging the oracle's norm weights by
