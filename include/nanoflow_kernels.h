@@ -84,6 +84,21 @@ NF_API size_t nf_gemm_workspace_bytes_upto(int max_M, int N, int K);
 NF_API int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
                           float alpha, float beta, int b_col_major, void* workspace, size_t workspace_bytes,
                           nf_stream_t stream);
+/* nf_gemm_f16_ws for callers that cannot allocate or pass a workspace (code under hipGraph
+ * capture, serving loops and harnesses that forbid hipMalloc): the partial sums of a launch split
+ * over K go to a static device array inside the library, nf_gemm_noalloc_scratch_bytes() = 32 MiB,
+ * which every device the library runs on holds until the process ends.  Calls no hipMalloc / hipFree
+ * or any allocating routine; the first call on a device looks up the array's address
+ * (hipGetSymbolAddress), so make that call outside a capture.  A shape whose split needs more than
+ * the array holds is rejected (NF_ERR_INVALID_ARGUMENT, nothing launched); shapes that are not
+ * split run as nf_gemm_f16 and never touch the array.  Nothing in the array has to start at zero
+ * (every share overwrites its sums before the reduction reads them), but all calls on one device
+ * share it: calls that overlap in time on one device (two streams) race.
+ * Results are bit-identical to nf_gemm_f16_ws with a workspace of nf_gemm_workspace_bytes().
+ * No counterpart in the reference. */
+NF_API int nf_gemm_f16_noalloc(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
+                               int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
+NF_API size_t nf_gemm_noalloc_scratch_bytes(void);
 /* the same for the fused gate/up pair: both products are split, their fp32 sums rounded to fp16 and
  * put through SiLU-mul by the reduction (workspace: nf_dual_swiglu_workspace_bytes(M, N, K)) */
 NF_API size_t nf_dual_swiglu_workspace_bytes(int M, int N, int K);

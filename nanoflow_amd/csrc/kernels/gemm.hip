@@ -797,6 +797,33 @@ static int dual_ws_entry(const char* who, const uint16_t* A, const uint16_t* Bga
   return launch_splitk<E, 128, 128, 2, 2, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
 }
 
+// ---- the entry point that allocates nothing: split-K partial sums in a static device array.
+// In host code the array's name is only a stand-in for the symbol; its device address is looked
+// up once per device (each device holds its own copy) and only that address is handed to kernels.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices] = {};  // benign race: every caller stores the same address
+
+static int static_scratch(const char* who, void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("%s: cannot tell the current device", who);
+    return NF_ERR_RUNTIME;
+  }
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      set_error("%s: hipGetSymbolAddress(scratch) on device %d: %s", who, dev, hipGetErrorString(e));
+      return NF_ERR_RUNTIME;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return NF_OK;
+}
+
 extern "C" {
 
 int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
@@ -841,6 +868,24 @@ int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint
   return gemm_ws_entry<F16>("nf_gemm_f16_ws", A, B, C, D, M, N, K, alpha, beta, b_col_major, workspace,
                             workspace_bytes, stream);
 }
+
+int nf_gemm_f16_noalloc(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
+                        float alpha, float beta, int b_col_major, nf_stream_t stream) {
+  const size_t need = nf_gemm_workspace_bytes(M, N, K);
+  NF_REQUIRE(need <= kStaticScratchBytes,
+             "nf_gemm_f16_noalloc: %d x %d x %d is split over K through %zu bytes of partial sums; the static "
+             "scratch array holds %zu (use nf_gemm_f16_ws with a workspace of your own, or nf_gemm_f16)",
+             M, N, K, need, kStaticScratchBytes);
+  void* ws = nullptr;
+  if (need) {  // shapes that are not split never touch the array
+    const int rc = static_scratch("nf_gemm_f16_noalloc", &ws);
+    if (rc) return rc;
+  }
+  return gemm_ws_entry<F16>("nf_gemm_f16_noalloc", A, B, C, D, M, N, K, alpha, beta, b_col_major, ws,
+                            need ? kStaticScratchBytes : 0, stream);
+}
+
+size_t nf_gemm_noalloc_scratch_bytes(void) { return kStaticScratchBytes; }
 
 int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M, int N,
                         int K, float alpha, float beta, int b_col_major, void* workspace, size_t workspace_bytes,

@@ -25,6 +25,7 @@ SYMBOLS = [
     "nf_gemm_f8w_f16", "nf_rope_append_f16", "nf_attention_workspace_bytes",
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
     "nf_calibrate_mfma", "nf_calibrate_hbm_read", "nf_calibrate_paged_read",
+    "nf_gemm_f16_noalloc", "nf_gemm_noalloc_scratch_bytes",
 ]
 
 
@@ -79,6 +80,9 @@ def lib() -> C.CDLL:
         l.nf_dual_swiglu_f8w_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, C.c_size_t, vp]
         l.nf_move_kv_pages.argtypes = [i32, vp, vp, vp, vp, vp, sz, i32, vp]
         l.nf_rope_append_f16.argtypes = [vp] * 7 + [i32] * 5 + [f32] * 4 + [vp]
+        l.nf_gemm_f16_noalloc.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
+        l.nf_gemm_noalloc_scratch_bytes.restype = sz
+        l.nf_gemm_noalloc_scratch_bytes.argtypes = []
         dp = C.POINTER(C.c_double)
         l.nf_calibrate_mfma.argtypes = [i32, i32, i32, vp, sz, dp, dp, vp]
         l.nf_calibrate_hbm_read.argtypes = [vp, sz, i32, vp, sz, dp, vp]
