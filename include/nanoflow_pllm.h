@@ -131,6 +131,13 @@ NF_PLLM_API int pllm_model_weight_to_gpu(const nf_vortex_model_weight* host_weig
  * freed.  layers must have room for the model's layer count; *weight points at it. */
 NF_PLLM_API int pllm_create_model_weight(nf_vortex_model_weight* weight, nf_vortex_layer_weight* layers,
                                          int layers_capacity);
+/* createModelWeightCPU (vortexData.cu:375-384), which is what the reference's Python module exports
+ * as createModelWeight (pybind.cu:281): HOST memory for every weight of the configured model
+ * (zero-filled, never freed), to be uploaded by pllm_model_weight_to_gpu as pllm_python.init does. */
+NF_PLLM_API int pllm_create_model_weight_host(nf_vortex_model_weight* weight, nf_vortex_layer_weight* layers,
+                                              int layers_capacity);
+/* Layers of the configured model (0 before pllm_set_model_config): the capacity the builders ask for. */
+NF_PLLM_API int pllm_num_layers(void);
 /* pllm_python.createInitData (pybind.cu:229, vortexData.cu:33-56): the tmp buffer and one zeroed
  * KV pool per layer for the configured model (never freed) around the given weights.  kv_data
  * must have room for the model's layer count. */

@@ -156,6 +156,21 @@ int pllm_create_model_weight(nf_vortex_model_weight* weight, nf_vortex_layer_wei
   return NF_PLLM_OK;
 }
 
+int pllm_create_model_weight_host(nf_vortex_model_weight* weight, nf_vortex_layer_weight* layers,
+                                  int layers_capacity) {
+  if (!g_config_loaded)
+    return fail(NF_PLLM_ERR_STATE, "pllm_create_model_weight_host: call pllm_set_model_config first");
+  if (!weight || !layers || layers_capacity < ModelConfig.model_layer)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_create_model_weight_host: room for %d layers needed",
+                ModelConfig.model_layer);
+  vortexModelWeight h;
+  createModelWeightCPU(h, 0);
+  layers_to_c(h, weight, layers);
+  return NF_PLLM_OK;
+}
+
+int pllm_num_layers(void) { return g_config_loaded ? ModelConfig.model_layer : 0; }
+
 int pllm_create_init_data(nf_vortex_init_data* data, uint16_t** kv_data, int layers_capacity,
                           const nf_vortex_model_weight* weight) {
   if (!g_config_loaded) return fail(NF_PLLM_ERR_STATE, "pllm_create_init_data: call pllm_set_model_config first");

@@ -75,3 +75,30 @@ def test_split_over_k_plan_without_a_gpu():
     dual = lambda M, N, K: l.nf_dual_swiglu_workspace_bytes(M, N, K) // (2 * M * N * 4)
     assert dual(64, 14336, 4096) == 2 and dual(64, 28672, 8192) == 0 and dual(256, 14336, 4096) == 0
     assert l.nf_gemm_f8w_workspace_bytes(2048, 4096) == 2048 * 4096 + 2048 * 4
+
+
+def test_extension_module_imports_without_a_gpu_and_has_the_reference_names():
+    """nanoflow_amd/ext/pllm_python.*.so (pybind11 over the control-plane C ABI): the reference's
+    module surface (pipeline/src/pybind.cu:189-284), importable with no device present."""
+    import importlib.util
+    ext = os.path.join(ROOT, "nanoflow_amd", "ext")
+    files = [f for f in os.listdir(ext) if f.startswith("pllm_python.") and f.endswith(".so")] if os.path.isdir(ext) else []
+    assert files, "extension module missing: run __graft_entry__.build()"
+    spec = importlib.util.spec_from_file_location("pllm_python", os.path.join(ext, files[0]))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    for name in ("init", "config", "update", "run", "run_async", "run_async_wait", "finalize", "getPipelineOutput",
+                 "setRank", "setModelConfig", "createModelWeight", "createInitData", "VortexInitData",
+                 "VortexUpdateData", "VortexConfigData", "VortexWeight", "VortexLayerWeight", "VortexModelWeight",
+                 "VortexOutputData", "PipelineType"):
+        assert hasattr(mod, name), name
+    u = mod.VortexUpdateData()
+    u.decodePrefillBorder = 7
+    u.setKVIndices(0)
+    u.setGemvBatchSize(__import__("numpy").array([1, 2, 3, 4], dtype="int32"))
+    assert u.decodePrefillBorder == 7
+    c = mod.VortexConfigData()
+    c.setGemmOpTag(["a", "b"])
+    assert c.gemmOpTag == ["a", "b"]
+    with pytest.raises(RuntimeError):
+        mod.setRank(2, 2)              # one rank only
