@@ -78,6 +78,8 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restric
 //     chunk c at c ^ (r & 15) (16-byte A-operand reads), V row r keeps chunk c at
 //     c ^ ((r & 7) << 1) and is read with the transposing LDS read (ds_read_b64_tr_b16), which
 //     hands each lane 4 consecutive keys of one feature: the V^T operand with no permutes.
+//   * The loads carry the non-temporal hint: every K and V byte is read once per launch, and
+//     without the hint the same pattern streams 10 % slower.
 //   * A page is addressed through its own buffer descriptor (base = page, 64 KiB range), so
 //     pools larger than 4 GiB need no 64-bit per-lane arithmetic and out-of-page offsets
 //     (used to zero-fill V rows past the end of the sequence) read as zero.
@@ -162,9 +164,9 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
         const rsrc_t ra = page_rsrc(2 * pp), rb = page_rsrc(2 * pp + 1);
         const uint32_t dst = wlds + buf * 8192;
 #pragma unroll
-        for (int t4 = 0; t4 < 4; ++t4) load16_to_lds(ra, k_src[t4], dst + t4 * 1024);
+        for (int t4 = 0; t4 < 4; ++t4) load16_to_lds_nt(ra, k_src[t4], dst + t4 * 1024);
 #pragma unroll
-        for (int t4 = 0; t4 < 4; ++t4) load16_to_lds(rb, k_src[t4], dst + 4096 + t4 * 1024);
+        for (int t4 = 0; t4 < 4; ++t4) load16_to_lds_nt(rb, k_src[t4], dst + 4096 + t4 * 1024);
       };
       auto dma_v = [&](int pp, int buf) {
         const rsrc_t ra = page_rsrc(2 * pp), rb = page_rsrc(2 * pp + 1);
@@ -173,10 +175,10 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
         const int first_key = pp * 32 + (lane >> 4);
 #pragma unroll
         for (int t4 = 0; t4 < 4; ++t4)
-          load16_to_lds(ra, first_key + 4 * t4 < kv_len ? v_src[t4] : kOob, dst + t4 * 1024);
+          load16_to_lds_nt(ra, first_key + 4 * t4 < kv_len ? v_src[t4] : kOob, dst + t4 * 1024);
 #pragma unroll
         for (int t4 = 0; t4 < 4; ++t4)
-          load16_to_lds(rb, first_key + 16 + 4 * t4 < kv_len ? v_src[t4] : kOob, dst + 4096 + t4 * 1024);
+          load16_to_lds_nt(rb, first_key + 16 + 4 * t4 < kv_len ? v_src[t4] : kOob, dst + 4096 + t4 * 1024);
       };
       // vmcnt(n): everything but the n youngest load instructions of this wavefront has landed
       auto wait_but = [&](int younger) {

@@ -107,8 +107,8 @@ __global__ __launch_bounds__(256) void calib_hbm_read_kernel(const rsrc_t* __res
 
 // Paged decode attention's traffic without its arithmetic.  Workgroup = (request, kv head), head
 // fastest; 2 wavefronts take alternate 32-key steps; a step pulls 32 K rows and 32 V rows of
-// 256 bytes (two pages each) straight into the wavefront's LDS ring of 2 K + 2 V tiles, and waits
-// only for the tile it is about to reuse.
+// 256 bytes (two pages each) straight into the wavefront's LDS ring of 2 K + 2 V tiles (non-temporal
+// loads, as the attention kernel issues them), and waits only for the tile it is about to reuse.
 __global__ __launch_bounds__(128) void calib_paged_read_kernel(const uint16_t* __restrict__ pool,
                                                                const int32_t* __restrict__ kv_indptr,
                                                                const int32_t* __restrict__ kv_indices,
@@ -139,7 +139,7 @@ __global__ __launch_bounds__(128) void calib_paged_read_kernel(const uint16_t* _
       for (int kv = 0; kv < 2; ++kv)
 #pragma unroll
         for (int t = 0; t < 4; ++t)  // 4 rows per instruction, 16 rows per page
-          load16_to_lds(rk, (uint32_t)kv * 16u * row_stride + (uint32_t)t * 4u * row_stride + lane_off,
+          load16_to_lds_nt(rk, (uint32_t)kv * 16u * row_stride + (uint32_t)t * 4u * row_stride + lane_off,
                         lds + (uint32_t)(kv * 2 + slot) * 8192u + (uint32_t)(half * 4 + t) * 1024u);
     }
   }
