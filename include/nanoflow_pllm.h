@@ -28,13 +28,19 @@ extern "C" {
 #define NF_PLLM_OK 0
 #define NF_PLLM_ERR_INVALID_ARGUMENT (-1)
 #define NF_PLLM_ERR_STATE (-2)       /* call out of order (e.g. update before config) */
-#define NF_PLLM_ERR_UNSUPPORTED (-3) /* tensor-parallel pipeline types, more than one rank */
+#define NF_PLLM_ERR_UNSUPPORTED (-3) /* more than one rank, a model shape the kernels are not built for */
 
 /* Worker::PipelineType (pipeline/include/computeBound.cuh:22-34). */
 enum nf_pipeline_type {
+  /* The reference's main Pipeline (pipeline/src/pipeline.cu): QKV projection, RoPE-append and
+   * decode attention as four nano-batches (sizes kqv1, nano1 - kqv1, kqv3, T - nano1 - kqv3), O and
+   * the FFN as two, attention on a stream of its own; on this one rank without its exchange steps. */
   NF_PIPE_PLLM = 0,
-  NF_PIPE_NONOVERLAP = 1,
-  NF_PIPE_NANOBATCH = 2,
+  NF_PIPE_NONOVERLAP = 1,  /* its sequential schedule: runs as NON_OVERLAP_LOCAL */
+  NF_PIPE_NANOBATCH = 2,   /* PLLM's nano-batches on one stream */
+  /* PLLM plus the KV offload round trip of pipeline.cu:37-59,701-726: every layer the pages of the
+   * iteration's first two requests are gathered, copied to pinned host memory, copied back and
+   * scattered into the pool again (results are PLLM's). */
   NF_PIPE_PLLMOFFLOAD = 3,
   /* models with a bias on the q/k/v projections (Qwen2; pipeline/src/computeBound.cu:234-242):
    * on this one device they run as LOCAL / NON_OVERLAP_LOCAL / NANOBATCH_LOCAL with
@@ -285,7 +291,8 @@ NF_PLLM_API int pllm_get_graph_counters(long counters[3]);
 NF_PLLM_API int pllm_reset_timings(void);
 /* Device address of an intermediate of the current pipeline, for parity checks:
  * name in {"hidden" (residual stream after the last layer, [T, hidden]),
- *          "logits" ([T, vocab])}; for the non-overlap pipeline also the last layer's operator
+ *          "logits" ([T, vocab])}; for PLLMOFFLOAD also "offload_host" (PINNED HOST memory,
+ *          [pages moved, halves per page]: what the last layer's offload round trip left); for the non-overlap pipeline also the last layer's operator
  *          inputs and outputs: "ln_attn" (QKV input), "kqv", "attn_out" (O input), "o_out",
  *          "ln_ffn" (gate/up input), "act" (down input). */
 NF_PLLM_API int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols);

@@ -68,8 +68,8 @@ int main(int argc, char** argv) {
     return 2;
   }
   if (nranks != 1 || vnranks != 1 || !Worker::isSupported(pipe)) {
-    std::fprintf(stderr, "this build runs LOCAL, NON_OVERLAP_LOCAL, NANOBATCH_LOCAL and the three *_KQVBIAS "
-                         "types on one GPU (got %s, %d ranks, gpu_num %d)\n", pipe_name.c_str(), nranks, vnranks);
+    std::fprintf(stderr, "this build runs every pipeline type on ONE GPU (got %s, %d ranks, gpu_num %d)\n",
+                 pipe_name.c_str(), nranks, vnranks);
     return 2;
   }
 

@@ -64,10 +64,7 @@ void init(int nranks, int vnranks, std::vector<vortexInitData>& input,
     std::exit(EXIT_FAILURE);
   }
   if (!Worker::isSupported(pipeTy)) {
-    std::fprintf(stderr,
-                 "init: pipeline type %d is the offload pipeline, whose host and SSD tiers this build does not "
-                 "have; every other type runs (the tensor-parallel ones as their one-device schedules)\n",
-                 static_cast<int>(pipeTy));
+    std::fprintf(stderr, "init: unknown pipeline type %d\n", static_cast<int>(pipeTy));
     std::exit(EXIT_FAILURE);
   }
   if (!workers.empty()) {
@@ -168,20 +165,19 @@ void Worker::as_thread(int core) {
 
 void Worker::init() {
   HIP_CHECK(hipSetDevice(rank));
-  // The *_KQVBIAS types name the tensor-parallel pipelines with a QKV bias
-  // (pipeline/src/computeBound.cu:234-242); on one device, with no exchange steps left, they are
-  // the local schedules with the bias switched on.
-  // So are PLLM, NANOBATCH and NONOVERLAP without the bias.
-  const bool nanobatch_only = PipeTy == PipelineType::NANOBATCH_LOCAL || PipeTy == PipelineType::NANOBATCH;
-  if (PipeTy == PipelineType::LOCAL || PipeTy == PipelineType::PLLM || nanobatch_only)
-    pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks, nanobatch_only);
-  else if (PipeTy == PipelineType::NON_OVERLAP_LOCAL || PipeTy == PipelineType::NONOVERLAP)
-    pipeline = std::make_unique<NonOverlapLocalPipeline>(input, rank, nranks, vnranks);
-  else if ((PipeTy == PipelineType::KQVBIAS || PipeTy == PipelineType::NANOBATCH_KQVBIAS) && nranks == 1)
-    pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks,
-                                               PipeTy == PipelineType::NANOBATCH_KQVBIAS, true);
-  else if (PipeTy == PipelineType::NONOVERLAP_KQVBIAS && nranks == 1)
-    pipeline = std::make_unique<NonOverlapLocalPipeline>(input, rank, nranks, vnranks, true);
+  // Type -> schedule as the reference maps them (pipeline/src/computeBound.cu:234-247): the five
+  // types of its main Pipeline run the four-way nano-batch schedule, without their exchange steps.
+  const bool bias = hasKQVBias(PipeTy);
+  if (PipeTy == PipelineType::PLLM || PipeTy == PipelineType::PLLMOFFLOAD || PipeTy == PipelineType::NANOBATCH ||
+      PipeTy == PipelineType::KQVBIAS || PipeTy == PipelineType::NANOBATCH_KQVBIAS)
+    pipeline = std::make_unique<Pipeline>(input, rank, nranks, vnranks, PipeTy == PipelineType::PLLMOFFLOAD,
+                                          PipeTy == PipelineType::NANOBATCH || PipeTy == PipelineType::NANOBATCH_KQVBIAS,
+                                          bias);
+  else if (PipeTy == PipelineType::NONOVERLAP || PipeTy == PipelineType::NONOVERLAP_KQVBIAS ||
+           PipeTy == PipelineType::NON_OVERLAP_LOCAL)
+    pipeline = std::make_unique<NonOverlapLocalPipeline>(input, rank, nranks, vnranks, bias);
+  else if (PipeTy == PipelineType::LOCAL || PipeTy == PipelineType::NANOBATCH_LOCAL)
+    pipeline = std::make_unique<LocalPipeline>(input, rank, nranks, vnranks, PipeTy == PipelineType::NANOBATCH_LOCAL);
   else
     NF_LOG_ERROR("Unknown pipeline type %d", static_cast<int>(PipeTy));
   if (pipeline && g_profiling) pipeline->setProfiling(g_profiling);

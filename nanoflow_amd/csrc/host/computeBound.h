@@ -59,12 +59,12 @@ public:
     NANOBATCH_LOCAL,
   };
   static PipelineType PipeTy;
-  // Everything but the offload pipeline.  PLLM, NONOVERLAP and NANOBATCH name the tensor-parallel
-  // schedules (pipeline/src/computeBound.cu:225-233); on the one rank of this build their exchange
-  // steps move nothing, and they run as LOCAL, NON_OVERLAP_LOCAL and NANOBATCH_LOCAL, so that the
-  // reference's multi-GPU pipeline files serve here once their gpu_num is 1.
-  static bool isSupported(PipelineType t) { return t != PipelineType::PLLMOFFLOAD; }
-  // the three bias types run as the local schedules with the QKV bias switched on
+  // Every type runs on the one rank of this build.  PLLM, NANOBATCH, PLLMOFFLOAD and the two
+  // nano-batched bias types are the reference's main Pipeline (four QKV / attention nano-batches)
+  // without its exchange steps, NONOVERLAP its sequential schedule, so that the reference's multi-GPU
+  // pipeline files serve here once their gpu_num is 1.
+  static bool isSupported(PipelineType t) { return static_cast<int>(t) >= 0 && static_cast<int>(t) <= 9; }
+  // the QKV GEMMs add vortexLayerWeight::B_KQV
   static bool hasKQVBias(PipelineType t) {
     return t == PipelineType::KQVBIAS || t == PipelineType::NONOVERLAP_KQVBIAS ||
            t == PipelineType::NANOBATCH_KQVBIAS;

@@ -6,7 +6,13 @@
 //   NonOverlapLocalPipeline   same math on one stream, no nano-batching
 //                             (pipeline/include/pipeline.h:405-465,
 //                              pipeline/src/pipeline_nonoverlap_local.cu)
-// The tensor-parallel pipelines of the reference are outside this build.
+//   Pipeline                  the reference's main schedule (pipeline/include/pipeline.h:53-170,
+//                             pipeline/src/pipeline.cu) on one device: the QKV projection, RoPE-append
+//                             and decode attention run as FOUR nano-batches, O / FFN as two; its
+//                             all-gather / all-reduce steps have nothing to move on one rank and are
+//                             left out.  With enable_offload it also round-trips KV pages through host
+//                             memory every layer (pipeline.cu:37-59,701-726).
+// More than one rank (the collectives) is outside this build.
 #pragma once
 #include <array>
 #include <memory>
@@ -292,6 +298,90 @@ public:
 
 private:
   double totalCompute();
+};
+
+class Pipeline : public PipelineBase {
+public:
+  enum class GEMM_NAME { O1 = 0, O2, D1, D2, KQV1, KQV2, KQV3, KQV4, LOGITS, NUM };
+  static constexpr std::array gemmConfig = {
+      "128_128_32_64_64_32_3_5_RowMajor_RowMajor_RowMajor",  // O1
+      "128_128_32_64_64_32_1_4_RowMajor_RowMajor_RowMajor",  // O2
+      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // D1
+      "128_128_32_64_64_32_1_4_RowMajor_RowMajor_RowMajor",  // D2
+      "128_64_64_64_32_64_2_3_RowMajor_RowMajor_RowMajor",   // KQV1
+      "128_128_32_64_64_32_2_5_RowMajor_RowMajor_RowMajor",  // KQV2
+      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV3
+      "128_64_64_64_32_64_2_3_RowMajor_RowMajor_RowMajor",   // KQV4
+      "128_256_32_64_64_32_2_3_RowMajor_RowMajor_RowMajor",  // LOGITS
+  };
+  static constexpr int gemmNum = static_cast<int>(GEMM_NAME::NUM);
+  std::array<BaseGEMMWrapper*, gemmNum> gemms{};
+  GEMM_ALIAS(O1);
+  GEMM_ALIAS(O2);
+  GEMM_ALIAS(D1);
+  GEMM_ALIAS(D2);
+  GEMM_ALIAS(KQV1);
+  GEMM_ALIAS(KQV2);
+  GEMM_ALIAS(KQV3);
+  GEMM_ALIAS(KQV4);
+  GEMM_ALIAS(LOGITS);
+
+  DualWrapper dual1, dual2;
+  GenEmbedding genEmbedding1, genEmbedding2_1, genEmbedding2_2;
+  DecodeGemvWrapper GEMV1, GEMV2, GEMV3, GEMV4;
+  std::array<DecodeGemvWrapper*, 4> gemvs{&GEMV1, &GEMV2, &GEMV3, &GEMV4};
+  PrefillGemvWrapper prefill;
+  LayerNorm layerNormAttention1, layerNormAttention2_1, layerNormAttention2_2;
+  LayerNorm layerNormFFN1, layerNormFFN2;
+  LayerNorm layerNormModel1;
+  BaseGEMMWrapper* KQV_ptrs[4] = {nullptr, nullptr, nullptr, nullptr};
+  RoPEAppend roPEAppends[4];
+  PageAggregator pageAgg;
+  PageDispatcher pageDisp;
+  MaxSampling maxSampler;
+  KeepToken keepToken;
+
+  pllmTensor<half> gemvQ, gemvAggregateOutput, KQV_output;
+  vortexOutputData output_data;
+  hipStream_t stream_gemm = nullptr, stream_gemv = nullptr, stream_cpy = nullptr;
+  int update_token_num = 0;
+  bool enable_offload = false;
+  bool nanobatch_only = false;
+
+  // KV offload round trip (enable_offload): the pages of the iteration's first offload_reqs
+  // requests are gathered from the layer's pool into deviceOffloadKVCache, copied to the pinned
+  // host buffer offloadKVCache, copied back into deviceLoadKVCache and scattered into the pages
+  // the requests own -- the data path of evicting and re-admitting a request, paid every layer
+  // as in the reference (whose lists and copy sizes are fixed constants: a cost model).
+  static constexpr int kOffloadReqs = 2;
+  half* offloadKVCache = nullptr;        // pinned host
+  half* deviceOffloadKVCache = nullptr;  // device staging, laid out like kv_indices
+  half* deviceLoadKVCache = nullptr;
+  int32_t* finished_idx = nullptr;       // device: 0, 1, 2, ...
+  int32_t* load_idx = nullptr;
+  size_t offload_pages_cap = 0;          // pages the staging buffers hold
+  size_t offload_pages = 0;              // pages moved per layer in this iteration
+  int offload_reqs = 0;
+  hipEvent_t offload_done = nullptr;
+
+  Pipeline(vortexInitData* input_data, int nrank, int nranks, int vnranks, bool enable_offload = false,
+           bool nanobatch_only = false, bool kqv_bias = false);
+  ~Pipeline() override;
+  void ScheduleInit();
+  void GEMMOpInit();
+  void GEMVOpInit();
+  void OtherOpInit();
+  void setWeight(int layer);
+  vortexOutputData run() override;
+  void update(vortexUpdateData* update_data) override;
+  void config(vortexConfigData* config_data) override;
+  void GEMVOpUpdate();
+  void setName() override;
+  hipStream_t uploadStream() override { return stream_gemm; }
+  void setProfiling(int level) override;
+
+private:
+  void enqueueIteration();
 };
 
 // Creates a stream restricted to `num_cus` compute units starting at CU `first_cu` of every

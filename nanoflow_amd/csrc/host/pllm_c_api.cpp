@@ -91,12 +91,7 @@ int pllm_init(const nf_vortex_init_data* input, int pipeline_type) {
   if (pipeline_type < 0 || pipeline_type > NF_PIPE_NANOBATCH_LOCAL)
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_init: unknown pipeline type %d", pipeline_type);
   auto ty = static_cast<Worker::PipelineType>(pipeline_type);
-  if (!Worker::isSupported(ty))
-    return fail(NF_PLLM_ERR_UNSUPPORTED,
-                "pllm_init: pipeline type %d is the offload pipeline, whose host and SSD tiers are not "
-                "built; every other type runs (PLLM(0), NONOVERLAP(1), NANOBATCH(2) as LOCAL(7), "
-                "NON_OVERLAP_LOCAL(8), NANOBATCH_LOCAL(9); the *_KQVBIAS types as those with a QKV bias)",
-                pipeline_type);
+  if (!Worker::isSupported(ty)) return fail(NF_PLLM_ERR_UNSUPPORTED, "pllm_init: unknown pipeline type %d", pipeline_type);
   if (getWeightFormat() == WeightFormat::E4M3 && Worker::hasKQVBias(ty))
     return fail(NF_PLLM_ERR_UNSUPPORTED, "pllm_init: the QKV bias pipelines take fp16 weights only");
   if (input->weight.num_layers < ModelConfig.model_layer)
@@ -429,6 +424,11 @@ int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols) {
   if (auto* lp = dynamic_cast<LocalPipeline*>(p)) {
     if (!std::strcmp(name, "hidden")) t = lp->keepToken.input;
     else if (!std::strcmp(name, "logits")) t = lp->maxSampler.d_matrix;
+  } else if (auto* pp = dynamic_cast<Pipeline*>(p)) {
+    if (!std::strcmp(name, "hidden")) t = pp->keepToken.input;
+    else if (!std::strcmp(name, "logits")) t = pp->maxSampler.d_matrix;
+    else if (!std::strcmp(name, "offload_host") && pp->offloadKVCache)  // pinned host memory: what the last layer's round trip left
+      t = pllmTensor<half>(pp->offloadKVCache, pp->offload_pages, ModelConfig.page_mem_size / sizeof(half), PllmLayout::ROW_MAJOR);
   } else if (auto* np = dynamic_cast<NonOverlapLocalPipeline*>(p)) {
     // the intermediates hold the LAST layer's values once an iteration has run
     if (!std::strcmp(name, "hidden")) t = np->keepToken.input;

@@ -77,7 +77,7 @@ class Engine:
         self.dev = torch.device("cuda:0")
         fd, self.cfg_path = tempfile.mkstemp(suffix=".json", prefix="nanoflow_cfg_")
         os.close(fd)
-        n_tags = 4 if pipeline_type.is_sequential else 7
+        n_tags = pipeline_type.gemm_tags
         write_config(self.cfg_path, shape, global_batch=global_batch, nano1=nano1, kqv1=self.kqv1,
                      kqv3=self.kqv3, pipeline_type=pipeline_type, kv_pages=kv_pages,
                      run_layer=run_layer, distinct_layers=distinct_layers, n_tags=n_tags)
@@ -216,7 +216,7 @@ class Engine:
         import ctypes as C
         hip = C.CDLL("libamdhip64.so")
         rc = hip.hipMemcpy(C.c_void_p(out.data_ptr()), C.c_void_p(ptr), C.c_size_t(rows * cols * 2),
-                           C.c_int(3))  # hipMemcpyDeviceToDevice
+                           C.c_int(4))  # hipMemcpyDefault: the source may be device or pinned host memory
         if rc != 0:
             raise RuntimeError(f"hipMemcpy failed: {rc}")
         return out

@@ -8,6 +8,10 @@
     python -m nanoflow_amd.kernel_bench --op attn --requests 1792 --kv-lo 1024 --kv-hi 1536
     python -m nanoflow_amd.kernel_bench --op prefill --chunks 755:269,0:1024,0:74
     python -m nanoflow_amd.kernel_bench --op copy                     # counter-calibration kernel
+    python -m nanoflow_amd.kernel_bench --op calibrate                # measured MFMA / HBM / paged-read ceilings
+    python -m nanoflow_amd.kernel_bench --op blas --m 2048            # the same GEMM shapes through torch.matmul (hipBLASLt / rocBLAS)
+    python -m nanoflow_amd.kernel_bench --op corun                    # GEMM and decode attention alone and together: time and board power
+    python -m nanoflow_amd.kernel_bench --op cusplit                  # the same pair on CU-masked streams (whole XCDs each)
 
 Each line reports the average launch time over --iters launches (HIP events on the launch
 stream) and the algorithmic rate: 2*M*N*K flops (4*M*N*K for the fused gate/up pair), or the
@@ -47,9 +51,122 @@ def layer_shapes(shape: synth.ModelShape, M: int):
             ("down", M, shape.hidden, shape.ffn), ("lm_head", (M + 127) // 128 * 128, shape.vocab, shape.hidden)]
 
 
+class PowerSampler:
+    """Board power from the amdgpu hwmon file (microwatts), sampled every 50 ms on a thread."""
+
+    def __init__(self):
+        import glob, threading
+        self.paths = [p for d in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")
+                      for p in (os.path.join(d, "power1_input"), os.path.join(d, "power1_average")) if os.path.exists(p)]
+        self.samples, self.stop = [], False
+        self.thread = threading.Thread(target=self._run, daemon=True)
+        self.thread.start()
+
+    def _run(self):
+        import time
+        while not self.stop:
+            try:
+                w = max(int(open(p).read()) / 1e6 for p in self.paths)
+            except (OSError, ValueError):
+                w = float("nan")
+            self.samples.append((time.perf_counter(), w))
+            time.sleep(0.05)
+
+    def mean(self, t0, t1):
+        v = [w for t, w in self.samples if t0 <= t <= t1 and w == w]
+        return sum(v) / len(v) if v else float("nan")
+
+
+def masked_stream(first_xcd: int, n_xcd: int):
+    """A stream restricted to whole XCDs (CU mask word i = XCD i on this part)."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    s = C.c_void_p()
+    mask = (C.c_uint32 * 8)(*[0xFFFFFFFF if first_xcd <= i < first_xcd + n_xcd else 0 for i in range(8)])
+    rc = hip.hipExtStreamCreateWithCUMask(C.byref(s), 8, mask)
+    assert rc == 0, f"hipExtStreamCreateWithCUMask: {rc}"
+    return torch.cuda.ExternalStream(s.value)
+
+
+def corun(a, shape, rnd):
+    """The fused gate/up GEMM (M rows) and decode attention (the offline cycle's request mix), each alone
+    and both at once on two streams: time per pair against the serial sum, and board power."""
+    import time
+    M = a.m
+    A, Bg, Bu = rnd(M, shape.hidden), rnd(shape.hidden, shape.ffn, std=0.02), rnd(shape.hidden, shape.ffn, std=0.02)
+    out = torch.empty(M, shape.ffn, dtype=torch.float16, device=DEV)
+    gemm = lambda: K.dual_swiglu(A, Bg, Bu, out=out)
+    fl = 4.0 * M * shape.ffn * shape.hidden
+    b = synth.config2_batch(seed=0, n_decode=a.requests, lo=a.kv_lo, hi=a.kv_hi, prefill_chunk=16)
+    nd = b.decodePrefillBorder
+    pool = rnd(b.num_pages, 2, shape.page_size, shape.Hkv, shape.d)
+    q = rnd(b.tokens, shape.Hq * shape.d)
+    o = torch.zeros_like(q)
+    t = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(DEV)
+    qi, kvp, kvi, kvl = t(b.input_indptr[:nd + 1]), t(b.kv_indptr[:nd + 1]), t(b.kv_indices), t(b.kv_last_page_len[:nd])
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+    attn = lambda: K.attention_paged(q, qi, pool, kvp, kvi, kvl, shape.Hq, shape.Hkv, causal=False, out=o, batch=nd,
+                                     max_qo_rows=nd, workspace=ws)
+    L = b.kv_len[:nd].astype(np.int64)
+    nb = int((2 * L * shape.Hkv * shape.d * 2).sum())
+    power = PowerSampler()
+
+    def phase(name, fn, note=None, secs=2.5):
+        torch.cuda.synchronize()
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < secs:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            n += 5
+        t1 = time.perf_counter()
+        per = (t1 - t0) / n
+        print(f"{name:44s} {per * 1e6:9.1f} us  board power {power.mean(t0 + 0.5, t1):7.1f} W"
+              + (f"  {note(per)}" if note else ""), flush=True)
+        return per
+
+    time.sleep(1.0)
+    print(f"idle: board power {power.mean(0, time.perf_counter()):7.1f} W", flush=True)
+    tg = phase(f"gate/up GEMM {M}x{shape.ffn}x{shape.hidden} alone", gemm, lambda p: f"{fl / p / 1e12:7.1f} TFLOP/s")
+    ta = phase(f"decode attention {nd} requests alone", attn, lambda p: f"{nb / p / 1e9:7.1f} GB/s")
+    if a.op == "corun":
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        splits = [("both, two unmasked streams", s1, s2)]
+    else:
+        splits = [(f"both, GEMM on {gx} XCDs + attention on {8 - gx} XCDs", masked_stream(0, gx), masked_stream(gx, 8 - gx))
+                  for gx in (6, 5, 4, 3)]
+    for name, sg, sa in splits:
+        def both():
+            with torch.cuda.stream(sg):
+                gemm()
+            with torch.cuda.stream(sa):
+                attn()
+        if a.op == "cusplit":
+            def g_only():
+                with torch.cuda.stream(sg):
+                    gemm()
+            def a_only():
+                with torch.cuda.stream(sa):
+                    attn()
+            phase("  GEMM alone on its XCDs", g_only, lambda p: f"{fl / p / 1e12:7.1f} TFLOP/s", secs=1.5)
+            phase("  attention alone on its XCDs", a_only, lambda p: f"{nb / p / 1e9:7.1f} GB/s", secs=1.5)
+        phase(name, both, lambda p: f"serial sum {(tg + ta) * 1e6:7.1f} us -> x{(tg + ta) / p:.3f}")
+    if a.op == "corun":
+        phase("mfma loop f16, pseudo-random operands", lambda: K.calibrate_mfma(False, True, 2000), secs=2.0)
+        phase("mfma loop f16, zero operands", lambda: K.calibrate_mfma(False, False, 2000), secs=2.0)
+        buf = torch.empty(4 << 30, dtype=torch.uint8, device=DEV).random_()
+        sc = torch.zeros(8192, dtype=torch.uint8, device=DEV)
+        import ctypes as C
+        gb = C.c_double()
+        phase("hbm read stream 4 GiB x 2", lambda: K.lib().nf_calibrate_hbm_read(buf.data_ptr(), buf.numel(), 2, sc.data_ptr(),
+                                                                                 8192, C.byref(gb), None), secs=2.0)
+    power.stop = True
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--op", required=True, choices=["gemm", "dual", "gemm_f8", "dual_f8", "attn", "prefill", "copy"])
+    ap.add_argument("--op", required=True, choices=["gemm", "dual", "gemm_f8", "dual_f8", "attn", "prefill", "copy", "calibrate", "blas",
+                                                  "corun", "cusplit"])
     ap.add_argument("--chunks", default="755:269,0:1024,0:74",
                     help="prefill: prev_len:chunk_len per request (default: a steady-state offline iteration)")
     ap.add_argument("--model", default="8b", choices=["8b", "70b"])
@@ -139,6 +256,40 @@ def main():
         flops = sum(l * (2 * (p + l) - l) * 2 * shape.Hq * shape.d for p, l in chunks)
         print(f"chunked-prefill attention {chunks}: {ms * 1e3:9.1f} us  {flops / ms / 1e9:8.1f} TFLOP/s "
               f"(causal flops of gemv/src/bench_batch_prefill.cu:133-134)", flush=True)
+    elif a.op == "calibrate":
+        for fp8 in (False, True):
+            K.calibrate_mfma(fp8, True, 4000)
+            for rand in (True, False):
+                tf, mhz = K.calibrate_mfma(fp8, rand, 40000)
+                print(f"mfma loop {'fp8 32x32x64' if fp8 else 'f16 32x32x16'} {'pseudo-random' if rand else 'zero':13s} operands: "
+                      f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
+        print(f"hbm read stream, 8 GiB x 4: {K.calibrate_hbm_read(8.0, 4):8.1f} GB/s", flush=True)
+        b = synth.config2_batch(seed=0, n_decode=a.requests, lo=a.kv_lo, hi=a.kv_hi, prefill_chunk=16)
+        nd = b.decodePrefillBorder
+        pool = rnd(b.num_pages, 2, shape.page_size, shape.Hkv, shape.d)
+        t = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(DEV)
+        kvb = int(2 * b.kv_len[:nd].astype(np.int64).sum() * shape.Hkv * shape.d * 2)
+        gbps = K.calibrate_paged_read(pool, t(b.kv_indptr[:nd + 1]), t(b.kv_indices), t(b.kv_last_page_len[:nd]), nd,
+                                      shape.Hkv, kvb, 10)
+        print(f"paged read without arithmetic, {nd} requests KV [{a.kv_lo},{a.kv_hi}]: {gbps:8.1f} GB/s", flush=True)
+    elif a.op == "blas":
+        shapes = layer_shapes(shape, a.m) + [("gate/up (2 GEMMs)", a.m, shape.ffn, shape.hidden)]
+        for name, M, N, Kd in shapes:
+            A = rnd(M, Kd)
+            Bkn, Bnk = rnd(Kd, N, std=0.02), rnd(N, Kd, std=0.02)
+            out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+            reps = 2 if name.startswith("gate") else 1
+            ms_kn = timeit(lambda: [torch.matmul(A, Bkn, out=out) for _ in range(reps)], a.iters, a.warm)
+            ms_nk = timeit(lambda: [torch.matmul(A, Bnk.t(), out=out) for _ in range(reps)], a.iters, a.warm)
+            if name.startswith("gate"):
+                ms_us = timeit(lambda: K.dual_swiglu(A, Bkn, Bkn, out=out), a.iters, a.warm)
+            else:
+                ms_us = timeit(lambda: K.gemm(A, Bkn, out=out), a.iters, a.warm)
+            fl = 2.0 * reps * M * N * Kd
+            print(f"{name:18s} {M}x{N}x{Kd}: torch.matmul [K,N] weights {fl / ms_kn / 1e9:7.1f}  [N,K] weights "
+                  f"{fl / ms_nk / 1e9:7.1f}  this library ([K,N]) {fl / ms_us / 1e9:7.1f} TFLOP/s", flush=True)
+    elif a.op in ("corun", "cusplit"):
+        corun(a, shape, rnd)
     else:
         n = a.mib << 20
         src = torch.empty(n, dtype=torch.uint8, device=DEV).random_(generator=g)

@@ -42,8 +42,7 @@ class PipelineType(enum.IntEnum):
 
     @property
     def has_kqv_bias(self) -> bool:
-        """The three bias types (pipeline/src/computeBound.cu:234-242) run on this one device as
-        LOCAL / NON_OVERLAP_LOCAL / NANOBATCH_LOCAL with B_KQV added by the QKV GEMMs."""
+        """The three bias types (pipeline/src/computeBound.cu:234-242): B_KQV is added by the QKV GEMMs."""
         return self in (PipelineType.KQVBIAS, PipelineType.NONOVERLAP_KQVBIAS, PipelineType.NANOBATCH_KQVBIAS)
 
     @property
@@ -51,10 +50,21 @@ class PipelineType(enum.IntEnum):
         """One stream, no nano-batch split: four GEMM tags, one decode-attention group."""
         return self in (PipelineType.NON_OVERLAP_LOCAL, PipelineType.NONOVERLAP_KQVBIAS, PipelineType.NONOVERLAP)
 
+    @property
+    def is_four_way(self) -> bool:
+        """The reference's main Pipeline: QKV / RoPE-append / decode attention as four nano-batches, nine
+        GEMM tags (O1, O2, D1, D2, KQV1-4, LOGITS)."""
+        return self in (PipelineType.PLLM, PipelineType.NANOBATCH, PipelineType.PLLMOFFLOAD, PipelineType.KQVBIAS,
+                        PipelineType.NANOBATCH_KQVBIAS)
+
+    @property
+    def gemm_tags(self) -> int:
+        return 4 if self.is_sequential else 9 if self.is_four_way else 7
+
 
 # serve_configs.pipeline_type of the reference's pipeline files (pipeline/utils/serve_8B.py:48-59).
-# PLLM, NON_OVERLAP and NANOBATCH, the tensor-parallel schedules, run on this one device as LOCAL,
-# NON_OVERLAP_LOCAL and NANOBATCH_LOCAL; PLLM_OFFLOAD is refused by init.
+# PLLM, NANOBATCH, PLLM_OFFLOAD and the nano-batched bias types run the reference's main schedule (four
+# QKV / attention nano-batches) without its exchange steps; NON_OVERLAP runs as NON_OVERLAP_LOCAL.
 pipeline_map = {
     "LOCAL": PipelineType.LOCAL,
     "PLLM": PipelineType.PLLM,

@@ -12,9 +12,10 @@ reference's pipeline/utils/serve_8B.py:
   tokenizer such rows are rejected.
 * config: the reference's pipeline JSON (pipeline/config_all/llama3-8B/1024.json schema);
   ``serve_configs.pipeline_type`` is one of the reference's names (serve_8B.py:48-59): LOCAL,
-  NON_OVERLAP_LOCAL, NANOBATCH_LOCAL; PLLM, NON_OVERLAP, NANOBATCH (the tensor-parallel schedules, which
-  on this one device run as the three above); for models with a bias on the q/k/v projections (Qwen2)
-  KQVBIAS, NONOVERLAP_KQVBIAS, NANOBATCH_KQVBIAS.  PLLM_OFFLOAD is refused.
+  NON_OVERLAP_LOCAL, NANOBATCH_LOCAL; PLLM, NANOBATCH, PLLM_OFFLOAD (the reference's main schedule with
+  four QKV / attention nano-batches, here without its exchange steps; PLLM_OFFLOAD adds the KV offload
+  round trip), NON_OVERLAP (runs as NON_OVERLAP_LOCAL); for models with a bias on the q/k/v
+  projections (Qwen2) KQVBIAS, NONOVERLAP_KQVBIAS, NANOBATCH_KQVBIAS.
 * ``--empty_weight True``: random-init weights on the device, as the reference's own evaluation
   runs (pipeline/eval/eval-fix-offline/run.py:42-50).  Otherwise the weights come from
   ``serve_configs.weight_path``/weight_rank_0.pt (nanoflow_amd/weights.py; serve_8B.py:611-629);

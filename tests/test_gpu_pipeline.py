@@ -229,8 +229,8 @@ def test_kqv_bias_schedules_match_oracle(oracle, case):
 
     w_zero = dict(w, b_kqv=[np.zeros_like(b) for b in w["b_kqv"]])
     pairs = [(P.PipelineType.NONOVERLAP_KQVBIAS, P.PipelineType.NON_OVERLAP_LOCAL),
-             (P.PipelineType.NANOBATCH_KQVBIAS, P.PipelineType.NANOBATCH_LOCAL),
-             (P.PipelineType.KQVBIAS, P.PipelineType.LOCAL)]
+             (P.PipelineType.NANOBATCH_KQVBIAS, P.PipelineType.NANOBATCH),
+             (P.PipelineType.KQVBIAS, P.PipelineType.PLLM)]
     for bias_pt, plain_pt in pairs:
         s, h, l, kv = run(bias_pt, w)
         assert _max_rel(h, hid) < E2E_RTOL, (bias_pt, "hidden", _max_rel(h, hid))
@@ -361,17 +361,74 @@ def test_llama31_rope_scaling_reaches_the_kernel_through_the_config(oracle):
         assert _max_rel(h, hid) < E2E_RTOL, (pt, _max_rel(h, hid))
 
 
-def test_the_offload_pipeline_type_is_rejected():
+FOUR_WAY_CASES = {
+    # name: (T, nano1, kqv1, kqv3, decode kv lens, prefill chunks (prev, len))
+    "decode_in_first_two_groups": (96, 40, 20, 28, list(range(5, 35)), [(7, 30), (0, 36)]),     # 30 decode rows: groups 20 + 10
+    "decode_fills_nano1": (96, 40, 20, 28, list(range(3, 43)), [(0, 23), (16, 17)]),            # 40 decode rows = nano1: O1 waits GEMV2
+    "decode_reaches_last_group": (96, 40, 20, 28, list(range(3, 78)), [(0, 11)]),               # 75 decode rows: all four groups
+    "prefill_only": (96, 40, 20, 28, [], [(0, 50), (5, 31)]),
+    "cut_on_the_border": (96, 40, 40, 56, list(range(5, 25)), [(7, 30), (0, 46)]),              # kqv1 == nano1, kqv3 == T - nano1: two empty pieces
+}
+
+
+@pytest.mark.parametrize("case", list(FOUR_WAY_CASES))
+def test_four_way_nanobatch_pipeline_matches_oracle_and_local(oracle, case):
+    """PLLM / NANOBATCH / PLLMOFFLOAD (the reference's main Pipeline, pipeline/src/pipeline.cu:599-789, on one
+    rank): four QKV / RoPE-append / decode-attention nano-batches and one prefill launch must give the
+    oracle's residual stream, samples and KV pages, and agree with LOCAL (same kernels, other row partition)."""
     from nanoflow_amd import engine, pllm_python as P
-    shape = synth.tiny_shape(layers=1, vocab=512, Hq=4, Hkv=2, ffn=256)
-    with pytest.raises(P.NanoflowPipelineError, match="offload"):
-        engine.Engine(shape, P.PipelineType.PLLMOFFLOAD, global_batch=32, nano1=16, kv_pages=64)
-    P.finalize()
+    T, nano1, kqv1, kqv3, dlens, chunks = FOUR_WAY_CASES[case]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=0)
+    b = synth.make_batch(dlens, chunks, vocab=shape.vocab, seed=23, extra_pages=40)
+    rng = np.random.default_rng(5)
+    pools0 = [synth.make_kv_pool(b.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok = b.input_tokens.copy()
+    tok[:b.decodePrefillBorder] = 1
+    d = b.as_dict()
+    d["input_tokens"] = tok
+    pools_ref = [p.copy() for p in pools0]
+    hid_ref, log_ref, samp_ref = oracle.decoder_forward(shape.as_dict(), w, pools_ref, d, want_logits=True)
+    top2 = np.sort(log_ref.astype(np.float32), axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 2 * E2E_RTOL * np.abs(log_ref.astype(np.float32)).max()
+
+    out = {}
+    for pt in (P.PipelineType.LOCAL, P.PipelineType.PLLM, P.PipelineType.NANOBATCH, P.PipelineType.PLLMOFFLOAD):
+        print(f"four-way case={case} pipeline={pt.name}", flush=True)
+        with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=kqv1, kqv3=kqv3, kv_pages=b.num_pages,
+                           weights=w, kv_pools=pools0) as e:
+            e.update(b, keep_token_list=np.ones(b.decodePrefillBorder, np.int32))
+            ids = e.run().copy()
+            hid = e.buffer("hidden").cpu().numpy()[:b.tokens]
+            kv = [p[:b.num_pages].cpu().numpy() for p in e.kv]
+            staged = e.buffer("offload_host").cpu().numpy() if pt == P.PipelineType.PLLMOFFLOAD else None
+        out[pt] = (ids, hid, kv)
+        assert _max_rel(hid, hid_ref) < E2E_RTOL, (pt, _max_rel(hid, hid_ref))
+        assert np.array_equal(ids[clear], samp_ref[clear]), pt
+        for l in range(shape.layers):
+            assert np.array_equal((pools_ref[l] != pools0[l]).any(axis=(3, 4)), (kv[l] != pools0[l]).any(axis=(3, 4))), (pt, l)
+            assert _max_rel(kv[l], pools_ref[l]) < E2E_RTOL, (pt, l)
+        if staged is not None:
+            # what the last layer's round trip left in pinned host memory: the pages of the first two
+            # requests, laid out like kv_indices -- the oracle's gather on the device's final pool
+            n_pages = int(b.kv_indptr[min(2, b.req_num)])
+            assert staged.shape[0] == n_pages
+            want = np.zeros((n_pages,) + kv[-1].shape[1:], np.float16)
+            oracle.move_kv_pages(list(range(min(2, b.req_num))), b.kv_indptr, b.kv_indices, want, kv[-1], to_pool=False)
+            assert np.array_equal(staged.reshape(want.shape).view(np.uint16), want.view(np.uint16))
+    base = out[P.PipelineType.LOCAL]
+    for pt in (P.PipelineType.PLLM, P.PipelineType.NANOBATCH, P.PipelineType.PLLMOFFLOAD):
+        assert _max_rel(out[pt][1], base[1]) < 2e-3, pt            # few-row GEMMs are split over K differently
+        assert np.array_equal(out[pt][0][clear], base[0][clear]), pt
+    # one stream or two, with or without the offload round trip: the same launches, the same bits
+    for pt in (P.PipelineType.NANOBATCH, P.PipelineType.PLLMOFFLOAD):
+        assert np.array_equal(out[pt][0], out[P.PipelineType.PLLM][0]) and np.array_equal(out[pt][1], out[P.PipelineType.PLLM][1])
+        assert all(np.array_equal(x, y) for x, y in zip(out[pt][2], out[P.PipelineType.PLLM][2]))
 
 
-def test_tensor_parallel_schedule_types_run_as_their_one_device_schedules():
-    """PLLM, NONOVERLAP and NANOBATCH (pipeline/src/computeBound.cu:225-233) on one rank: no exchange step
-    moves anything, so they are LOCAL, NON_OVERLAP_LOCAL and NANOBATCH_LOCAL, bit for bit."""
+def test_sequential_tensor_parallel_type_runs_as_the_sequential_local_schedule():
+    """NONOVERLAP (pipeline/src/computeBound.cu:243-244) on one rank has no exchange step left: it is
+    NON_OVERLAP_LOCAL, bit for bit."""
     from nanoflow_amd import engine, pllm_python as P
     shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
     b = synth.make_batch(list(range(5, 25)), [(7, 30), (0, 46)], vocab=shape.vocab, seed=31, extra_pages=40)
@@ -385,13 +442,10 @@ def test_tensor_parallel_schedule_types_run_as_their_one_device_schedules():
             e.update(b)
             ids = e.run().copy()
             return ids, e.buffer("hidden").cpu().numpy()[:b.tokens], [p.cpu().numpy() for p in e.kv]
-    for tp, local in ((P.PipelineType.PLLM, P.PipelineType.LOCAL), (P.PipelineType.NONOVERLAP, P.PipelineType.NON_OVERLAP_LOCAL),
-                      (P.PipelineType.NANOBATCH, P.PipelineType.NANOBATCH_LOCAL)):
-        print("pipeline type", tp.name, flush=True)
-        assert tp.is_sequential == local.is_sequential
-        a, b_ = run(tp), run(local)
-        assert np.array_equal(a[0], b_[0]) and np.array_equal(a[1], b_[1])
-        assert all(np.array_equal(x, y) for x, y in zip(a[2], b_[2]))
+    assert P.PipelineType.NONOVERLAP.is_sequential and P.PipelineType.NONOVERLAP.gemm_tags == 4
+    a, b_ = run(P.PipelineType.NONOVERLAP), run(P.PipelineType.NON_OVERLAP_LOCAL)
+    assert np.array_equal(a[0], b_[0]) and np.array_equal(a[1], b_[1])
+    assert all(np.array_equal(x, y) for x, y in zip(a[2], b_[2]))
 
 
 def _serve_requests(n=14, seed=3):
