@@ -488,9 +488,10 @@ def main():
                          "(80 layers, hidden 8192, 64 Q / 8 KV heads, FFN 28672) resident on the one GPU")
     ap.add_argument("--weights", default="f16", choices=["f16", "e4m3"],
                     help="e4m3: the five per-layer GEMM weights in fp8 with per-output-channel scales")
-    ap.add_argument("--pipeline", default="auto", choices=["auto", "LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL"],
+    ap.add_argument("--pipeline", default="auto", choices=["auto", "LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL", "PLLM", "NANOBATCH", "PLLMOFFLOAD"],
                     help="auto = the fastest schedule measured on MI355X for both workloads: NON_OVERLAP_LOCAL\n"
-                         "(one stream); LOCAL measures the two-stream overlapped schedule")
+                         "(one stream); LOCAL measures the two-stream overlapped schedule, PLLM the reference's main\n"
+                         "schedule (four QKV / attention nano-batches), PLLMOFFLOAD that with the KV offload round trip")
     ap.add_argument("--nano1", type=int, default=1024, help="rows of nano-batch 1")
     ap.add_argument("--kqv1", type=int, default=512)
     ap.add_argument("--kqv3", type=int, default=512)

@@ -9,9 +9,9 @@ the candidates on the device and writes that block:
     python -m nanoflow_amd.autosearch -c config_all/llama3-8B/1024.json -o tuned.json \\
            [--decode 681 --kv-lo 1024 --kv-hi 1536 --prefill 755:269,0:1024,0:74] [--layers 8]
 
-Candidates: NON_OVERLAP_LOCAL (one stream, no split), and NANOBATCH_LOCAL / LOCAL (two
-nano-batches, LOCAL on two streams) over a grid of nano-batch-1 sizes and QKV sub-splits, all
-multiples of ``--step`` rows.  Optional ``--cu-masks`` adds, for LOCAL, static compute-unit splits
+Candidates: NON_OVERLAP_LOCAL (one stream, no split), NANOBATCH_LOCAL / LOCAL (two nano-batches,
+LOCAL on two streams) and PLLM (four QKV / attention nano-batches, two streams) over a grid of
+nano-batch-1 sizes and QKV sub-splits, all multiples of ``--step`` rows.  Optional ``--cu-masks`` adds, for LOCAL, static compute-unit splits
 between the GEMM and the attention stream (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS: CU counts, given
 here in whole XCDs of 32).
 Each candidate runs the same iteration (the decode requests and prefill chunks given, on
@@ -65,7 +65,7 @@ def measure(shape, batch, T, cand, layers, iters, warm, env=None):
     os.environ.update(env or {})
     try:
         eng = engine.Engine(shape, P.PipelineType[name], global_batch=T, nano1=n1, kqv1=k1, kqv3=k3,
-                            kv_pages=batch.num_pages, run_layer=layers, distinct_layers=layers, kv_fill="zeros")
+                            kv_pages=batch.num_pages, run_layer=layers, distinct_layers=layers)
     finally:
         for k, v in saved.items():
             if v is None:
@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--prefill", default="755:269,0:1024,0:74", help="prefill chunks prev_len:chunk_len,...")
     ap.add_argument("--layers", type=int, default=8, help="layers executed per measurement")
     ap.add_argument("--step", type=int, default=128, help="granularity of the nano-batch sizes")
-    ap.add_argument("--types", default="NON_OVERLAP_LOCAL,NANOBATCH_LOCAL,LOCAL")
+    ap.add_argument("--types", default="NON_OVERLAP_LOCAL,NANOBATCH_LOCAL,LOCAL,PLLM")
     ap.add_argument("--fine", action="store_true", help="also try 1/4 and 3/4 QKV sub-splits")
     ap.add_argument("--cu-masks", default="", help="LOCAL only: GEMM:attention XCD counts to try, e.g. 6:2,5:3,4:4")
     ap.add_argument("--iters", type=int, default=5)
