@@ -51,7 +51,13 @@ struct GemmSmem {
   // stages-1 slabs before they are needed
   static constexpr int stages = (144 * 1024) / stage_bytes > 4 ? 4 : (144 * 1024) / stage_bytes;
   static_assert(stages >= 2, "tile too large for two LDS stages");
-  static constexpr size_t bytes = (size_t)stages * stage_bytes;
+  // Tiles with room for two stages only (256 x 256, the 256 x 128 pair: 64 KB per slab) would have to
+  // land every load of a slab within the slab before it -- less than a microsecond, which a load
+  // that misses the L2 does not make.  They keep the activations in a ring of two stages and give
+  // the weights (the operand that streams from HBM) a ring of three: 2 x 32 + 3 x 32 KB = all 160 KB.
+  static constexpr bool split = stages == 2 && 2 * a_bytes + 3 * NB * b_bytes <= 160 * 1024;
+  static constexpr int b_ring = 2 * a_bytes;  // split rings: activation stages first, then the weight stages
+  static constexpr size_t bytes = split ? (size_t)2 * a_bytes + (size_t)3 * NB * b_bytes : (size_t)stages * stage_bytes;
 };
 
 // Element types of the family: how 16-bit storage is multiplied, widened and rounded.
@@ -171,28 +177,29 @@ __device__ __forceinline__ void gemm_tile(
   constexpr int NS = SM::stages;
   constexpr int LOADS = A_LOADS + NB * B_LOADS;  // per wave per slab
   constexpr int PARTS = NS == 2 ? 3 : 4;         // k-steps the loads of one slab are spread over
-  // k_ok: this lane's 16 bytes of the slab's 128-byte rows lie below K.
-  auto load_one = [&](auto t_c, uint32_t st, bool k_ok) {
+  // k_ok: this lane's 16 bytes of the slab's 128-byte rows lie below K.  la / lb: LDS address of
+  // the stage the activations / the weights of the slab go to, + wave * 1024.
+  auto load_one = [&](auto t_c, uint32_t la, uint32_t lb, bool k_ok) {
     constexpr int t = decltype(t_c)::value;
     if constexpr (t < A_LOADS) {
-      load16_to_lds<t * 4096>(a_rsrc, k_ok ? a_off[t] : kOob, st);
+      load16_to_lds<t * 4096>(a_rsrc, k_ok ? a_off[t] : kOob, la);
       a_off[t] += BK * 2;
     } else {
       constexpr int b = (t - A_LOADS) / B_LOADS, tt = (t - A_LOADS) % B_LOADS;
-      constexpr int dst = SM::a_bytes + b * SM::b_bytes + tt * 4096;
+      constexpr int dst = b * SM::b_bytes + tt * 4096;
       if constexpr (kBCol) {
-        load16_to_lds<dst>(b_rsrc[b], k_ok ? b_off[b][tt] : kOob, st);
+        load16_to_lds<dst>(b_rsrc[b], k_ok ? b_off[b][tt] : kOob, lb);
         b_off[b][tt] += BK * 2;
       } else {
-        load16_to_lds<dst>(b_rsrc[b], b_off[b][tt], st);
+        load16_to_lds<dst>(b_rsrc[b], b_off[b][tt], lb);
         b_off[b][tt] += b_slab;
       }
     }
   };
-  auto load_slab = [&](int stage, int k0) {  // every load of one slab, back to back
+  auto load_slab = [&](int stage, int k0) {  // every load of one slab, back to back (one ring for both operands)
     const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::stage_bytes + wave * 1024);
     const bool k_ok = k0 + a_kc < K;
-    static_for<LOADS>([&](auto t_c) { load_one(t_c, st, k_ok); });
+    static_for<LOADS>([&](auto t_c) { load_one(t_c, st, st + SM::a_bytes, k_ok); });
   };
 
   // ---- LDS -> MFMA operand fragments, double-buffered across k-steps
@@ -217,13 +224,14 @@ __device__ __forceinline__ void gemm_tile(
   half8_t af[2][TM];
   half8_t bf[2][NB][TN];
   constexpr int READS = TM + NB * TN;  // fragment reads per k-step: q < TM activations, then weights
-  auto read_one = [&](auto q_c, auto kk_c, auto buf_c, const uint8_t* st) {
+  // sa / sb: the stage holding the slab's activations / weights
+  auto read_one = [&](auto q_c, auto kk_c, auto buf_c, const uint8_t* sa, const uint8_t* sb) {
     constexpr int q = decltype(q_c)::value, kk = decltype(kk_c)::value, buf = decltype(buf_c)::value;
     if constexpr (q < TM) {
-      af[buf][q] = *reinterpret_cast<const half8_t*>(st + a_rd + swz[kk] + q * 32 * 128);
+      af[buf][q] = *reinterpret_cast<const half8_t*>(sa + a_rd + swz[kk] + q * 32 * 128);
     } else {
       constexpr int b = (q - TM) / TN, j = (q - TM) % TN;
-      const uint8_t* bs = st + SM::a_bytes + b * SM::b_bytes;
+      const uint8_t* bs = sb + b * SM::b_bytes;
       if constexpr (kBCol) {
         bf[buf][b][j] = *reinterpret_cast<const half8_t*>(bs + bc_rd + swz[kk] + j * 32 * 128);
       } else {
@@ -240,12 +248,13 @@ __device__ __forceinline__ void gemm_tile(
   // One k-step: the MFMAs on fragment buffer kk & 1, with the step's side work dealt out
   // between them and the order pinned -- a wavefront is alone on its SIMD, so whatever it issues
   // between two MFMAs must fit into the 32 cycles the first one occupies the matrix pipe:
-  //   loads LP, LP + PARTS, ... of the slab being fetched (LP < 0: none), into stage address ld_st;
-  //   then the fragment reads of k-step RK from stage rd_st into the other buffer (RK < 0: none).
+  //   loads L0, L0 + LSTR, ... (NL of them) of a slab being fetched, into the stages at la / lb;
+  //   then the fragment reads of k-step RK from the stages sa / sb into the other buffer (RK < 0: none).
   constexpr int NM = NB * TN * TM;
-  auto step = [&](auto kk_c, auto lp_c, auto rk_c, uint32_t ld_st, bool ld_ok, const uint8_t* rd_st) {
-    constexpr int kk = decltype(kk_c)::value, LP = decltype(lp_c)::value, RK = decltype(rk_c)::value;
-    constexpr int NL = LP < 0 ? 0 : (LOADS - LP + PARTS - 1) / PARTS;
+  auto step = [&](auto kk_c, auto l0_c, auto lstr_c, auto nl_c, auto rk_c, uint32_t la, uint32_t lb, bool ld_ok,
+                  const uint8_t* sa, const uint8_t* sb) {
+    constexpr int kk = decltype(kk_c)::value, L0 = decltype(l0_c)::value, LSTR = decltype(lstr_c)::value;
+    constexpr int NL = decltype(nl_c)::value, RK = decltype(rk_c)::value;
     constexpr int NR = RK < 0 ? 0 : READS;
     constexpr int S = NL + NR;
     static_for<NM>([&](auto n_c) {
@@ -258,12 +267,83 @@ __device__ __forceinline__ void gemm_tile(
       constexpr int lo = n * S / NM, hi = (n + 1) * S / NM;
       static_for<hi - lo>([&](auto d_c) {
         constexpr int q = lo + decltype(d_c)::value;
-        if constexpr (q < NL) load_one(ic<(LP < 0 ? 0 : LP) + PARTS * q>{}, ld_st, ld_ok);
-        else read_one(ic<q - NL>{}, ic<(RK < 0 ? 0 : RK)>{}, ic<(kk + 1) & 1>{}, rd_st);
+        if constexpr (q < NL) load_one(ic<L0 + LSTR * q>{}, la, lb, ld_ok);
+        else read_one(ic<q - NL>{}, ic<(RK < 0 ? 0 : RK)>{}, ic<(kk + 1) & 1>{}, sa, sb);
       });
       __builtin_amdgcn_sched_barrier(0);
     });
   };
+  using T_ = std::true_type;
+  using F_ = std::false_type;
+  const int nslab = (K + BK - 1) / BK;
+
+  if constexpr (SM::split) {
+    // ---- two activation stages, three weight stages.  Slab s has its activations in stage s % 2
+    // and its weights in stage s % 3.  During slab s a wavefront issues, in this order: the second
+    // half of the activation loads of slab s+1 (k-step 0; the first half went out in k-step 3 of
+    // slab s-1), all weight loads of slab s+2 (k-steps 1 and 2), then waits until everything but
+    // those weight loads has landed -- its loads of slab s+1 -- and meets the others at the barrier;
+    // k-step 3 prefetches the first fragments of slab s+1 and issues the first half of the
+    // activation loads of slab s+2 into the stage the barrier has just freed.  A weight load has
+    // five to six k-steps to land, an activation load three.
+    constexpr int HA = (A_LOADS + 1) / 2;               // activation loads issued in k-step 3
+    constexpr int BL = NB * B_LOADS, HB = (BL + 1) / 2;  // weight loads, and those issued in k-step 1
+    static_assert(BL < 64, "vmcnt range");
+    constexpr int wait_but_b = 0x0070 | (BL & 15) | ((BL >> 4) << 14);  // vmcnt(BL), lgkmcnt(0)
+    auto a_lds = [&](int stage) { return __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::a_bytes + wave * 1024); };
+    auto b_lds = [&](int stage) {
+      return __builtin_amdgcn_readfirstlane(smem_lds + SM::b_ring + stage * NB * SM::b_bytes + wave * 1024);
+    };
+    auto a_ptr = [&](int stage) { return smem + stage * SM::a_bytes; };
+    auto b_ptr = [&](int stage) { return smem + SM::b_ring + stage * NB * SM::b_bytes; };
+    auto k_ok_of = [&](int slab_idx) { return slab_idx * BK + a_kc < K; };
+    // prologue: activations and weights of slab 0, weights of slab 1
+    {
+      const uint32_t la = a_lds(0), lb0 = b_lds(0), lb1 = b_lds(1);
+      static_for<A_LOADS>([&](auto t_c) { load_one(t_c, la, lb0, k_ok_of(0)); });
+      static_for<BL>([&](auto t_c) { load_one(ic<A_LOADS + decltype(t_c)::value>{}, la, lb0, k_ok_of(0)); });
+      if (nslab > 1) {
+        static_for<BL>([&](auto t_c) { load_one(ic<A_LOADS + decltype(t_c)::value>{}, la, lb1, k_ok_of(1)); });
+        __builtin_amdgcn_s_waitcnt(wait_but_b);
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0070);
+      }
+    }
+    __syncthreads();
+    static_for<READS>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, a_ptr(0), b_ptr(0)); });
+    if (nslab > 1) {  // what k-step 3 of a slab before slab 0 would have issued
+      const uint32_t la = a_lds(1);
+      static_for<HA>([&](auto t_c) { load_one(t_c, la, la, k_ok_of(1)); });
+    }
+    // H1: slab s+1 exists, H2: slab s+2 exists
+    auto slab2 = [&](auto h1_c, auto h2_c, int s, int bs) {
+      constexpr bool H1 = decltype(h1_c)::value, H2 = decltype(h2_c)::value;
+      const uint8_t *sa = a_ptr(s & 1), *sb = b_ptr(bs);
+      const int bs1 = bs == 2 ? 0 : bs + 1, bs2 = bs1 == 2 ? 0 : bs1 + 1;
+      const uint32_t la1 = a_lds((s + 1) & 1), lb2 = b_lds(bs2);
+      step(ic<0>{}, ic<HA>{}, ic<1>{}, ic<H1 ? A_LOADS - HA : 0>{}, ic<1>{}, la1, la1, k_ok_of(s + 1), sa, sb);
+      step(ic<1>{}, ic<A_LOADS>{}, ic<1>{}, ic<H2 ? HB : 0>{}, ic<2>{}, lb2, lb2, k_ok_of(s + 2), sa, sb);
+      step(ic<2>{}, ic<A_LOADS + HB>{}, ic<1>{}, ic<H2 ? BL - HB : 0>{}, ic<3>{}, lb2, lb2, k_ok_of(s + 2), sa, sb);
+      if constexpr (H1) {
+        __builtin_amdgcn_s_waitcnt(H2 ? wait_but_b : 0x0070);
+        __syncthreads();
+      }
+      const uint32_t la2 = a_lds(s & 1);  // slab s+2's activations reuse this slab's stage
+      step(ic<3>{}, ic<0>{}, ic<1>{}, ic<H2 ? HA : 0>{}, ic<H1 ? 0 : -1>{}, la2, la2, k_ok_of(s + 2), a_ptr((s + 1) & 1),
+           b_ptr(bs1));
+    };
+    int s = 0, bs = 0;
+    for (; s + 2 < nslab; ++s) {
+      slab2(T_{}, T_{}, s, bs);
+      bs = bs == 2 ? 0 : bs + 1;
+    }
+    if (s + 1 < nslab) {
+      slab2(T_{}, F_{}, s, bs);
+      bs = bs == 2 ? 0 : bs + 1;
+      ++s;
+    }
+    slab2(F_{}, F_{}, s, bs);
+  } else {
 
   // vmcnt(n) with lgkmcnt(0): n in bits [3:0] and [15:14]
   auto wait_loads = [&](int younger) {
@@ -272,6 +352,7 @@ __device__ __forceinline__ void gemm_tile(
   };
   static_assert(LOADS * (NS - 2) < 64, "vmcnt range");
   auto next = [](int st) { return st + 1 == NS ? 0 : st + 1; };
+  constexpr auto nl = [](int lp) { return (LOADS - lp + PARTS - 1) / PARTS; };  // loads lp, lp + PARTS, ...
 
   // Slab s lives in LDS stage s % NS.  Its k-steps 0..2 prefetch the fragments of the step after
   // them; then the wavefront waits until its own loads of slab s+1 have landed and its fragment
@@ -285,21 +366,22 @@ __device__ __forceinline__ void gemm_tile(
   auto slab = [&](auto ia_c, auto ib_c, auto last_c, int s, int cs, int ls) {
     constexpr bool IA = decltype(ia_c)::value, IB = decltype(ib_c)::value, LAST = decltype(last_c)::value;
     const uint8_t* st = smem + cs * SM::stage_bytes;
+    const uint8_t* sb = st + SM::a_bytes;
     const uint32_t ld_a = __builtin_amdgcn_readfirstlane(smem_lds + ls * SM::stage_bytes + wave * 1024);
     const bool ok_a = (s + NS - 1) * BK + a_kc < K;
-    step(ic<0>{}, ic<(IA && PARTS > 1) ? 1 : -1>{}, ic<1>{}, ld_a, ok_a, st);
-    step(ic<1>{}, ic<(IA && PARTS > 2) ? 2 : -1>{}, ic<2>{}, ld_a, ok_a, st);
-    step(ic<2>{}, ic<(IA && PARTS > 3) ? 3 : -1>{}, ic<3>{}, ld_a, ok_a, st);
+    step(ic<0>{}, ic<1>{}, ic<PARTS>{}, ic<(IA && PARTS > 1) ? nl(1) : 0>{}, ic<1>{}, ld_a, ld_a + SM::a_bytes, ok_a, st, sb);
+    step(ic<1>{}, ic<2>{}, ic<PARTS>{}, ic<(IA && PARTS > 2) ? nl(2) : 0>{}, ic<2>{}, ld_a, ld_a + SM::a_bytes, ok_a, st, sb);
+    step(ic<2>{}, ic<3>{}, ic<PARTS>{}, ic<(IA && PARTS > 3) ? nl(3) : 0>{}, ic<3>{}, ld_a, ld_a + SM::a_bytes, ok_a, st, sb);
     if constexpr (!LAST) {
       wait_loads(IA ? 1 : 0);
       __syncthreads();
     }
     const uint32_t ld_b = __builtin_amdgcn_readfirstlane(smem_lds + cs * SM::stage_bytes + wave * 1024);
-    step(ic<3>{}, ic<IB ? 0 : -1>{}, ic<LAST ? -1 : 0>{}, ld_b, (s + NS) * BK + a_kc < K,
-         smem + next(cs) * SM::stage_bytes);
+    const uint8_t* nst = smem + next(cs) * SM::stage_bytes;
+    step(ic<3>{}, ic<0>{}, ic<PARTS>{}, ic<IB ? nl(0) : 0>{}, ic<LAST ? -1 : 0>{}, ld_b, ld_b + SM::a_bytes,
+         (s + NS) * BK + a_kc < K, nst, nst + SM::a_bytes);
   };
 
-  const int nslab = (K + BK - 1) / BK;
 #pragma unroll
   for (int p = 0; p < NS - 1; ++p)
     if (p < nslab) load_slab(p, p * BK);
@@ -307,15 +389,13 @@ __device__ __forceinline__ void gemm_tile(
   // matters for speed: waiting for everything is always correct)
   wait_loads(nslab >= NS - 1 ? 1 : 0);
   __syncthreads();
-  static_for<READS>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, smem); });
+  static_for<READS>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, smem, smem + SM::a_bytes); });
   if (NS - 1 < nslab) {  // the share of slab NS-1 that a slab's k-step 3 would have issued
     const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + (NS - 1) * SM::stage_bytes + wave * 1024);
     const bool k_ok = (NS - 1) * BK + a_kc < K;
-    static_for<(LOADS + PARTS - 1) / PARTS>([&](auto q_c) { load_one(ic<PARTS * decltype(q_c)::value>{}, st, k_ok); });
+    static_for<(LOADS + PARTS - 1) / PARTS>([&](auto q_c) { load_one(ic<PARTS * decltype(q_c)::value>{}, st, st + SM::a_bytes, k_ok); });
   }
   int cs = 0, ls = NS - 1, s = 0;
-  using T_ = std::true_type;
-  using F_ = std::false_type;
   for (; s + NS < nslab; ++s) {  // steady state
     slab(T_{}, T_{}, F_{}, s, cs, ls);
     cs = next(cs);
@@ -328,6 +408,7 @@ __device__ __forceinline__ void gemm_tile(
     ls = next(ls);
   }
   slab(F_{}, F_{}, T_{}, s, cs, ls);  // the last slab: nothing left to fetch or prefetch
+  }  // one ring for both operands
 
   // Epilogue.  acc[.][i][j][r] holds D[m][n] with m = tile row l32 and
   // n = (r/4)*8 + lg*4 + r%4 of the 32x32 tile: a lane owns 4 consecutive columns of 32 different
