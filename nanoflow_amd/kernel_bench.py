@@ -33,10 +33,21 @@ from nanoflow_amd import kernels as K, synth  # noqa: E402
 DEV = "cuda"
 
 
+WARM_MS = 0.0   # --warm-ms: keep launching for this long before timing (the clocks of a part that sat
+                # idle take tens of milliseconds of load to settle; short cold runs read 5-15 % low)
+
+
 def timeit(fn, iters, warm):
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
+    if WARM_MS > 0:
+        import time
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < WARM_MS:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s.record()
     for _ in range(iters):
@@ -180,9 +191,13 @@ def main():
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"], help="gemm, dual: element type")
     ap.add_argument("--b-col-major", action="store_true", help="gemm: weights stored [N][K] (k contiguous)")
     ap.add_argument("--ws", action="store_true", help="gemm: the entry point with a workspace (split over K where it pays)")
+    ap.add_argument("--warm-ms", type=float, default=300.0,
+                    help="gemm, dual, blas, attn: keep launching this long before timing (0: only --warm launches)")
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--warm", type=int, default=3)
     a = ap.parse_args()
+    global WARM_MS
+    WARM_MS = a.warm_ms if a.iters > 2 else 0.0      # counter-collection runs (--iters 1 or 2) stay short
     assert torch.cuda.is_available(), "needs the MI355X"
     shape = synth.LLAMA3_8B if a.model == "8b" else synth.LLAMA3_70B
     g = torch.Generator(device=DEV).manual_seed(0)
@@ -279,15 +294,21 @@ def main():
             Bkn, Bnk = rnd(Kd, N, std=0.02), rnd(N, Kd, std=0.02)
             out = torch.empty(M, N, dtype=torch.float16, device=DEV)
             reps = 2 if name.startswith("gate") else 1
+            # every measurement follows --warm-ms of the same launches: all three are timed warm
             ms_kn = timeit(lambda: [torch.matmul(A, Bkn, out=out) for _ in range(reps)], a.iters, a.warm)
             ms_nk = timeit(lambda: [torch.matmul(A, Bnk.t(), out=out) for _ in range(reps)], a.iters, a.warm)
             if name.startswith("gate"):
-                ms_us = timeit(lambda: K.dual_swiglu(A, Bkn, Bkn, out=out), a.iters, a.warm)
+                Bkn2 = rnd(Kd, N, std=0.02)
+                ms_us = timeit(lambda: K.dual_swiglu(A, Bkn, Bkn2, out=out), a.iters, a.warm)
+                ms_same = timeit(lambda: K.dual_swiglu(A, Bkn, Bkn, out=out), a.iters, a.warm)
             else:
                 ms_us = timeit(lambda: K.gemm(A, Bkn, out=out), a.iters, a.warm)
             fl = 2.0 * reps * M * N * Kd
             print(f"{name:18s} {M}x{N}x{Kd}: torch.matmul [K,N] weights {fl / ms_kn / 1e9:7.1f}  [N,K] weights "
                   f"{fl / ms_nk / 1e9:7.1f}  this library ([K,N]) {fl / ms_us / 1e9:7.1f} TFLOP/s", flush=True)
+            if name.startswith("gate"):
+                print(f"{'':18s} this library's fused pair with ONE buffer given as both weight matrices (half the weight "
+                      f"bytes, same flops): {fl / ms_same / 1e9:7.1f} TFLOP/s", flush=True)
     elif a.op in ("corun", "cusplit"):
         corun(a, shape, rnd)
     else:
