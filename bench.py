@@ -42,7 +42,7 @@ A100_PUBLISHED_TOKENS_PER_S = 12756.0   # reference, 1x A100 80GB, same offline 
 # HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
 # by what the same counter reads for a 1 GiB device copy), as a ratio to the algorithmic bytes of
 # the same launch: profiles/decode_attention_config2_pmc.txt.
-DECODE_ATTN_TRAFFIC_RATIO = 1.0072
+DECODE_ATTN_TRAFFIC_RATIO = 1.0069
 
 
 def decode_attention_bytes(kv_len: np.ndarray, Hq=32, Hkv=8, d=128, page=16) -> int:
@@ -106,9 +106,15 @@ def calibrate(fp8: bool):
     K.calibrate_mfma(fp8, True, 4000)                      # power state settles
     tf_rand, mhz_rand = K.calibrate_mfma(fp8, True, 40000)
     tf_zero, mhz_zero = K.calibrate_mfma(fp8, False, 40000)
+    tf_lds, mhz_lds = (None, None) if fp8 else K.calibrate_mfma(False, 2, 40000)
+    tf_ld, mhz_ld = (None, None) if fp8 else K.calibrate_mfma(False, 3, 40000)
     hbm = K.calibrate_hbm_read(8.0, 4)
     return {"mfma_tflops_random_operands": tf_rand, "mfma_clock_mhz_random_operands": mhz_rand,
             "mfma_tflops_zero_operands": tf_zero, "mfma_clock_mhz_zero_operands": mhz_zero,
+            # the same loop with its operand fragments re-read from LDS at the GEMM main loop's rate
+            "mfma_tflops_random_operands_from_lds": tf_lds, "mfma_clock_mhz_random_operands_from_lds": mhz_lds,
+            # ... and with a 256x256 tile's operand loads (L2 -> LDS) beside them: a main loop without barriers
+            "mfma_tflops_with_operand_loads": tf_ld, "mfma_clock_mhz_with_operand_loads": mhz_ld,
             "mfma_dtype": "f8e4m3" if fp8 else "f16", "hbm_read_stream_gbps": hbm,
             "how": "nf_calibrate_mfma: 1024 workgroups x 4 wavefronts x 40000 x 16 independent 32x32 MFMAs, "
                    "registers only; nf_calibrate_hbm_read: 2048 workgroups stream 8 GiB 4 times"}
@@ -145,8 +151,8 @@ def _attention_roofline(tm, bytes_per_launch, name="roofline", calib=None):
 # Memory-side bytes per dense GEMM launch over algorithmic bytes (operands once + output), measured
 # with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernels at M = 2048 (LM head: 684 rows) and
 # scaled by the copy-kernel calibration: profiles/gemm_hbm_traffic_pmc.txt.  The activations are
-# fetched once per XCD; most of the repeats hit the Infinity Cache.
-GEMM_TRAFFIC_RATIO = 2.66
+# fetched once per XCD and round of tiles; most of the repeats hit the Infinity Cache.
+GEMM_TRAFFIC_RATIO = 2.44
 
 
 def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows, weight_bytes=2):
@@ -309,6 +315,29 @@ def run_iteration(args):
     return rec
 
 
+def _serve_whole_job(former, chunk=512):
+    """The whole job, `chunk` timed cycles per call of the serving loop, with a progress line
+    after each (a 70B job runs for minutes).  Each call starts and ends with the GPU idle: one
+    cycle in `chunk` loses the overlap of batch formation with the device."""
+    import types
+    tot = types.SimpleNamespace(cycles=0, retired=0, wall_s=0.0, tokens_processed=0, cycle_ms=0.0, form_ms=0.0,
+                                wait_ms=0.0, update_ms=0.0, gpu_iter_ms=0.0)
+    while True:
+        st = former.serve(0, chunk, warmup_cycles=0)
+        for f in ("cycle_ms", "form_ms", "wait_ms", "update_ms", "gpu_iter_ms"):   # means over cycles
+            setattr(tot, f, (getattr(tot, f) * tot.cycles + getattr(st, f) * st.cycles) / max(tot.cycles + st.cycles, 1))
+        tot.cycles += st.cycles
+        tot.retired += st.retired
+        tot.wall_s += st.wall_s
+        tot.tokens_processed += st.tokens_processed
+        state = former.state()
+        left = state["queued"] + state["decoding"] + state["prefilling"]
+        print(f"[bench] {tot.cycles} cycles, {tot.retired} requests retired, {left} left, {tot.wall_s:.1f} s",
+              file=sys.stderr, flush=True)
+        if st.cycles < chunk or left == 0:
+            return tot
+
+
 def run_offline(args):
     import torch
     from nanoflow_amd import engine, synth, pllm_python as P
@@ -352,14 +381,14 @@ def run_offline(args):
     P.setGraphMode(graph)
     prime = 0
     if args.full_run:
-        skip, warmup, steps = 0, 0, 1 << 30
+        skip, warmup = 0, 0
     else:
         skip = args.skip_cycles
         prime = args.prime_cycles if graph else 0
         if prime:
             former.serve(skip, prime, warmup_cycles=0)
             skip = 0
-    st = former.serve(skip, steps, warmup_cycles=warmup)
+    st = _serve_whole_job(former) if args.full_run else former.serve(skip, steps, warmup_cycles=warmup)
     counters = P.getGraphCounters()
     P.setGraphMode(False)
 

@@ -241,7 +241,12 @@ NF_API int nf_argmax_f16(const uint16_t* logits, uint16_t* max_vals, int32_t* ar
  * events on `stream`); `scratch` is at least 8192 bytes of device memory the kernels may write.
  * nf_calibrate_mfma: a register-only loop of independent 32x32 MFMA instructions (fp8 == 0:
  *   v_mfma_f32_32x32x16_f16; else the 32x32x64 fp8 form), one wavefront per SIMD, `iters` x 16
- *   instructions per wavefront, on zero operands (random_operands == 0) or pseudo-random ones;
+ *   instructions per wavefront, on zero operands (random_operands == 0), on pseudo-random ones
+ *   (1), or (2, fp16 only) on pseudo-random operands that each wavefront re-reads from LDS before
+ *   every 16 instructions, the way the main loop of the 256x256 GEMM tile is fed, or (3, fp16
+ *   only; `scratch` then holds 8192 + 8 MiB bytes) with that tile's operand loads beside them as
+ *   well, from a window of scratch the L2 holds straight into LDS, or (10 + n, n <= 64) as 1 with
+ *   n x 64 idle cycles after every 16 instructions;
  *   *tflops = the rate, *clock_mhz = shader clock the wavefronts saw while running.
  * nf_calibrate_hbm_read: all CUs stream `bytes` of `buf` (16-byte aligned, much larger than the
  *   last-level cache) `reps` times; *gbps = the read rate.

@@ -5,8 +5,17 @@
 //                          32x32x64 fp8) instructions, one wavefront per SIMD like the GEMM kernels,
 //                          on zero operands (the least switching activity: the highest clock the
 //                          part holds) or on pseudo-random ones (what a GEMM on N(0,1) data feeds
-//                          the matrix pipe); reports TFLOP/s and the shader clock the wavefronts
-//                          saw (shader-clock ticks over real-time ticks).
+//                          the matrix pipe), or (random_operands = 2, fp16) on pseudo-random operands
+//                          that every wavefront re-reads from LDS before each 16 MFMAs, as the main
+//                          loop of the 256x256 GEMM tile does (8 reads of 16 bytes per lane): the
+//                          matrix pipe plus the fragment traffic, still without a byte from memory;
+//                          or (3) with the operand loads of that tile beside them as well (64 KB
+//                          per workgroup per 64 MFMAs, straight into LDS, from a window the L2
+//                          holds): the GEMM's main loop without barriers, prologue or epilogue;
+//                          or (10 + n) as 1 with n x 64 idle cycles after every 16 MFMAs: how much
+//                          of an idle matrix pipe the power management gives back as clock;
+//                          reports TFLOP/s and the shader clock the wavefronts saw (shader-clock
+//                          ticks over real-time ticks).
 //   nf_calibrate_hbm_read  every CU streams its share of a buffer far larger than the last-level
 //                          cache with 16-byte loads; reports GB/s.
 //   nf_calibrate_paged_read  the access pattern of paged decode attention without its arithmetic:
@@ -72,6 +81,8 @@ __global__ __launch_bounds__(256) void calib_mfma_kernel(int iters, int random_o
         else
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b16[j], a16[i], acc[i][j], 0, 0, 0);
       }
+    // random_operands = 10 + n: n x 64 idle cycles after every 16 MFMAs (512 busy cycles)
+    for (int q = 10; q < random_operands; ++q) asm volatile("s_nop 15" ::: "memory");
   }
   const uint64_t c1 = __builtin_readcyclecounter(), r1 = wall_clock64();
   float s = 0.f;
@@ -82,6 +93,93 @@ __global__ __launch_bounds__(256) void calib_mfma_kernel(int iters, int random_o
 #pragma unroll
       for (int r = 0; r < 16; ++r) s += acc[i][j][r];
   sink[gid & 1023u] = s;  // keeps the loop alive; the value is never read
+  if (threadIdx.x == 0 && blockIdx.x < 64) {
+    clocks[blockIdx.x * 2 + 0] = c1 - c0;
+    clocks[blockIdx.x * 2 + 1] = r1 - r0;
+  }
+}
+
+// The same 16 accumulators, with the 4 + 4 operand fragments of every 16 MFMAs read from LDS one
+// step ahead (two sets of pseudo-random fragments per wavefront, taken in turn): what the matrix
+// pipe sustains when it is fed the way the GEMM's main loop feeds it.
+__device__ __forceinline__ half8_t lds_read16(uint32_t addr) {
+  rsrc_t v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr));
+  return __builtin_bit_cast(half8_t, v);
+}
+// kLoads: every wavefront also issues 4 direct-to-LDS loads of 1 KB per 16 MFMAs (the 64 KB a
+// 256x256 tile fetches per 64-deep slab), from a 2 MB window of `src` that 64 workgroups share and
+// the L2 holds, into a second 64 KB of LDS, with at most two steps of loads in flight.
+template <bool kLoads>
+__global__ __launch_bounds__(256) void calib_mfma_lds_kernel(int iters, uint64_t* clocks, float* sink,
+                                                             const uint8_t* __restrict__ src) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // 64 KB of fragments (+ 64 KB of landing area)
+  const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int c = 0; c < 16; ++c) {  // 256 bytes of fragments per thread
+    half8_t v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      v[e] = (_Float16)(((int)(mix32(gid * 128u + c * 8u + e) >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
+    *reinterpret_cast<half8_t*>(smem + (c * 256 + threadIdx.x) * 16) = v;
+  }
+  __syncthreads();
+  float16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  // the wavefront's 16 KB: fragment f of set s at s * 8192 + f * 1024 + lane * 16
+  const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem + wave * 16384 + lane * 16;
+  half8_t a[2][4], b[2][4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    a[0][f] = lds_read16(base + f * 1024);
+    b[0][f] = lds_read16(base + (4 + f) * 1024);
+  }
+  constexpr uint32_t kWindow = 2u << 20;
+  const rsrc_t rsrc = make_rsrc(kLoads ? src + (size_t)(blockIdx.x / 8 % 4) * kWindow : nullptr, kLoads ? kWindow : 0);
+  const uint32_t land = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem + 65536 + wave * 1024);
+  uint32_t goff = (uint32_t)(wave * 1024 + lane * 16);
+  const uint64_t c0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+  for (int it = 0; it < iters; it += 2) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      if constexpr (kLoads) {
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // the loads of the step before last have landed
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          load16_to_lds(rsrc, goff + (uint32_t)q * 4096u, land + (uint32_t)s * 32768u + (uint32_t)q * 4096u);
+        goff = (goff + 16384u) & (kWindow - 1);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // set s, requested one step ago
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        a[s ^ 1][f] = lds_read16(base + (s ^ 1) * 8192 + f * 1024);
+        b[s ^ 1][f] = lds_read16(base + (s ^ 1) * 8192 + (4 + f) * 1024);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[s][j], a[s][i], acc[i][j], 0, 0, 0);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  const uint64_t c1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s += acc[i][j][r];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) s += (float)a[0][f][0] + (float)b[0][f][0];  // the last reads are consumed too
+  sink[gid & 1023u] = s;
   if (threadIdx.x == 0 && blockIdx.x < 64) {
     clocks[blockIdx.x * 2 + 0] = c1 - c0;
     clocks[blockIdx.x * 2 + 1] = r1 - r0;
@@ -174,6 +272,20 @@ extern "C" {
 int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, size_t scratch_bytes, double* tflops,
                       double* clock_mhz, nf_stream_t stream) {
   NF_REQUIRE(iters > 0 && scratch && scratch_bytes >= 8192 && tflops && clock_mhz, "nf_calibrate_mfma: bad arguments");
+  NF_REQUIRE(random_operands >= 0 && (random_operands <= 3 || (random_operands >= 10 && random_operands <= 74)) &&
+                 !(fp8 && random_operands >= 2 && random_operands <= 3),
+             "nf_calibrate_mfma: random_operands = %d (0, 1, 10 + n = 1 with n x 64 idle cycles per 16 MFMAs, or fp16 "
+             "only: 2 = operands re-read from LDS, 3 = and operand loads from L2 into LDS beside them)", random_operands);
+  NF_REQUIRE(random_operands != 3 || scratch_bytes >= 8192 + ((size_t)8 << 20),
+             "nf_calibrate_mfma: random_operands = 3 reads 8 MiB of scratch behind its first 8192 bytes");
+  if (random_operands == 2 || random_operands == 3) {
+    iters = (iters + 1) / 2 * 2;
+    for (auto k : {reinterpret_cast<const void*>(calib_mfma_lds_kernel<false>), reinterpret_cast<const void*>(calib_mfma_lds_kernel<true>)})
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) {
+        set_error("nf_calibrate_mfma: cannot reserve 128 KB of LDS");
+        return NF_ERR_RUNTIME;
+      }
+  }
   hipStream_t s = (hipStream_t)stream;
   uint64_t* clocks = static_cast<uint64_t*>(scratch);                       // 64 x 2 x 8 bytes
   float* sink = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + 2048);  // 1024 floats
@@ -185,7 +297,11 @@ int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, si
     return NF_ERR_RUNTIME;
   }
   auto launch = [&](int n) {
-    if (fp8) calib_mfma_kernel<true><<<grid, 256, 0, s>>>(n, random_operands, clocks, sink);
+    if (random_operands == 2) calib_mfma_lds_kernel<false><<<grid, 256, 65536, s>>>((n + 1) / 2 * 2, clocks, sink, nullptr);
+    else if (random_operands == 3)
+      calib_mfma_lds_kernel<true><<<grid, 256, 131072, s>>>((n + 1) / 2 * 2, clocks, sink,
+                                                            static_cast<const uint8_t*>(scratch) + 8192);
+    else if (fp8) calib_mfma_kernel<true><<<grid, 256, 0, s>>>(n, random_operands, clocks, sink);
     else calib_mfma_kernel<false><<<grid, 256, 0, s>>>(n, random_operands, clocks, sink);
   };
   launch(std::max(iters / 8, 1));  // warm-up: clocks and power state settle
