@@ -59,6 +59,12 @@ NF_API int nf_move_kv_pages(int req_num, const int32_t* req_idx, const int32_t* 
  * LayerNorm::work (pipeline/include/otherWrapper.cuh:94-102). */
 NF_API int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* weight, int rows, int hidden,
                    float eps, nf_stream_t stream);
+/* nf_rmsnorm_f16 whose result is also written in the form an fp8-weight GEMM takes: out_q [rows,
+ * hidden] e4m3 bytes and row_scale [rows], bit for bit what nf_quantize_rows_e4m3 makes of `out`
+ * (which is written as well), in the same launch.  hidden % 16 == 0, hidden <= 8192.  No counterpart
+ * in the reference (its GEMMs are fp16 only). */
+NF_API int nf_rmsnorm_quantize_e4m3(uint16_t* out, const uint16_t* in, const uint16_t* weight, uint8_t* out_q,
+                                    float* row_scale, int rows, int hidden, float eps, nf_stream_t stream);
 
 /* D = half(alpha * A.B + beta * C), fp16 operands, fp32 accumulate on MFMA.
  * A [M,K] row-major; B [K,N] row-major when b_col_major == 0, [N,K] row-major
@@ -153,7 +159,11 @@ NF_API int nf_dual_swiglu_bf16(const uint16_t* A, const uint16_t* Bgate, const u
  * nf_dual_swiglu_f8_f16: out = half(silu(g) * u) with g = half(a_scale[m] * g_scale[n] * sum_k
  *   Aq[m][k] * Gq[n][k]) and u likewise from Uq, u_scale: nf_dual_swiglu_f16 on fp8 operands
  *   (products rounded to fp16 before SiLU-mul, as there).  nf_dual_swiglu_f8w_f16: the same from
- *   fp16 activations, quantised into `workspace` (nf_gemm_f8w_workspace_bytes(M, K) bytes). */
+ *   fp16 activations, quantised into `workspace` (nf_gemm_f8w_workspace_bytes(M, K) bytes).
+ * nf_gemm_f8q_f16 / nf_dual_swiglu_f8q_f16: nf_gemm_f8w_f16 / nf_dual_swiglu_f8w_f16 on activations
+ *   that are quantised already (Aq, a_scale: by nf_quantize_rows_e4m3 or nf_rmsnorm_quantize_e4m3);
+ *   `workspace` (may be NULL) is the one the f8w form would be given and is used, at the same
+ *   offsets, for the sums of a launch split over K only. */
 /* nf_gemm_f8w_f16 and nf_dual_swiglu_f8w_f16 split launches of at most 256 rows over K, like
  * nf_gemm_f16_ws, when the workspace also has room for the fp32 sums behind the quantised rows:
  * nf_gemm_f8w_split_workspace_bytes(M, N, K) / nf_dual_swiglu_f8w_split_workspace_bytes(M, N, K)
@@ -176,6 +186,12 @@ NF_API int nf_quantize_rows_e4m3(const uint16_t* X, uint8_t* Xq, float* row_scal
 NF_API int nf_gemm_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, const float* b_scale,
                           const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha, float beta,
                           nf_stream_t stream);
+NF_API int nf_gemm_f8q_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, const float* b_scale,
+                           const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha, float beta,
+                           void* workspace, size_t workspace_bytes, nf_stream_t stream);
+NF_API int nf_dual_swiglu_f8q_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Gq, const float* g_scale,
+                                  const uint8_t* Uq, const float* u_scale, uint16_t* out, int M, int N, int K,
+                                  void* workspace, size_t workspace_bytes, nf_stream_t stream);
 NF_API size_t nf_gemm_f8w_workspace_bytes(int M, int K);
 NF_API int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* b_scale, const uint16_t* C,
                            uint16_t* D, int M, int N, int K, float alpha, float beta, void* workspace,

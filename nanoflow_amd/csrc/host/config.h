@@ -63,6 +63,9 @@ struct vortexModelConfig {
     // quantised activations of the fp8-weight GEMMs (one byte per element of the QKV, O, gate/up
     // and down inputs, a scale per row, 256-byte alignment of up to 8 wrappers)
     k_temp_size += (size_t)max_batch_size * (3 * model_hidden_dim + model_ff_dim + 32) / 2 + 8 * 256;
+    // the same form of the two RMSNorm outputs, written by the RMSNorms themselves (a byte per
+    // element, a scale per row, per nano-batch piece)
+    k_temp_size += (size_t)max_batch_size * (2 * model_hidden_dim + 8) / 2 + 12 * 256;
     // fp32 partial sums of GEMM launches split over K: shares x M x N is at most CUs x the largest
     // split tile (256 x 256 x 256 elements = 67 MB) per wrapper, up to 7 wrappers, 256-byte
     // alignment (the fused gate/up pair keeps two sets of sums of 128 x 128 tiles, 34 MB together,

@@ -18,6 +18,15 @@ struct DualWrapper : public OperatorWrapper {
   void set_live_rows(int r) { live_rows = r; }
   int rows() const { return live_rows >= 0 && live_rows < M ? live_rows : M; }
   bool e4m3 = false;
+  // e4m3 weights: the rows of A as e4m3 bytes [M, K] + one fp32 scale per row, when the producer
+  // of A has written them (nf_rmsnorm_quantize_e4m3); the launch then skips its quantiser
+  const uint8_t* a_q = nullptr;
+  const float* a_q_scale = nullptr;
+  bool setQuantizedA(const uint8_t* q, const float* scale) {
+    a_q = q;
+    a_q_scale = scale;
+    return e4m3 && q && scale;
+  }
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
   void setWeightFormat(WeightFormat f) { e4m3 = f == WeightFormat::E4M3; }
@@ -41,6 +50,12 @@ struct DualWrapper : public OperatorWrapper {
       const uint8_t* g = reinterpret_cast<const uint8_t*>(pllm_tensor_b1.ptr);
       const uint8_t* u = reinterpret_cast<const uint8_t*>(pllm_tensor_b2.ptr);
       const size_t so = e4m3WeightScaleOffset((size_t)N, (size_t)K);
+      if (a_q && a_q_scale) {
+        NF_KERNEL_CHECK(nf_dual_swiglu_f8q_f16(a_q, a_q_scale, g, reinterpret_cast<const float*>(g + so), u,
+                                               reinterpret_cast<const float*>(u + so), pllm_tensor_d2.ptr, rows(), N, K,
+                                               workspace, workspace_bytes, stream));
+        return;
+      }
       NF_KERNEL_CHECK(nf_dual_swiglu_f8w_f16(pllm_tensor_a.ptr, g, reinterpret_cast<const float*>(g + so), u,
                                              reinterpret_cast<const float*>(u + so), pllm_tensor_d2.ptr, rows(), N, K,
                                              workspace, workspace_bytes, stream));

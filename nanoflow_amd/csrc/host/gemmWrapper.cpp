@@ -51,6 +51,11 @@ BaseGEMMWrapper* generateGEMM(const std::string& tag, WeightFormat format) {
 void HipGEMMWrapperF8W::work() {
   const uint8_t* bq = reinterpret_cast<const uint8_t*>(pllm_tensor_b.ptr);
   const float* bs = reinterpret_cast<const float*>(bq + e4m3WeightScaleOffset(N, K));
+  if (a_q && a_q_scale) {
+    NF_KERNEL_CHECK(nf_gemm_f8q_f16(a_q, a_q_scale, bq, bs, pllm_tensor_c.ptr, pllm_tensor_d.ptr, (int)rows(), (int)N,
+                                    (int)K, alpha, beta, workspace, workspace_bytes, stream));
+    return;
+  }
   NF_KERNEL_CHECK(nf_gemm_f8w_f16(pllm_tensor_a.ptr, bq, bs, pllm_tensor_c.ptr, pllm_tensor_d.ptr, (int)rows(),
                                   (int)N, (int)K, alpha, beta, workspace, workspace_bytes, stream));
 }

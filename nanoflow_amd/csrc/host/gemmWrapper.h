@@ -57,6 +57,14 @@ struct BaseGEMMWrapper : public OperatorWrapper {
   virtual pllmTensor<ElementOutput> getC() = 0;
   virtual void set_alpha(float alpha_) = 0;
   virtual void set_beta(float beta_) = 0;
+  // Not in the reference's interface: the rows of A as e4m3 bytes [M, K] with one fp32 scale per
+  // row, written by the producer of A (nf_rmsnorm_quantize_e4m3) at the same row positions.  A
+  // wrapper on e4m3 weights then skips its own quantiser launch and returns true; others ignore it.
+  virtual bool setQuantizedA(const uint8_t* a_q, const float* a_scale) {
+    (void)a_q;
+    (void)a_scale;
+    return false;
+  }
   // Not in the reference's interface: C = one row [1, N] added (times beta) to every row of the
   // product, read by the kernel's epilogue.  Takes the place of setC() with the bias replicated
   // over max-batch rows (replicateKQVBias, pipeline/src/pipeline.cu:520-533,1048-1058).
@@ -165,7 +173,14 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
 struct HipGEMMWrapperF8W : public HipGEMMWrapper {
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
+  const uint8_t* a_q = nullptr;   // rows of A quantised by their producer (setQuantizedA), or null
+  const float* a_q_scale = nullptr;
   explicit HipGEMMWrapperF8W(const GemmTag& t) : HipGEMMWrapper(t) {}
+  bool setQuantizedA(const uint8_t* q, const float* scale) override {
+    a_q = q;
+    a_q_scale = scale;
+    return q && scale;
+  }
   void work() override;
   void set_weight(half* blob) override {  // see WeightFormat::E4M3
     pllm_tensor_b = pllmTensor<half>(blob, N, K, PllmLayout::COL_MAJOR);

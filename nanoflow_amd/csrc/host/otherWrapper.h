@@ -55,11 +55,29 @@ public:
   // rows that hold tokens in this iteration (-1: all rows of the input); the rest is left as it was
   int live_rows = -1;
   void set_live_rows(int r) { live_rows = r; }
+  // Not in the reference's interface: the output rows also as e4m3 bytes [rows, hidden] with one
+  // fp32 scale per row, for a consumer GEMM on e4m3 weights (BaseGEMMWrapper::setQuantizedA); the
+  // fp16 output is written all the same.  Hidden sizes the fused kernel does not take are refused.
+  uint8_t* output_q = nullptr;
+  float* output_q_scale = nullptr;
+  static bool canQuantize() { return ModelConfig.model_hidden_dim % 16 == 0 && ModelConfig.model_hidden_dim <= 8192; }
+  bool setQuantOutput(uint8_t* q, float* scale) {
+    if (!canQuantize() || !q || !scale) return false;
+    output_q = q;
+    output_q_scale = scale;
+    return true;
+  }
   void work() override {
     assert(pllm_tensor_input.dim2 == (size_t)ModelConfig.model_hidden_dim);
     const int all = (int)(input_size / ModelConfig.model_hidden_dim);
-    NF_KERNEL_CHECK(nf_rmsnorm_f16(output, input, weight, live_rows >= 0 && live_rows < all ? live_rows : all,
-                                   ModelConfig.model_hidden_dim, ModelConfig.rms_norm_eps, stream));
+    const int rows = live_rows >= 0 && live_rows < all ? live_rows : all;
+    if (output_q) {
+      NF_KERNEL_CHECK(nf_rmsnorm_quantize_e4m3(output, input, weight, output_q, output_q_scale, rows,
+                                               ModelConfig.model_hidden_dim, ModelConfig.rms_norm_eps, stream));
+      return;
+    }
+    NF_KERNEL_CHECK(nf_rmsnorm_f16(output, input, weight, rows, ModelConfig.model_hidden_dim,
+                                   ModelConfig.rms_norm_eps, stream));
   }
 };
 

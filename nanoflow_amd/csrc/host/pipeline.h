@@ -80,6 +80,23 @@ protected:
     return true;
   }
 
+  // e4m3 weights: the RMSNorm in front of the QKV and of the gate/up projection writes its rows
+  // as e4m3 bytes + one fp32 scale per row as well, into a [rows, hidden] image carved from the tmp
+  // buffer, and the GEMMs read their rows there instead of launching a quantiser of their own.
+  struct QuantRows {
+    uint8_t* q = nullptr;
+    float* scale = nullptr;
+    QuantRows at(size_t row) const { return {q + row * (size_t)ModelConfig.model_hidden_dim, scale + row}; }
+    explicit operator bool() const { return q != nullptr; }
+  };
+  QuantRows allocQuantRows(size_t rows) {
+    if (weight_format != WeightFormat::E4M3 || !LayerNorm::canQuantize() || rows == 0) return {};
+    QuantRows r;
+    r.q = static_cast<uint8_t*>(tmpBufferM.allocBytes(rows * (size_t)ModelConfig.model_hidden_dim));
+    r.scale = static_cast<float*>(tmpBufferM.allocBytes(rows * sizeof(float)));
+    return r;
+  }
+
   // hipGraph replay of an iteration.  Everything that shapes a launch (grid sizes, row counts,
   // which operators are skipped) is a function of the configuration and of a few integers of
   // the update data; those integers form the signature a captured graph is filed under.  A

@@ -322,6 +322,15 @@ void LocalPipeline::ScheduleInit() {
     gemms[i]->setWorkspace(tmpBufferM.allocBytes(gemms[i]->workspaceBytes()), gemms[i]->workspaceBytes());
   dual1.setWorkspace(tmpBufferM.allocBytes(dual1.workspaceBytes()), dual1.workspaceBytes());
   dual2.setWorkspace(tmpBufferM.allocBytes(dual2.workspaceBytes()), dual2.workspaceBytes());
+  // e4m3 weights: the RMSNorms hand their consumers quantised rows
+  if (const QuantRows q = allocQuantRows(KQV1->M); q && KQV1->setQuantizedA(q.q, q.scale))
+    layerNormAttention1.setQuantOutput(q.q, q.scale);
+  if (const QuantRows q = allocQuantRows(KQV2->M); q && KQV2->setQuantizedA(q.q, q.scale))
+    layerNormAttention2.setQuantOutput(q.q, q.scale);
+  if (const QuantRows q = allocQuantRows(dual1.M); q && dual1.setQuantizedA(q.q, q.scale))
+    layerNormFFN1.setQuantOutput(q.q, q.scale);
+  if (const QuantRows q = allocQuantRows(dual2.M); q && dual2.setQuantizedA(q.q, q.scale))
+    layerNormFFN2.setQuantOutput(q.q, q.scale);
   NF_LOG_INFO("allocated num: %zu", tmpBufferM.getAllocation());
 }
 

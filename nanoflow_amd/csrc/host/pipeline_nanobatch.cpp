@@ -249,6 +249,25 @@ void Pipeline::ScheduleInit() {
     gemms[i]->setWorkspace(tmpBufferM.allocBytes(gemms[i]->workspaceBytes()), gemms[i]->workspaceBytes());
   dual1.setWorkspace(tmpBufferM.allocBytes(dual1.workspaceBytes()), dual1.workspaceBytes());
   dual2.setWorkspace(tmpBufferM.allocBytes(dual2.workspaceBytes()), dual2.workspaceBytes());
+  // e4m3 weights: the RMSNorms hand their consumers quantised rows (one image of all T rows for
+  // the attention side: layerNormAttention1 covers the rows of KQV1 and KQV2)
+  if (const QuantRows q = allocQuantRows(T)) {
+    const size_t row0[4] = {0, k[0], k[0] + k[1], k[0] + k[1] + k[2]};
+    bool all = true;
+    for (int i = 0; i < 4; ++i)
+      if (k[i] > 0) all &= KQV_ptrs[i]->setQuantizedA(q.at(row0[i]).q, q.at(row0[i]).scale);
+    if (all) {
+      layerNormAttention1.setQuantOutput(q.q, q.scale);
+      if (k[2] > 0) layerNormAttention2_1.setQuantOutput(q.at(row0[2]).q, q.at(row0[2]).scale);
+      if (k[3] > 0) layerNormAttention2_2.setQuantOutput(q.at(row0[3]).q, q.at(row0[3]).scale);
+    } else {
+      for (int i = 0; i < 4; ++i) KQV_ptrs[i]->setQuantizedA(nullptr, nullptr);
+    }
+  }
+  if (const QuantRows q = allocQuantRows(dual1.M); q && dual1.setQuantizedA(q.q, q.scale))
+    layerNormFFN1.setQuantOutput(q.q, q.scale);
+  if (const QuantRows q = allocQuantRows(dual2.M); q && dual2.setQuantizedA(q.q, q.scale))
+    layerNormFFN2.setQuantOutput(q.q, q.scale);
   NF_LOG_INFO("allocated num: %zu", tmpBufferM.getAllocation());
 }
 

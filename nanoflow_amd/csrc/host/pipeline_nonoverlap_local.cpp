@@ -236,6 +236,11 @@ void NonOverlapLocalPipeline::ScheduleInit() {
   for (int i = 0; i < gemmNum; ++i)
     gemms[i]->setWorkspace(tmpBufferM.allocBytes(gemms[i]->workspaceBytes()), gemms[i]->workspaceBytes());
   dual.setWorkspace(tmpBufferM.allocBytes(dual.workspaceBytes()), dual.workspaceBytes());
+  // e4m3 weights: the two RMSNorms hand their consumers quantised rows
+  if (const QuantRows qa = allocQuantRows(KQV->M); qa && KQV->setQuantizedA(qa.q, qa.scale))
+    layerNormAttention.setQuantOutput(qa.q, qa.scale);
+  if (const QuantRows qf = allocQuantRows(dual.M); qf && dual.setQuantizedA(qf.q, qf.scale))
+    layerNormFFN.setQuantOutput(qf.q, qf.scale);
   NF_LOG_INFO("allocated %zu halfs", tmpBufferM.getAllocation());
 }
 

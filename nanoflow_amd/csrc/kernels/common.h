@@ -76,6 +76,38 @@ __device__ __forceinline__ float h2f_bits(uint32_t bits16) {
 __device__ __forceinline__ uint32_t f2h_bits(float f) {
   return (uint32_t)__half_as_ushort(__float2half_rn(f));
 }
+
+// Round-to-nearest-even OCP e4m3 (bias 7, no infinities, max 448), saturating.
+__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  const float a = fabsf(x);
+  uint32_t code;
+  if (!(a < 464.f)) {
+    code = 0x7Eu;                                // 448; also where NaN ends up
+  } else if (a < 0.015625f) {
+    code = (uint32_t)(int)rintf(a * 512.f);      // subnormals: steps of 2^-9 (8 -> smallest normal)
+  } else {
+    uint32_t ua = __float_as_uint(a);
+    ua += 0x7FFFFu + ((ua >> 20) & 1u);          // RNE at mantissa bit 20
+    code = (((ua >> 23) - 120u) << 3) | ((ua >> 20) & 7u);
+  }
+  return sign | code;
+}
+// Eight halves (a 16-byte chunk) divided by s and rounded to e4m3: 8 bytes.
+__device__ __forceinline__ u32x2 quantize_chunk_e4m3(const u32x4& v, float s) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  uint32_t q[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    q[2 * i] = f32_to_e4m3(h2f_bits(w[i] & 0xffffu) / s);
+    q[2 * i + 1] = f32_to_e4m3(h2f_bits(w[i] >> 16) / s);
+  }
+  u32x2 o;
+  o.x = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+  o.y = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
+  return o;
+}
 // Two floats rounded to nearest-even fp16, lo in bits 15:0 (one v_cvt_pk_f16_f32 on gfx950).
 __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
   typedef float f32x2_t __attribute__((ext_vector_type(2)));

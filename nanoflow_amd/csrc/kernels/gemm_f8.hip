@@ -34,24 +34,10 @@ struct F8Smem {
   static constexpr size_t bytes = (size_t)stages * stage_bytes;
 };
 
-// Round-to-nearest-even OCP e4m3 (bias 7, no infinities, max 448), saturating.
-__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
-  const uint32_t u = __float_as_uint(x);
-  const uint32_t sign = (u >> 24) & 0x80u;
-  const float a = fabsf(x);
-  uint32_t code;
-  if (!(a < 464.f)) {
-    code = 0x7Eu;                                // 448; also where NaN ends up
-  } else if (a < 0.015625f) {
-    code = (uint32_t)(int)rintf(a * 512.f);      // subnormals: steps of 2^-9 (8 -> smallest normal)
-  } else {
-    uint32_t ua = __float_as_uint(a);
-    ua += 0x7FFFFu + ((ua >> 20) & 1u);          // RNE at mantissa bit 20
-    code = (((ua >> 23) - 120u) << 3) | ((ua >> 20) & 7u);
-  }
-  return sign | code;
-}
-
+// One workgroup per row.  kChunks > 0: the row (at most kChunks x 256 chunks of 8 halves) stays in
+// registers between the maximum and the rounding, so it is read once; kChunks == 0: any length, the
+// second pass reads the row again.
+template <int kChunks>
 __global__ __launch_bounds__(256) void quantize_rows_e4m3_kernel(const uint16_t* __restrict__ X,
                                                                  uint8_t* __restrict__ Xq,
                                                                  float* __restrict__ scale, int K) {
@@ -59,15 +45,26 @@ __global__ __launch_bounds__(256) void quantize_rows_e4m3_kernel(const uint16_t*
   const int row = blockIdx.x, tid = threadIdx.x;
   const u32x4* src = reinterpret_cast<const u32x4*>(X + (size_t)row * K);
   const int chunks = K / 8;
+  constexpr int kHeld = kChunks > 0 ? kChunks : 1;
+  u32x4 held[kHeld];
   float amax = 0.f;
-  for (int c = tid; c < chunks; c += 256) {
-    const u32x4 v = src[c];
+  auto chunk_max = [&](const u32x4& v) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       amax = fmaxf(amax, fabsf(h2f_bits(w[i] & 0xffffu)));
       amax = fmaxf(amax, fabsf(h2f_bits(w[i] >> 16)));
     }
+  };
+  if constexpr (kChunks > 0) {
+#pragma unroll
+    for (int u = 0; u < kChunks; ++u)
+      if (tid + u * 256 < chunks) held[u] = src[tid + u * 256];
+#pragma unroll
+    for (int u = 0; u < kChunks; ++u)
+      if (tid + u * 256 < chunks) chunk_max(held[u]);
+  } else {
+    for (int c = tid; c < chunks; c += 256) chunk_max(src[c]);
   }
 #pragma unroll
   for (int m = 32; m > 0; m >>= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
@@ -77,19 +74,12 @@ __global__ __launch_bounds__(256) void quantize_rows_e4m3_kernel(const uint16_t*
   const float s = amax > 0.f ? amax / 448.f : 1.f;
   if (tid == 0) scale[row] = s;
   u32x2* dst = reinterpret_cast<u32x2*>(Xq + (size_t)row * K);
-  for (int c = tid; c < chunks; c += 256) {
-    const u32x4 v = src[c];
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-    uint32_t q[8];
+  if constexpr (kChunks > 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      q[2 * i] = f32_to_e4m3(h2f_bits(w[i] & 0xffffu) / s);
-      q[2 * i + 1] = f32_to_e4m3(h2f_bits(w[i] >> 16) / s);
-    }
-    u32x2 o;
-    o.x = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
-    o.y = q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24);
-    dst[c] = o;
+    for (int u = 0; u < kChunks; ++u)
+      if (tid + u * 256 < chunks) dst[tid + u * 256] = quantize_chunk_e4m3(held[u], s);
+  } else {
+    for (int c = tid; c < chunks; c += 256) dst[c] = quantize_chunk_e4m3(src[c], s);
   }
 }
 
@@ -600,7 +590,10 @@ int nf_quantize_rows_e4m3(const uint16_t* X, uint8_t* Xq, float* row_scale, int 
   NF_REQUIRE(M == 0 || (X && Xq && row_scale), "nf_quantize_rows_e4m3: null pointer");
   NF_REQUIRE(((uintptr_t)X | (uintptr_t)Xq) % 16 == 0, "nf_quantize_rows_e4m3: operands must be 16-byte aligned");
   if (M == 0) return NF_OK;
-  quantize_rows_e4m3_kernel<<<M, 256, 0, (hipStream_t)stream>>>(X, Xq, row_scale, K);
+  hipStream_t s = (hipStream_t)stream;
+  if (K <= 4 * 2048) quantize_rows_e4m3_kernel<4><<<M, 256, 0, s>>>(X, Xq, row_scale, K);
+  else if (K <= 16 * 2048) quantize_rows_e4m3_kernel<16><<<M, 256, 0, s>>>(X, Xq, row_scale, K);
+  else quantize_rows_e4m3_kernel<0><<<M, 256, 0, s>>>(X, Xq, row_scale, K);
   return check_launch("quantize_rows_e4m3 launch");
 }
 
@@ -666,6 +659,27 @@ size_t nf_gemm_f8w_workspace_bytes(int M, int K) {
   return ((size_t)M * K + 255) / 256 * 256 + (size_t)M * sizeof(float);
 }
 
+// The GEMM on rows that are quantised already: split over K when the launch has few rows against a
+// narrow N and the workspace holds the partial sums behind the place of the quantised rows.
+static int gemm_f8q(const uint8_t* Aq, const float* sa, const uint8_t* Bq, const float* b_scale, const uint16_t* C,
+                    uint16_t* D, int M, int N, int K, float alpha, float beta, void* workspace, size_t workspace_bytes,
+                    nf_stream_t stream) {
+  int k_per = 0;
+  const int shares = N > 0 && N % 8 == 0 && K % 16 == 0 ? splitk_plan_f8(M, N, K, false, &k_per) : 1;
+  const size_t p_at = (nf_gemm_f8w_workspace_bytes(M, K) + 255) / 256 * 256;
+  if (shares >= 2 && workspace && (uintptr_t)workspace % 16 == 0 &&
+      workspace_bytes >= p_at + (size_t)shares * M * N * sizeof(float) && Bq && b_scale && D &&
+      ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull &&
+      (beta == 0.f || C) && ((uintptr_t)Bq | (uintptr_t)b_scale) % 16 == 0 && ((uintptr_t)D | (uintptr_t)C) % 8 == 0) {
+    float* P = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p_at);
+    hipStream_t s = (hipStream_t)stream;
+    if (M <= 64)
+      return launch_splitk_f8<64, 256, 1, 4, false>(Aq, Bq, nullptr, sa, b_scale, nullptr, C, D, M, N, K, alpha, beta, shares, k_per, P, s);
+    return launch_splitk_f8<128, 128, 2, 2, false>(Aq, Bq, nullptr, sa, b_scale, nullptr, C, D, M, N, K, alpha, beta, shares, k_per, P, s);
+  }
+  return nf_gemm_f8_f16(Aq, sa, Bq, b_scale, C, D, M, N, K, alpha, beta, stream);
+}
+
 int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* b_scale, const uint16_t* C,
                     uint16_t* D, int M, int N, int K, float alpha, float beta, void* workspace,
                     size_t workspace_bytes, nf_stream_t stream) {
@@ -681,20 +695,15 @@ int nf_gemm_f8w_f16(const uint16_t* A, const uint8_t* Bq, const float* b_scale, 
   float* sa = reinterpret_cast<float*>(Aq + ((size_t)M * K + 255) / 256 * 256);
   int rc = nf_quantize_rows_e4m3(A, Aq, sa, M, K, stream);
   if (rc) return rc;
-  // few rows against a narrow N: split over K when the workspace also holds the partial sums
-  int k_per = 0;
-  const int shares = N > 0 && N % 8 == 0 && K % 16 == 0 ? splitk_plan_f8(M, N, K, false, &k_per) : 1;
-  const size_t p_at = (need + 255) / 256 * 256;
-  if (shares >= 2 && workspace_bytes >= p_at + (size_t)shares * M * N * sizeof(float) && Bq && b_scale && D &&
-      ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull &&
-      (beta == 0.f || C) && ((uintptr_t)Bq | (uintptr_t)b_scale) % 16 == 0 && ((uintptr_t)D | (uintptr_t)C) % 8 == 0) {
-    float* P = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p_at);
-    hipStream_t s = (hipStream_t)stream;
-    if (M <= 64)
-      return launch_splitk_f8<64, 256, 1, 4, false>(Aq, Bq, nullptr, sa, b_scale, nullptr, C, D, M, N, K, alpha, beta, shares, k_per, P, s);
-    return launch_splitk_f8<128, 128, 2, 2, false>(Aq, Bq, nullptr, sa, b_scale, nullptr, C, D, M, N, K, alpha, beta, shares, k_per, P, s);
-  }
-  return nf_gemm_f8_f16(Aq, sa, Bq, b_scale, C, D, M, N, K, alpha, beta, stream);
+  return gemm_f8q(Aq, sa, Bq, b_scale, C, D, M, N, K, alpha, beta, workspace, workspace_bytes, stream);
+}
+
+int nf_gemm_f8q_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, const float* b_scale,
+                    const uint16_t* C, uint16_t* D, int M, int N, int K, float alpha, float beta, void* workspace,
+                    size_t workspace_bytes, nf_stream_t stream) {
+  NF_REQUIRE(M >= 0 && K > 0, "nf_gemm_f8q_f16: bad shape M=%d K=%d", M, K);
+  if (M == 0) return NF_OK;
+  return gemm_f8q(Aq, a_scale, Bq, b_scale, C, D, M, N, K, alpha, beta, workspace, workspace_bytes, stream);
 }
 
 size_t nf_gemm_f8w_split_workspace_bytes(int M, int N, int K) {
@@ -725,6 +734,26 @@ size_t nf_dual_swiglu_f8w_split_workspace_bytes_upto(int max_M, int N, int K) {
   return need;
 }
 
+static int dual_swiglu_f8q(const uint8_t* Aq, const float* sa, const uint8_t* Gq, const float* g_scale,
+                           const uint8_t* Uq, const float* u_scale, uint16_t* out, int M, int N, int K, void* workspace,
+                           size_t workspace_bytes, nf_stream_t stream) {
+  int k_per = 0;
+  const int shares = N > 0 && N % 8 == 0 && K % 16 == 0 ? splitk_plan_f8(M, N, K, true, &k_per) : 1;
+  const size_t p_at = (nf_gemm_f8w_workspace_bytes(M, K) + 255) / 256 * 256;
+  if (shares >= 2 && workspace && (uintptr_t)workspace % 16 == 0 &&
+      workspace_bytes >= p_at + (size_t)2 * shares * M * N * sizeof(float) && Gq && g_scale && Uq &&
+      ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull &&
+      u_scale && out &&
+      ((uintptr_t)Gq | (uintptr_t)Uq | (uintptr_t)g_scale | (uintptr_t)u_scale) % 16 == 0 && (uintptr_t)out % 8 == 0) {
+    float* P = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p_at);
+    hipStream_t s = (hipStream_t)stream;
+    if (M <= 64)
+      return launch_splitk_f8<64, 128, 2, 2, true>(Aq, Gq, Uq, sa, g_scale, u_scale, nullptr, out, M, N, K, 1.f, 0.f, shares, k_per, P, s);
+    return launch_splitk_f8<128, 128, 2, 2, true>(Aq, Gq, Uq, sa, g_scale, u_scale, nullptr, out, M, N, K, 1.f, 0.f, shares, k_per, P, s);
+  }
+  return nf_dual_swiglu_f8_f16(Aq, sa, Gq, g_scale, Uq, u_scale, out, M, N, K, stream);
+}
+
 int nf_dual_swiglu_f8w_f16(const uint16_t* A, const uint8_t* Gq, const float* g_scale, const uint8_t* Uq,
                            const float* u_scale, uint16_t* out, int M, int N, int K, void* workspace,
                            size_t workspace_bytes, nf_stream_t stream) {
@@ -740,20 +769,15 @@ int nf_dual_swiglu_f8w_f16(const uint16_t* A, const uint8_t* Gq, const float* g_
   float* sa = reinterpret_cast<float*>(Aq + ((size_t)M * K + 255) / 256 * 256);
   int rc = nf_quantize_rows_e4m3(A, Aq, sa, M, K, stream);
   if (rc) return rc;
-  int k_per = 0;
-  const int shares = N > 0 && N % 8 == 0 && K % 16 == 0 ? splitk_plan_f8(M, N, K, true, &k_per) : 1;
-  const size_t p_at = (need + 255) / 256 * 256;
-  if (shares >= 2 && workspace_bytes >= p_at + (size_t)2 * shares * M * N * sizeof(float) && Gq && g_scale && Uq &&
-      ((size_t)N + 256) * ((size_t)K + 1024) < 0xFFFFFF00ull &&
-      u_scale && out &&
-      ((uintptr_t)Gq | (uintptr_t)Uq | (uintptr_t)g_scale | (uintptr_t)u_scale) % 16 == 0 && (uintptr_t)out % 8 == 0) {
-    float* P = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p_at);
-    hipStream_t s = (hipStream_t)stream;
-    if (M <= 64)
-      return launch_splitk_f8<64, 128, 2, 2, true>(Aq, Gq, Uq, sa, g_scale, u_scale, nullptr, out, M, N, K, 1.f, 0.f, shares, k_per, P, s);
-    return launch_splitk_f8<128, 128, 2, 2, true>(Aq, Gq, Uq, sa, g_scale, u_scale, nullptr, out, M, N, K, 1.f, 0.f, shares, k_per, P, s);
-  }
-  return nf_dual_swiglu_f8_f16(Aq, sa, Gq, g_scale, Uq, u_scale, out, M, N, K, stream);
+  return dual_swiglu_f8q(Aq, sa, Gq, g_scale, Uq, u_scale, out, M, N, K, workspace, workspace_bytes, stream);
+}
+
+int nf_dual_swiglu_f8q_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Gq, const float* g_scale,
+                           const uint8_t* Uq, const float* u_scale, uint16_t* out, int M, int N, int K, void* workspace,
+                           size_t workspace_bytes, nf_stream_t stream) {
+  NF_REQUIRE(M >= 0 && K > 0, "nf_dual_swiglu_f8q_f16: bad shape M=%d K=%d", M, K);
+  if (M == 0) return NF_OK;
+  return dual_swiglu_f8q(Aq, a_scale, Gq, g_scale, Uq, u_scale, out, M, N, K, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -35,11 +35,17 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const int32_t* __restr
 
 // One workgroup per row.  Two passes over the row (second pass hits L1/L2); fp32 math,
 // single rounding on output.
+// kQuant: the rounded row (at most 4 x 256 chunks of 8 halves: hidden <= 8192) stays in registers
+// and is also written as e4m3 bytes with one fp32 scale per row, exactly what the row quantiser
+// makes of the fp16 output: the fp8-weight GEMM that follows needs no quantiser launch.
+template <bool kQuant>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
                                                       const u32x4* __restrict__ in,
                                                       const u32x4* __restrict__ w, int vec_per_row,
-                                                      float inv_n, float eps) {
+                                                      float inv_n, float eps, uint8_t* __restrict__ q_out,
+                                                      float* __restrict__ q_scale) {
   __shared__ float s_part[4];
+  __shared__ float s_max[4];
   const int r = blockIdx.x;
   const u32x4* x = in + (long long)r * vec_per_row;
   u32x4* y = out + (long long)r * vec_per_row;
@@ -50,7 +56,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float a = h2f_bits(p[j] & 0xffffu), b = h2f_bits(p[j] >> 16);
-      ss += a * a + b * b;
+      ss = fmaf(a, a, ss);
+      ss = fmaf(b, b, ss);
     }
   }
   ss = wave_sum(ss);
@@ -58,7 +65,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
   __syncthreads();
   const float tot = s_part[0] + s_part[1] + s_part[2] + s_part[3];
   const float scale = 1.0f / sqrtf(tot * inv_n + eps);
-  for (int i = threadIdx.x; i < vec_per_row; i += 256) {
+  u32x4 held[kQuant ? 4 : 1];
+  float amax = 0.f;
+  auto normalise = [&](int i) {  // chunk i of the row: scaled, weighted, rounded once, stored
     u32x4 v = x[i];
     u32x4 g = w[i];
     const uint32_t p[4] = {v.x, v.y, v.z, v.w};
@@ -69,8 +78,34 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
       float a = h2f_bits(p[j] & 0xffffu) * scale * h2f_bits(q[j] & 0xffffu);
       float b = h2f_bits(p[j] >> 16) * scale * h2f_bits(q[j] >> 16);
       o[j] = f2h_bits(a) | (f2h_bits(b) << 16);
+      if constexpr (kQuant) {
+        amax = fmaxf(amax, fabsf(h2f_bits(o[j] & 0xffffu)));
+        amax = fmaxf(amax, fabsf(h2f_bits(o[j] >> 16)));
+      }
     }
-    y[i] = u32x4{o[0], o[1], o[2], o[3]};
+    const u32x4 yv = u32x4{o[0], o[1], o[2], o[3]};
+    y[i] = yv;
+    return yv;
+  };
+  if constexpr (kQuant) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if ((int)threadIdx.x + k * 256 < vec_per_row) held[k] = normalise(threadIdx.x + k * 256);
+  } else {
+    for (int i = threadIdx.x; i < vec_per_row; i += 256) normalise(i);
+  }
+  if constexpr (kQuant) {
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) amax = fmaxf(amax, __shfl_xor(amax, m, 64));
+    if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    const float s = amax > 0.f ? amax / 448.f : 1.f;
+    if (threadIdx.x == 0) q_scale[r] = s;
+    u32x2* dst = reinterpret_cast<u32x2*>(q_out + (size_t)r * vec_per_row * 8);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if ((int)threadIdx.x + k * 256 < vec_per_row) dst[threadIdx.x + k * 256] = quantize_chunk_e4m3(held[k], s);
   }
 }
 
@@ -290,10 +325,25 @@ int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* weight, in
              "nf_rmsnorm_f16: hidden=%d must be a positive multiple of 8 (rows=%d)", hidden, rows);
   if (rows == 0) return NF_OK;
   NF_REQUIRE(out && in && weight, "nf_rmsnorm_f16: null pointer");
-  rmsnorm_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(
+  rmsnorm_kernel<false><<<rows, 256, 0, (hipStream_t)stream>>>(
       reinterpret_cast<u32x4*>(out), reinterpret_cast<const u32x4*>(in),
-      reinterpret_cast<const u32x4*>(weight), hidden / 8, 1.0f / (float)hidden, eps);
+      reinterpret_cast<const u32x4*>(weight), hidden / 8, 1.0f / (float)hidden, eps, nullptr, nullptr);
   return check_launch("nf_rmsnorm_f16");
+}
+
+int nf_rmsnorm_quantize_e4m3(uint16_t* out, const uint16_t* in, const uint16_t* weight, uint8_t* out_q,
+                             float* row_scale, int rows, int hidden, float eps, nf_stream_t stream) {
+  NF_REQUIRE(rows >= 0 && hidden > 0 && hidden % 16 == 0 && hidden <= 8192,
+             "nf_rmsnorm_quantize_e4m3: hidden=%d must be a positive multiple of 16, at most 8192 (rows=%d)", hidden,
+             rows);
+  if (rows == 0) return NF_OK;
+  NF_REQUIRE(out && in && weight && out_q && row_scale, "nf_rmsnorm_quantize_e4m3: null pointer");
+  NF_REQUIRE(((uintptr_t)out | (uintptr_t)in | (uintptr_t)weight | (uintptr_t)out_q) % 16 == 0,
+             "nf_rmsnorm_quantize_e4m3: operands must be 16-byte aligned");
+  rmsnorm_kernel<true><<<rows, 256, 0, (hipStream_t)stream>>>(
+      reinterpret_cast<u32x4*>(out), reinterpret_cast<const u32x4*>(in),
+      reinterpret_cast<const u32x4*>(weight), hidden / 8, 1.0f / (float)hidden, eps, out_q, row_scale);
+  return check_launch("nf_rmsnorm_quantize_e4m3");
 }
 
 int nf_argmax_f16(const uint16_t* logits, uint16_t* max_vals, int32_t* argmax, int rows, int cols,

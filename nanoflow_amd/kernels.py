@@ -26,6 +26,7 @@ SYMBOLS = [
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
     "nf_calibrate_mfma", "nf_calibrate_hbm_read", "nf_calibrate_paged_read",
     "nf_gemm_f16_noalloc", "nf_gemm_noalloc_scratch_bytes",
+    "nf_rmsnorm_quantize_e4m3", "nf_gemm_f8q_f16", "nf_dual_swiglu_f8q_f16",
 ]
 
 
@@ -76,6 +77,9 @@ def lib() -> C.CDLL:
             getattr(l, name).restype = sz
             getattr(l, name).argtypes = [i32, i32, i32]
         l.nf_quantize_weight_e4m3.argtypes = [vp, vp, vp, i32, i32, vp]
+        l.nf_rmsnorm_quantize_e4m3.argtypes = [vp, vp, vp, vp, vp, i32, i32, f32, vp]
+        l.nf_gemm_f8q_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, f32, f32, vp, C.c_size_t, vp]
+        l.nf_dual_swiglu_f8q_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, C.c_size_t, vp]
         l.nf_dual_swiglu_f8_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp]
         l.nf_dual_swiglu_f8w_f16.argtypes = [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp, C.c_size_t, vp]
         l.nf_move_kv_pages.argtypes = [i32, vp, vp, vp, vp, vp, sz, i32, vp]
@@ -141,6 +145,18 @@ def rmsnorm(x, w, eps=1e-5, out=None):
     out = torch.empty_like(x) if out is None else out
     _check(lib().nf_rmsnorm_f16(_p(out), _p(x), _p(w), rows, H, eps, _stream()), "nf_rmsnorm_f16")
     return out
+
+
+def rmsnorm_quantize_e4m3(x, w, eps=1e-5):
+    """(fp16 RMSNorm output, its e4m3 bytes, fp32 row scales) from one launch."""
+    _f16(x); _f16(w)
+    rows, H = x.shape
+    out = torch.empty_like(x)
+    q = torch.empty((rows, H), dtype=torch.uint8, device=x.device)
+    scale = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    _check(lib().nf_rmsnorm_quantize_e4m3(_p(out), _p(x), _p(w), _p(q), _p(scale), rows, H, eps, _stream()),
+           "nf_rmsnorm_quantize_e4m3")
+    return out, q, scale
 
 
 def _elem(t, dtype):
@@ -268,6 +284,31 @@ def gemm_f8w(A, Bq_nk, b_scale, Cmat=None, alpha=1.0, beta=0.0, out=None, worksp
     _check(lib().nf_gemm_f8w_f16(_p(A), _p(Bq_nk), _p(b_scale), _p(Cmat), _p(out), M, N, K, alpha, beta,
                                  _p(workspace), workspace.numel() * workspace.element_size(), _stream()),
            "nf_gemm_f8w_f16")
+    return out
+
+
+def gemm_f8q(Aq, a_scale, Bq_nk, b_scale, Cmat=None, alpha=1.0, beta=0.0, out=None, workspace=None):
+    """nf_gemm_f8w_f16 on rows that are quantised already; the workspace only holds the sums of a split over K."""
+    M, K = Aq.shape
+    N = Bq_nk.shape[0]
+    need = lib().nf_gemm_f8w_split_workspace_bytes(M, N, K)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=Aq.device)
+    out = torch.empty((M, N), dtype=torch.float16, device=Aq.device) if out is None else out
+    _check(lib().nf_gemm_f8q_f16(_p(Aq), _p(a_scale), _p(Bq_nk), _p(b_scale), _p(Cmat), _p(out), M, N, K, alpha, beta,
+                                 _p(workspace), workspace.numel(), _stream()), "nf_gemm_f8q_f16")
+    return out
+
+
+def dual_swiglu_f8q(Aq, a_scale, Gq, g_scale, Uq, u_scale, out=None, workspace=None):
+    M, Kd = Aq.shape
+    N = Gq.shape[0]
+    need = lib().nf_dual_swiglu_f8w_split_workspace_bytes(M, N, Kd)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=Aq.device)
+    out = torch.empty((M, N), dtype=torch.float16, device=Aq.device) if out is None else out
+    _check(lib().nf_dual_swiglu_f8q_f16(_p(Aq), _p(a_scale), _p(Gq), _p(g_scale), _p(Uq), _p(u_scale), _p(out), M, N,
+                                        Kd, _p(workspace), workspace.numel(), _stream()), "nf_dual_swiglu_f8q_f16")
     return out
 
 

@@ -363,7 +363,9 @@ def _quantize_weights_nk(W):
     return q, sc
 
 
-@pytest.mark.parametrize("M,K_", [(1, 16), (5, 4096), (33, 144), (64, 28672)])
+# row lengths on both sides of what the quantiser keeps in registers (8192 and 32768 halves)
+@pytest.mark.parametrize("M,K_", [(1, 16), (5, 4096), (33, 144), (64, 28672), (7, 8192), (6, 8208), (9, 14336),
+                                  (4, 32768), (3, 32784), (3, 40960)])
 def test_quantize_rows_e4m3_bit_exact(K, oracle, M, K_):
     rng = np.random.default_rng(M * 7 + K_)
     X = (rng.normal(0, 1, (M, K_)) * rng.uniform(0.01, 20, (M, 1))).astype(np.float16)
@@ -506,6 +508,46 @@ def test_dual_swiglu_f8w_split_over_k_matches_oracle(K, oracle, M, N, K_):
     assert_close(got, ref, 2 * RTOL, what="split-K fp8 gate/up pair")       # two fp16 roundings before SiLU-mul
     small = torch.empty(l.nf_gemm_f8w_workspace_bytes(M, K_), dtype=torch.uint8, device="cuda")
     assert_close(host(K.dual_swiglu_f8w(dev(A), Gq, sg, Uq, su, workspace=small)), ref, 2 * RTOL, what="unsplit pair")
+
+
+@pytest.mark.parametrize("rows,H", [(1, 16), (5, 4096), (130, 8192), (33, 1040), (64, 2048)])
+def test_rmsnorm_quantize_is_rmsnorm_then_the_row_quantiser(K, oracle, rows, H):
+    """The fused launch writes the fp16 output of nf_rmsnorm_f16 bit for bit, and the e4m3 bytes and
+    row scales that nf_quantize_rows_e4m3 makes of it (the oracle's quantiser applied to the output)."""
+    rng = np.random.default_rng(rows + H)
+    x = (rng.normal(0, 1, (rows, H)) * rng.uniform(0.01, 30, (rows, 1))).astype(np.float16)
+    if rows > 2:
+        x[2] = 0                                   # an all-zero row: output 0, scale 1, codes 0
+    w = (1 + rng.normal(0, 0.1, H)).astype(np.float16)
+    y = K.rmsnorm(dev(x), dev(w))
+    out, q, s = K.rmsnorm_quantize_e4m3(dev(x), dev(w))
+    assert np.array_equal(host(out).view(np.uint16), host(y).view(np.uint16))
+    q_ref, s_ref = oracle.quantize_rows_e4m3(host(y))
+    assert np.array_equal(host(s), s_ref)
+    assert np.array_equal(host(q), q_ref)
+    assert_close(host(out), oracle.rmsnorm(x, w), what="rmsnorm in the fused launch")
+
+
+def test_rmsnorm_quantize_refuses_rows_it_cannot_hold(K):
+    from nanoflow_amd import kernels
+    x = torch.zeros((2, 8208), dtype=torch.float16, device="cuda")
+    with pytest.raises(kernels.NanoflowKernelError, match="8192"):
+        K.rmsnorm_quantize_e4m3(x, torch.ones(8208, dtype=torch.float16, device="cuda"))
+
+
+@pytest.mark.parametrize("M,N,K_", [(16, 6144, 4096), (200, 1160, 4112), (700, 1024, 4096)])
+def test_f8q_entries_equal_the_f8w_entries_on_prequantised_rows(K, M, N, K_):
+    """nf_gemm_f8q_f16 / nf_dual_swiglu_f8q_f16 take rows that are quantised already: same bits as the
+    f8w entries that quantise them themselves, split over K (few rows) or not."""
+    rng = np.random.default_rng(M + N + 3)
+    A = dev(rng.normal(0, 1, (M, K_)).astype(np.float16))
+    Cm = dev(rng.normal(0, 1, (M, N)).astype(np.float16))
+    Wq, sc = K.quantize_weight_e4m3(dev(rng.normal(0, 0.02, (K_, N)).astype(np.float16)))
+    Uq, su = K.quantize_weight_e4m3(dev(rng.normal(0, 0.02, (K_, N)).astype(np.float16)))
+    q, s = K.quantize_rows_e4m3(A)
+    assert np.array_equal(host(K.gemm_f8q(q, s, Wq, sc, Cm, alpha=0.5, beta=1.0)),
+                          host(K.gemm_f8w(A, Wq, sc, Cm, alpha=0.5, beta=1.0)))
+    assert np.array_equal(host(K.dual_swiglu_f8q(q, s, Wq, sc, Uq, su)), host(K.dual_swiglu_f8w(A, Wq, sc, Uq, su)))
 
 
 def test_gemm_f8w_rejects_short_workspace(K):
