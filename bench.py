@@ -152,7 +152,7 @@ def _attention_roofline(tm, bytes_per_launch, name="roofline", calib=None):
 # with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernels at M = 2048 (LM head: 684 rows) and
 # scaled by the copy-kernel calibration: profiles/gemm_hbm_traffic_pmc.txt.  The activations are
 # fetched once per XCD and round of tiles; most of the repeats hit the Infinity Cache.
-GEMM_TRAFFIC_RATIO = 2.44
+GEMM_TRAFFIC_RATIO = 2.41
 
 
 def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows, weight_bytes=2):
