@@ -13,7 +13,7 @@ Candidates: NON_OVERLAP_LOCAL (one stream, no split), NANOBATCH_LOCAL / LOCAL (t
 LOCAL on two streams) and PLLM (four QKV / attention nano-batches, two streams) over a grid of
 nano-batch-1 sizes and QKV sub-splits, all multiples of ``--step`` rows.  Optional ``--cu-masks`` adds, for LOCAL, static compute-unit splits
 between the GEMM and the attention stream (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS: CU counts, given
-here in whole XCDs of 32).
+here in eighths of the chip: 32 CUs, which a CU mask spreads as 4 CUs over each of the 8 XCDs).
 Each candidate runs the same iteration (the decode requests and prefill chunks given, on
 ``--layers`` layers of random-init weights: the per-layer schedule is what is being compared) and is
 timed over ``--iters`` runs after ``--warm``.  The output JSON is the input config with the winning
@@ -99,7 +99,7 @@ def main():
     ap.add_argument("--step", type=int, default=128, help="granularity of the nano-batch sizes")
     ap.add_argument("--types", default="NON_OVERLAP_LOCAL,NANOBATCH_LOCAL,LOCAL,PLLM")
     ap.add_argument("--fine", action="store_true", help="also try 1/4 and 3/4 QKV sub-splits")
-    ap.add_argument("--cu-masks", default="", help="LOCAL only: GEMM:attention XCD counts to try, e.g. 6:2,5:3,4:4")
+    ap.add_argument("--cu-masks", default="", help="LOCAL only: GEMM:attention shares of the CUs to try, in eighths (4 CUs of every XCD each), e.g. 6:2,5:3,4:4")
     ap.add_argument("--iters", type=int, default=5)
     ap.add_argument("--warm", type=int, default=2)
     ap.add_argument("--seed", type=int, default=0)
@@ -134,12 +134,12 @@ def main():
         cand = ("LOCAL", best_local["nanobatch_1_size"], best_local["kqv1_size"], best_local["kqv3_size"])
         for g, v in masks:
             if g <= 0 or v <= 0 or g + v > 8:
-                raise SystemExit(f"--cu-masks {g}:{v}: XCD counts must be positive and sum to at most 8")
-            env = {"NANOFLOW_GEMM_CUS": str(32 * g), "NANOFLOW_GEMV_CUS": str(32 * v)}   # 32 CUs per XCD
+                raise SystemExit(f"--cu-masks {g}:{v}: the shares (eighths of the CUs) must be positive and sum to at most 8")
+            env = {"NANOFLOW_GEMM_CUS": str(32 * g), "NANOFLOW_GEMV_CUS": str(32 * v)}   # 32 CUs per eighth
             ms = measure(shape, batch, T, cand, layers, a.iters, a.warm, env)
             rows.append({"pipeline_type": "LOCAL", "nanobatch_1_size": cand[1], "kqv1_size": cand[2],
-                         "kqv3_size": cand[3], "gemm_xcds": g, "attention_xcds": v, "ms": ms, **env})
-            print(f"  LOCAL with {g} XCDs for GEMM, {v} for attention: {ms:8.3f} ms", flush=True)
+                         "kqv3_size": cand[3], "gemm_cu_eighths": g, "attention_cu_eighths": v, "ms": ms, **env})
+            print(f"  LOCAL with {4 * g} CUs of every XCD for GEMM, {4 * v} for attention: {ms:8.3f} ms", flush=True)
     best = min(rows, key=lambda r: r["ms"])
     out = copy.deepcopy(cfg)
     pc = out.setdefault("pipeline_configs", {})

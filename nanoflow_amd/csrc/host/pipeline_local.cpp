@@ -33,6 +33,9 @@ static int env_int(const char* name, int dflt) {
   return v && *v ? std::atoi(v) : dflt;
 }
 
+// CUs first_cu .. first_cu + num_cus - 1 in the numbering of the CU mask, whose bit i is a CU of XCD
+// i % 8 on this part: a range of 8 n bits is n CUs of every XCD, so both streams of a split keep
+// all eight L2s and memory ports.
 hipStream_t createPipelineStream(int first_cu, int num_cus) {
   hipStream_t s = nullptr;
   if (num_cus <= 0) {

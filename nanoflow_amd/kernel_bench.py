@@ -11,7 +11,7 @@
     python -m nanoflow_amd.kernel_bench --op calibrate                # measured MFMA / HBM / paged-read ceilings
     python -m nanoflow_amd.kernel_bench --op blas --m 2048            # the same GEMM shapes through torch.matmul (hipBLASLt / rocBLAS)
     python -m nanoflow_amd.kernel_bench --op corun                    # GEMM and decode attention alone and together: time and board power
-    python -m nanoflow_amd.kernel_bench --op cusplit                  # the same pair on CU-masked streams (whole XCDs each)
+    python -m nanoflow_amd.kernel_bench --op cusplit                  # the same pair on CU-masked streams (disjoint CU sets, the same on every XCD)
 
 Each line reports the average launch time over --iters launches (HIP events on the launch
 stream) and the algorithmic rate: 2*M*N*K flops (4*M*N*K for the fused gate/up pair), or the
@@ -88,12 +88,15 @@ class PowerSampler:
         return sum(v) / len(v) if v else float("nan")
 
 
-def masked_stream(first_xcd: int, n_xcd: int):
-    """A stream restricted to whole XCDs (CU mask word i = XCD i on this part)."""
+def masked_stream(first_cu: int, n_cu: int):
+    """A stream restricted to CUs first_cu .. first_cu + n_cu - 1 (multiples of 4) of EVERY XCD.  Bit i
+    of the CU mask is a CU of XCD i % 8 on this part (a kernel that records its XCC id under a mask
+    shows it), so one 32-bit word holds 4 CUs of each of the 8 XCDs."""
     import ctypes as C
+    assert first_cu % 4 == 0 and n_cu % 4 == 0 and 0 < n_cu and first_cu + n_cu <= 32
     hip = C.CDLL("libamdhip64.so")
     s = C.c_void_p()
-    mask = (C.c_uint32 * 8)(*[0xFFFFFFFF if first_xcd <= i < first_xcd + n_xcd else 0 for i in range(8)])
+    mask = (C.c_uint32 * 8)(*[0xFFFFFFFF if first_cu // 4 <= i < (first_cu + n_cu) // 4 else 0 for i in range(8)])
     rc = hip.hipExtStreamCreateWithCUMask(C.byref(s), 8, mask)
     assert rc == 0, f"hipExtStreamCreateWithCUMask: {rc}"
     return torch.cuda.ExternalStream(s.value)
@@ -144,8 +147,8 @@ def corun(a, shape, rnd):
         s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
         splits = [("both, two unmasked streams", s1, s2)]
     else:
-        splits = [(f"both, GEMM on {gx} XCDs + attention on {8 - gx} XCDs", masked_stream(0, gx), masked_stream(gx, 8 - gx))
-                  for gx in (6, 5, 4, 3)]
+        splits = [(f"both, GEMM on {gc} + attention on {32 - gc} CUs of every XCD", masked_stream(0, gc),
+                   masked_stream(gc, 32 - gc)) for gc in (24, 20, 16, 12)]
     for name, sg, sa in splits:
         def both():
             with torch.cuda.stream(sg):
@@ -159,8 +162,8 @@ def corun(a, shape, rnd):
             def a_only():
                 with torch.cuda.stream(sa):
                     attn()
-            phase("  GEMM alone on its XCDs", g_only, lambda p: f"{fl / p / 1e12:7.1f} TFLOP/s", secs=1.5)
-            phase("  attention alone on its XCDs", a_only, lambda p: f"{nb / p / 1e9:7.1f} GB/s", secs=1.5)
+            phase("  GEMM alone on its CUs", g_only, lambda p: f"{fl / p / 1e12:7.1f} TFLOP/s", secs=1.5)
+            phase("  attention alone on its CUs", a_only, lambda p: f"{nb / p / 1e9:7.1f} GB/s", secs=1.5)
         phase(name, both, lambda p: f"serial sum {(tg + ta) * 1e6:7.1f} us -> x{(tg + ta) / p:.3f}")
     if a.op == "corun":
         phase("mfma loop f16, pseudo-random operands", lambda: K.calibrate_mfma(False, True, 2000), secs=2.0)

@@ -124,7 +124,7 @@ def test_three_schedules_match_oracle(oracle, case):
 
 @pytest.mark.parametrize("gemm_cus,gemv_cus", [(128, 128), (160, 96)])
 def test_local_pipeline_on_cu_masked_streams_matches_unmasked_and_oracle(oracle, gemm_cus, gemv_cus):
-    """LocalPipeline with its two streams restricted to disjoint sets of whole XCDs
+    """LocalPipeline with its two streams restricted to disjoint CU sets (16 + 16 and 20 + 12 CUs of every XCD)
     (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS -> hipExtStreamCreateWithCUMask): where a workgroup runs
     must not change a bit of the result, and the result must be the oracle's."""
     import os
