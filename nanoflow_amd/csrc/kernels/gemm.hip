@@ -776,7 +776,10 @@ static int splitk_plan_dual(int M, int N, int K, int* k_per) {
 // Tile choice.  A launch takes ceil(tiles / CUs) rounds of one tile each, a round costing the
 // tile's area over its relative efficiency (bigger tiles re-read less through LDS); the cheapest
 // candidate wins.  So 192 tiles of 256x256 beat 1.5 rounds of 128x256, and 2048 x 6144 takes
-// 256 tiles of 128x384 rather than 192 of 256x256.  Short M uses a 64-row tile so that padding
+// 256 tiles of 128x384 rather than 192 of 256x256.  The efficiencies are the measured rates of
+// one-round launches at 2048 rows relative to the 256x256 tile's (1.28 PFLOP/s on the LM head:
+// 128x384 1.17 on QKV, 128x256 1.13-1.21 on O and down, 128x128 about 1.0), rounded towards the
+// larger tile.  Short M uses a 64-row tile so that padding
 // rows do not dominate.
 template <class E, bool kBCol>
 static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
