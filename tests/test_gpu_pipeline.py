@@ -820,7 +820,7 @@ def test_autosearch_writes_a_tuned_pipeline_config(tmp_path):
     rows = t["search"]["measurements"]
     kinds = {m["pipeline_type"] for m in rows}
     assert kinds == {"NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL", "LOCAL", "PLLM"}
-    assert any("gemm_xcds" in m for m in rows)
+    assert any("gemm_cu_eighths" in m for m in rows)
     best = min(rows, key=lambda m: m["ms"])
     pc = t["pipeline_configs"]
     assert t["serve_configs"]["pipeline_type"] == best["pipeline_type"] and best["ms"] > 0
