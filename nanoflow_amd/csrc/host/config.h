@@ -71,6 +71,9 @@ struct vortexModelConfig {
     // alignment (the fused gate/up pair keeps two sets of sums of 128 x 128 tiles, 34 MB together,
     // for up to 2 of its wrappers)
     k_temp_size += (size_t)(7 + 2) * ((size_t)256 * 65536 * 2 + 128);
+    // ... and 84 MB for each of the pair's wrappers from 257 to 320 rows (two sets of sums of
+    // 320 x 128 tiles)
+    k_temp_size += (size_t)2 * ((size_t)256 * 320 * 128 * 2 * 2 - (size_t)256 * 65536 * 2);
     if (!rope_3_1) {
       smooth_a = 0;
       smooth_b = 0;

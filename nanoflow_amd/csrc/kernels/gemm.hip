@@ -93,6 +93,8 @@ __device__ __forceinline__ float swiglu_rounded(float g_acc, float u_acc) {
   return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
 }
 
+// WM x WN wavefronts: four (one per SIMD, up to 512 registers each) or eight (two per SIMD, up to
+// 256 each: for tiles whose accumulators do not fit four wavefronts, the 320 x 128 gate/up pair).
 // kDual: two weight matrices, SwiGLU epilogue.  kBCol: weights stored [N][K].
 // One BM x BN output tile at (m_base, n_base), computed by the whole workgroup.
 // K is the extent of the contraction and lda the row stride (elements) of the k-contiguous
@@ -109,10 +111,12 @@ __device__ __forceinline__ void gemm_tile(
   using SM = GemmSmem<BM, BN, NB>;
   constexpr int TM = BM / WM / 32;  // MFMA tiles per wave along M
   constexpr int TN = BN / WN / 32;
-  static_assert(WM * WN == 4, "four wavefronts");
-  static_assert((BN / WN) % 64 == 0 && BM % 32 == 0 && BN % 64 == 0, "tile shape");
-  constexpr int A_LOADS = BM / 32;   // 1 KB load instructions per wave per slab
-  constexpr int B_LOADS = BN / 32;   // ... per weight matrix
+  // four wavefronts (one per SIMD) or eight (two per SIMD, at most 256 registers each)
+  constexpr int NW = WM * WN;
+  static_assert(NW == 4 || NW == 8, "four or eight wavefronts");
+  static_assert((BN / WN) % 32 == 0 && (BM / WM) % 32 == 0 && BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile shape");
+  constexpr int A_LOADS = BM / (8 * NW);   // 1 KB load instructions per wave per slab
+  constexpr int B_LOADS = BN / (8 * NW);   // ... per weight matrix
   constexpr int ROWB = BN * 2;       // bytes per k row of a [K][N] weight slab
   constexpr int B_CPR = BN / 8;      // 16-byte chunks per such row
 
@@ -151,7 +155,7 @@ __device__ __forceinline__ void gemm_tile(
   uint32_t a_off[A_LOADS];
 #pragma unroll
   for (int t = 0; t < A_LOADS; ++t) {
-    const int gm = m_base + (t * 4 + wave) * 8 + (lane >> 3);
+    const int gm = m_base + (t * NW + wave) * 8 + (lane >> 3);
     a_off[t] = ((uint32_t)gm * (uint32_t)lda + a_kc) * 2u;
   }
   uint32_t b_off[NB][B_LOADS];
@@ -160,10 +164,10 @@ __device__ __forceinline__ void gemm_tile(
   for (int t = 0; t < B_LOADS; ++t) {
     uint32_t off;
     if constexpr (kBCol) {
-      const int gn = n_base + (t * 4 + wave) * 8 + (lane >> 3);
+      const int gn = n_base + (t * NW + wave) * 8 + (lane >> 3);
       off = ((uint32_t)gn * (uint32_t)lda + a_kc) * 2u;
     } else {
-      const int g = (t * 4 + wave) * 64 + lane;  // 16-byte slot of the slab's LDS image
+      const int g = (t * NW + wave) * 64 + lane;  // 16-byte slot of the slab's LDS image
       const int row = g / B_CPR;
       const int c = (g % B_CPR) ^ ((row & 3) << 2);
       off = ((uint32_t)row * (uint32_t)N + n_base + c * 8) * 2u;
@@ -182,11 +186,11 @@ __device__ __forceinline__ void gemm_tile(
   auto load_one = [&](auto t_c, uint32_t la, uint32_t lb, bool k_ok) {
     constexpr int t = decltype(t_c)::value;
     if constexpr (t < A_LOADS) {
-      load16_to_lds<t * 4096>(a_rsrc, k_ok ? a_off[t] : kOob, la);
+      load16_to_lds<t * NW * 1024>(a_rsrc, k_ok ? a_off[t] : kOob, la);
       a_off[t] += BK * 2;
     } else {
       constexpr int b = (t - A_LOADS) / B_LOADS, tt = (t - A_LOADS) % B_LOADS;
-      constexpr int dst = b * SM::b_bytes + tt * 4096;
+      constexpr int dst = b * SM::b_bytes + tt * NW * 1024;
       if constexpr (kBCol) {
         load16_to_lds<dst>(b_rsrc[b], k_ok ? b_off[b][tt] : kOob, lb);
         b_off[b][tt] += BK * 2;
@@ -419,7 +423,7 @@ __device__ __forceinline__ void gemm_tile(
   constexpr int CW = BN / WN;        // columns of the wavefront's block
   constexpr int ROWP = CW * 4 + 16;  // bytes per padded fp32 row
   constexpr int CPR = CW / 4;        // 4-column groups per row
-  static_assert(4 * 32 * ROWP <= (int)SM::bytes && (32 * CPR) % 64 == 0, "epilogue staging");
+  static_assert(NW * 32 * ROWP <= (int)SM::bytes && (32 * CPR) % 64 == 0, "epilogue staging");
   __syncthreads();  // every wavefront has read its last fragments
   uint8_t* ep = smem + wave * (32 * ROWP);
   constexpr int ITER = 32 * CPR / 64;  // 4-column groups per lane and pass
@@ -553,7 +557,7 @@ __device__ __forceinline__ bool xcd_tile(int bid, int tiles_m, int tiles_n, int*
 }
 
 template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
-__global__ __launch_bounds__(256) void gemm_f16_kernel(
+__global__ __launch_bounds__(WM * WN * 64) void gemm_f16_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B0,
     const uint16_t* __restrict__ B1, const uint16_t* C, uint16_t* D,
     int M, int N, int K, float alpha, float beta, int ldc, int tiles_m, int tiles_n) {
@@ -594,7 +598,7 @@ __global__ __launch_bounds__(256) void gemm_f16_hybrid_kernel(
 // as fp32 to P[share][M][N]; splitk_reduce_kernel adds the shares and applies alpha, beta and C.
 // kDual: two weight matrices; the sums of the second go to P1[share][M][N].
 template <class E, int BM, int BN, int WM, int WN, bool kDual, bool kBCol>
-__global__ __launch_bounds__(256) void gemm_f16_splitk_kernel(
+__global__ __launch_bounds__(WM * WN * 64) void gemm_f16_splitk_kernel(
     const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, const uint16_t* __restrict__ B1,
     float* __restrict__ P, float* __restrict__ P1, int M, int N, int K, int shares, int k_per, int tiles_m,
     int tiles_n) {
@@ -667,7 +671,7 @@ static int launch_splitk(const uint16_t* A, const uint16_t* B, const uint16_t* C
   }
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int grid = ((tiles_m * tiles_n * shares + 7) / 8) * 8;
-  kern<<<grid, 256, SM::bytes, stream>>>(A, B, B1, P, P1, M, N, K, shares, k_per, tiles_m, tiles_n);
+  kern<<<grid, WM * WN * 64, SM::bytes, stream>>>(A, B, B1, P, P1, M, N, K, shares, k_per, tiles_m, tiles_n);
   int rc = check_launch("gemm split-K launch");
   if (rc) return rc;
   const size_t groups = (size_t)M * N / 4;
@@ -696,7 +700,7 @@ static int launch_gemm(const uint16_t* A, const uint16_t* B0, const uint16_t* B1
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int ntiles = tiles_m * tiles_n;
   const int grid = ((ntiles + 7) / 8) * 8;
-  kern<<<grid, 256, SM::bytes, stream>>>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc, tiles_m, tiles_n);
+  kern<<<grid, WM * WN * 64, SM::bytes, stream>>>(A, B0, B1, C, D, M, N, K, alpha, beta, ldc, tiles_m, tiles_n);
   return check_launch("gemm launch");
 }
 
@@ -761,11 +765,11 @@ static int splitk_plan(int M, int N, int K, int* k_per) {
   return (K + *k_per - 1) / *k_per;  // shares that are not empty
 }
 
-// The same for the fused gate/up pair (tiles of 64 x 128 up to 64 rows, else 128 x 128; a
-// 320 x 128 pair of accumulators does not fit the register file).
+// The same for the fused gate/up pair (tiles of 64 x 128 up to 64 rows, 128 x 128 up to 256,
+// 320 x 128 on eight wavefronts up to 320).
 static int splitk_plan_dual(int M, int N, int K, int* k_per) {
-  if (M > 256 || K < 1024) return 1;
-  const int bm = M <= 64 ? 64 : 128;
+  if (M > kTallRows || K < 1024) return 1;
+  const int bm = M <= 64 ? 64 : M <= 256 ? 128 : 320;
   const int tiles = ((M + bm - 1) / bm) * ((N + 127) / 128);
   const int shares = std::min(std::min(cu_count() / tiles, K / 512), kMaxShares);
   if (shares < 2) return 1;
@@ -872,6 +876,11 @@ static int dual_entry(const char* who, const uint16_t* A, const uint16_t* Bgate,
   hipStream_t s = (hipStream_t)stream;
   if (M <= 64)
     return launch_gemm<E, 64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
+  // 257 .. 320 rows against enough column panels to fill the chip: one 320-row tile per panel, so
+  // the weights pass through LDS once instead of three times; its two 320 x 128 accumulators are
+  // spread over eight wavefronts (160 registers each)
+  if (M > 256 && M <= kTallRows && (N + 127) / 128 >= 192)
+    return launch_gemm<E, 320, 128, 2, 4, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
   const long long t256 = (long long)((M + 255) / 256) * ((N + 127) / 128);
   const int tail = M % 256;  // rows in the last 256-row tile: half-empty tiles go to the 128-row kernel
   if (t256 >= 192 && (tail == 0 || tail > 128)) {
@@ -899,6 +908,8 @@ static int dual_ws_entry(const char* who, const uint16_t* A, const uint16_t* Bga
   float* P = static_cast<float*>(workspace);
   if (M <= 64)
     return launch_splitk<E, 64, 128, 2, 2, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
+  if (M > 256)
+    return launch_splitk<E, 320, 128, 2, 4, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
   return launch_splitk<E, 128, 128, 2, 2, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
 }
 
@@ -958,7 +969,7 @@ size_t nf_dual_swiglu_workspace_bytes(int M, int N, int K) {
 
 size_t nf_dual_swiglu_workspace_bytes_upto(int max_M, int N, int K) {
   size_t need = 0;
-  for (int m = 1; m <= max_M && m <= 256; ++m) need = std::max(need, nf_dual_swiglu_workspace_bytes(m, N, K));
+  for (int m = 1; m <= max_M && m <= kTallRows; ++m) need = std::max(need, nf_dual_swiglu_workspace_bytes(m, N, K));
   return need;
 }
 

@@ -233,7 +233,10 @@ def test_gemm_identity_is_exact(K):
 @pytest.mark.parametrize("M,N,K_", [(64, 14336, 4096), (5, 136, 72), (200, 512, 256), (640, 2048, 512),
                                     (2048, 14336, 128),    # 3.5 rounds of 256-row tiles: two tile heights in one launch
                                     (1992, 14328, 200),    # the same with M, N and K tails
-                                    (267, 1160, 264)])     # a few hundred rows, N and K tails
+                                    (267, 1160, 264),      # a few hundred rows, N and K tails
+                                    (267, 24584, 328),     # 257 .. 320 rows against 193 column panels: the
+                                    (320, 24576, 128),     # 320-row tile on eight wavefronts (N and K tails; exact fit)
+                                    (257, 28672, 72)])
 def test_dual_swiglu(K, oracle, M, N, K_):
     rng = np.random.default_rng(7)
     A = synth.normal_f16(rng, (M, K_))
@@ -243,7 +246,8 @@ def test_dual_swiglu(K, oracle, M, N, K_):
                  what="dual swiglu")
 
 
-@pytest.mark.parametrize("M,N,K_", [(16, 14336, 4096), (64, 1160, 2056), (128, 14336, 1024), (200, 2048, 4096)])
+@pytest.mark.parametrize("M,N,K_", [(16, 14336, 4096), (64, 1160, 2056), (128, 14336, 1024), (200, 2048, 4096),
+                                    (300, 14336, 1024), (267, 1160, 2056)])    # the 320-row tile, split
 def test_dual_swiglu_split_over_k_matches_oracle(K, oracle, M, N, K_):
     """Few rows: both products of the gate/up pair are split over K, summed in fp32, rounded to fp16 and
     put through SiLU-mul by the reduction.  Twice the fp16 tolerance, as for the bf16 and fp8 pairs: a
