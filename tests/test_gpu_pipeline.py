@@ -250,7 +250,7 @@ def test_kqv_bias_schedules_match_oracle(oracle, case):
 
 @pytest.mark.parametrize("case", ["decode_crosses_border", "prefill_straddles_border"])
 def test_fp8_weight_pipelines_match_oracle(oracle, case):
-    """The three schedules with the five per-layer GEMM weights in e4m3 (quantised on the device from
+    """The four schedules with the five per-layer GEMM weights in e4m3 (quantised on the device from
     the same fp16 weights, per-output-channel scales), against the oracle's forward with the same
     arithmetic (input rows re-quantised per GEMM, fp8 x fp8 products) and against fp16 activations
     on the dequantised weights, the definition the fp8 tolerance of 3e-2 per GEMM is stated for.
@@ -286,7 +286,8 @@ def test_fp8_weight_pipelines_match_oracle(oracle, case):
     keep = np.ones(b1.decodePrefillBorder, np.int32)
     results = {}
     try:
-        for pt in (P.PipelineType.NON_OVERLAP_LOCAL, P.PipelineType.NANOBATCH_LOCAL, P.PipelineType.LOCAL):
+        for pt in (P.PipelineType.NON_OVERLAP_LOCAL, P.PipelineType.NANOBATCH_LOCAL, P.PipelineType.LOCAL,
+                   P.PipelineType.PLLM):
             print(f"case={case} pipeline={pt.name} weights=e4m3", flush=True)
             with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=max(nano1 // 2, 1), kqv3=(T - nano1) // 2,
                                kv_pages=b1.num_pages, weights=w, kv_pools=pools0, weight_format="e4m3") as e:
@@ -311,7 +312,7 @@ def test_fp8_weight_pipelines_match_oracle(oracle, case):
     finally:
         P.setWeightFormat(P.WeightFormat.F16)
     base = results[P.PipelineType.NON_OVERLAP_LOCAL]
-    for pt in (P.PipelineType.NANOBATCH_LOCAL, P.PipelineType.LOCAL):
+    for pt in (P.PipelineType.NANOBATCH_LOCAL, P.PipelineType.LOCAL, P.PipelineType.PLLM):
         # per-row activation scales and a fixed k order: splitting the rows differently changes no
         # bit of a row, which is what keeps the schedules comparable despite the discontinuity
         assert np.array_equal(results[pt][0], base[0]), (pt, "samples differ between schedules")
