@@ -356,7 +356,7 @@ def run_offline(args):
     shape = synth.LLAMA3_70B if args.shape == "70b" else synth.LLAMA3_8B
     wb = 1 if args.weights == "e4m3" else 2                    # bytes per element of the per-layer GEMM weights
     shape_name = "Llama-3-70B" if args.shape == "70b" else "Llama-3-8B"
-    T, n_req, in_len, out_len = 2048, args.requests, 1024, 512
+    T, n_req, in_len, out_len = args.global_batch, args.requests, 1024, 512
     steps = args.steps or 256
     warmup = 8 if args.warmup is None else args.warmup
 
@@ -532,6 +532,9 @@ def main():
                     help="auto = the fastest schedule measured on MI355X for both workloads: NON_OVERLAP_LOCAL\n"
                          "(one stream); LOCAL measures the two-stream overlapped schedule, PLLM the reference's main\n"
                          "schedule (four QKV / attention nano-batches), PLLMOFFLOAD that with the KV offload round trip")
+    ap.add_argument("--global-batch", type=int, default=2048,
+                    help="offline workload: tokens per iteration the scheduler keeps (the measured configuration is 2048; "
+                         "more is a what-if for a part with room for it)")
     ap.add_argument("--nano1", type=int, default=1024, help="rows of nano-batch 1")
     ap.add_argument("--kqv1", type=int, default=512)
     ap.add_argument("--kqv3", type=int, default=512)
