@@ -16,7 +16,10 @@ between the GEMM and the attention stream (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS
 here in eighths of the chip: 32 CUs, which a CU mask spreads as 4 CUs over each of the 8 XCDs).
 Each candidate runs the same iteration (the decode requests and prefill chunks given, on
 ``--layers`` layers of random-init weights: the per-layer schedule is what is being compared) and is
-timed over ``--iters`` runs after ``--warm``.  The output JSON is the input config with the winning
+timed over ``--iters`` runs after ``--warm``; one further run with HIP events around every attention and dense
+GEMM launch records what justifies the choice: the TFLOP/s of the GEMM launches and the GB/s of decode attention
+while they ran, and the share of the iteration each kind was running (shares that add up to more than 1 overlap).
+The output JSON is the input config with the winning
 ``pipeline_configs`` / ``pipeline_type`` and a ``search`` block holding every measurement.
 """
 from __future__ import annotations
@@ -57,7 +60,9 @@ def candidates(T: int, step: int, types, fine: bool):
 
 
 def measure(shape, batch, T, cand, layers, iters, warm, env=None):
-    """Milliseconds per iteration of one candidate (median of iters runs)."""
+    """(milliseconds per iteration of one candidate: median of iters runs; utilisation record of one
+    further run with HIP events around every attention and dense GEMM launch: the rate each kind of
+    launch reached while it ran, and the share of the iteration each kind was running)."""
     import torch
     from nanoflow_amd import engine, pllm_python as P
     name, n1, k1, k3 = cand
@@ -82,7 +87,29 @@ def measure(shape, batch, T, cand, layers, iters, warm, env=None):
             t0 = time.perf_counter()
             eng.run()
             ts.append((time.perf_counter() - t0) * 1e3)
-        return float(np.median(ts))
+        util = {}
+        try:
+            P.setProfilingStride(1)
+            P.setProfiling(2)
+            eng.run()
+            P.resetTimings()
+            eng.run()
+            torch.cuda.synchronize()
+            tm = P.getTimings()
+            nd = batch.decodePrefillBorder
+            kv = batch.kv_len[:nd].astype(np.int64)
+            attn_bytes = float((2 * kv * shape.Hkv * shape.d * 2 + 2 * shape.Hq * shape.d * 2
+                                + 4 * ((kv + shape.page_size - 1) // shape.page_size + 2)).sum()) * layers
+            if tm.gemm_ms > 0:
+                util["gemm_tflops_while_running"] = tm.gemm_flop / (tm.gemm_ms * 1e-3) / 1e12
+                util["gemm_share_of_iteration"] = tm.gemm_ms / tm.iter_ms
+            if tm.decode_attn_ms > 0:
+                util["decode_attention_gbps_while_running"] = attn_bytes / (tm.decode_attn_ms * 1e-3) / 1e9
+                util["attention_share_of_iteration"] = (tm.decode_attn_ms + tm.prefill_attn_ms) / tm.iter_ms
+        finally:
+            P.setProfiling(0)
+            P.setProfilingStride(0)
+        return float(np.median(ts)), util
     finally:
         eng.close()
 
@@ -123,10 +150,13 @@ def main():
     rows = []
     print(f"{len(cands)} candidates, {batch.tokens} tokens ({batch.decodePrefillBorder} decode), {layers} layers each", flush=True)
     for cand in cands:
-        ms = measure(shape, batch, T, cand, layers, a.iters, a.warm)
+        ms, util = measure(shape, batch, T, cand, layers, a.iters, a.warm)
         rows.append({"pipeline_type": cand[0], "nanobatch_1_size": cand[1], "kqv1_size": cand[2],
-                     "kqv3_size": cand[3], "ms": ms})
-        print(f"  {cand[0]:18s} nano1 {cand[1]:5d} kqv1 {cand[2]:5d} kqv3 {cand[3]:5d}: {ms:8.3f} ms", flush=True)
+                     "kqv3_size": cand[3], "ms": ms, **util})
+        print(f"  {cand[0]:18s} nano1 {cand[1]:5d} kqv1 {cand[2]:5d} kqv3 {cand[3]:5d}: {ms:8.3f} ms   "
+              f"GEMM {util.get('gemm_tflops_while_running', 0):6.0f} TFLOP/s over {util.get('gemm_share_of_iteration', 0):4.2f} of the iteration, "
+              f"decode attention {util.get('decode_attention_gbps_while_running', 0):6.0f} GB/s, attention over "
+              f"{util.get('attention_share_of_iteration', 0):4.2f}", flush=True)
     masks = [tuple(int(x) for x in m.split(":")) for m in a.cu_masks.split(",") if m]
     local = [r for r in rows if r["pipeline_type"] == "LOCAL"]
     if masks and local:
@@ -136,9 +166,9 @@ def main():
             if g <= 0 or v <= 0 or g + v > 8:
                 raise SystemExit(f"--cu-masks {g}:{v}: the shares (eighths of the CUs) must be positive and sum to at most 8")
             env = {"NANOFLOW_GEMM_CUS": str(32 * g), "NANOFLOW_GEMV_CUS": str(32 * v)}   # 32 CUs per eighth
-            ms = measure(shape, batch, T, cand, layers, a.iters, a.warm, env)
+            ms, util = measure(shape, batch, T, cand, layers, a.iters, a.warm, env)
             rows.append({"pipeline_type": "LOCAL", "nanobatch_1_size": cand[1], "kqv1_size": cand[2],
-                         "kqv3_size": cand[3], "gemm_cu_eighths": g, "attention_cu_eighths": v, "ms": ms, **env})
+                         "kqv3_size": cand[3], "gemm_cu_eighths": g, "attention_cu_eighths": v, "ms": ms, **util, **env})
             print(f"  LOCAL with {4 * g} CUs of every XCD for GEMM, {4 * v} for attention: {ms:8.3f} ms", flush=True)
     best = min(rows, key=lambda r: r["ms"])
     out = copy.deepcopy(cfg)
