@@ -777,14 +777,19 @@ static int splitk_plan_dual(int M, int N, int K, int* k_per) {
   return (K + *k_per - 1) / *k_per;
 }
 
-// Tile choice.  A launch takes ceil(tiles / CUs) rounds of one tile each, a round costing the
-// tile's area over its relative efficiency (bigger tiles re-read less through LDS); the cheapest
-// candidate wins.  So 192 tiles of 256x256 beat 1.5 rounds of 128x256, and 2048 x 6144 takes
-// 256 tiles of 128x384 rather than 192 of 256x256.  The efficiencies are the measured rates of
-// one-round launches at 2048 rows relative to the 256x256 tile's (1.28 PFLOP/s on the LM head:
-// 128x384 1.17 on QKV, 128x256 1.13-1.21 on O and down, 128x128 about 1.0), rounded towards the
-// larger tile.  Short M uses a 64-row tile so that padding
-// rows do not dominate.
+// Tile choice.  A launch takes tiles / CUs rounds of one tile per CU, a round costing the tile's
+// area over its relative efficiency (bigger tiles re-read less through LDS); the cheapest candidate
+// wins.  A last, partly filled round is not charged in full: the part is power-bound, so the
+// fewer CUs clock higher, and measured it costs 0.47 + 0.53 x its fill (a quarter-full round 0.61,
+// three quarters 0.86 of a full one).  Efficiencies and that rule are fitted to launches of 1024
+// and 2048 rows on the Llama-3-8B and -70B layer shapes WITH THE WEIGHTS STREAMED FROM HBM, as a
+// layer's weights are (multiplying by the same weights again finds the smaller matrices in the
+// 256 MB last-level cache and flatters tiles with two LDS stages): the model picks the fastest of
+// the three tiles in all ten cases.  2048 x 6144 x 4096 runs on 192 tiles of 256x256 (93-98 us)
+// rather than 384 of 128x256 (116-122) or 768 of 128x128 (118-120).  A 128x384 tile, which fills
+// the chip exactly once on that shape, has room for two LDS stages only, and a load that misses
+// the cache does not land within a slab: 102-105 us, and last or second to last in every case;
+// it is not a candidate.  Short M uses a 64-row tile so that padding rows do not dominate.
 template <class E, bool kBCol>
 static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
                           int M, int N, int K, float alpha, float beta, int ldc, hipStream_t s) {
@@ -792,13 +797,24 @@ static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* 
   const int cus = cu_count();
   auto cost = [&](int bm, int bn, double eff) {
     const long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-    return (double)((tiles + cus - 1) / cus) * bm * bn / eff;
+    const long long full = tiles / cus, rest = tiles % cus;
+    const double rounds = (double)full + (rest ? 0.47 + 0.53 * (double)rest / cus : 0.0);
+    return rounds * bm * bn / eff;
   };
-  const double c256 = cost(256, 256, 1.0), c384 = cost(128, 384, 0.97), c128x256 = cost(128, 256, 0.95),
-               c128 = cost(128, 128, 0.80);
-  const double best = std::min(std::min(c256, c384), std::min(c128x256, c128));
+  double c256 = cost(256, 256, 1.0);
+  const double c128x256 = cost(128, 256, 0.95), c128 = cost(128, 128, 0.80);
+  // 256x256 tiles that fill the chip a whole number of times plus at most half a round: the tiles of
+  // that last round are computed as two 128-row halves by two workgroups each, in the same launch
+  // (2048 x 10240 x 8192, 320 tiles: 256 + 2 x 64)
+  const long long t256 = (long long)((M + 255) / 256) * ((N + 255) / 256);
+  const int rest256 = (int)(t256 % cus);
+  const bool two_heights = t256 > cus && rest256 > 0 && rest256 <= cus / 2;
+  if (two_heights)
+    c256 = ((double)(t256 / cus) + 0.5 * (0.47 + 0.53 * 2.0 * rest256 / cus) / 0.95) * 256 * 256;
+  const double best = std::min(c256, std::min(c128x256, c128));
+  if (best == c256 && two_heights)
+    return launch_hybrid<E, 256, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, (int)(t256 - rest256), s);
   if (best == c256) return launch_gemm<E, 256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
-  if (best == c384) return launch_gemm<E, 128, 384, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
   if (best == c128x256) return launch_gemm<E, 128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
   return launch_gemm<E, 128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
 }

@@ -611,10 +611,28 @@ int nf_gemm_f8_f16(const uint8_t* Aq, const float* a_scale, const uint8_t* Bq, c
              "nf_gemm_f8_f16: an operand of %d x %d x %d exceeds the 4 GiB buffer-addressing limit", M, N, K);
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
-  auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   if (M <= 64) return launch_gemm_f8<64, 256, 1, 4>(Aq, Bq, a_scale, b_scale, C, D, M, N, K, alpha, beta, s);
-  if (tiles(256, 256) >= 224) return launch_gemm_f8<256, 256, 2, 2>(Aq, Bq, a_scale, b_scale, C, D, M, N, K, alpha, beta, s);
-  if (tiles(128, 256) >= 224 || M <= 128) return launch_gemm_f8<128, 256, 2, 2>(Aq, Bq, a_scale, b_scale, C, D, M, N, K, alpha, beta, s);
+  // Tile choice by cost, as for the fp16 kernels: rounds of one tile per CU, a partly filled last
+  // round charged 0.47 + 0.53 x its fill, a round costing the tile's area over its efficiency
+  // (1 / 0.80 / 0.60 for 256x256 / 128x256 / 128x128, from full rounds with the weights streamed
+  // from HBM).  Picks the fastest tile on the Llama-3-8B and -70B layer shapes at 1024 and 2048
+  // rows (2048 x 6144 x 4096: 49 us on 192 tiles of 256x256, 64 us on 384 of 128x256).
+  static int cus = 0;  // benign race: every thread computes the same value
+  if (cus == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    cus = v;
+  }
+  auto cost = [&](int bm, int bn, double eff) {
+    const long long tiles = (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    const long long full = tiles / cus, rest = tiles % cus;
+    return ((double)full + (rest ? 0.47 + 0.53 * (double)rest / cus : 0.0)) * bm * bn / eff;
+  };
+  const double c256 = cost(256, 256, 1.0), c128x256 = cost(128, 256, 0.80), c128 = cost(128, 128, 0.60);
+  const double best = std::min(c256, std::min(c128x256, c128));
+  if (best == c256) return launch_gemm_f8<256, 256, 2, 2>(Aq, Bq, a_scale, b_scale, C, D, M, N, K, alpha, beta, s);
+  if (best == c128x256) return launch_gemm_f8<128, 256, 2, 2>(Aq, Bq, a_scale, b_scale, C, D, M, N, K, alpha, beta, s);
   return launch_gemm_f8<128, 128, 2, 2>(Aq, Bq, a_scale, b_scale, C, D, M, N, K, alpha, beta, s);
 }
 

@@ -57,6 +57,17 @@ def timeit(fn, iters, warm):
     return s.elapsed_time(e) / iters
 
 
+def cold_copies(W, cold: bool):
+    """An endless iterator over W, or (--cold) over enough copies of it that a launch never finds its
+    weights in the 256 MB last-level cache: the way a layer's weights arrive in the pipeline, where
+    a model's 15 to 140 GB of weights pass through between two uses of the same matrix."""
+    import itertools
+    if not cold:
+        return itertools.repeat(W)
+    n = max(2, -(-(1 << 30) // (W.numel() * W.element_size())))   # at least 1 GiB of distinct weights
+    return itertools.cycle([W] + [W.clone() for _ in range(n - 1)])
+
+
 def layer_shapes(shape: synth.ModelShape, M: int):
     return [("kqv", M, shape.kqv_n, shape.hidden), ("o", M, shape.hidden, shape.Hq * shape.d),
             ("down", M, shape.hidden, shape.ffn), ("lm_head", (M + 127) // 128 * 128, shape.vocab, shape.hidden)]
@@ -195,6 +206,8 @@ def main():
     ap.add_argument("--mib", type=int, default=1024, help="copy: MiB moved")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"], help="gemm, dual: element type")
     ap.add_argument("--b-col-major", action="store_true", help="gemm: weights stored [N][K] (k contiguous)")
+    ap.add_argument("--cold", action="store_true",
+                    help="gemm, dual, gemm_f8, dual_f8: cycle through 1 GiB of weight copies so that every launch streams its weights from HBM")
     ap.add_argument("--ws", action="store_true", help="gemm: the entry point with a workspace (split over K where it pays)")
     ap.add_argument("--warm-ms", type=float, default=300.0,
                     help="gemm, dual, blas, attn: keep launching this long before timing (0: only --warm launches)")
@@ -217,23 +230,26 @@ def main():
             if a.op == "gemm":
                 A = rnd(M, Kd).to(edt)
                 B = (rnd(N, Kd, std=0.02) if a.b_col_major else rnd(Kd, N, std=0.02)).to(edt)
+                Bs = cold_copies(B, a.cold)
                 if a.ws:
                     ws = torch.empty((max(K.lib().nf_gemm_workspace_bytes(M, N, Kd), 16),), dtype=torch.uint8, device=DEV)
-                    fn = lambda: K.gemm_ws(A, B, out=out, b_col_major=a.b_col_major, workspace=ws)
+                    fn = lambda: K.gemm_ws(A, next(Bs), out=out, b_col_major=a.b_col_major, workspace=ws)
                 else:
-                    fn = lambda: K.gemm(A, B, out=out, b_col_major=a.b_col_major)
+                    fn = lambda: K.gemm(A, next(Bs), out=out, b_col_major=a.b_col_major)
             else:
                 Aq = torch.randint(0, 120, (M, Kd), dtype=torch.uint8, device=DEV)
                 Bq = torch.randint(0, 120, (N, Kd), dtype=torch.uint8, device=DEV)
                 sa, sb = torch.ones(M, device=DEV), torch.ones(N, device=DEV)
-                fn = lambda: K.gemm_f8(Aq, sa, Bq, sb, out=out)
+                Bqs = cold_copies(Bq, a.cold)
+                fn = lambda: K.gemm_f8(Aq, sa, next(Bqs), sb, out=out)
             ms = timeit(fn, a.iters, a.warm)
             print(f"{a.op} {name:8s} {M}x{N}x{Kd}: {ms * 1e3:9.1f} us  {2.0 * M * N * Kd / ms / 1e9:8.1f} TFLOP/s", flush=True)
     elif a.op == "dual":
         A, Bg, Bu = (t.to(edt) for t in (rnd(a.m, shape.hidden), rnd(shape.hidden, shape.ffn, std=0.02),
                                          rnd(shape.hidden, shape.ffn, std=0.02)))
         out = torch.empty(a.m, shape.ffn, dtype=edt, device=DEV)
-        ms = timeit(lambda: K.dual_swiglu(A, Bg, Bu, out=out), a.iters, a.warm)
+        Gs, Us = cold_copies(Bg, a.cold), cold_copies(Bu, a.cold)
+        ms = timeit(lambda: K.dual_swiglu(A, next(Gs), next(Us), out=out), a.iters, a.warm)
         print(f"dual gate/up {a.m}x{shape.ffn}x{shape.hidden}: {ms * 1e3:9.1f} us  "
               f"{4.0 * a.m * shape.ffn * shape.hidden / ms / 1e9:8.1f} TFLOP/s", flush=True)
     elif a.op == "dual_f8":
@@ -243,7 +259,8 @@ def main():
         Uq = torch.randint(0, 120, (N, Kd), dtype=torch.uint8, device=DEV)
         sa, sg, su = torch.ones(M, device=DEV), torch.full((N,), 1e-4, device=DEV), torch.full((N,), 1e-4, device=DEV)
         out = torch.empty(M, N, dtype=torch.float16, device=DEV)
-        ms = timeit(lambda: K.dual_swiglu_f8(Aq, sa, Gq, sg, Uq, su, out=out), a.iters, a.warm)
+        Gqs, Uqs = cold_copies(Gq, a.cold), cold_copies(Uq, a.cold)
+        ms = timeit(lambda: K.dual_swiglu_f8(Aq, sa, next(Gqs), sg, next(Uqs), su, out=out), a.iters, a.warm)
         print(f"dual_f8 gate/up {M}x{N}x{Kd}: {ms * 1e3:9.1f} us  {4.0 * M * N * Kd / ms / 1e9:8.1f} TFLOP/s", flush=True)
     elif a.op == "attn":
         b = synth.config2_batch(seed=0, n_decode=a.requests, lo=a.kv_lo, hi=a.kv_hi, prefill_chunk=16)

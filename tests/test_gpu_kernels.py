@@ -96,8 +96,10 @@ GEMM_SHAPES = [
     (257, 512, 128),      # M tail of one row
     (384, 4096, 4096),    # nano-batch O projection
     (1408, 6144, 512),    # 256x256 tiles with an M tail, XCD-remapped grid
-    (2048, 6144, 256),    # one round of 128x384 tiles (the QKV projection of a full batch)
-    (1930, 5000, 264),    # 128x384 tiles with M, N and K tails
+    (2048, 6144, 256),    # 192 tiles of 256x256: three quarters of a round (the QKV projection of a full batch)
+    (1930, 5000, 264),    # the same with M, N and K tails
+    (2048, 10240, 136),   # 320 tiles of 256x256: one round, then 64 tiles as two 128-row halves each
+    (1950, 10200, 72),    # the same with M, N and K tails
     (267, 1160, 520),     # a few hundred rows (the KV-bound 70B serving regime), N and K tails
 ]
 
