@@ -115,8 +115,20 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
   for (int i = 0; i < 8; ++i)
     vx[i] = (uint32_t)((g * 4 + (i16 >> 2)) * 256 + ((i ^ vx_x) * 32) + (i16 & 3) * 8);
 
+  // Work item w -> (request, kv head).  Workgroup ids go round the 8 XCDs, so in groups of 8
+  // requests the item order is (head, request): the workgroups an XCD starts one after the other
+  // are then the heads of ONE request, which walk the same pages at about the same time and pull
+  // each key's 256-byte rows of all heads -- one contiguous Hkv x 256 bytes in the pool -- together
+  // (the bare load pattern: 6.55 -> 6.76 TB/s).  The requests past the last whole group of 8 keep
+  // (request, head) order.
+  const long long grouped = (long long)(batch / 8) * 8 * Hkv;
   for (long long w = blockIdx.x; w < (long long)batch * Hkv; w += gridDim.x) {
-    const int req = (int)(w / Hkv), kvh = (int)(w % Hkv);
+    int req = (int)(w / Hkv), kvh = (int)(w % Hkv);
+    if (w < grouped) {
+      const int j = (int)(w % (8 * Hkv));
+      req = (int)(w / (8 * Hkv)) * 8 + j % 8;
+      kvh = j / 8;
+    }
     const int qo0 = qo_indptr[req];
     const int qo_len = qo_indptr[req + 1] - qo0;
     const int pg0 = kv_indptr[req];
