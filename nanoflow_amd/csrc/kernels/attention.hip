@@ -209,6 +209,12 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
         dma_k(wave + NW, 1);
         dma_v(wave + NW, 1);
       }
+      // The compiler does not see the DMA loads above but does see the Q loads: left alone it waits
+      // for them where Q is first used, inside the loop below, with vmcnt(0) on EVERY pass -- which
+      // also waits for every K and V tile in flight and leaves the ring one step deep.  A use of Q
+      // here makes it wait once, now (for Q and the tiles just requested).
+#pragma unroll
+      for (int j = 0; j < 4; ++j) asm volatile("" ::"v"(qf[j].w[0]));
       int buf = 0;
       for (int pp = wave; pp < npairs; pp += NW, buf ^= 1) {
         const int t_base = pp * 32;
