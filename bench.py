@@ -42,7 +42,7 @@ A100_PUBLISHED_TOKENS_PER_S = 12756.0   # reference, 1x A100 80GB, same offline 
 # HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
 # by what the same counter reads for a 1 GiB device copy), as a ratio to the algorithmic bytes of
 # the same launch: profiles/decode_attention_config2_pmc.txt.
-DECODE_ATTN_TRAFFIC_RATIO = 1.0069
+DECODE_ATTN_TRAFFIC_RATIO = 1.0061
 
 
 def decode_attention_bytes(kv_len: np.ndarray, Hq=32, Hkv=8, d=128, page=16) -> int:
@@ -152,7 +152,7 @@ def _attention_roofline(tm, bytes_per_launch, name="roofline", calib=None):
 # with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernels at M = 2048 (LM head: 684 rows) and
 # scaled by the copy-kernel calibration: profiles/gemm_hbm_traffic_pmc.txt.  The activations are
 # fetched once per XCD and round of tiles; most of the repeats hit the Infinity Cache.
-GEMM_TRAFFIC_RATIO = 2.41
+GEMM_TRAFFIC_RATIO = 2.43
 
 
 def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows, weight_bytes=2):

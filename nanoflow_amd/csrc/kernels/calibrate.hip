@@ -203,17 +203,25 @@ __global__ __launch_bounds__(256) void calib_hbm_read_kernel(const rsrc_t* __res
   if (x == 0x9e3779b9u) sink[blockIdx.x & 1023] = x;  // practically never true; keeps the loads alive
 }
 
-// Paged decode attention's traffic without its arithmetic.  Workgroup = (request, kv head), head
-// fastest; 2 wavefronts take alternate 32-key steps; a step pulls 32 K rows and 32 V rows of
-// 256 bytes (two pages each) straight into the wavefront's LDS ring of 2 K + 2 V tiles (non-temporal
-// loads, as the attention kernel issues them), and waits only for the tile it is about to reuse.
+// Paged decode attention's traffic without its arithmetic.  Workgroup = (request, kv head), in
+// the attention kernel's order; 2 wavefronts take alternate 32-key steps; a step pulls 32 K rows
+// and 32 V rows of 256 bytes (two pages each) straight into the wavefront's LDS ring of 2 K + 2 V
+// tiles (non-temporal loads, as the attention kernel issues them), and waits only for the tile it
+// is about to reuse.
 __global__ __launch_bounds__(128) void calib_paged_read_kernel(const uint16_t* __restrict__ pool,
                                                                const int32_t* __restrict__ kv_indptr,
                                                                const int32_t* __restrict__ kv_indices,
                                                                const int32_t* __restrict__ kv_last_page_len,
-                                                               int num_kv_heads, uint32_t* sink) {
+                                                               int batch, int num_kv_heads, uint32_t* sink) {
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * 4 * 8192];
-  const int req = blockIdx.x / num_kv_heads, head = blockIdx.x % num_kv_heads;
+  // (request, head) of a workgroup id as attn_decode_kernel orders its items: inside groups of 8
+  // requests (head, request), so that one XCD starts the heads of one request together
+  int req = blockIdx.x / num_kv_heads, head = blockIdx.x % num_kv_heads;
+  if ((int)blockIdx.x < (batch / 8) * 8 * num_kv_heads) {
+    const int j = blockIdx.x % (8 * num_kv_heads);
+    req = (int)(blockIdx.x / (8 * num_kv_heads)) * 8 + j % 8;
+    head = j / 8;
+  }
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int p0 = kv_indptr[req], p1 = kv_indptr[req + 1];
   const int kv_len = (p1 - p0 - 1) * 16 + kv_last_page_len[req];
@@ -375,7 +383,7 @@ int nf_calibrate_paged_read(const uint16_t* kv_data, const int32_t* kv_indptr, c
   }
   auto launch = [&] {
     calib_paged_read_kernel<<<batch * num_kv_heads, 128, 0, s>>>(kv_data, kv_indptr, kv_indices, kv_last_page_len,
-                                                                 num_kv_heads, static_cast<uint32_t*>(scratch));
+                                                                 batch, num_kv_heads, static_cast<uint32_t*>(scratch));
   };
   launch();
   (void)hipEventRecord(ev.a, s);

@@ -207,7 +207,7 @@ def main():
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"], help="gemm, dual: element type")
     ap.add_argument("--b-col-major", action="store_true", help="gemm: weights stored [N][K] (k contiguous)")
     ap.add_argument("--cold", action="store_true",
-                    help="gemm, dual, gemm_f8, dual_f8: cycle through 1 GiB of weight copies so that every launch streams its weights from HBM")
+                    help="gemm, dual, gemm_f8, dual_f8, blas: cycle through 1 GiB of weight copies so that every launch streams its weights from HBM")
     ap.add_argument("--ws", action="store_true", help="gemm: the entry point with a workspace (split over K where it pays)")
     ap.add_argument("--warm-ms", type=float, default=300.0,
                     help="gemm, dual, blas, attn: keep launching this long before timing (0: only --warm launches)")
@@ -327,15 +327,17 @@ def main():
             Bkn, Bnk = rnd(Kd, N, std=0.02), rnd(N, Kd, std=0.02)
             out = torch.empty(M, N, dtype=torch.float16, device=DEV)
             reps = 2 if name.startswith("gate") else 1
-            # every measurement follows --warm-ms of the same launches: all three are timed warm
-            ms_kn = timeit(lambda: [torch.matmul(A, Bkn, out=out) for _ in range(reps)], a.iters, a.warm)
-            ms_nk = timeit(lambda: [torch.matmul(A, Bnk.t(), out=out) for _ in range(reps)], a.iters, a.warm)
+            # every measurement follows --warm-ms of the same launches: all are timed warm; with --cold
+            # every launch (each of the two gate/up GEMMs too) takes the next of 1 GiB of weight copies
+            kn, nk = cold_copies(Bkn, a.cold), cold_copies(Bnk, a.cold)
+            ms_kn = timeit(lambda: [torch.matmul(A, next(kn), out=out) for _ in range(reps)], a.iters, a.warm)
+            ms_nk = timeit(lambda: [torch.matmul(A, next(nk).t(), out=out) for _ in range(reps)], a.iters, a.warm)
             if name.startswith("gate"):
-                Bkn2 = rnd(Kd, N, std=0.02)
-                ms_us = timeit(lambda: K.dual_swiglu(A, Bkn, Bkn2, out=out), a.iters, a.warm)
+                kn2 = cold_copies(rnd(Kd, N, std=0.02), a.cold)
+                ms_us = timeit(lambda: K.dual_swiglu(A, next(kn), next(kn2), out=out), a.iters, a.warm)
                 ms_same = timeit(lambda: K.dual_swiglu(A, Bkn, Bkn, out=out), a.iters, a.warm)
             else:
-                ms_us = timeit(lambda: K.gemm(A, Bkn, out=out), a.iters, a.warm)
+                ms_us = timeit(lambda: K.gemm(A, next(kn), out=out), a.iters, a.warm)
             fl = 2.0 * reps * M * N * Kd
             print(f"{name:18s} {M}x{N}x{Kd}: torch.matmul [K,N] weights {fl / ms_kn / 1e9:7.1f}  [N,K] weights "
                   f"{fl / ms_nk / 1e9:7.1f}  this library ([K,N]) {fl / ms_us / 1e9:7.1f} TFLOP/s", flush=True)
