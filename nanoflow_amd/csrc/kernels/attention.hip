@@ -13,8 +13,8 @@
 // exactly zero (the reference's -5e4 mask underflows to zero in fp32 as well).
 //
 // Decode: a workgroup's wavefronts split the request's pages (32 keys per step each) and
-// merge (m, l, O) through LDS; work item = (request, kv head), head fastest, so that
-// concurrently running workgroups stream the same 64 KiB pages.  Prefill: a workgroup is a
+// merge (m, l, O) through LDS; work item = (request, kv head), ordered so that the workgroups
+// one XCD starts together are the heads of one request and stream the same 64 KiB pages.  Prefill: a workgroup is a
 // 16-token tile (for GQA 4) whose wavefronts share the streamed K/V tiles; tiles are planned
 // on the device from qo_indptr (prefix of tiles per request) -- no host round trip in either mode.
 #include <type_traits>
