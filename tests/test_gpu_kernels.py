@@ -157,7 +157,7 @@ def test_gemm_alpha_beta_and_in_place_residual(K, oracle):
 
 def test_gemm_column_major_weights(K, oracle):
     rng = np.random.default_rng(5)
-    for (M, N, K_) in [(64, 512, 256), (300, 384, 320), (1930, 5000, 264)]:
+    for (M, N, K_) in [(64, 512, 256), (300, 384, 320), (1930, 5000, 264), (1950, 10200, 72)]:
         A = synth.normal_f16(rng, (M, K_))
         Bt = synth.normal_f16(rng, (N, K_), 0.05)
         assert_close(host(K.gemm(dev(A), dev(Bt), b_col_major=True)),
@@ -289,7 +289,8 @@ def _bf16_host(t):
     return t.view(torch.int16).cpu().numpy().view(np.uint16)
 
 
-@pytest.mark.parametrize("M,N,K_", [(64, 512, 256), (33, 136, 200), (300, 384, 320), (2048, 6144, 256), (1408, 6144, 512)])
+@pytest.mark.parametrize("M,N,K_", [(64, 512, 256), (33, 136, 200), (300, 384, 320), (2048, 6144, 256), (1408, 6144, 512),
+                                    (2048, 10240, 72)])
 def test_gemm_bf16(K, oracle, M, N, K_):
     rng = np.random.default_rng(31)
     A = oracle.float_to_bf16(rng.standard_normal((M, K_), dtype=np.float32))
