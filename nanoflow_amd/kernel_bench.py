@@ -307,6 +307,12 @@ def main():
                 tf, mhz = K.calibrate_mfma(False, 3, 40000)
                 print(f"   ... with 64 KB of operand loads per workgroup per 64 MFMAs (L2 -> LDS) beside them: "
                       f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
+                tf, mhz = K.calibrate_mfma(False, 5, 40000)
+                print(f"   ... with the same operand bytes routed through registers (buffer_load, ds_write_b128) instead: "
+                      f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
+                tf, mhz = K.calibrate_mfma(False, 4, 40000)
+                print(f"mfma loop f16 16x16x32 pseudo-random operands (32 accumulators, the same flops per pass): "
+                      f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
                 for n in (1, 2, 3, 4, 6, 8):
                     tf, mhz = K.calibrate_mfma(False, 10 + n, 40000)
                     print(f"mfma loop f16 32x32x16 pseudo-random operands, {64 * n:4d} idle cycles after every 16 MFMAs "

@@ -674,3 +674,43 @@ def test_attention_page_permutation_invariance(K):
                            dev(perm[b.kv_indices].astype(np.int32)), dev(b.kv_last_page_len), Hq, Hkv,
                            max_qo_rows=3)
     assert np.array_equal(host(o1), host(o2))
+
+
+# ---------------------------------------------------------------- calibration micro-benchmarks
+
+def test_calibration_loops_report_rates_this_part_can_have(K):
+    """The ceilings bench.py reports its rates against: every mode runs, and orders as the hardware
+    must order it (zero operands above random ones, fp8 above fp16, feeding the loop from LDS and
+    loading operands beside it cost something; nothing exceeds the published peaks)."""
+    from nanoflow_amd import kernels
+    zero, mhz0 = K.calibrate_mfma(False, False, 4000)
+    rnd, mhz1 = K.calibrate_mfma(False, True, 4000)
+    lds, _ = K.calibrate_mfma(False, 2, 4000)
+    direct, _ = K.calibrate_mfma(False, 3, 4000)
+    via_regs, _ = K.calibrate_mfma(False, 5, 4000)
+    small, _ = K.calibrate_mfma(False, 4, 4000)
+    idle, _ = K.calibrate_mfma(False, 14, 4000)
+    f8, _ = K.calibrate_mfma(True, True, 4000)
+    print(f"mfma f16 zero {zero:.0f} random {rnd:.0f} from LDS {lds:.0f} + loads {direct:.0f} (through registers {via_regs:.0f}) "
+          f"16x16x32 {small:.0f} duty 2/3 {idle:.0f} fp8 {f8:.0f} TFLOP/s", flush=True)
+    assert 500 < rnd <= zero <= 2600 and 1000 < mhz1 <= mhz0 < 2600
+    assert 500 < direct < lds * 1.03 and lds < rnd * 1.03 and 500 < via_regs < lds * 1.03
+    assert 500 < small < 2600 and 500 < idle < rnd * 1.03 and rnd < f8 <= 5200
+    with pytest.raises(kernels.NanoflowKernelError, match="random_operands"):
+        K.calibrate_mfma(False, 6, 100)
+    with pytest.raises(kernels.NanoflowKernelError, match="random_operands"):
+        K.calibrate_mfma(True, 2, 100)
+
+
+def test_calibration_read_streams(K):
+    gbps = K.calibrate_hbm_read(2.0, 2)
+    shape = synth.ModelShape()
+    b = synth.config2_batch(seed=0, n_decode=128, lo=256, hi=512, prefill_chunk=16)
+    nd = b.decodePrefillBorder
+    pool = torch.randn(b.num_pages * 2 * shape.page_size * shape.Hkv * shape.d // 2, device="cuda").view(torch.float16)
+    assert pool.numel() == b.num_pages * 2 * shape.page_size * shape.Hkv * shape.d
+    kvb = int(2 * b.kv_len[:nd].astype(np.int64).sum() * shape.Hkv * shape.d * 2)
+    paged = K.calibrate_paged_read(pool, dev(b.kv_indptr[:nd + 1]), dev(b.kv_indices), dev(b.kv_last_page_len[:nd]), nd,
+                                   shape.Hkv, kvb, reps=5)
+    print(f"read stream {gbps:.0f} GB/s, paged read of 128 requests {paged:.0f} GB/s", flush=True)
+    assert 2000 < gbps < 8000 and 300 < paged < 8000
