@@ -101,34 +101,35 @@ __global__ __launch_bounds__(256) void calib_mfma_kernel(int iters, int random_o
   }
 }
 
-// The same flops per pass from v_mfma_f32_16x16x32_f16: 32 independent 16x16 accumulators, 8 + 4
-// operand fragments that never change, pseudo-random operands.
+// The same flops from v_mfma_f32_16x16x32_f16: 64 independent 16x16 accumulators (the 128x128
+// register tile again), 8 + 8 operand fragments that never change, pseudo-random operands; one
+// pass of its loop is two passes of calib_mfma_kernel's.
 __global__ __launch_bounds__(256) void calib_mfma16_kernel(int iters, uint64_t* clocks, float* sink) {
   const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
-  float4_t acc[8][4];
-  half8_t a[8], b[4];
+  float4_t acc[8][8];
+  half8_t a[8], b[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       a[i][e] = (_Float16)(((int)(mix32(gid * 128u + i * 8u + e) >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
-      if (i < 4) b[i][e] = (_Float16)(((int)(mix32(gid * 128u + 64u + i * 8u + e) >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
+      b[i][e] = (_Float16)(((int)(mix32(gid * 128u + 64u + i * 8u + e) >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 8; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
   const uint64_t c0 = __builtin_readcyclecounter(), r0 = wall_clock64();
-  for (int it = 0; it < iters; ++it)
+  for (int it = 0; it < iters; it += 2)
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < 8; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j], a[i], acc[i][j], 0, 0, 0);
   const uint64_t c1 = __builtin_readcyclecounter(), r1 = wall_clock64();
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 8; ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) s += acc[i][j][r];
   sink[gid & 1023u] = s;
@@ -356,6 +357,7 @@ int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, si
   const bool l2_loads = random_operands == 3 || random_operands == 5;
   NF_REQUIRE(!l2_loads || scratch_bytes >= 8192 + ((size_t)8 << 20),
              "nf_calibrate_mfma: random_operands = 3 and 5 read 8 MiB of scratch behind its first 8192 bytes");
+  if (random_operands == 4) iters = (iters + 1) / 2 * 2;
   if (random_operands == 2 || l2_loads) {
     iters = (iters + 1) / 2 * 2;
     for (auto k : {reinterpret_cast<const void*>(calib_mfma_lds_kernel<0>), reinterpret_cast<const void*>(calib_mfma_lds_kernel<1>),
@@ -383,7 +385,7 @@ int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, si
     else if (random_operands == 5)
       calib_mfma_lds_kernel<2><<<grid, 256, 131072, s>>>((n + 1) / 2 * 2, clocks, sink,
                                                          static_cast<const uint8_t*>(scratch) + 8192);
-    else if (random_operands == 4) calib_mfma16_kernel<<<grid, 256, 0, s>>>(n, clocks, sink);
+    else if (random_operands == 4) calib_mfma16_kernel<<<grid, 256, 0, s>>>((n + 1) / 2 * 2, clocks, sink);
     else if (fp8) calib_mfma_kernel<true><<<grid, 256, 0, s>>>(n, random_operands, clocks, sink);
     else calib_mfma_kernel<false><<<grid, 256, 0, s>>>(n, random_operands, clocks, sink);
   };

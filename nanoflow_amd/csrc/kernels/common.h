@@ -117,6 +117,34 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
 
 // ---- global memory -> LDS without passing through registers (gfx950 buffer_load ... lds)
 typedef short short4_t __attribute__((ext_vector_type(4)));
+
+// The accumulators of G adjacent 16x16 MFMA tiles are kept as ONE vector of 4 G floats (a register
+// tuple the allocator places as a unit, like a 32x32 tile's 16), and a tile's 4 floats are taken
+// out of it and put back by constant shuffles, which cost no instruction: as 64 separate 4-float
+// values the compiler assigned them differently on either side of the slab loop's back edge and
+// permuted all 256 accumulator registers once per slab.
+template <int G> struct AccVec;
+template <> struct AccVec<1> { typedef float4_t type; };
+template <> struct AccVec<2> { typedef float type __attribute__((ext_vector_type(8))); };
+template <> struct AccVec<4> { typedef float16_t type; };
+template <int Q, class V, int... I>
+__device__ __forceinline__ float4_t acc_get_impl(const V& v, std::integer_sequence<int, I...>) {
+  return __builtin_shufflevector(v, v, (4 * Q + I)...);
+}
+template <int Q, class V>
+__device__ __forceinline__ float4_t acc_get(const V& v) {
+  return acc_get_impl<Q>(v, std::make_integer_sequence<int, 4>{});
+}
+template <int Q, int N, class V, int... I>
+__device__ __forceinline__ void acc_put_impl(V& v, float4_t c, std::integer_sequence<int, I...>) {
+  const V w = __builtin_shufflevector(c, c, (I < 4 ? I : -1)...);                       // c widened to N floats
+  v = __builtin_shufflevector(v, w, ((I >= 4 * Q && I < 4 * Q + 4) ? N + I - 4 * Q : I)...);
+}
+template <int Q, int N, class V>
+__device__ __forceinline__ void acc_put(V& v, float4_t c) {
+  acc_put_impl<Q, N>(v, c, std::make_integer_sequence<int, N>{});
+}
+
 // Out-of-range per-lane offsets read as zero (also into LDS), so tile edges need no branches:
 // out-of-range chunks just get the kOob offset.  Only the per-lane offset is range-checked by
 // the hardware, so the whole address stays in it.

@@ -35,8 +35,13 @@
 // through LDS so that D is stored, and C read, in whole 512-byte runs.
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 
 #include "common.h"
+
+#ifndef NF_GEMM_MFMA16
+#define NF_GEMM_MFMA16 1
+#endif
 
 namespace nf {
 
@@ -65,6 +70,9 @@ struct F16 {
   static __device__ __forceinline__ float16_t mfma(half8_t b, half8_t a, float16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(b, a, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ float4_t mfma16(half8_t b, half8_t a, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(b, a, c, 0, 0, 0);
+  }
   static __device__ __forceinline__ float widen(uint32_t bits) { return h2f_bits(bits); }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
   static __device__ __forceinline__ float rounded(float x) { return __half2float(__float2half_rn(x)); }
@@ -75,6 +83,9 @@ struct BF16 {
   typedef float f32x2_t __attribute__((ext_vector_type(2)));
   static __device__ __forceinline__ float16_t mfma(half8_t b, half8_t a, float16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, b), __builtin_bit_cast(bf16x8_t, a), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float4_t mfma16(half8_t b, half8_t a, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b), __builtin_bit_cast(bf16x8_t, a), c, 0, 0, 0);
   }
   static __device__ __forceinline__ float widen(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // round to nearest even
@@ -109,10 +120,24 @@ __device__ __forceinline__ void gemm_tile(
     const int lda) {
   constexpr int NB = kDual ? 2 : 1;
   using SM = GemmSmem<BM, BN, NB>;
-  constexpr int TM = BM / WM / 32;  // MFMA tiles per wave along M
-  constexpr int TN = BN / WN / 32;
   // four wavefronts (one per SIMD) or eight (two per SIMD, at most 256 registers each)
   constexpr int NW = WM * WN;
+  // The MFMA the tile is computed with.  kM16: v_mfma_f32_16x16x32 -- at this part's power cap the
+  // register-only loop delivers 19 % more flops on it than on 32x32x16 (half the accumulator
+  // traffic per flop), for the same LDS bytes per flop; its fragments are 32 deep, so a 64-deep
+  // slab is two k-steps, each issued as two sub-steps: one half of the wavefront's tile columns
+  // each, column by column.  The activation fragments of a k-step stay in registers for the step
+  // (double-buffered by k-step); the weight fragments are double-buffered by sub-step -- a
+  // sub-step reads the columns of the next one -- so that everything but the accumulators fits
+  // the 256 architectural registers and the compiler has no reason to shuffle accumulators
+  // between the two register files.
+  // Eight-wavefront tiles keep 32x32x16 (256 registers per wavefront in all).
+  constexpr bool kM16 = NW == 4 && NF_GEMM_MFMA16;
+  constexpr int MT = kM16 ? 16 : 32;  // rows and columns of an MFMA tile
+  constexpr int TM = BM / WM / MT;    // MFMA tiles per wave along M
+  constexpr int TN = BN / WN / MT;
+  constexpr int CH = NB * TN / 2;  // kM16: columns of MFMA tiles per sub-step, over both weight matrices
+  static_assert(!kM16 || (NB * TN) % 2 == 0, "a sub-step takes half of the tile columns");
   static_assert(NW == 4 || NW == 8, "four or eight wavefronts");
   static_assert((BN / WN) % 32 == 0 && (BM / WM) % 32 == 0 && BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile shape");
   constexpr int A_LOADS = BM / (8 * NW);   // 1 KB load instructions per wave per slab
@@ -127,16 +152,21 @@ __device__ __forceinline__ void gemm_tile(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int l32 = lane & 31, lg = lane >> 5;
+  const int l16 = lane & 15, lq = lane >> 4;
 
-  float16_t acc[NB][TM][TN];
+  // kM16: G adjacent column tiles share one accumulator vector (see AccVec)
+  constexpr int G = !kM16 ? 1 : TN % 4 == 0 ? 4 : TN % 2 == 0 ? 2 : 1;
+  constexpr int TNG = TN / G;
+  using acc_t = std::conditional_t<kM16, typename AccVec<G>::type, float16_t>;
+  acc_t acc[NB][TM][TNG];
 #pragma unroll
   for (int b = 0; b < NB; ++b)
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TNG; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[b][i][j][r] = 0.f;
+        for (int r = 0; r < (kM16 ? 4 * G : 16); ++r) acc[b][i][j][r] = 0.f;
 
   // ---- global -> LDS: per-lane byte offsets of the chunks this lane fetches
   const rsrc_t a_rsrc = make_rsrc(A, ((size_t)(M - 1) * lda + K) * 2);
@@ -208,43 +238,53 @@ __device__ __forceinline__ void gemm_tile(
 
   // ---- LDS -> MFMA operand fragments, double-buffered across k-steps
   // A-style: row r = l32 (+ multiples of 32), logical chunk kk*2+lg sits at chunk ^ ((r>>1)&7).
-  const uint32_t a_rd = (uint32_t)(wm * (BM / WM) + l32) * 128u;
-  const uint32_t bc_rd = (uint32_t)(wn * (BN / WN) + l32) * 128u;  // [N][K] weights
+  // kM16: row r = l16 (+ multiples of 16), logical chunk kk*4 + lq of k-step kk (32 deep), same
+  // permutation: the 16 rows of a read cycle land on 16 different 16-byte slots as well.
+  const int lrow = kM16 ? l16 : l32;
+  const uint32_t a_rd = (uint32_t)(wm * (BM / WM) + lrow) * 128u;
+  const uint32_t bc_rd = (uint32_t)(wn * (BN / WN) + lrow) * 128u;  // [N][K] weights
   uint32_t swz[4];
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) swz[kk] = (uint32_t)(((kk * 2 + lg) ^ ((l32 >> 1) & 7)) << 4);
+  for (int kk = 0; kk < 4; ++kk)
+    swz[kk] = kM16 ? (uint32_t)((((kk & 1) * 4 + lq) ^ ((l16 >> 1) & 7)) << 4) : (uint32_t)(((kk * 2 + lg) ^ ((l32 >> 1) & 7)) << 4);
   // [K][N] weights: 16-lane group g reads the 4(k) x 16(n) block at rows lg*8 + 4h.., columns
   // (g&1)*16.. of the MFMA tile, lane i of the group addressing row i/4, columns (i&3)*4..+3.
   // 32-byte unit u of a row sits at u ^ ((row & 3) << 1), row & 3 = (i/4) & 3.
+  // kM16: the 16-lane group lq holds k rows lq*8.. of the 32-deep k-step, all four groups the
+  // same 16 columns (one 32-byte unit per MFMA tile).
   const int i16 = lane & 15, bx = (i16 >> 2) & 3, g1 = (lane >> 4) & 1;
-  const uint32_t br_row = (uint32_t)(lg * 8 + (i16 >> 2)) * ROWB + (uint32_t)(i16 & 3) * 8u;
+  const uint32_t br_row = (uint32_t)((kM16 ? lq : lg) * 8 + (i16 >> 2)) * ROWB + (uint32_t)(i16 & 3) * 8u;
   uint32_t br_tbl[TN];  // byte offset inside the row of this lane's 8 bytes, per MFMA tile j
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int unit = (wn * (BN / WN)) / 16 + 2 * j + g1;  // logical 32-byte unit
+    const int unit = kM16 ? (wn * (BN / WN)) / 16 + j : (wn * (BN / WN)) / 16 + 2 * j + g1;  // logical 32-byte unit
     br_tbl[j] = (uint32_t)((unit ^ (bx << 1)) * 32);
   }
 
   half8_t af[2][TM];
   half8_t bf[2][NB][TN];
+  half8_t bh[2][CH > 0 ? CH : 1];  // kM16: the weight fragments of a sub-step's columns
   constexpr int READS = TM + NB * TN;  // fragment reads per k-step: q < TM activations, then weights
+  constexpr int KSTEP = kM16 ? 32 : 16;
   // sa / sb: the stage holding the slab's activations / weights
   auto read_one = [&](auto q_c, auto kk_c, auto buf_c, const uint8_t* sa, const uint8_t* sb) {
     constexpr int q = decltype(q_c)::value, kk = decltype(kk_c)::value, buf = decltype(buf_c)::value;
     if constexpr (q < TM) {
-      af[buf][q] = *reinterpret_cast<const half8_t*>(sa + a_rd + swz[kk] + q * 32 * 128);
+      af[buf][q] = *reinterpret_cast<const half8_t*>(sa + a_rd + swz[kk] + q * MT * 128);
     } else {
       constexpr int b = (q - TM) / TN, j = (q - TM) % TN;
       const uint8_t* bs = sb + b * SM::b_bytes;
+      // kM16: `buf` is the sub-step's slot, the fragment goes to its place among the sub-step's columns
+      half8_t& dst = kM16 ? bh[buf][(q - TM) % (CH > 0 ? CH : 1)] : bf[buf][b][j];
       if constexpr (kBCol) {
-        bf[buf][b][j] = *reinterpret_cast<const half8_t*>(bs + bc_rd + swz[kk] + j * 32 * 128);
+        dst = *reinterpret_cast<const half8_t*>(bs + bc_rd + swz[kk] + j * MT * 128);
       } else {
-        const uint8_t* p = bs + br_row + br_tbl[j] + kk * 16 * ROWB;
+        const uint8_t* p = bs + br_row + br_tbl[j] + kk * KSTEP * ROWB;
         const short4_t lo = lds_read_tr16(p);
         const short4_t hi = lds_read_tr16(p + 4 * ROWB);
         typedef short short8_t __attribute__((ext_vector_type(8)));
         const short8_t v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        bf[buf][b][j] = __builtin_bit_cast(half8_t, v);
+        dst = __builtin_bit_cast(half8_t, v);
       }
     }
   };
@@ -259,12 +299,39 @@ __device__ __forceinline__ void gemm_tile(
                   const uint8_t* sa, const uint8_t* sb) {
     constexpr int kk = decltype(kk_c)::value, L0 = decltype(l0_c)::value, LSTR = decltype(lstr_c)::value;
     constexpr int NL = decltype(nl_c)::value, RK = decltype(rk_c)::value;
+    if constexpr (kM16) {
+      // Sub-step kk of the slab: the MFMAs of k-step kk / 2 (32 deep) on half kk % 2 of the tile
+      // columns, column by column.  Fragment reads dealt out between them: the weight fragments of
+      // the next sub-step's columns (from the stage at sb: the next slab's for sub-step 3, which
+      // runs past the slab's barrier), and activation fragments -- sub-steps 0 and 1 one half each
+      // of k-step 1's, sub-step 2 none, sub-step 3 all of the next slab's k-step 0.  The callers
+      // name the 16-deep k-step the step would prefetch: RK = kk + 1, 0 past the barrier, -1 for none.
+      constexpr int K2 = kk >> 1, H = kk & 1, NMH = CH * TM;
+      constexpr int NXT = (kk + 1) & 3, K2N = NXT >> 1, HN = NXT & 1;  // the sub-step the weight reads are for
+      constexpr int NRB = RK < 0 ? 0 : CH;
+      constexpr int A0 = RK == 2 ? TM / 2 : 0, A1 = RK == 1 ? TM / 2 : (RK == 0 || RK == 2) ? TM : 0;
+      constexpr int NRA = A1 - A0, AK = RK == 0 ? 0 : 1;  // the k-step (and buffer) those activation fragments are of
+      constexpr int S16 = NL + NRB + NRA;
+      static_for<NMH>([&](auto n_c) {
+        constexpr int n = decltype(n_c)::value;
+        constexpr int c = n / TM, i = n % TM, col = H * CH + c, b = col / TN, j = col % TN;
+        acc_put<j % G, 4 * G>(acc[b][i][j / G], E::mfma16(bh[H][c], af[K2][i], acc_get<j % G>(acc[b][i][j / G])));
+        constexpr int lo = n * S16 / NMH, hi = (n + 1) * S16 / NMH;
+        static_for<hi - lo>([&](auto d_c) {
+          constexpr int q = lo + decltype(d_c)::value;
+          if constexpr (q < NL) load_one(ic<L0 + LSTR * q>{}, la, lb, ld_ok);
+          else if constexpr (q < NL + NRB) read_one(ic<TM + HN * CH + (q - NL)>{}, ic<K2N>{}, ic<HN>{}, sa, sb);
+          else read_one(ic<A0 + (q - NL - NRB)>{}, ic<AK>{}, ic<AK>{}, sa, sb);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    } else {
     constexpr int NR = RK < 0 ? 0 : READS;
     constexpr int S = NL + NR;
     static_for<NM>([&](auto n_c) {
       constexpr int n = decltype(n_c)::value;
       constexpr int b = n / (TN * TM), j = (n / TM) % TN, i = n % TM;
-      acc[b][i][j] = E::mfma(bf[kk & 1][b][j], af[kk & 1][i], acc[b][i][j]);
+      if constexpr (!kM16) acc[b][i][j] = E::mfma(bf[kk & 1][b][j], af[kk & 1][i], acc[b][i][j]);
       // Side work is dealt out evenly, the loads ahead of the fragment reads.  Measured the other
       // way round (reads first, in the order the next step consumes them): 3-5 % slower on the
       // 256-row tiles -- the loads then queue behind each other at the end of the step.
@@ -276,6 +343,7 @@ __device__ __forceinline__ void gemm_tile(
       });
       __builtin_amdgcn_sched_barrier(0);
     });
+    }
   };
   using T_ = std::true_type;
   using F_ = std::false_type;
@@ -314,7 +382,7 @@ __device__ __forceinline__ void gemm_tile(
       }
     }
     __syncthreads();
-    static_for<READS>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, a_ptr(0), b_ptr(0)); });
+    static_for<(kM16 ? TM + CH : READS)>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, a_ptr(0), b_ptr(0)); });
     if (nslab > 1) {  // what k-step 3 of a slab before slab 0 would have issued
       const uint32_t la = a_lds(1);
       static_for<HA>([&](auto t_c) { load_one(t_c, la, la, k_ok_of(1)); });
@@ -393,7 +461,7 @@ __device__ __forceinline__ void gemm_tile(
   // matters for speed: waiting for everything is always correct)
   wait_loads(nslab >= NS - 1 ? 1 : 0);
   __syncthreads();
-  static_for<READS>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, smem, smem + SM::a_bytes); });
+  static_for<(kM16 ? TM + CH : READS)>([&](auto q_c) { read_one(q_c, ic<0>{}, ic<0>{}, smem, smem + SM::a_bytes); });
   if (NS - 1 < nslab) {  // the share of slab NS-1 that a slab's k-step 3 would have issued
     const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + (NS - 1) * SM::stage_bytes + wave * 1024);
     const bool k_ok = (NS - 1) * BK + a_kc < K;
@@ -424,12 +492,38 @@ __device__ __forceinline__ void gemm_tile(
   constexpr int ROWP = CW * 4 + 16;  // bytes per padded fp32 row
   constexpr int CPR = CW / 4;        // 4-column groups per row
   static_assert(NW * 32 * ROWP <= (int)SM::bytes && (32 * CPR) % 64 == 0, "epilogue staging");
+  constexpr int PASSES = BM / WM / 32;  // 32 rows of the wavefront's block per pass
+  auto ep_of = [&](int row) { return smem + wave * (32 * ROWP) + row * ROWP; };
+  // the pass's rows as the MFMA left them: a lane's 4 consecutive columns of a row, 16 bytes
+  auto stage_pass = [&](int i, auto value) {
+    if constexpr (kM16) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          float4_t v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = value(2 * i + ii, j, e);
+          *reinterpret_cast<float4_t*>(ep_of(ii * 16 + l16) + (j * 16 + lq * 4) * 4) = v;
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          float4_t v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = value(i, j, qd * 4 + e);
+          *reinterpret_cast<float4_t*>(ep_of(l32) + (j * 32 + qd * 8 + lg * 4) * 4) = v;
+        }
+    }
+  };
   __syncthreads();  // every wavefront has read its last fragments
   uint8_t* ep = smem + wave * (32 * ROWP);
   constexpr int ITER = 32 * CPR / 64;  // 4-column groups per lane and pass
   typedef unsigned int u32v2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int i = 0; i < PASSES; ++i) {
     // C and D go through buffer descriptors based at the pass's first row and ending with the
     // matrix (rows >= M fall outside and are dropped by the hardware; columns >= N get an
     // out-of-range offset), so the pass has no branches and all its loads are in flight together.
@@ -466,15 +560,7 @@ __device__ __forceinline__ void gemm_tile(
       typedef unsigned int u32v4_t __attribute__((ext_vector_type(4)));
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int qd = 0; qd < 4; ++qd) {
-            float4_t v;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[b][i][j][qd * 4 + e];
-            *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
-          }
+        stage_pass(i, [&](int ti, int tj, int r) { return kM16 ? acc[b][ti][tj / G][(tj % G) * 4 + r] : acc[b][ti][tj][r]; });
         float* dst = b == 0 ? reinterpret_cast<float*>(D) : reinterpret_cast<float*>(const_cast<uint16_t*>(C));
         const __amdgpu_buffer_rsrc_t p_rsrc =
             __builtin_amdgcn_make_buffer_rsrc(dst + row0, 0, rows > 0 ? rows * N * 4 : 0, 0x00020000);
@@ -488,18 +574,11 @@ __device__ __forceinline__ void gemm_tile(
       }
       continue;
     }
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        float4_t v;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (kDual) v[e] = swiglu_rounded<E>(acc[0][i][j][qd * 4 + e], acc[1][i][j][qd * 4 + e]);
-          else v[e] = acc[0][i][j][qd * 4 + e];
-        }
-        *reinterpret_cast<float4_t*>(ep + l32 * ROWP + (j * 32 + qd * 8 + lg * 4) * 4) = v;
-      }
+    stage_pass(i, [&](int ti, int tj, int r) {
+      const int gj = kM16 ? tj / G : tj, gr = kM16 ? (tj % G) * 4 + r : r;
+      if constexpr (kDual) return swiglu_rounded<E>(acc[0][ti][gj][gr], acc[1][ti][gj][gr]);
+      else return acc[0][ti][gj][gr];
+    });
     float4_t a4[ITER];
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {

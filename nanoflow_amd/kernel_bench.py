@@ -181,6 +181,8 @@ def corun(a, shape, rnd):
         phase("mfma loop f16, zero operands", lambda: K.calibrate_mfma(False, False, 2000), secs=2.0)
         phase("mfma loop f16, pseudo-random operands re-read from LDS", lambda: K.calibrate_mfma(False, 2, 2000), secs=2.0)
         phase("   ... with the tile's operand loads (L2 -> LDS) beside them", lambda: K.calibrate_mfma(False, 3, 2000), secs=2.0)
+        phase("   ... with those loads routed through registers instead", lambda: K.calibrate_mfma(False, 5, 2000), secs=2.0)
+        phase("mfma loop f16 on 16x16x32 instructions, pseudo-random operands", lambda: K.calibrate_mfma(False, 4, 2000), secs=2.0)
         buf = torch.empty(4 << 30, dtype=torch.uint8, device=DEV).random_()
         sc = torch.zeros(8192, dtype=torch.uint8, device=DEV)
         import ctypes as C
@@ -311,7 +313,7 @@ def main():
                 print(f"   ... with the same operand bytes routed through registers (buffer_load, ds_write_b128) instead: "
                       f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
                 tf, mhz = K.calibrate_mfma(False, 4, 40000)
-                print(f"mfma loop f16 16x16x32 pseudo-random operands (32 accumulators, the same flops per pass): "
+                print(f"mfma loop f16 16x16x32 pseudo-random operands (64 accumulators: the same register tile): "
                       f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
                 for n in (1, 2, 3, 4, 6, 8):
                     tf, mhz = K.calibrate_mfma(False, 10 + n, 40000)
