@@ -1,12 +1,13 @@
-// 16-bit x 16-bit -> fp32 -> 16-bit GEMM family for gfx950 on v_mfma_f32_32x32x16_f16 (fp16, the
-// pipeline's type) and v_mfma_f32_32x32x16_bf16 (bf16: same kernels, other element type).
+// 16-bit x 16-bit -> fp32 -> 16-bit GEMM family for gfx950 on v_mfma_f32_16x16x32_f16 (fp16, the
+// pipeline's type; 32x32x16 for the tiles on eight wavefronts) and the bf16 forms of the same
+// instructions (bf16: same kernels, other element type).
 //
 //   D = half(alpha * A.B + beta * C)                     (plain; QKV, O, down, LM head)
 //   D = half(silu(half(A.Bg)) * half(A.Bu))              (dual; gate/up SwiGLU)
 //
 // Workgroup = 256 threads = 4 wavefronts in a WM x WN grid; each wavefront owns a
-// (BM/WM) x (BN/WN) block of 32x32 MFMA tiles.  K is walked in slabs of 64 through a ring of
-// two to four LDS stages (as many as fit 144 KB).
+// (BM/WM) x (BN/WN) block of 16x16 (or 32x32) MFMA tiles.  K is walked in slabs of 64 through a
+// ring of two to four LDS stages (as many as fit 144 KB).
 //
 // Operands go from global memory STRAIGHT INTO LDS (buffer_load_dwordx4 ... lds): a CU moves
 // about 38 GB/s through the load-to-register path but well over 100 GB/s through this one, and
@@ -31,7 +32,7 @@
 // current k-step, in a pinned order; one barrier per slab.
 //
 // The MFMA is issued as D^T = B^T.A^T (weights as the first operand): a lane ends up with 4
-// consecutive output columns of 32 rows.  The epilogue turns each wavefront's block around
+// consecutive output columns of a row (of 32 rows with the 32x32 instruction).  The epilogue turns each wavefront's block around
 // through LDS so that D is stored, and C read, in whole 512-byte runs.
 #include <algorithm>
 #include <type_traits>
@@ -230,6 +231,35 @@ __device__ __forceinline__ void gemm_tile(
       }
     }
   };
+  // The same load in two pieces, for steps whose MFMAs leave room for two or three other
+  // instructions each: the offset (masked, and advanced for the next slab) first, the M0 write and
+  // the load instruction one MFMA later.
+  uint32_t pend = 0;
+  auto load_prepare = [&](auto t_c, bool k_ok) {
+    constexpr int t = decltype(t_c)::value;
+    if constexpr (t < A_LOADS) {
+      pend = k_ok ? a_off[t] : kOob;
+      a_off[t] += BK * 2;
+    } else {
+      constexpr int b = (t - A_LOADS) / B_LOADS, tt = (t - A_LOADS) % B_LOADS;
+      if constexpr (kBCol) {
+        pend = k_ok ? b_off[b][tt] : kOob;
+        b_off[b][tt] += BK * 2;
+      } else {
+        pend = b_off[b][tt];
+        b_off[b][tt] += b_slab;
+      }
+    }
+  };
+  auto load_issue = [&](auto t_c, uint32_t la, uint32_t lb) {
+    constexpr int t = decltype(t_c)::value;
+    if constexpr (t < A_LOADS) {
+      load16_to_lds<t * NW * 1024>(a_rsrc, pend, la);
+    } else {
+      constexpr int b = (t - A_LOADS) / B_LOADS, tt = (t - A_LOADS) % B_LOADS;
+      load16_to_lds<b * SM::b_bytes + tt * NW * 1024>(b_rsrc[b], pend, lb);
+    }
+  };
   auto load_slab = [&](int stage, int k0) {  // every load of one slab, back to back (one ring for both operands)
     const uint32_t st = __builtin_amdgcn_readfirstlane(smem_lds + stage * SM::stage_bytes + wave * 1024);
     const bool k_ok = k0 + a_kc < K;
@@ -311,7 +341,7 @@ __device__ __forceinline__ void gemm_tile(
       constexpr int NRB = RK < 0 ? 0 : CH;
       constexpr int A0 = RK == 2 ? TM / 2 : 0, A1 = RK == 1 ? TM / 2 : (RK == 0 || RK == 2) ? TM : 0;
       constexpr int NRA = A1 - A0, AK = RK == 0 ? 0 : 1;  // the k-step (and buffer) those activation fragments are of
-      constexpr int S16 = NL + NRB + NRA;
+      constexpr int S16 = 2 * NL + NRB + NRA;  // a load counts twice: prepared, then issued
       static_for<NMH>([&](auto n_c) {
         constexpr int n = decltype(n_c)::value;
         constexpr int c = n / TM, i = n % TM, col = H * CH + c, b = col / TN, j = col % TN;
@@ -319,9 +349,14 @@ __device__ __forceinline__ void gemm_tile(
         constexpr int lo = n * S16 / NMH, hi = (n + 1) * S16 / NMH;
         static_for<hi - lo>([&](auto d_c) {
           constexpr int q = lo + decltype(d_c)::value;
-          if constexpr (q < NL) load_one(ic<L0 + LSTR * q>{}, la, lb, ld_ok);
-          else if constexpr (q < NL + NRB) read_one(ic<TM + HN * CH + (q - NL)>{}, ic<K2N>{}, ic<HN>{}, sa, sb);
-          else read_one(ic<A0 + (q - NL - NRB)>{}, ic<AK>{}, ic<AK>{}, sa, sb);
+          if constexpr (q < 2 * NL) {
+            if constexpr (q % 2 == 0) load_prepare(ic<L0 + LSTR * (q / 2)>{}, ld_ok);
+            else load_issue(ic<L0 + LSTR * (q / 2)>{}, la, lb);
+          } else if constexpr (q < 2 * NL + NRB) {
+            read_one(ic<TM + HN * CH + (q - 2 * NL)>{}, ic<K2N>{}, ic<HN>{}, sa, sb);
+          } else {
+            read_one(ic<A0 + (q - 2 * NL - NRB)>{}, ic<AK>{}, ic<AK>{}, sa, sb);
+          }
         });
         __builtin_amdgcn_sched_barrier(0);
       });
