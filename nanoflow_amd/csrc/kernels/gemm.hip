@@ -21,10 +21,11 @@
 //       logical chunk c at position c ^ ((r >> 1) & 7).  An MFMA fragment is one 16-byte read;
 //       the 16 rows of a read cycle (two per 256 bytes) land on 16 different 16-byte slots.
 //   [K][N] weights               kept row-major, 64 rows of BN*2 bytes; row r keeps chunk c at
-//       position c ^ ((r & 3) << 2).  The k-contiguous MFMA operand is produced by the
-//       transposing LDS read (ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(n) block row-wise
-//       and receive it column-wise), two per operand; the 4 rows x 64 bytes a read cycle
-//       touches sit in 4 different 64-byte bank groups.
+//       position c ^ ((r & 3) << 2) ^ (((r >> 3) & 1) << 1).  The k-contiguous MFMA operand is
+//       produced by the transposing LDS read (ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(n)
+//       block row-wise and receive it column-wise), two per operand; the 2 x 4 rows x 32 bytes a
+//       read cycle touches (two k-groups of 8 rows, 8 rows apart) sit in 8 different 32-byte
+//       bank groups.
 // With these two permutations SQ_LDS_BANK_CONFLICT reads zero for the kernel.
 // No staging registers, no permutes, no LDS stores in the main loop.  A wavefront is alone on
 // its SIMD, so nothing hides a stall of its instruction stream: the loads of later slabs and
@@ -200,7 +201,7 @@ __device__ __forceinline__ void gemm_tile(
     } else {
       const int g = (t * NW + wave) * 64 + lane;  // 16-byte slot of the slab's LDS image
       const int row = g / B_CPR;
-      const int c = (g % B_CPR) ^ ((row & 3) << 2);
+      const int c = (g % B_CPR) ^ ((row & 3) << 2) ^ (((row >> 3) & 1) << 1);
       off = ((uint32_t)row * (uint32_t)N + n_base + c * 8) * 2u;
     }
 #pragma unroll
@@ -279,7 +280,8 @@ __device__ __forceinline__ void gemm_tile(
     swz[kk] = kM16 ? (uint32_t)((((kk & 1) * 4 + lq) ^ ((l16 >> 1) & 7)) << 4) : (uint32_t)(((kk * 2 + lg) ^ ((l32 >> 1) & 7)) << 4);
   // [K][N] weights: 16-lane group g reads the 4(k) x 16(n) block at rows lg*8 + 4h.., columns
   // (g&1)*16.. of the MFMA tile, lane i of the group addressing row i/4, columns (i&3)*4..+3.
-  // 32-byte unit u of a row sits at u ^ ((row & 3) << 1), row & 3 = (i/4) & 3.
+  // 32-byte unit u of a row sits at u ^ ((row & 3) << 1) ^ ((row >> 3) & 1), row & 3 = (i/4) & 3 and
+  // (row >> 3) & 1 = the parity of the lane group's k rows.
   // kM16: the 16-lane group lq holds k rows lq*8.. of the 32-deep k-step, all four groups the
   // same 16 columns (one 32-byte unit per MFMA tile).
   const int i16 = lane & 15, bx = (i16 >> 2) & 3, g1 = (lane >> 4) & 1;
@@ -288,7 +290,7 @@ __device__ __forceinline__ void gemm_tile(
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int unit = kM16 ? (wn * (BN / WN)) / 16 + j : (wn * (BN / WN)) / 16 + 2 * j + g1;  // logical 32-byte unit
-    br_tbl[j] = (uint32_t)((unit ^ (bx << 1)) * 32);
+    br_tbl[j] = (uint32_t)((unit ^ (bx << 1) ^ (kM16 ? (lq & 1) : lg)) * 32);
   }
 
   half8_t af[2][TM];
