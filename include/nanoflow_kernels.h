@@ -261,8 +261,9 @@ NF_API int nf_argmax_f16(const uint16_t* logits, uint16_t* max_vals, int32_t* ar
  *   (1), or (2, fp16 only) on pseudo-random operands that each wavefront re-reads from LDS before
  *   every 16 instructions, the way the main loop of the 256x256 GEMM tile is fed, or (3, fp16
  *   only; `scratch` then holds 8192 + 8 MiB bytes) with that tile's operand loads beside them as
- *   well, from a window of scratch the L2 holds straight into LDS, or (4, fp16 only) as 1 with
- *   v_mfma_f32_16x16x32_f16 instead (the same flops per pass), or (5, fp16 only; scratch as for 3)
+ *   well, from a window of scratch the L2 holds straight into LDS, or (4) as 1 with the 16x16
+ *   instruction of the type instead (16x16x32 f16, 16x16x128 fp8; the same flops per pass on 64
+ *   accumulators), or (5, fp16 only; scratch as for 3)
  *   as 3 with the operand bytes routed through registers (buffer_load_dwordx4, ds_write_b128), or
  *   (10 + n, n <= 64) as 1 with n x 64 idle cycles after every 16 instructions;
  *   *tflops = the rate, *clock_mhz = shader clock the wavefronts saw while running.

@@ -104,16 +104,21 @@ __global__ __launch_bounds__(256) void calib_mfma_kernel(int iters, int random_o
 // The same flops from v_mfma_f32_16x16x32_f16: 64 independent 16x16 accumulators (the 128x128
 // register tile again), 8 + 8 operand fragments that never change, pseudo-random operands; one
 // pass of its loop is two passes of calib_mfma_kernel's.
+template <bool kF8>
 __global__ __launch_bounds__(256) void calib_mfma16_kernel(int iters, uint64_t* clocks, float* sink) {
   const uint32_t gid = blockIdx.x * 256u + threadIdx.x;
   float4_t acc[8][8];
   half8_t a[8], b[8];
+  v8i32 a8[8], b8[8];  // kF8: v_mfma_f32_16x16x128_f8f6f4 on e4m3 codes with |x| < 1
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      a[i][e] = (_Float16)(((int)(mix32(gid * 128u + i * 8u + e) >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
-      b[i][e] = (_Float16)(((int)(mix32(gid * 128u + 64u + i * 8u + e) >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
+      const uint32_t ha = mix32(gid * 128u + i * 8u + e), hb = mix32(gid * 128u + 64u + i * 8u + e);
+      a[i][e] = (_Float16)(((int)(ha >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
+      b[i][e] = (_Float16)(((int)(hb >> 8) - (1 << 23)) * (1.0f / (1 << 23)));
+      a8[i][e] = (int)(ha & 0xb7b7b7b7u);
+      b8[i][e] = (int)(hb & 0xb7b7b7b7u);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -123,7 +128,12 @@ __global__ __launch_bounds__(256) void calib_mfma16_kernel(int iters, uint64_t* 
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < 8; ++j) {
+        if constexpr (kF8)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b8[j], a8[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+        else
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+      }
   const uint64_t c1 = __builtin_readcyclecounter(), r1 = wall_clock64();
   float s = 0.f;
 #pragma unroll
@@ -350,7 +360,7 @@ int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, si
                       double* clock_mhz, nf_stream_t stream) {
   NF_REQUIRE(iters > 0 && scratch && scratch_bytes >= 8192 && tflops && clock_mhz, "nf_calibrate_mfma: bad arguments");
   NF_REQUIRE(random_operands >= 0 && (random_operands <= 5 || (random_operands >= 10 && random_operands <= 74)) &&
-                 !(fp8 && random_operands >= 2 && random_operands <= 5),
+                 !(fp8 && random_operands >= 2 && random_operands <= 5 && random_operands != 4),
              "nf_calibrate_mfma: random_operands = %d (0, 1, 10 + n = 1 with n x 64 idle cycles per 16 MFMAs, or fp16 "
              "only: 2 = operands re-read from LDS, 3 = and operand loads from L2 into LDS beside them, 4 = 1 with "
              "16x16x32 MFMAs, 5 = 3 with the operand loads routed through registers)", random_operands);
@@ -385,7 +395,8 @@ int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, si
     else if (random_operands == 5)
       calib_mfma_lds_kernel<2><<<grid, 256, 131072, s>>>((n + 1) / 2 * 2, clocks, sink,
                                                          static_cast<const uint8_t*>(scratch) + 8192);
-    else if (random_operands == 4) calib_mfma16_kernel<<<grid, 256, 0, s>>>((n + 1) / 2 * 2, clocks, sink);
+    else if (random_operands == 4 && fp8) calib_mfma16_kernel<true><<<grid, 256, 0, s>>>((n + 1) / 2 * 2, clocks, sink);
+    else if (random_operands == 4) calib_mfma16_kernel<false><<<grid, 256, 0, s>>>((n + 1) / 2 * 2, clocks, sink);
     else if (fp8) calib_mfma_kernel<true><<<grid, 256, 0, s>>>(n, random_operands, clocks, sink);
     else calib_mfma_kernel<false><<<grid, 256, 0, s>>>(n, random_operands, clocks, sink);
   };

@@ -351,13 +351,17 @@ __device__ __forceinline__ void gemm_tile(
         constexpr int lo = n * S16 / NMH, hi = (n + 1) * S16 / NMH;
         static_for<hi - lo>([&](auto d_c) {
           constexpr int q = lo + decltype(d_c)::value;
-          if constexpr (q < 2 * NL) {
-            if constexpr (q % 2 == 0) load_prepare(ic<L0 + LSTR * (q / 2)>{}, ld_ok);
-            else load_issue(ic<L0 + LSTR * (q / 2)>{}, la, lb);
-          } else if constexpr (q < 2 * NL + NRB) {
-            read_one(ic<TM + HN * CH + (q - 2 * NL)>{}, ic<K2N>{}, ic<HN>{}, sa, sb);
+          // reads first (activation fragments, then weight fragments), then the load pieces: the
+          // fragments are what the next sub-step waits for
+          constexpr int NRD = NRB + NRA;
+          constexpr int qq = q < NRA ? 2 * NL + NRB + q : q < NRD ? 2 * NL + (q - NRA) : q - NRD;
+          if constexpr (qq < 2 * NL) {
+            if constexpr (qq % 2 == 0) load_prepare(ic<L0 + LSTR * (qq / 2)>{}, ld_ok);
+            else load_issue(ic<L0 + LSTR * (qq / 2)>{}, la, lb);
+          } else if constexpr (qq < 2 * NL + NRB) {
+            read_one(ic<TM + HN * CH + (qq - 2 * NL)>{}, ic<K2N>{}, ic<HN>{}, sa, sb);
           } else {
-            read_one(ic<A0 + (q - 2 * NL - NRB)>{}, ic<AK>{}, ic<AK>{}, sa, sb);
+            read_one(ic<A0 + (qq - 2 * NL - NRB)>{}, ic<AK>{}, ic<AK>{}, sa, sb);
           }
         });
         __builtin_amdgcn_sched_barrier(0);

@@ -302,6 +302,10 @@ def main():
                 tf, mhz = K.calibrate_mfma(fp8, rand, 40000)
                 print(f"mfma loop {'fp8 32x32x64' if fp8 else 'f16 32x32x16'} {'pseudo-random' if rand else 'zero':13s} operands: "
                       f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
+            if fp8:
+                tf, mhz = K.calibrate_mfma(True, 4, 40000)
+                print(f"mfma loop fp8 16x16x128 pseudo-random operands (64 accumulators: the same register tile): "
+                      f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
             if not fp8:
                 tf, mhz = K.calibrate_mfma(False, 2, 40000)
                 print(f"mfma loop f16 32x32x16 pseudo-random operands re-read from LDS every 16 MFMAs (8 x 16 B per lane): "
