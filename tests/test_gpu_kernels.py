@@ -643,6 +643,15 @@ def test_attention_decode_many_requests(K, oracle, Hq, Hkv):
     _attn_case(K, oracle, Hq, Hkv, lens, [], seed=16)
 
 
+@pytest.mark.parametrize("Hq,Hkv,n", [(32, 8, 77), (8, 8, 13), (4, 2, 139), (32, 8, 5)])
+def test_attention_decode_request_counts_off_the_group_of_eight(K, oracle, Hq, Hkv, n):
+    """The decode kernel orders its work items (head, request) inside groups of 8 requests and
+    (request, head) past the last whole group: counts that leave a remainder, fewer than 8
+    requests, and kv-head counts other than 8."""
+    lens = [int(x) for x in np.random.default_rng(17).integers(1, 200, size=n)]
+    _attn_case(K, oracle, Hq, Hkv, lens, [], seed=17)
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (64, 8), (8, 4), (4, 4)])
 def test_attention_chunked_prefill(K, oracle, Hq, Hkv):
     _attn_case(K, oracle, Hq, Hkv, [], [(0, 1), (0, 37), (100, 64), (5, 130), (256, 3)], seed=12)
