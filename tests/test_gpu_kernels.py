@@ -700,11 +700,12 @@ def test_calibration_loops_report_rates_this_part_can_have(K):
     small, _ = K.calibrate_mfma(False, 4, 4000)
     idle, _ = K.calibrate_mfma(False, 14, 4000)
     f8, _ = K.calibrate_mfma(True, True, 4000)
+    f8_small, _ = K.calibrate_mfma(True, 4, 4000)
     print(f"mfma f16 zero {zero:.0f} random {rnd:.0f} from LDS {lds:.0f} + loads {direct:.0f} (through registers {via_regs:.0f}) "
           f"16x16x32 {small:.0f} duty 2/3 {idle:.0f} fp8 {f8:.0f} TFLOP/s", flush=True)
     assert 500 < rnd <= zero <= 2600 and 1000 < mhz1 <= mhz0 < 2600
     assert 500 < direct < lds * 1.03 and lds < rnd * 1.03 and 500 < via_regs < lds * 1.03
-    assert 500 < small < 2600 and 500 < idle < rnd * 1.03 and rnd < f8 <= 5200
+    assert 500 < small < 2600 and 500 < idle < rnd * 1.03 and rnd < f8 <= 5200 and rnd < f8_small <= 5200
     with pytest.raises(kernels.NanoflowKernelError, match="random_operands"):
         K.calibrate_mfma(False, 6, 100)
     with pytest.raises(kernels.NanoflowKernelError, match="random_operands"):
