@@ -263,9 +263,7 @@ NF_API int nf_argmax_f16(const uint16_t* logits, uint16_t* max_vals, int32_t* ar
  *   only; `scratch` then holds 8192 + 8 MiB bytes) with that tile's operand loads beside them as
  *   well, from a window of scratch the L2 holds straight into LDS, or (4) as 1 with the 16x16
  *   instruction of the type instead (16x16x32 f16, 16x16x128 fp8; the same flops per pass on 64
- *   accumulators), or (5, fp16 only; scratch as for 3)
- *   as 3 with the operand bytes routed through registers (buffer_load_dwordx4, ds_write_b128), or
- *   (10 + n, n <= 64) as 1 with n x 64 idle cycles after every 16 instructions;
+ *   accumulators);
  *   *tflops = the rate, *clock_mhz = shader clock the wavefronts saw while running.
  * nf_calibrate_hbm_read: all CUs stream `bytes` of `buf` (16-byte aligned, much larger than the
  *   last-level cache) `reps` times; *gbps = the read rate.

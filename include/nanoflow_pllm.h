@@ -151,6 +151,21 @@ NF_PLLM_API int pllm_create_init_data(nf_vortex_init_data* data, uint16_t** kv_d
                                       const nf_vortex_model_weight* weight);
 /* pllm_python.config (pybind.cu:106-108). */
 NF_PLLM_API int pllm_config(const nf_vortex_config_data* config);
+/* What pllm_config checks before it builds anything, callable on its own (no state, no device):
+ * 0 < global_batch_size <= max_batch_size; for the nano-batched types 0 < nanobatch_1_size <
+ * global_batch_size; for the types that run the four-way schedule (PLLM, NANOBATCH, PLLMOFFLOAD,
+ * KQVBIAS, NANOBATCH_KQVBIAS: pipeline/src/computeBound.cu:234-247) also 0 <= kqv1_size <=
+ * nanobatch_1_size and 0 <= kqv3_size <= global_batch_size - nanobatch_1_size.  The reference
+ * checks none of this (pipeline/src/pipeline.cu:279-470 sizes its buffers from the fields as given). */
+NF_PLLM_API int pllm_check_nanobatch_split(int pipeline_type, int max_batch_size, int global_batch_size,
+                                           int nanobatch_1_size, int kqv1_size, int kqv3_size);
+/* What pllm_update checks of gemv_batch_size[4] (serve_8B.py:391-394 produces it): the groups sum
+ * to the decode rows; nano-batched types: groups 0+1 = the decode rows of nano-batch 1; four-way
+ * types: the rows of groups 0..i lie inside QKV pieces 0..i (decode attention of group i starts as
+ * soon as QKV piece i and its RoPE-append are done, pipeline/src/pipeline.cu:640-676; a group that
+ * reaches further would read rows not yet written).  No state, no device. */
+NF_PLLM_API int pllm_check_gemv_split(int pipeline_type, int nanobatch_1_size, int kqv1_size, int kqv3_size,
+                                      int decode_rows, const int32_t* gemv_batch_size);
 /* pllm_python.update (pybind.cu:100-104 -> update(), computeBound.cu:115-161). */
 NF_PLLM_API int pllm_update(const nf_vortex_update_data* update);
 /* run / run_async / run_async_wait (computeBound.cu:27-61). */

@@ -168,8 +168,7 @@ void Worker::init() {
   // Type -> schedule as the reference maps them (pipeline/src/computeBound.cu:234-247): the five
   // types of its main Pipeline run the four-way nano-batch schedule, without their exchange steps.
   const bool bias = hasKQVBias(PipeTy);
-  if (PipeTy == PipelineType::PLLM || PipeTy == PipelineType::PLLMOFFLOAD || PipeTy == PipelineType::NANOBATCH ||
-      PipeTy == PipelineType::KQVBIAS || PipeTy == PipelineType::NANOBATCH_KQVBIAS)
+  if (isFourWay(PipeTy))
     pipeline = std::make_unique<Pipeline>(input, rank, nranks, vnranks, PipeTy == PipelineType::PLLMOFFLOAD,
                                           PipeTy == PipelineType::NANOBATCH || PipeTy == PipelineType::NANOBATCH_KQVBIAS,
                                           bias);

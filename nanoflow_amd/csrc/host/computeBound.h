@@ -69,6 +69,11 @@ public:
     return t == PipelineType::KQVBIAS || t == PipelineType::NONOVERLAP_KQVBIAS ||
            t == PipelineType::NANOBATCH_KQVBIAS;
   }
+  // the reference's main schedule: four QKV / attention nano-batches (class Pipeline)
+  static bool isFourWay(PipelineType t) {
+    return t == PipelineType::PLLM || t == PipelineType::PLLMOFFLOAD || t == PipelineType::NANOBATCH ||
+           t == PipelineType::KQVBIAS || t == PipelineType::NANOBATCH_KQVBIAS;
+  }
   static bool isSequential(PipelineType t) {
     return t == PipelineType::NON_OVERLAP_LOCAL || t == PipelineType::NONOVERLAP_KQVBIAS ||
            t == PipelineType::NONOVERLAP;

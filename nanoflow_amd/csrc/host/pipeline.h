@@ -15,6 +15,8 @@
 // More than one rank (the collectives) is outside this build.
 #pragma once
 #include <array>
+#include <cstdarg>
+#include <string>
 #include <memory>
 
 #include "allocManager.h"
@@ -69,6 +71,19 @@ protected:
   // GEMMs add vortexLayerWeight::B_KQV ([1, kqv_n], columns K|V|Q) to every row, beta = 1
   // (pipeline/src/pipeline.cu:520-533, pipeline_nonoverlap.cu:209-211).
   WeightFormat weight_format = getWeightFormat();  // of the five per-layer GEMM weights
+  // config() reports what it cannot build here and returns early instead of ending the process
+  // (the reference dereferences the null wrapper, pipeline_local.cu:850); the control plane turns
+  // it into an error code.
+  std::string config_error;
+  void configFail(const char* fmt, ...) __attribute__((format(printf, 2, 3))) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    config_error = buf;
+    std::fprintf(stderr, "%s\n", buf);
+  }
   bool kqv_bias = false;
   bool bindKQVBias(BaseGEMMWrapper* kqv, vortexWeight& bias) {
     if (!kqv_bias) return true;
@@ -162,6 +177,8 @@ public:
   // stream on which update data must be uploaded so that it is ordered before run()
   virtual hipStream_t uploadStream() = 0;
   // level 0: off; 1: attention launches; 2: attention and dense GEMM launches
+  // empty when the last config() built its schedule
+  const std::string& configError() const { return config_error; }
   virtual void setProfiling(int level) { profiling = level > 0; profile_gemms = level > 1; }
   // every stride-th launch of an operator is timed: the override, else 4 on schedules of 8 or
   // more layers (the event records themselves cost device time), else 1

@@ -627,6 +627,11 @@ double LocalPipeline::totalCompute() {
 void LocalPipeline::config(vortexConfigData* config_data_) {
   NF_LOG_INFO("Config local pipeline");
   clearGraphs();  // the buffer plan below may move every operand
+  config_error.clear();
+  for (auto*& g : gemms) {  // a second config() replaces the wrappers of the first
+    delete g;
+    g = nullptr;
+  }
   this->config_data = *config_data_;
   for (int i = 0; i < gemmNum; ++i) {
     const std::string& tag =
@@ -634,8 +639,8 @@ void LocalPipeline::config(vortexConfigData* config_data_) {
     // the LM head stays fp16 in both weight formats
     gemms[i] = generateGEMM(tag, i == static_cast<int>(GEMM_NAME::LOGITS) ? WeightFormat::F16 : weight_format);
     if (!gemms[i]) {
-      std::fprintf(stderr, "LocalPipeline::config: cannot build GEMM %d from tag \"%s\"\n", i, tag.c_str());
-      std::exit(EXIT_FAILURE);
+      configFail("LocalPipeline::config: cannot build GEMM %d from tag \"%s\"", i, tag.c_str());
+      return;
     }
   }
   KQV_ptrs[0] = KQV1;
@@ -644,9 +649,9 @@ void LocalPipeline::config(vortexConfigData* config_data_) {
   const int nano1 = config_data.nanobatch_1_size;
   const int nano2 = globalbatch - nano1;
   if (nano1 <= 0 || nano2 <= 0 || globalbatch > ModelConfig.max_batch_size) {
-    std::fprintf(stderr, "LocalPipeline::config: bad nano-batch split %d + %d (max batch %d)\n", nano1,
+    configFail("LocalPipeline::config: bad nano-batch split %d + %d (max batch %d)", nano1,
                  nano2, ModelConfig.max_batch_size);
-    std::exit(EXIT_FAILURE);
+      return;
   }
   const int kqv_n = (2 * ModelConfig.model_kv_heads_gpu + ModelConfig.model_qo_heads_gpu) *
                     ModelConfig.model_head_dim;

@@ -26,7 +26,8 @@ Pipeline::Pipeline(vortexInitData* input_data, int nrank, int nranks, int vnrank
   stream_gemv = createPipelineStream(0, 0);
   stream_cpy = createPipelineStream(0, 0);
   if (enable_offload) {
-    // room for two requests of 256 pages each (4096 tokens); longer ones move their first pages
+    // room for two requests of 256 pages each (4096 tokens): the iteration's leading requests are
+    // moved as long as their pages fit together; a first request longer than the room moves nothing
     offload_pages_cap = 512;
     const size_t bytes = offload_pages_cap * ModelConfig.page_mem_size;
     HIP_CHECK(hipHostMalloc(&offloadKVCache, bytes, hipHostMallocDefault));
@@ -342,6 +343,7 @@ vortexOutputData Pipeline::run() {
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_START], stream_gemm));
   std::vector<int> sig = baseSignature();
   sig.push_back((int)offload_pages);
+  sig.push_back(offload_reqs);  // baked into the gather / scatter launches
   runIteration(stream_gemm, sig, [this] { enqueueIteration(); });
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_END], stream_gemm));
   HIP_CHECK(hipMemcpyAsync(output_data.sampled_token_array, maxSampler.d_argMax.ptr,
@@ -475,6 +477,11 @@ void Pipeline::update(vortexUpdateData* update_data_) {
 void Pipeline::config(vortexConfigData* config_data_) {
   NF_LOG_INFO("Config pipeline (four QKV / attention nano-batches)");
   clearGraphs();  // the buffer plan below may move every operand
+  config_error.clear();
+  for (auto*& g : gemms) {  // a second config() replaces the wrappers of the first
+    delete g;
+    g = nullptr;
+  }
   this->config_data = *config_data_;
   for (int i = 0; i < gemmNum; ++i) {
     const std::string& tag =
@@ -482,8 +489,8 @@ void Pipeline::config(vortexConfigData* config_data_) {
     // the LM head stays fp16 in both weight formats
     gemms[i] = generateGEMM(tag, i == static_cast<int>(GEMM_NAME::LOGITS) ? WeightFormat::F16 : weight_format);
     if (!gemms[i]) {
-      std::fprintf(stderr, "Pipeline::config: cannot build GEMM %d from tag \"%s\"\n", i, tag.c_str());
-      std::exit(EXIT_FAILURE);
+      configFail("Pipeline::config: cannot build GEMM %d from tag \"%s\"", i, tag.c_str());
+      return;
     }
   }
   KQV_ptrs[0] = KQV1;
@@ -494,9 +501,9 @@ void Pipeline::config(vortexConfigData* config_data_) {
   const int nano1 = config_data.nanobatch_1_size, nano2 = T - nano1;
   const int k1 = config_data.kqv1_size, k3 = config_data.kqv3_size;
   if (nano1 <= 0 || nano2 <= 0 || T > ModelConfig.max_batch_size || k1 < 0 || k1 > nano1 || k3 < 0 || k3 > nano2) {
-    std::fprintf(stderr, "Pipeline::config: bad nano-batch split %d + %d with QKV cuts %d, %d (max batch %d)\n", nano1,
+    configFail("Pipeline::config: bad nano-batch split %d + %d with QKV cuts %d, %d (max batch %d)", nano1,
                  nano2, k1, k3, ModelConfig.max_batch_size);
-    std::exit(EXIT_FAILURE);
+      return;
   }
   const int kqv_n = (2 * ModelConfig.model_kv_heads_gpu + ModelConfig.model_qo_heads_gpu) * ModelConfig.model_head_dim;
   const int H = ModelConfig.model_hidden_dim;

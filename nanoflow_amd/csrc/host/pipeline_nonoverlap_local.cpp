@@ -127,6 +127,11 @@ void NonOverlapLocalPipeline::update(vortexUpdateData* update_data_) {
 void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
   NF_LOG_INFO("Config non-overlap local pipeline");
   clearGraphs();  // the buffer plan below may move every operand
+  config_error.clear();
+  for (auto*& g : gemms) {  // a second config() replaces the wrappers of the first
+    delete g;
+    g = nullptr;
+  }
   this->config_data = *config_data_;
   for (int i = 0; i < gemmNum; ++i) {
     const std::string& tag =
@@ -134,16 +139,16 @@ void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
     // the LM head stays fp16 in both weight formats
     gemms[i] = generateGEMM(tag, i == static_cast<int>(GEMM_NAME::LOGITS) ? WeightFormat::F16 : weight_format);
     if (!gemms[i]) {
-      std::fprintf(stderr, "NonOverlapLocalPipeline::config: cannot build GEMM %d from tag \"%s\"\n", i,
+      configFail("NonOverlapLocalPipeline::config: cannot build GEMM %d from tag \"%s\"", i,
                    tag.c_str());
-      std::exit(EXIT_FAILURE);
+      return;
     }
   }
   const int globalbatch = config_data.global_batch_size;
   if (globalbatch <= 0 || globalbatch > ModelConfig.max_batch_size) {
-    std::fprintf(stderr, "NonOverlapLocalPipeline::config: global batch %d exceeds max batch %d\n",
+    configFail("NonOverlapLocalPipeline::config: global batch %d exceeds max batch %d",
                  globalbatch, ModelConfig.max_batch_size);
-    std::exit(EXIT_FAILURE);
+      return;
   }
   O->set_shape(globalbatch, ModelConfig.model_hidden_dim_pergpu, ModelConfig.model_hidden_dim);
   D->set_shape(globalbatch, ModelConfig.model_hidden_dim, ModelConfig.model_ff_dim_gpu);

@@ -196,17 +196,72 @@ int pllm_model_weight_to_gpu(const nf_vortex_model_weight* host_weight,
   return NF_PLLM_OK;
 }
 
+static bool four_way(int pipeline_type) {
+  const auto t = static_cast<Worker::PipelineType>(pipeline_type);
+  return Worker::isSupported(t) && Worker::isFourWay(t);
+}
+
+int pllm_check_nanobatch_split(int pipeline_type, int max_batch_size, int global_batch_size, int nanobatch_1_size,
+                               int kqv1_size, int kqv3_size) {
+  const auto t = static_cast<Worker::PipelineType>(pipeline_type);
+  if (!Worker::isSupported(t)) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pipeline type %d unknown", pipeline_type);
+  if (global_batch_size <= 0 || global_batch_size > max_batch_size)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: global_batch_size %d not in (0, %d]", global_batch_size,
+                max_batch_size);
+  if (!Worker::isSequential(t) && (nanobatch_1_size <= 0 || nanobatch_1_size >= global_batch_size))
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: nanobatch_1_size %d not in (0, %d)", nanobatch_1_size,
+                global_batch_size);
+  // the four-way schedule cuts each nano-batch once more for the QKV projection and attention
+  if (four_way(pipeline_type)) {
+    if (kqv1_size < 0 || kqv1_size > nanobatch_1_size)
+      return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: kqv1_size %d not in [0, nanobatch_1_size = %d]",
+                  kqv1_size, nanobatch_1_size);
+    if (kqv3_size < 0 || kqv3_size > global_batch_size - nanobatch_1_size)
+      return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: kqv3_size %d not in [0, %d] (nano-batch 2)", kqv3_size,
+                  global_batch_size - nanobatch_1_size);
+  }
+  return NF_PLLM_OK;
+}
+
+int pllm_check_gemv_split(int pipeline_type, int nanobatch_1_size, int kqv1_size, int kqv3_size, int decode_rows,
+                          const int32_t* g) {
+  const auto t = static_cast<Worker::PipelineType>(pipeline_type);
+  if (!Worker::isSupported(t)) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pipeline type %d unknown", pipeline_type);
+  if (!g) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: null gemv_batch_size");
+  if (g[0] < 0 || g[1] < 0 || g[2] < 0 || g[3] < 0)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: negative gemv_batch_size");
+  const int gsum = g[0] + g[1] + g[2] + g[3];
+  if (gsum != decode_rows)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: gemv_batch_size sums to %d, decode requests %d", gsum,
+                decode_rows);
+  if (Worker::isSequential(t)) return NF_PLLM_OK;
+  // decode groups 0 and 1 are the decode rows of nano-batch 1, groups 2 and 3 those of
+  // nano-batch 2 (the O projection of nano-batch 1 waits for groups 0/1 only)
+  const int want = std::min(decode_rows, nanobatch_1_size);
+  if (g[0] + g[1] != want)
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT,
+                "pllm_update: decode groups 0+1 hold %d requests, nano-batch 1 has %d decode rows", g[0] + g[1], want);
+  if (four_way(pipeline_type)) {
+    // decode attention of group i starts once QKV piece i and its RoPE-append are done: the rows of
+    // groups 0..i must lie inside QKV pieces 0..i, or the launch reads Q and KV rows not yet written
+    if (g[0] > kqv1_size)
+      return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: decode group 0 holds %d requests, QKV piece 1 has %d rows",
+                  g[0], kqv1_size);
+    if (g[0] + g[1] + g[2] > nanobatch_1_size + kqv3_size)
+      return fail(NF_PLLM_ERR_INVALID_ARGUMENT,
+                  "pllm_update: decode groups 0..2 hold %d requests, QKV pieces 1..3 have %d rows", g[0] + g[1] + g[2],
+                  nanobatch_1_size + kqv3_size);
+  }
+  return NF_PLLM_OK;
+}
+
 int pllm_config(const nf_vortex_config_data* c) {
   if (!g_inited) return fail(NF_PLLM_ERR_STATE, "pllm_config: call pllm_init first");
   if (g_configured) return fail(NF_PLLM_ERR_STATE, "pllm_config: already configured");
   if (!c) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: null config");
-  const bool local = !Worker::isSequential(Worker::PipeTy);
-  if (c->global_batch_size <= 0 || c->global_batch_size > ModelConfig.max_batch_size)
-    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: global_batch_size %d not in (0, %d]",
-                c->global_batch_size, ModelConfig.max_batch_size);
-  if (local && (c->nanobatch_1_size <= 0 || c->nanobatch_1_size >= c->global_batch_size))
-    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: nanobatch_1_size %d not in (0, %d)",
-                c->nanobatch_1_size, c->global_batch_size);
+  if (int rc = pllm_check_nanobatch_split(static_cast<int>(Worker::PipeTy), ModelConfig.max_batch_size,
+                                          c->global_batch_size, c->nanobatch_1_size, c->kqv1_size, c->kqv3_size))
+    return rc;
   vortexConfigData d;
   for (int i = 0; i < c->num_gemm_op_tag; ++i) {
     GemmTag t;
@@ -229,6 +284,8 @@ int pllm_config(const nf_vortex_config_data* c) {
                 g_init[0].tmp_buffer_size, need);
   g_cfg[0] = d;
   config(g_nranks, g_cfg);
+  if (PipelineBase* p = currentPipeline(); p && !p->configError().empty())
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_config: %s", p->configError().c_str());
   g_configured = true;
   return NF_PLLM_OK;
 }
@@ -253,19 +310,9 @@ int pllm_update(const nf_vortex_update_data* u) {
   if ((size_t)u->kv_indptr[req] > ModelConfig.max_page_num)
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: %d pages in use, pool has %zu",
                 u->kv_indptr[req], ModelConfig.max_page_num);
-  const int gsum = u->gemv_batch_size[0] + u->gemv_batch_size[1] + u->gemv_batch_size[2] + u->gemv_batch_size[3];
-  if (gsum != u->decodePrefillBorder)
-    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: gemv_batch_size sums to %d, decode requests %d",
-                gsum, u->decodePrefillBorder);
-  if (!Worker::isSequential(Worker::PipeTy)) {
-    // decode groups 0 and 1 are the decode rows of nano-batch 1, groups 2 and 3 those of
-    // nano-batch 2 (the O projection of nano-batch 1 waits for groups 0/1 only)
-    const int want = std::min(u->decodePrefillBorder, g_cfg[0].nanobatch_1_size);
-    if (u->gemv_batch_size[0] + u->gemv_batch_size[1] != want)
-      return fail(NF_PLLM_ERR_INVALID_ARGUMENT,
-                  "pllm_update: decode groups 0+1 hold %d requests, nano-batch 1 has %d decode rows",
-                  u->gemv_batch_size[0] + u->gemv_batch_size[1], want);
-  }
+  if (int rc = pllm_check_gemv_split(static_cast<int>(Worker::PipeTy), g_cfg[0].nanobatch_1_size, g_cfg[0].kqv1_size,
+                                     g_cfg[0].kqv3_size, u->decodePrefillBorder, u->gemv_batch_size))
+    return rc;
   vortexUpdateData d;
   d.decodePrefillBorder = u->decodePrefillBorder;
   d.prefillNum = u->prefillNum;

@@ -12,10 +12,7 @@
 //                          or (3) with the operand loads of that tile beside them as well (64 KB
 //                          per workgroup per 64 MFMAs, straight into LDS, from a window the L2
 //                          holds): the GEMM's main loop without barriers, prologue or epilogue;
-//                          or (4) as 1 on v_mfma_f32_16x16x32_f16, or (5) as 3 with the operand
-//                          bytes routed through registers instead of straight into LDS;
-//                          or (10 + n) as 1 with n x 64 idle cycles after every 16 MFMAs: how much
-//                          of an idle matrix pipe the power management gives back as clock;
+//                          or (4) as 1 on v_mfma_f32_16x16x32_f16;
 //                          reports TFLOP/s and the shader clock the wavefronts saw (shader-clock
 //                          ticks over real-time ticks).
 //   nf_calibrate_hbm_read  every CU streams its share of a buffer far larger than the last-level
@@ -83,8 +80,6 @@ __global__ __launch_bounds__(256) void calib_mfma_kernel(int iters, int random_o
         else
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b16[j], a16[i], acc[i][j], 0, 0, 0);
       }
-    // random_operands = 10 + n: n x 64 idle cycles after every 16 MFMAs (512 busy cycles)
-    for (int q = 10; q < random_operands; ++q) asm volatile("s_nop 15" ::: "memory");
   }
   const uint64_t c1 = __builtin_readcyclecounter(), r1 = wall_clock64();
   float s = 0.f;
@@ -160,8 +155,6 @@ __device__ __forceinline__ half8_t lds_read16(uint32_t addr) {
 // kLoads = 1: every wavefront also issues 4 direct-to-LDS loads of 1 KB per 16 MFMAs (the 64 KB a
 // 256x256 tile fetches per 64-deep slab), from a 2 MB window of `src` that 64 workgroups share and
 // the L2 holds, into a second 64 KB of LDS, with at most two steps of loads in flight.
-// kLoads = 2: the same bytes by way of registers (buffer_load_dwordx4, then ds_write_b128 two steps
-// later), the route a kernel without the direct path would take.
 template <int kLoads>
 __global__ __launch_bounds__(256) void calib_mfma_lds_kernel(int iters, uint64_t* clocks, float* sink,
                                                              const uint8_t* __restrict__ src) {
@@ -193,24 +186,9 @@ __global__ __launch_bounds__(256) void calib_mfma_lds_kernel(int iters, uint64_t
   }
   constexpr uint32_t kWindow = 2u << 20;
   const rsrc_t rsrc = make_rsrc(kLoads ? src + (size_t)(blockIdx.x / 8 % 4) * kWindow : nullptr, kLoads ? kWindow : 0);
-  const uint32_t land_v = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem + 65536 + wave * 1024 + lane * 16;
-  rsrc_t st[2][4];  // kLoads = 2: the loads in flight
   const uint32_t land = __builtin_amdgcn_readfirstlane(
       (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem + 65536 + wave * 1024);
   uint32_t goff = (uint32_t)(wave * 1024 + lane * 16);
-#pragma unroll
-  for (int s = 0; s < 2; ++s)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) st[s][q] = rsrc_t{0, 0, 0, 0};
-  if constexpr (kLoads == 2) {  // two steps of loads in flight before the loop
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(st[s][q]) : "v"(goff + (uint32_t)q * 4096u), "s"(rsrc) : "memory");
-      goff = (goff + 16384u) & (kWindow - 1);
-    }
-  }
   const uint64_t c0 = __builtin_readcyclecounter(), r0 = wall_clock64();
   for (int it = 0; it < iters; it += 2) {
 #pragma unroll
@@ -220,17 +198,6 @@ __global__ __launch_bounds__(256) void calib_mfma_lds_kernel(int iters, uint64_t
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           load16_to_lds(rsrc, goff + (uint32_t)q * 4096u, land + (uint32_t)s * 32768u + (uint32_t)q * 4096u);
-        goff = (goff + 16384u) & (kWindow - 1);
-      } else if constexpr (kLoads == 2) {
-        // the four loads of two steps ago have landed in st[s] (the registers are named in the wait so
-        // that nothing reads them before it): store them to LDS, request four more
-        asm volatile("s_waitcnt vmcnt(4)" : "+v"(st[s][0]), "+v"(st[s][1]), "+v"(st[s][2]), "+v"(st[s][3])::"memory");
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          asm volatile("ds_write_b128 %0, %1" ::"v"(land_v + (uint32_t)s * 32768u + (uint32_t)q * 4096u), "v"(st[s][q]) : "memory");
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(st[s][q]) : "v"(goff + (uint32_t)q * 4096u), "s"(rsrc) : "memory");
         goff = (goff + 16384u) & (kWindow - 1);
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // set s, requested one step ago
@@ -257,7 +224,6 @@ __global__ __launch_bounds__(256) void calib_mfma_lds_kernel(int iters, uint64_t
       for (int r = 0; r < 16; ++r) s += acc[i][j][r];
 #pragma unroll
   for (int f = 0; f < 4; ++f) s += (float)a[0][f][0] + (float)b[0][f][0];  // the last reads are consumed too
-  if constexpr (kLoads == 2) s += __builtin_bit_cast(float, st[0][0][0]) * 0.f + __builtin_bit_cast(float, st[1][3][1]) * 0.f;
   sink[gid & 1023u] = s;
   if (threadIdx.x == 0 && blockIdx.x < 64) {
     clocks[blockIdx.x * 2 + 0] = c1 - c0;
@@ -359,19 +325,16 @@ extern "C" {
 int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, size_t scratch_bytes, double* tflops,
                       double* clock_mhz, nf_stream_t stream) {
   NF_REQUIRE(iters > 0 && scratch && scratch_bytes >= 8192 && tflops && clock_mhz, "nf_calibrate_mfma: bad arguments");
-  NF_REQUIRE(random_operands >= 0 && (random_operands <= 5 || (random_operands >= 10 && random_operands <= 74)) &&
-                 !(fp8 && random_operands >= 2 && random_operands <= 5 && random_operands != 4),
-             "nf_calibrate_mfma: random_operands = %d (0, 1, 10 + n = 1 with n x 64 idle cycles per 16 MFMAs, or fp16 "
-             "only: 2 = operands re-read from LDS, 3 = and operand loads from L2 into LDS beside them, 4 = 1 with "
-             "16x16x32 MFMAs, 5 = 3 with the operand loads routed through registers)", random_operands);
-  const bool l2_loads = random_operands == 3 || random_operands == 5;
+  NF_REQUIRE(random_operands >= 0 && random_operands <= 4 && !(fp8 && (random_operands == 2 || random_operands == 3)),
+             "nf_calibrate_mfma: random_operands = %d (0, 1, 4 = 1 with 16x16 MFMAs, or fp16 only: 2 = operands "
+             "re-read from LDS, 3 = and operand loads from L2 into LDS beside them)", random_operands);
+  const bool l2_loads = random_operands == 3;
   NF_REQUIRE(!l2_loads || scratch_bytes >= 8192 + ((size_t)8 << 20),
-             "nf_calibrate_mfma: random_operands = 3 and 5 read 8 MiB of scratch behind its first 8192 bytes");
+             "nf_calibrate_mfma: random_operands = 3 reads 8 MiB of scratch behind its first 8192 bytes");
   if (random_operands == 4) iters = (iters + 1) / 2 * 2;
   if (random_operands == 2 || l2_loads) {
     iters = (iters + 1) / 2 * 2;
-    for (auto k : {reinterpret_cast<const void*>(calib_mfma_lds_kernel<0>), reinterpret_cast<const void*>(calib_mfma_lds_kernel<1>),
-                   reinterpret_cast<const void*>(calib_mfma_lds_kernel<2>)})
+    for (auto k : {reinterpret_cast<const void*>(calib_mfma_lds_kernel<0>), reinterpret_cast<const void*>(calib_mfma_lds_kernel<1>)})
       if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) {
         set_error("nf_calibrate_mfma: cannot reserve 128 KB of LDS");
         return NF_ERR_RUNTIME;
@@ -391,9 +354,6 @@ int nf_calibrate_mfma(int fp8, int random_operands, int iters, void* scratch, si
     if (random_operands == 2) calib_mfma_lds_kernel<0><<<grid, 256, 65536, s>>>((n + 1) / 2 * 2, clocks, sink, nullptr);
     else if (random_operands == 3)
       calib_mfma_lds_kernel<1><<<grid, 256, 131072, s>>>((n + 1) / 2 * 2, clocks, sink,
-                                                         static_cast<const uint8_t*>(scratch) + 8192);
-    else if (random_operands == 5)
-      calib_mfma_lds_kernel<2><<<grid, 256, 131072, s>>>((n + 1) / 2 * 2, clocks, sink,
                                                          static_cast<const uint8_t*>(scratch) + 8192);
     else if (random_operands == 4 && fp8) calib_mfma16_kernel<true><<<grid, 256, 0, s>>>((n + 1) / 2 * 2, clocks, sink);
     else if (random_operands == 4) calib_mfma16_kernel<false><<<grid, 256, 0, s>>>((n + 1) / 2 * 2, clocks, sink);

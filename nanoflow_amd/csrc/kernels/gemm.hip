@@ -41,10 +41,6 @@
 
 #include "common.h"
 
-#ifndef NF_GEMM_MFMA16
-#define NF_GEMM_MFMA16 1
-#endif
-
 namespace nf {
 
 constexpr int BK = 64;  // K slab (halves); an A-style LDS row is 128 bytes
@@ -134,7 +130,7 @@ __device__ __forceinline__ void gemm_tile(
   // the 256 architectural registers and the compiler has no reason to shuffle accumulators
   // between the two register files.
   // Eight-wavefront tiles keep 32x32x16 (256 registers per wavefront in all).
-  constexpr bool kM16 = NW == 4 && NF_GEMM_MFMA16;
+  constexpr bool kM16 = NW == 4;
   constexpr int MT = kM16 ? 16 : 32;  // rows and columns of an MFMA tile
   constexpr int TM = BM / WM / MT;    // MFMA tiles per wave along M
   constexpr int TN = BN / WN / MT;

@@ -181,7 +181,6 @@ def corun(a, shape, rnd):
         phase("mfma loop f16, zero operands", lambda: K.calibrate_mfma(False, False, 2000), secs=2.0)
         phase("mfma loop f16, pseudo-random operands re-read from LDS", lambda: K.calibrate_mfma(False, 2, 2000), secs=2.0)
         phase("   ... with the tile's operand loads (L2 -> LDS) beside them", lambda: K.calibrate_mfma(False, 3, 2000), secs=2.0)
-        phase("   ... with those loads routed through registers instead", lambda: K.calibrate_mfma(False, 5, 2000), secs=2.0)
         phase("mfma loop f16 on 16x16x32 instructions, pseudo-random operands", lambda: K.calibrate_mfma(False, 4, 2000), secs=2.0)
         buf = torch.empty(4 << 30, dtype=torch.uint8, device=DEV).random_()
         sc = torch.zeros(8192, dtype=torch.uint8, device=DEV)
@@ -313,16 +312,9 @@ def main():
                 tf, mhz = K.calibrate_mfma(False, 3, 40000)
                 print(f"   ... with 64 KB of operand loads per workgroup per 64 MFMAs (L2 -> LDS) beside them: "
                       f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
-                tf, mhz = K.calibrate_mfma(False, 5, 40000)
-                print(f"   ... with the same operand bytes routed through registers (buffer_load, ds_write_b128) instead: "
-                      f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
                 tf, mhz = K.calibrate_mfma(False, 4, 40000)
                 print(f"mfma loop f16 16x16x32 pseudo-random operands (64 accumulators: the same register tile): "
                       f"{tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
-                for n in (1, 2, 3, 4, 6, 8):
-                    tf, mhz = K.calibrate_mfma(False, 10 + n, 40000)
-                    print(f"mfma loop f16 32x32x16 pseudo-random operands, {64 * n:4d} idle cycles after every 16 MFMAs "
-                          f"(512 cycles): {tf:8.1f} TFLOP/s at {mhz:6.0f} MHz shader clock", flush=True)
         print(f"hbm read stream, 8 GiB x 4: {K.calibrate_hbm_read(8.0, 4):8.1f} GB/s", flush=True)
         b = synth.config2_batch(seed=0, n_decode=a.requests, lo=a.kv_lo, hi=a.kv_hi, prefill_chunk=16)
         nd = b.decodePrefillBorder

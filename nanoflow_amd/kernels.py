@@ -425,10 +425,8 @@ def calibrate_mfma(fp8: bool = False, random_operands=True, iters: int = 20000):
     """(TFLOP/s, shader clock in MHz) of an MFMA loop on this device.  random_operands: False = zero
     operands in registers, True = pseudo-random ones, 2 = pseudo-random ones re-read from LDS before
     every 16 MFMAs (fp16 only), as a GEMM's main loop reads its fragments, 3 = with the operand loads
-    of a 256x256 tile (L2 -> LDS) beside them as well, 4 = as True with 16x16x32 MFMAs, 5 = as 3 with
-    the operand bytes routed through registers, 10 + n = as True with n x 64 idle cycles after every
-    16 MFMAs."""
-    scratch = torch.zeros(8192 + ((8 << 20) if int(random_operands) in (3, 5) else 0), dtype=torch.uint8, device="cuda")
+    of a 256x256 tile (L2 -> LDS) beside them as well, 4 = as True with 16x16 MFMAs."""
+    scratch = torch.zeros(8192 + ((8 << 20) if int(random_operands) == 3 else 0), dtype=torch.uint8, device="cuda")
     tf, mhz = C.c_double(), C.c_double()
     _check(lib().nf_calibrate_mfma(int(fp8), int(random_operands), iters, scratch.data_ptr(), scratch.numel(),
                                    C.byref(tf), C.byref(mhz), _stream()), "nf_calibrate_mfma")

@@ -102,3 +102,36 @@ def test_extension_module_imports_without_a_gpu_and_has_the_reference_names():
     assert c.gemmOpTag == ["a", "b"]
     with pytest.raises(RuntimeError):
         mod.setRank(2, 2)              # one rank only
+
+
+def test_nanobatch_split_and_attention_groups_are_checked_on_the_host():
+    """What pllm_config / pllm_update reject before anything is built or written, through the two
+    stateless checkers they call: a QKV cut outside its nano-batch, and decode-attention groups that
+    reach past the QKV pieces finished when the group's launch starts (four-way schedule)."""
+    lib = ctypes.CDLL(os.path.join(ROOT, "nanoflow_amd", "libnf_pipeline.so"))
+    lib.pllm_last_error.restype = ctypes.c_char_p
+    PLLM, NONOVERLAP, NANOBATCH, OFFLOAD, LOCAL, SEQ = 0, 1, 2, 3, 7, 8
+    cfg = lib.pllm_check_nanobatch_split
+    assert cfg(PLLM, 2048, 2048, 640, 256, 768) == 0
+    assert cfg(PLLM, 2048, 2048, 640, 0, 1408) == 0              # cuts on the borders are allowed
+    for bad in ((PLLM, 2048, 2048, 640, 641, 768), (NANOBATCH, 2048, 2048, 640, 256, 1409),
+                (OFFLOAD, 2048, 2048, 640, -1, 10), (PLLM, 2048, 2048, 2048, 1, 1), (PLLM, 1024, 2048, 640, 1, 1),
+                (LOCAL, 2048, 2048, 0, 0, 0), (42, 2048, 2048, 640, 1, 1)):
+        assert cfg(*bad) == -1, bad
+    assert b"kqv3_size" in (cfg(NANOBATCH, 2048, 2048, 640, 256, 1409), lib.pllm_last_error())[1]
+    assert cfg(LOCAL, 2048, 2048, 640, 9999, -5) == 0            # two-way schedules never read the QKV cuts
+    assert cfg(SEQ, 2048, 2048, 0, 0, 0) == 0 and cfg(NONOVERLAP, 2048, 2048, 0, 0, 0) == 0
+    grp = lib.pllm_check_gemv_split
+    g = lambda *v: (ctypes.c_int32 * 4)(*v)
+    # 1000 decode rows on 640 | 1408 with QKV pieces 256 | 384 | 768 | 640
+    assert grp(PLLM, 640, 256, 768, 1000, g(256, 384, 360, 0)) == 0
+    assert grp(PLLM, 640, 256, 768, 1000, g(200, 440, 360, 0)) == 0      # group 1 inside pieces 1..2
+    assert grp(PLLM, 640, 256, 768, 1000, g(300, 340, 360, 0)) == -1     # group 0 past QKV piece 1
+    assert b"group 0" in lib.pllm_last_error()
+    assert grp(PLLM, 640, 256, 768, 1800, g(256, 384, 800, 360)) == -1   # groups 0..2 past piece 3
+    assert grp(PLLM, 640, 256, 768, 1800, g(256, 384, 768, 392)) == 0
+    assert grp(PLLM, 640, 256, 768, 1000, g(256, 300, 444, 0)) == -1     # groups 0+1 != decode rows of nano-batch 1
+    assert grp(PLLM, 640, 256, 768, 1000, g(256, 384, 300, 0)) == -1     # does not sum to the decode rows
+    assert grp(LOCAL, 640, 256, 768, 1000, g(300, 340, 360, 0)) == 0     # two-way: only the 0+1 rule
+    assert grp(SEQ, 0, 0, 0, 1000, g(1000, 0, 0, 0)) == 0
+    assert grp(PLLM, 640, 256, 768, 1000, None) == -1

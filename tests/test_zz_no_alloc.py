@@ -53,7 +53,7 @@ def test_gemm_noalloc_matches_the_workspace_entry_point_on_two_calls_in_a_row(or
 def test_gemm_noalloc_rejects_what_the_static_array_cannot_hold():
     from nanoflow_amd import kernels as K
     l = K.lib()
-    # 512 rows x 8192 columns split 8 ways over K = 28672: 64 MiB of partial sums
+    # 512 rows x 8192 columns split 4 ways over K = 28672: four shares of 16 MiB of partial sums
     M, N, K_ = 512, 8192, 28672
     assert l.nf_gemm_workspace_bytes(M, N, K_) > l.nf_gemm_noalloc_scratch_bytes()
     A = torch.zeros((M, K_), dtype=torch.float16, device="cuda")
