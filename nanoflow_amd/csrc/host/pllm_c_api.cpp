@@ -474,6 +474,18 @@ int pllm_debug_buffer(const char* name, uint16_t** ptr, int* rows, int* cols) {
   } else if (auto* pp = dynamic_cast<Pipeline*>(p)) {
     if (!std::strcmp(name, "hidden")) t = pp->keepToken.input;
     else if (!std::strcmp(name, "logits")) t = pp->maxSampler.d_matrix;
+    // whole-iteration buffers (the nano-batch pieces are consecutive rows of them); they hold the
+    // LAST layer's values once an iteration has run
+    else if (!std::strcmp(name, "kqv")) t = pp->KQV_output;
+    else if (!std::strcmp(name, "attn_out")) t = pp->gemvAggregateOutput;
+    else if (!std::strcmp(name, "ln_attn") || !std::strcmp(name, "o_out") || !std::strcmp(name, "ln_ffn") ||
+             !std::strcmp(name, "act")) {
+      const pllmTensor<half> first = !std::strcmp(name, "ln_attn") ? pp->layerNormAttention1.getOutput()
+                                     : !std::strcmp(name, "o_out") ? pp->O1->getD()
+                                     : !std::strcmp(name, "ln_ffn") ? pp->dual1.getA()
+                                                                    : pp->D1->getA();
+      t = pllmTensor<half>(first.ptr, pp->KQV_output.dim1, first.dim2, PllmLayout::ROW_MAJOR);
+    }
     else if (!std::strcmp(name, "offload_host") && pp->offloadKVCache)  // pinned host memory: what the last layer's round trip left
       t = pllmTensor<half>(pp->offloadKVCache, pp->offload_pages, ModelConfig.page_mem_size / sizeof(half), PllmLayout::ROW_MAJOR);
   } else if (auto* np = dynamic_cast<NonOverlapLocalPipeline*>(p)) {
