@@ -242,7 +242,7 @@ def run_iteration(args):
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, run_layer=shape.layers,
                         distinct_layers=distinct, seed=args.seed, profiling=0,
-                        weight_format=args.weights)
+                        weight_format=args.weights, weight_layout=args.weight_layout)
     P.setGraphMode(args.graph)
     eng.update(batch)
     torch.cuda.synchronize()
@@ -298,6 +298,9 @@ def run_iteration(args):
                          + f"iteration: {n_dec} decode tokens (KV U[1024,1536], page 16, permuted page table)"
                          + (f" + one {n_pre}-token prefill chunk" if n_pre else "")),
             "weights": args.weights,
+            "weight_layout": ("[N][K] (k contiguous; GEMM tags say ColumnMajor for B)" if eng.weight_layout == "col" else
+                              "[K][N] (the reference's weight-file orientation; tags say RowMajor)") if wb == 2 else
+                             "e4m3 [N][K] + per-output-channel scales; LM head fp16 " + ("[V][H]" if eng.lm_head_layout == "col" else "[H][V]"),
             "pipeline": args.pipeline, "global_batch": T, "nanobatch_1_size": args.nano1,
             "kqv1_size": args.kqv1, "kqv3_size": args.kqv3, "layers_executed": shape.layers,
             "distinct_layers_in_hbm": distinct, "kv_pages_per_layer": int(pages),
@@ -382,7 +385,8 @@ def run_offline(args):
     # rows read must not be a run of zeros.
     eng = engine.Engine(shape, P.PipelineType[args.pipeline], global_batch=T, nano1=args.nano1,
                         kqv1=args.kqv1, kqv3=args.kqv3, kv_pages=pages, seed=args.seed,
-                        profiling=0, kv_fill=args.kv_fill, weight_format=args.weights)
+                        profiling=0, kv_fill=args.kv_fill, weight_format=args.weights,
+                        weight_layout=args.weight_layout)
     former = P.BatchFormer(pages, shape.page_size, T, args.nano1, args.kqv1, args.kqv3, in_len, out_len)
     rng = np.random.default_rng(args.seed)
     for i in range(n_req):
@@ -457,6 +461,9 @@ def run_offline(args):
         "dtype": "f16" if wb == 2 else "f8e4m3 weights and GEMM inputs, f16 activations and KV", "data": "synthetic",
         "config": {
             "weights": args.weights,
+            "weight_layout": ("[N][K] (k contiguous; GEMM tags say ColumnMajor for B)" if eng.weight_layout == "col" else
+                              "[K][N] (the reference's weight-file orientation; tags say RowMajor)") if wb == 2 else
+                             "e4m3 [N][K] + per-output-channel scales; LM head fp16 " + ("[V][H]" if eng.lm_head_layout == "col" else "[H][V]"),
             "workload": (f"{shape_name} shape, offline throughput: {n_req} requests, constant {in_len}-token "
                          f"prompts (ids uniform over the vocab) / {out_len} output tokens, greedy, EOS "
                          f"ignored, <= {T} tokens per iteration with chunked prefill; "
@@ -533,6 +540,9 @@ def main():
                          "(80 layers, hidden 8192, 64 Q / 8 KV heads, FFN 28672) resident on the one GPU")
     ap.add_argument("--weights", default="f16", choices=["f16", "e4m3"],
                     help="e4m3: the five per-layer GEMM weights in fp8 with per-output-channel scales")
+    ap.add_argument("--weight-layout", default="col", choices=["col", "row"],
+                    help="col: fp16 weights handed over [N][K], k contiguous (every GEMM tag says ColumnMajor for B; a\n"
+                         "Hugging Face checkpoint's own orientation); row: [K][N] as the reference's weight files hold them")
     ap.add_argument("--pipeline", default="auto", choices=["auto", "LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_LOCAL", "PLLM", "NANOBATCH", "PLLMOFFLOAD"],
                     help="auto = the fastest schedule measured on MI355X for both workloads: NON_OVERLAP_LOCAL\n"
                          "(one stream); LOCAL measures the two-stream overlapped schedule, PLLM the reference's main\n"

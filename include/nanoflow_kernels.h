@@ -110,7 +110,8 @@ NF_API size_t nf_gemm_noalloc_scratch_bytes(void);
 NF_API size_t nf_dual_swiglu_workspace_bytes(int M, int N, int K);
 NF_API size_t nf_dual_swiglu_workspace_bytes_upto(int max_M, int N, int K);
 NF_API int nf_dual_swiglu_f16_ws(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
-                                 int M, int N, int K, void* workspace, size_t workspace_bytes, nf_stream_t stream);
+                                 int M, int N, int K, int b_col_major, void* workspace, size_t workspace_bytes,
+                                 nf_stream_t stream);
 /* the same for nf_gemm_bias_f16 (declared below) */
 NF_API int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M, int N,
                                int K, float alpha, float beta, int b_col_major, void* workspace,
@@ -124,12 +125,14 @@ NF_API int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint1
 NF_API int nf_gemm_bias_f16(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M,
                      int N, int K, float alpha, float beta, int b_col_major, nf_stream_t stream);
 
-/* out = half(silu(float(half(A.Bgate))) * float(half(A.Bup))); A [M,K], Bgate/Bup [K,N],
- * out [M,N], all row-major.  K % 8 == 0, N % 8 == 0.
+/* out = half(silu(float(half(A.Bgate))) * float(half(A.Bup))); A [M,K] and out [M,N] row-major;
+ * Bgate/Bup [K,N] row-major (b_col_major = 0, the orientation the reference's weight files use)
+ * or [N,K], k contiguous (b_col_major = 1: the layout a GEMM tag calls ColumnMajor for B,
+ * pipeline/src/generate-gemm/genGEMM.py:44-49).  K % 8 == 0, N % 8 == 0.
  * Replaces DualWrapper::work / cutlass DualGemm + LeftSiLUAndMul
  * (pipeline/include/dualWrapper.cuh:95-144,192-194). */
 NF_API int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
-                       int M, int N, int K, nf_stream_t stream);
+                       int M, int N, int K, int b_col_major, nf_stream_t stream);
 
 /* The same two operators on bfloat16 storage (bf16 x bf16 -> fp32 -> bf16, products rounded to bf16
  * before SiLU-mul): same kernels, other element type.  The reference's wrappers are fp16 only

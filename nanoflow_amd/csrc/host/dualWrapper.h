@@ -30,6 +30,12 @@ struct DualWrapper : public OperatorWrapper {
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
   void setWeightFormat(WeightFormat f) { e4m3 = f == WeightFormat::E4M3; }
+  // fp16 weights: ROW_MAJOR = [K][N] as the reference's weight files hold them, COL_MAJOR = [N][K],
+  // k contiguous (what a GEMM tag calls ColumnMajor for B).  The reference's DualWrapper takes its
+  // layouts as template arguments (dualWrapper.cuh:47-60) and the pipeline JSON has no tag for it:
+  // the pipelines give the pair the layout that ALL per-layer GEMM tags agree on, RowMajor otherwise.
+  PllmLayout weight_layout = PllmLayout::ROW_MAJOR;
+  void setWeightLayout(PllmLayout l) { weight_layout = l; }
   // fp16 weights: scratch for launches of few rows that are split over K (nf_dual_swiglu_f16_ws)
   size_t workspaceBytes() const {
     return e4m3 ? nf_dual_swiglu_f8w_split_workspace_bytes_upto(M, N, K) : nf_dual_swiglu_workspace_bytes_upto(M, N, K);
@@ -61,8 +67,9 @@ struct DualWrapper : public OperatorWrapper {
                                              workspace, workspace_bytes, stream));
       return;
     }
-    NF_KERNEL_CHECK(nf_dual_swiglu_f16_ws(pllm_tensor_a.ptr, pllm_tensor_b1.ptr, pllm_tensor_b2.ptr,
-                                          pllm_tensor_d2.ptr, rows(), N, K, workspace, workspace_bytes, stream));
+    NF_KERNEL_CHECK(nf_dual_swiglu_f16_ws(pllm_tensor_a.ptr, pllm_tensor_b1.ptr, pllm_tensor_b2.ptr, pllm_tensor_d2.ptr,
+                                          rows(), N, K, weight_layout == PllmLayout::COL_MAJOR ? 1 : 0, workspace,
+                                          workspace_bytes, stream));
   }
   DualWrapper& setA(pllmTensor<half> a) {
     assert(a.layout == PllmLayout::ROW_MAJOR && (int)a.dim1 == M && (int)a.dim2 == K);
@@ -90,8 +97,13 @@ struct DualWrapper : public OperatorWrapper {
                    weight2.size(), K, N);
       return false;
     }
-    pllm_tensor_b1 = pllmTensor<half>(weight1.ptr, K, N, PllmLayout::ROW_MAJOR);
-    pllm_tensor_b2 = pllmTensor<half>(weight2.ptr, K, N, PllmLayout::ROW_MAJOR);
+    if (weight_layout == PllmLayout::COL_MAJOR && !e4m3) {
+      pllm_tensor_b1 = pllmTensor<half>(weight1.ptr, N, K, PllmLayout::COL_MAJOR);
+      pllm_tensor_b2 = pllmTensor<half>(weight2.ptr, N, K, PllmLayout::COL_MAJOR);
+    } else {
+      pllm_tensor_b1 = pllmTensor<half>(weight1.ptr, K, N, PllmLayout::ROW_MAJOR);
+      pllm_tensor_b2 = pllmTensor<half>(weight2.ptr, K, N, PllmLayout::ROW_MAJOR);
+    }
     return true;
   }
   double totalCompute() { return 4.0 * (double)rows() * (double)N * (double)K; }

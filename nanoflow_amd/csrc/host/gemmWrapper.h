@@ -77,6 +77,9 @@ struct BaseGEMMWrapper : public OperatorWrapper {
     (void)ptr;
     (void)bytes;
   }
+  // The layout of B the wrapper was built for (the tag's second layout field): ROW_MAJOR = [K][N],
+  // COL_MAJOR = [N][K].  Not in the reference's interface (there it is a template argument).
+  virtual PllmLayout weightLayout() const { return PllmLayout::ROW_MAJOR; }
 };
 
 struct GemmTag {
@@ -104,6 +107,7 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   bool c_is_row = false;  // pllm_tensor_c is a [1, N] row added to every row
 
   explicit HipGEMMWrapper(const GemmTag& t) : tag(t) {}
+  PllmLayout weightLayout() const override { return tag.layout_b; }
 
   void work() override;
 

@@ -95,6 +95,15 @@ protected:
     return true;
   }
 
+  // The weight layout the gate/up pair is given (it has no tag of its own): [N][K] when every
+  // per-layer GEMM tag says ColumnMajor for B, the reference's [K][N] otherwise.
+  template <class Gemms>
+  static PllmLayout pairWeightLayout(const Gemms& gemms, int logits_index) {
+    for (int i = 0; i < (int)gemms.size(); ++i)
+      if (i != logits_index && gemms[i]->weightLayout() != PllmLayout::COL_MAJOR) return PllmLayout::ROW_MAJOR;
+    return PllmLayout::COL_MAJOR;
+  }
+
   // e4m3 weights: the RMSNorm in front of the QKV and of the gate/up projection writes its rows
   // as e4m3 bytes + one fp32 scale per row as well, into a [rows, hidden] image carved from the tmp
   // buffer, and the GEMMs read their rows there instead of launching a quantiser of their own.

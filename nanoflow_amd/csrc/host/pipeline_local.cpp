@@ -665,7 +665,9 @@ void LocalPipeline::config(vortexConfigData* config_data_) {
   dual1.set_shape(nano1, ModelConfig.model_ff_dim_gpu, ModelConfig.model_hidden_dim);
   dual2.set_shape(nano2, ModelConfig.model_ff_dim_gpu, ModelConfig.model_hidden_dim);
   dual1.setWeightFormat(weight_format);
+  dual1.setWeightLayout(pairWeightLayout(gemms, static_cast<int>(GEMM_NAME::LOGITS)));
   dual2.setWeightFormat(weight_format);
+  dual2.setWeightLayout(pairWeightLayout(gemms, static_cast<int>(GEMM_NAME::LOGITS)));
 
   setName();
   ScheduleInit();

@@ -519,7 +519,9 @@ void Pipeline::config(vortexConfigData* config_data_) {
   dual1.set_shape(nano1, ModelConfig.model_ff_dim_gpu, H);
   dual2.set_shape(nano2, ModelConfig.model_ff_dim_gpu, H);
   dual1.setWeightFormat(weight_format);
+  dual1.setWeightLayout(pairWeightLayout(gemms, static_cast<int>(GEMM_NAME::LOGITS)));
   dual2.setWeightFormat(weight_format);
+  dual2.setWeightLayout(pairWeightLayout(gemms, static_cast<int>(GEMM_NAME::LOGITS)));
 
   setName();
   ScheduleInit();

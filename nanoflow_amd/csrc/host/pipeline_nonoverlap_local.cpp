@@ -159,6 +159,7 @@ void NonOverlapLocalPipeline::config(vortexConfigData* config_data_) {
   LOGITS->set_shape(globalbatch, (int)ModelConfig.vocab_size, ModelConfig.model_hidden_dim);
   dual.set_shape(globalbatch, ModelConfig.model_ff_dim_gpu, ModelConfig.model_hidden_dim);
   dual.setWeightFormat(weight_format);
+  dual.setWeightLayout(pairWeightLayout(gemms, static_cast<int>(GEMM_NAME::LOGITS)));
   ScheduleInit();
   GEMMOpInit();
   GEMVOpInit();

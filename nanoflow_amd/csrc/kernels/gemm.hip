@@ -997,7 +997,7 @@ static int gemm_ws_entry(const char* who, const uint16_t* A, const uint16_t* B, 
                      : launch_splitk<E, 128, 128, 2, 2, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
 }
 
-template <class E>
+template <class E, bool kBCol>
 static int dual_entry(const char* who, const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup,
                       uint16_t* out, int M, int N, int K, nf_stream_t stream) {
   int rc = check_gemm_args(who, A, Bgate, out, M, N, K);
@@ -1007,42 +1007,42 @@ static int dual_entry(const char* who, const uint16_t* A, const uint16_t* Bgate,
   if (M == 0) return NF_OK;
   hipStream_t s = (hipStream_t)stream;
   if (M <= 64)
-    return launch_gemm<E, 64, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
+    return launch_gemm<E, 64, 128, 2, 2, true, kBCol>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
   // 257 .. 320 rows against enough column panels to fill the chip: one 320-row tile per panel, so
   // the weights pass through LDS once instead of three times; its two 320 x 128 accumulators are
   // spread over eight wavefronts (160 registers each)
   if (M > 256 && M <= kTallRows && (N + 127) / 128 >= 192)
-    return launch_gemm<E, 320, 128, 2, 4, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
+    return launch_gemm<E, 320, 128, 2, 4, true, kBCol>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
   const long long t256 = (long long)((M + 255) / 256) * ((N + 127) / 128);
   const int tail = M % 256;  // rows in the last 256-row tile: half-empty tiles go to the 128-row kernel
   if (t256 >= 192 && (tail == 0 || tail > 128)) {
     const int cus = cu_count();
     const int rest = (int)(t256 % cus);  // tiles of the last, partial round
     if (t256 > cus && rest > 0 && rest <= cus / 2)
-      return launch_hybrid<E, 128, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, (int)(t256 - rest), s);
-    return launch_gemm<E, 256, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
+      return launch_hybrid<E, 128, true, kBCol>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, (int)(t256 - rest), s);
+    return launch_gemm<E, 256, 128, 2, 2, true, kBCol>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
   }
-  return launch_gemm<E, 128, 128, 2, 2, true, false>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
+  return launch_gemm<E, 128, 128, 2, 2, true, kBCol>(A, Bgate, Bup, nullptr, out, M, N, K, 1.f, 0.f, N, s);
 }
 
-template <class E>
+template <class E, bool kBCol>
 static int dual_ws_entry(const char* who, const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup,
                          uint16_t* out, int M, int N, int K, void* workspace, size_t workspace_bytes,
                          nf_stream_t stream) {
   int k_per = 0;
   const int shares = M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0 ? splitk_plan_dual(M, N, K, &k_per) : 1;
   if (shares < 2 || !workspace || workspace_bytes < (size_t)2 * shares * M * N * sizeof(float))
-    return dual_entry<E>(who, A, Bgate, Bup, out, M, N, K, stream);
+    return dual_entry<E, kBCol>(who, A, Bgate, Bup, out, M, N, K, stream);
   int rc = check_gemm_args(who, A, Bgate, out, M, N, K);
   if (rc) return rc;
   NF_REQUIRE(Bup && ((uintptr_t)Bup | (uintptr_t)workspace) % 16 == 0, "%s: Bup and the workspace must be 16-byte aligned", who);
   hipStream_t s = (hipStream_t)stream;
   float* P = static_cast<float*>(workspace);
   if (M <= 64)
-    return launch_splitk<E, 64, 128, 2, 2, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
+    return launch_splitk<E, 64, 128, 2, 2, kBCol, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
   if (M > 256)
-    return launch_splitk<E, 320, 128, 2, 4, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
-  return launch_splitk<E, 128, 128, 2, 2, false, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
+    return launch_splitk<E, 320, 128, 2, 4, kBCol, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
+  return launch_splitk<E, 128, 128, 2, 2, kBCol, true>(A, Bgate, nullptr, out, M, N, K, 1.f, 0.f, N, shares, k_per, P, s, Bup);
 }
 
 // ---- the entry point that allocates nothing: split-K partial sums in a static device array.
@@ -1106,8 +1106,11 @@ size_t nf_dual_swiglu_workspace_bytes_upto(int max_M, int N, int K) {
 }
 
 int nf_dual_swiglu_f16_ws(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out, int M,
-                          int N, int K, void* workspace, size_t workspace_bytes, nf_stream_t stream) {
-  return dual_ws_entry<F16>("nf_dual_swiglu_f16_ws", A, Bgate, Bup, out, M, N, K, workspace, workspace_bytes, stream);
+                          int N, int K, int b_col_major, void* workspace, size_t workspace_bytes, nf_stream_t stream) {
+  return b_col_major ? dual_ws_entry<F16, true>("nf_dual_swiglu_f16_ws", A, Bgate, Bup, out, M, N, K, workspace,
+                                                workspace_bytes, stream)
+                     : dual_ws_entry<F16, false>("nf_dual_swiglu_f16_ws", A, Bgate, Bup, out, M, N, K, workspace,
+                                                 workspace_bytes, stream);
 }
 
 int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
@@ -1150,8 +1153,9 @@ int nf_gemm_bias_f16(const uint16_t* A, const uint16_t* B, const uint16_t* bias,
 }
 
 int nf_dual_swiglu_f16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
-                       int M, int N, int K, nf_stream_t stream) {
-  return dual_entry<F16>("nf_dual_swiglu_f16", A, Bgate, Bup, out, M, N, K, stream);
+                       int M, int N, int K, int b_col_major, nf_stream_t stream) {
+  return b_col_major ? dual_entry<F16, true>("nf_dual_swiglu_f16", A, Bgate, Bup, out, M, N, K, stream)
+                     : dual_entry<F16, false>("nf_dual_swiglu_f16", A, Bgate, Bup, out, M, N, K, stream);
 }
 
 int nf_gemm_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
@@ -1161,7 +1165,7 @@ int nf_gemm_bf16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16
 
 int nf_dual_swiglu_bf16(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
                         int M, int N, int K, nf_stream_t stream) {
-  return dual_entry<BF16>("nf_dual_swiglu_bf16", A, Bgate, Bup, out, M, N, K, stream);
+  return dual_entry<BF16, false>("nf_dual_swiglu_bf16", A, Bgate, Bup, out, M, N, K, stream);
 }
 
 }  // extern "C"

@@ -17,12 +17,34 @@ import torch
 from . import pllm_python as P
 from . import synth
 
-# Tags are accepted for interface parity; tiling is chosen by the kernel layer.
+# The tag grammar of the reference's pipeline files (pipeline/include/gemmShape.cuh:5-6).  The second
+# layout field is B's: RowMajor = [K][N] weights as the reference's weight files hold them,
+# ColumnMajor = [N][K] (k contiguous, a Hugging Face checkpoint's own orientation).
 DEFAULT_TAG = "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor"
+DEFAULT_TAG_NK = "128_128_32_64_64_32_1_5_RowMajor_ColumnMajor_RowMajor"
+
+
+def tag_weight_layout(tag: str) -> str:
+    """"row" ([K][N]) or "col" ([N][K]): the layout a GEMM tag gives its weight."""
+    parts = tag.split("_")
+    if len(parts) != 11 or parts[9] not in ("RowMajor", "ColumnMajor"):
+        raise ValueError(f"malformed GEMM tag {tag!r}")
+    return "col" if parts[9] == "ColumnMajor" else "row"
+
+
+def layouts_of_tags(tags):
+    """(layout of the per-layer GEMM weights, layout of the LM head) of a pipeline file's tag list
+    (the LM head's tag is the last one in every schedule).  The per-layer tags must agree: one weight
+    serves every nano-batch's GEMM of its role, and the gate/up pair, which has no tag, follows them."""
+    per_layer = {tag_weight_layout(t) for t in tags[:-1]}
+    if len(per_layer) != 1:
+        raise ValueError("the per-layer GEMM tags disagree on B's layout (RowMajor / ColumnMajor): "
+                         "a weight is stored in one orientation")
+    return per_layer.pop(), tag_weight_layout(tags[-1])
 
 
 def write_config(path, shape: synth.ModelShape, *, global_batch, nano1, kqv1, kqv3, pipeline_type,
-                 kv_pages, run_layer=None, distinct_layers=None, max_batch=None, n_tags=7):
+                 kv_pages, run_layer=None, distinct_layers=None, max_batch=None, n_tags=7, tags=None):
     """Writes a pipeline JSON in the reference's schema (pipeline/config_all/llama3-8B/1024.json)."""
     layers = shape.layers if distinct_layers is None else distinct_layers
     cfg = {
@@ -38,7 +60,7 @@ def write_config(path, shape: synth.ModelShape, *, global_batch, nano1, kqv1, kq
             "max_batch_size": global_batch if max_batch is None else max_batch,
         },
         "pipeline_configs": {
-            "gemm_op_tag": [DEFAULT_TAG] * n_tags, "global_batch_size": global_batch,
+            "gemm_op_tag": list(tags) if tags else [DEFAULT_TAG] * n_tags, "global_batch_size": global_batch,
             "nanobatch_1_size": nano1, "kqv1_size": kqv1, "kqv3_size": kqv3,
         },
         "serve_configs": {"actual_gpu_num": 1, "pipeline_type": {v: k for k, v in P.pipeline_map.items()}[pipeline_type]},
@@ -62,7 +84,14 @@ class Engine:
 
     def __init__(self, shape: synth.ModelShape, pipeline_type=P.PipelineType.LOCAL, *, global_batch,
                  nano1, kqv1=None, kqv3=None, kv_pages, weights=None, kv_pools=None, run_layer=None,
-                 distinct_layers=None, seed=0, profiling=False, kv_fill="randn", weight_format="f16"):
+                 distinct_layers=None, seed=0, profiling=False, kv_fill="randn", weight_format="f16",
+                 weight_layout="row", gemm_tags=None):
+        """weight_layout: "row" = [K][N] weights (the reference's orientation), "col" = [N][K]
+        (k contiguous): the five per-layer GEMM weights and the LM head are handed over in that
+        orientation and every GEMM tag says so.  With e4m3 weights only the LM head follows it (the
+        fp8 form has one layout).  gemm_tags: the tag list of a pipeline file instead; its layout
+        fields then decide (layouts_of_tags).  ``weights`` is always given in the [K][N] orientation
+        and turned around on the device when the layout asks for it."""
         self.shape = shape
         self.pipeline_type = pipeline_type
         # "e4m3": the five GEMM weights of every layer are quantised on the device as they are
@@ -78,9 +107,23 @@ class Engine:
         fd, self.cfg_path = tempfile.mkstemp(suffix=".json", prefix="nanoflow_cfg_")
         os.close(fd)
         n_tags = pipeline_type.gemm_tags
+        e4m3 = self.weight_format == P.WeightFormat.E4M3
+        if gemm_tags is not None:
+            if len(gemm_tags) != n_tags:
+                raise ValueError(f"{pipeline_type.name} takes {n_tags} GEMM tags, the list has {len(gemm_tags)}")
+            self.tags = list(gemm_tags)
+            layer_layout, head_layout = layouts_of_tags(self.tags)
+            if e4m3 and layer_layout != "row":
+                raise ValueError("e4m3 weights have one layout: the per-layer GEMM tags must say RowMajor for B")
+        else:
+            assert weight_layout in ("row", "col"), weight_layout
+            layer_layout, head_layout = ("row" if e4m3 else weight_layout), weight_layout
+            tag_of = {"row": DEFAULT_TAG, "col": DEFAULT_TAG_NK}
+            self.tags = [tag_of[layer_layout]] * (n_tags - 1) + [tag_of[head_layout]]
+        self.weight_layout, self.lm_head_layout = layer_layout, head_layout
         write_config(self.cfg_path, shape, global_batch=global_batch, nano1=nano1, kqv1=self.kqv1,
                      kqv3=self.kqv3, pipeline_type=pipeline_type, kv_pages=kv_pages,
-                     run_layer=run_layer, distinct_layers=distinct_layers, n_tags=n_tags)
+                     run_layer=run_layer, distinct_layers=distinct_layers, n_tags=n_tags, tags=self.tags)
         P.setRank(1, 1)
         P.setModelConfig(self.cfg_path)
         self.max_pages = P.maxPageNum()
@@ -88,25 +131,27 @@ class Engine:
         H, V, F, d = shape.hidden, shape.vocab, shape.ffn, shape.d
         kqv_n = shape.kqv_n
 
-        def mk(key, layer, rows, cols, std=0.02, mean=0.0):
+        def mk(key, layer, rows, cols, std=0.02, mean=0.0, layout="row"):
+            """A [rows, cols] tensor; layout "col" stores its transpose [cols, rows] (for a GEMM
+            weight [K, N]: [N][K])."""
             if weights is not None:
                 a = weights[key] if layer is None else weights[key][layer]
-                return torch.from_numpy(np.ascontiguousarray(a)).to(self.dev)
-            t = torch.empty((rows, cols), dtype=torch.float16, device=self.dev)
+                t = torch.from_numpy(np.ascontiguousarray(a)).to(self.dev)
+                return t.t().contiguous() if layout == "col" else t
+            t = torch.empty((cols, rows) if layout == "col" else (rows, cols), dtype=torch.float16, device=self.dev)
             t.normal_(mean, std, generator=gen)
             return t
 
-        self.t = {"embedding": mk("embedding", None, V, H), "lm_head": mk("lm_head", None, H, V),
+        self.t = {"embedding": mk("embedding", None, V, H), "lm_head": mk("lm_head", None, H, V, layout=head_layout),
                   "model_norm": mk("model_norm", None, 1, H, 0.02, 1.0), "layers": []}
         mw = P.VortexModelWeight()
         mw.lm_head = _weight(self.t["lm_head"], H, V)
         mw.embedding = _weight(self.t["embedding"], V, H)
         mw.model_layernorm = _weight(self.t["model_norm"], H, 1)
-        e4m3 = self.weight_format == P.WeightFormat.E4M3
 
         def gemm_weight(key, layer, rows, cols):
             """(tensor to keep alive, VortexWeight) of a [rows = K, cols = N] GEMM weight."""
-            t = mk(key, layer, rows, cols)
+            t = mk(key, layer, rows, cols, layout=layer_layout)
             if not e4m3:
                 return t, _weight(t, cols, rows)
             blob = torch.empty((P.e4m3WeightBytes(cols, rows),), dtype=torch.uint8, device=self.dev)
@@ -164,7 +209,7 @@ class Engine:
         self._open = True
         try:
             cfg = P.VortexConfigData()
-            cfg.setGemmOpTag([DEFAULT_TAG] * n_tags)
+            cfg.setGemmOpTag(self.tags)
             cfg.globalBatchSize, cfg.nanobatch1Size = global_batch, nano1
             cfg.kqv1Size, cfg.kqv3Size = self.kqv1, self.kqv3
             P.config([cfg])

@@ -246,12 +246,12 @@ def main():
             ms = timeit(fn, a.iters, a.warm)
             print(f"{a.op} {name:8s} {M}x{N}x{Kd}: {ms * 1e3:9.1f} us  {2.0 * M * N * Kd / ms / 1e9:8.1f} TFLOP/s", flush=True)
     elif a.op == "dual":
-        A, Bg, Bu = (t.to(edt) for t in (rnd(a.m, shape.hidden), rnd(shape.hidden, shape.ffn, std=0.02),
-                                         rnd(shape.hidden, shape.ffn, std=0.02)))
+        wshape = (shape.ffn, shape.hidden) if a.b_col_major else (shape.hidden, shape.ffn)
+        A, Bg, Bu = (t.to(edt) for t in (rnd(a.m, shape.hidden), rnd(*wshape, std=0.02), rnd(*wshape, std=0.02)))
         out = torch.empty(a.m, shape.ffn, dtype=edt, device=DEV)
         Gs, Us = cold_copies(Bg, a.cold), cold_copies(Bu, a.cold)
-        ms = timeit(lambda: K.dual_swiglu(A, next(Gs), next(Us), out=out), a.iters, a.warm)
-        print(f"dual gate/up {a.m}x{shape.ffn}x{shape.hidden}: {ms * 1e3:9.1f} us  "
+        ms = timeit(lambda: K.dual_swiglu(A, next(Gs), next(Us), out=out, b_col_major=a.b_col_major), a.iters, a.warm)
+        print(f"dual gate/up {'[N][K] weights ' if a.b_col_major else ''}{a.m}x{shape.ffn}x{shape.hidden}: {ms * 1e3:9.1f} us  "
               f"{4.0 * a.m * shape.ffn * shape.hidden / ms / 1e9:8.1f} TFLOP/s", flush=True)
     elif a.op == "dual_f8":
         M, N, Kd = a.m, shape.ffn, shape.hidden

@@ -61,10 +61,10 @@ def lib() -> C.CDLL:
         l.nf_dual_swiglu_workspace_bytes.argtypes = [i32, i32, i32]
         l.nf_dual_swiglu_workspace_bytes_upto.restype = sz
         l.nf_dual_swiglu_workspace_bytes_upto.argtypes = [i32, i32, i32]
-        l.nf_dual_swiglu_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp, sz, vp]
+        l.nf_dual_swiglu_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, vp, sz, vp]
         l.nf_gemm_bias_f16_ws.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp, sz, vp]
         l.nf_gemm_bias_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
-        l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
+        l.nf_dual_swiglu_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, vp]
         l.nf_gemm_bf16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_dual_swiglu_bf16.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
         l.nf_quantize_rows_e4m3.argtypes = [vp, vp, vp, i32, i32, vp]
@@ -216,33 +216,38 @@ def gemm_ws(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, w
     return out, need
 
 
-def dual_swiglu_ws(A, Bg, Bu, out=None, workspace=None):
-    """nf_dual_swiglu_f16_ws; returns (out, bytes of workspace the shape asks for: 0 = not split)."""
+def dual_swiglu_ws(A, Bg, Bu, out=None, workspace=None, b_col_major=False):
+    """nf_dual_swiglu_f16_ws; returns (out, bytes of workspace the shape asks for: 0 = not split).
+    b_col_major: Bg / Bu are [N, K] (k contiguous) instead of [K, N]."""
     _f16(A); _f16(Bg); _f16(Bu)
     M, K = A.shape
-    N = Bg.shape[1]
-    assert tuple(Bg.shape) == (K, N) and tuple(Bu.shape) == (K, N)
+    N = Bg.shape[0] if b_col_major else Bg.shape[1]
+    assert tuple(Bg.shape) == ((N, K) if b_col_major else (K, N)) and Bu.shape == Bg.shape
     need = lib().nf_dual_swiglu_workspace_bytes(M, N, K)
     if workspace is None:
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
     out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
-    _check(lib().nf_dual_swiglu_f16_ws(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, _p(workspace), workspace.numel(),
-                                       _stream()), "nf_dual_swiglu_f16_ws")
+    _check(lib().nf_dual_swiglu_f16_ws(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, int(b_col_major), _p(workspace),
+                                       workspace.numel(), _stream()), "nf_dual_swiglu_f16_ws")
     return out, need
 
 
-def dual_swiglu(A, Bg, Bu, out=None):
+def dual_swiglu(A, Bg, Bu, out=None, b_col_major=False):
+    """b_col_major (fp16 only): Bg / Bu are [N, K] (k contiguous) instead of [K, N]."""
     dt = A.dtype
     assert dt in (torch.float16, torch.bfloat16), dt
     _elem(A, dt); _elem(Bg, dt); _elem(Bu, dt)
     M, K = A.shape
-    N = Bg.shape[1]
-    assert tuple(Bg.shape) == (K, N) and tuple(Bu.shape) == (K, N)
+    N = Bg.shape[0] if b_col_major else Bg.shape[1]
+    assert tuple(Bg.shape) == ((N, K) if b_col_major else (K, N)) and Bu.shape == Bg.shape
     out = torch.empty((M, N), dtype=dt, device=A.device) if out is None else out
     _elem(out, dt)
-    fn, name = (lib().nf_dual_swiglu_f16, "nf_dual_swiglu_f16") if dt == torch.float16 else \
-        (lib().nf_dual_swiglu_bf16, "nf_dual_swiglu_bf16")
-    _check(fn(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, _stream()), name)
+    if dt == torch.float16:
+        _check(lib().nf_dual_swiglu_f16(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, int(b_col_major), _stream()),
+               "nf_dual_swiglu_f16")
+    else:
+        assert not b_col_major, "the bf16 pair takes [K, N] weights only"
+        _check(lib().nf_dual_swiglu_bf16(_p(A), _p(Bg), _p(Bu), _p(out), M, N, K, _stream()), "nf_dual_swiglu_bf16")
     return out
 
 

@@ -132,6 +132,10 @@ def main():
     cfg = json.load(open(a.config_path))
     mc, sc = cfg["model_configs"], cfg["serve_configs"]
     shape, pt, (T, nano1, kqv1, kqv3), pages = parse_config(cfg)
+    # the file's GEMM tags (their B layout decides the orientation the weights are handed over in);
+    # a list written for another schedule's GEMM count falls back to the default tags
+    tags = cfg["pipeline_configs"].get("gemm_op_tag") or []
+    tags = list(tags) if len(tags) == pt.gemm_tags else None
 
     weights = None
     if not empty_weight:
@@ -160,7 +164,7 @@ def main():
     avg_out = sum(r[2] for r in reqs) // len(reqs)
     eng = engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=kqv1, kqv3=kqv3, kv_pages=pages,
                         run_layer=mc.get("run_layer", shape.layers), kv_fill="zeros", weights=weights,
-                        weight_format=sc.get("weight_format", "f16"))
+                        weight_format=sc.get("weight_format", "f16"), gemm_tags=tags)
     former = P.BatchFormer(pages, shape.page_size, T, nano1, kqv1, kqv3, avg_in, avg_out)
 
     pending = list(reqs)                  # not yet released, in arrival order

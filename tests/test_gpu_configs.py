@@ -25,7 +25,7 @@ def _max_rel(got, ref):
     return np.abs(got.astype(np.float64) - ref).max() / np.abs(ref).max()
 
 
-def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines, weight_format="f16"):
+def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines, weight_format="f16", weight_layout="row"):
     """Iteration 0 prefills the last prompt token of every request (so that the decode iteration
     is fed distinct tokens: the samples of iteration 0); iteration 1 is the decode step under test."""
     from nanoflow_amd import engine, pllm_python as P
@@ -55,10 +55,10 @@ def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines, weight_format="f
                            num_pages=b0.num_pages)
 
     for pt in pipelines:
-        print(f"shape hidden={shape.hidden} pipeline={pt.name}", flush=True)
+        print(f"shape hidden={shape.hidden} pipeline={pt.name} weight layout={weight_layout}", flush=True)
         T = max(64, (n + 63) // 64 * 64)
-        with engine.Engine(shape, pt, global_batch=T, nano1=T // 2, kqv1=T // 4, kqv3=T // 4,
-                           kv_pages=b0.num_pages, weights=w, kv_pools=pools0, weight_format=weight_format) as e:
+        with engine.Engine(shape, pt, global_batch=T, nano1=T // 2, kqv1=T // 4, kqv3=T // 4, kv_pages=b0.num_pages,
+                           weights=w, kv_pools=pools0, weight_format=weight_format, weight_layout=weight_layout) as e:
             e.update(b0, keep_token_list=np.zeros(0, np.int32))
             s0 = e.run()
             kv_after0 = [p[:b0.num_pages].cpu().numpy() for p in e.kv]
@@ -141,19 +141,22 @@ def _decode_layer_case(oracle, shape, kv_lens, seed, pipelines, weight_format="f
             assert _max_rel(kv[l][wrote_got], pools_ref[l][wrote_ref]) < kv_tol, (pt, l, "appended K/V rows")
 
 
-def test_llama3_8b_layer_64_decode_tokens(oracle):
+@pytest.mark.parametrize("weight_layout", ["row", "col"])
+def test_llama3_8b_layer_64_decode_tokens(oracle, weight_layout):
     from nanoflow_amd import pllm_python as P
     shape = synth.ModelShape(layers=1, vocab=4096)                      # 8B layer dimensions
     kv_lens = np.random.default_rng(2).integers(512, 1025, size=64)
-    _decode_layer_case(oracle, shape, kv_lens, seed=0,
+    _decode_layer_case(oracle, shape, kv_lens, seed=0, weight_layout=weight_layout,
                        pipelines=(P.PipelineType.NON_OVERLAP_LOCAL, P.PipelineType.LOCAL))
 
 
-def test_llama3_70b_shaped_layer(oracle):
+@pytest.mark.parametrize("weight_layout", ["row", "col"])
+def test_llama3_70b_shaped_layer(oracle, weight_layout):
     from nanoflow_amd import pllm_python as P
     shape = synth.ModelShape(hidden=8192, Hq=64, Hkv=8, ffn=28672, vocab=2048, layers=1)
     kv_lens = np.random.default_rng(3).integers(200, 400, size=16)
-    _decode_layer_case(oracle, shape, kv_lens, seed=1, pipelines=(P.PipelineType.NON_OVERLAP_LOCAL,))
+    _decode_layer_case(oracle, shape, kv_lens, seed=1, pipelines=(P.PipelineType.NON_OVERLAP_LOCAL,),
+                       weight_layout=weight_layout)
 
 
 def test_llama3_70b_shaped_layer_with_e4m3_weights(oracle):
@@ -243,7 +246,8 @@ def _teacher_forced_e4m3(oracle, w, wq, inter, hid, x_in, tag):
 
 def _full_width_iteration(oracle, shape, batch, schedules, weight_format="f16", seed=11):
     """One iteration of `batch` through ONE full-width decoder layer on each schedule of
-    `schedules` = ((pipeline type, (nano1, kqv1, kqv3)), ...), against the oracle.
+    `schedules` = ((pipeline type, (nano1, kqv1, kqv3)[, weight layout "row" | "col"]), ...), against
+    the oracle (one oracle forward serves them all: the layouts hold the same matrices).
 
     fp16 weights: the residual stream end to end and the appended K / V rows within 2e-3 on every
     schedule, sampled ids; on the schedules that expose their whole-iteration buffers (the sequential
@@ -269,12 +273,14 @@ def _full_width_iteration(oracle, shape, batch, schedules, weight_format="f16", 
     gidx = lambda a: torch.from_numpy(a.astype(np.int64)).cuda()
     names = ("ln_attn", "kqv", "attn_out", "o_out", "ln_ffn", "act")
     try:
-        for pt, split in schedules:
-            tag = f"{pt.name} {weight_format}"
+        for pt, split, *rest in schedules:
+            layout = rest[0] if rest else "row"
+            tag = f"{pt.name} {weight_format} {layout}"
             print(f"full-width iteration against the oracle: hidden={shape.hidden} rows={T} ({nd} decode) {tag}", flush=True)
             G = (T + 63) // 64 * 64
             with engine.Engine(shape, pt, global_batch=G, nano1=split[0], kqv1=split[1], kqv3=split[2],
-                               kv_pages=batch.num_pages, weights=w, seed=seed, weight_format=weight_format) as e:  # KV pool: N(0, 1) drawn on the device
+                               kv_pages=batch.num_pages, weights=w, seed=seed, weight_format=weight_format,
+                               weight_layout=layout) as e:  # KV pool: N(0, 1) drawn on the device
                 if ref is None:
                     kv0 = e.kv[0][:batch.num_pages].cpu().numpy()
                 e.update(batch, keep_token_list=np.ones(nd, np.int32))
@@ -330,8 +336,10 @@ def test_one_iteration_workload_matches_oracle_at_full_width(oracle):
     shape = synth.ModelShape(layers=1, vocab=4096)
     batch = synth.config2_batch(seed=0, vocab=shape.vocab)
     assert batch.tokens == 2048 and batch.decodePrefillBorder == 1792
-    _full_width_iteration(oracle, shape, batch, ((P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512)),
-                                                 (P.PipelineType.PLLM, (640, 256, 768))))
+    _full_width_iteration(oracle, shape, batch, ((P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512), "row"),
+                                                 (P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512), "col"),
+                                                 (P.PipelineType.PLLM, (640, 256, 768), "row"),
+                                                 (P.PipelineType.PLLM, (640, 256, 768), "col")))
 
 
 LLAMA3_70B_LAYER = dict(hidden=8192, Hq=64, Hkv=8, ffn=28672, vocab=2048, layers=1)
@@ -348,8 +356,10 @@ def test_llama3_70b_layer_on_the_dense_iteration_mix(oracle, weight_format):
     shape = synth.ModelShape(**LLAMA3_70B_LAYER)
     batch = synth.config2_batch(seed=3, vocab=shape.vocab)
     assert batch.tokens == 2048 and batch.decodePrefillBorder == 1792
-    _full_width_iteration(oracle, shape, batch, ((P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512)),
-                                                 (P.PipelineType.PLLM, (640, 256, 768))), weight_format=weight_format)
+    layouts = ("row", "col") if weight_format == "f16" else ("col",)     # e4m3: only the LM head follows the layout
+    _full_width_iteration(oracle, shape, batch,
+                          [(P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512), lay) for lay in layouts] +
+                          [(P.PipelineType.PLLM, (640, 256, 768), layouts[-1])], weight_format=weight_format)
 
 
 def _offline_steady_state_batch(vocab, kv_pages=98304, T=2048, cycles=1300):
@@ -393,8 +403,9 @@ def test_llama3_8b_layer_on_the_offline_steady_state_batch(oracle):
     print(f"steady-state batch: {nd} decode rows, {pre} prefill requests of {np.diff(batch.input_indptr[nd:]).tolist()} tokens "
           f"continuing at {prev.tolist()}", flush=True)
     assert 600 < nd < 760 and batch.tokens > 1900 and pre >= 2 and prev.max() > 0
-    _full_width_iteration(oracle, shape, batch, ((P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512)),
-                                                 (P.PipelineType.LOCAL, (1024, 512, 512))))
+    _full_width_iteration(oracle, shape, batch, ((P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512), "col"),
+                                                 (P.PipelineType.NON_OVERLAP_LOCAL, (1024, 512, 512), "row"),
+                                                 (P.PipelineType.LOCAL, (1024, 512, 512), "col")))
 
 
 def test_one_iteration_workload_is_schedule_independent_at_full_width():

@@ -268,6 +268,30 @@ def test_dual_swiglu_split_over_k_matches_oracle(K, oracle, M, N, K_):
     assert need == 0
 
 
+@pytest.mark.parametrize("M,N,K_", [(5, 136, 72), (64, 14336, 256), (200, 1160, 264), (267, 24584, 328), (300, 14336, 1024),
+                                    (16, 14336, 4096), (2048, 14336, 256), (1992, 14328, 200), (1792, 28672, 128)])
+def test_dual_swiglu_with_k_contiguous_weights(K, oracle, M, N, K_):
+    """The gate/up pair on [N][K] weights (the layout a GEMM tag calls ColumnMajor for B), plain and
+    split over K: against the oracle, and bit for bit what the [K][N] path gives for the same
+    matrices (the same products summed in the same order; only the way the fragments reach the
+    registers differs)."""
+    rng = np.random.default_rng(M + N + K_)
+    A = synth.normal_f16(rng, (M, K_))
+    Bg = synth.normal_f16(rng, (K_, N), 0.03)
+    Bu = synth.normal_f16(rng, (K_, N), 0.03)
+    gt, ut = dev(np.ascontiguousarray(Bg.T)), dev(np.ascontiguousarray(Bu.T))
+    ref = oracle.dual_swiglu(A, Bg, Bu)
+    got = host(K.dual_swiglu(dev(A), gt, ut, b_col_major=True))
+    assert_close(got, ref, what="dual swiglu, [N][K] weights")
+    assert np.array_equal(got, host(K.dual_swiglu(dev(A), dev(Bg), dev(Bu))))
+    got_ws, need = K.dual_swiglu_ws(dev(A), gt, ut, b_col_major=True)
+    row_ws, need_row = K.dual_swiglu_ws(dev(A), dev(Bg), dev(Bu))
+    assert need == need_row
+    assert_close(host(got_ws), ref, 2 * RTOL if need else RTOL, what="dual swiglu with workspace, [N][K] weights")
+    assert np.array_equal(host(got_ws), host(row_ws))
+    assert not np.array_equal(got, host(K.dual_swiglu(dev(A), ut, gt, b_col_major=True)))     # gate is the first
+
+
 def test_dual_known_answer_inputs(K, oracle):
     # inputs of the reference's dual-GEMM test program (all operands (j+k)/2560, 128^3)
     j, k = np.meshgrid(np.arange(128), np.arange(128), indexing="ij")

@@ -912,3 +912,44 @@ def test_python_builders_follow_the_reference_call_sequence(tmp_path):
         assert len(out) == nd + b.prefillNum and np.array_equal(out, np.zeros(len(out), np.int32))
     finally:
         P.finalize()
+
+
+@pytest.mark.parametrize("pt_name", ["NON_OVERLAP_LOCAL", "LOCAL", "NANOBATCH_LOCAL", "PLLM", "NANOBATCH", "PLLMOFFLOAD",
+                                     "KQVBIAS", "NONOVERLAP_KQVBIAS"])
+def test_k_contiguous_weights_give_the_same_results_on_every_schedule(oracle, pt_name):
+    """The same model handed over as [N][K] weights (every GEMM tag says ColumnMajor for B; the gate/up
+    pair follows the tags) and as the reference's [K][N]: against the oracle, and bit for bit the same
+    residual stream, logits and samples (same products, same order of summation).  Also through an
+    explicit tag list, as a pipeline file gives it, and the refusal of tags that disagree."""
+    from nanoflow_amd import engine, pllm_python as P
+    pt = P.PipelineType[pt_name]
+    T, nano1, dlens, chunks = CASES["prefill_straddles_border"]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=0)
+    if pt.has_kqv_bias:
+        w["b_kqv"] = synth.make_weights(shape, seed=9, kqv_bias=True)["b_kqv"]
+    b1 = synth.make_batch(dlens, chunks, vocab=shape.vocab, seed=21, extra_pages=40)
+    rng = np.random.default_rng(5)
+    pools0 = [synth.make_kv_pool(b1.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok1 = b1.input_tokens.copy()
+    tok1[:b1.decodePrefillBorder] = 1
+    d1 = b1.as_dict()
+    d1["input_tokens"] = tok1
+    hid, log, samp = oracle.decoder_forward(shape.as_dict(), w, [p.copy() for p in pools0], d1, want_logits=True)
+    out = {}
+    nk = [engine.DEFAULT_TAG_NK] * pt.gemm_tags
+    for name, kw in (("row", dict(weight_layout="row")), ("col", dict(weight_layout="col")), ("tags", dict(gemm_tags=nk))):
+        print(f"pipeline={pt_name} weights {name}", flush=True)
+        with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=max(nano1 // 2, 1), kqv3=(T - nano1) // 2,
+                           kv_pages=b1.num_pages, weights=w, kv_pools=pools0, **kw) as e:
+            assert e.weight_layout == ("row" if name == "row" else "col")
+            e.update(b1, keep_token_list=np.ones(b1.decodePrefillBorder, np.int32))
+            s = e.run().copy()
+            out[name] = (s, e.buffer("hidden").cpu().numpy()[:b1.tokens], e.buffer("logits").cpu().numpy()[:b1.req_num])
+        assert _max_rel(out[name][1], hid) < E2E_RTOL and _max_rel(out[name][2], log) < E2E_RTOL, (pt_name, name)
+    for name in ("col", "tags"):
+        for a, c in zip(out["row"], out[name]):
+            assert np.array_equal(a, c), (pt_name, name)
+    mixed = [engine.DEFAULT_TAG_NK] + [engine.DEFAULT_TAG] * (pt.gemm_tags - 1)
+    with pytest.raises(ValueError, match="disagree"):
+        engine.Engine(shape, pt, global_batch=T, nano1=nano1, kv_pages=b1.num_pages, gemm_tags=mixed)

@@ -235,3 +235,23 @@ def test_shipped_pipeline_files_parse_and_fit_one_mi355x():
         assert kv > 0.25 * (288 << 30), (f, kv / 1e9)                      # and the pool is not a token gesture
         if "3.1" in f:
             assert shape.rope_scaling and shape.rope_scaling["factor"] == 8.0
+
+
+def test_gemm_tag_layout_fields_decide_the_weight_orientation():
+    """engine.layouts_of_tags: the B layout field of the per-layer tags and of the LM head's tag (the last
+    one) of a pipeline file; the shipped fp16 files ask for [N][K] weights throughout, the e4m3 ones for
+    the fp8 form's own layout (RowMajor tags) with a k-contiguous LM head."""
+    import glob, json, os
+    from nanoflow_amd import engine
+    assert engine.layouts_of_tags([engine.DEFAULT_TAG] * 4) == ("row", "row")
+    assert engine.layouts_of_tags([engine.DEFAULT_TAG_NK] * 7) == ("col", "col")
+    assert engine.layouts_of_tags([engine.DEFAULT_TAG] * 8 + [engine.DEFAULT_TAG_NK]) == ("row", "col")
+    with pytest.raises(ValueError, match="disagree"):
+        engine.layouts_of_tags([engine.DEFAULT_TAG, engine.DEFAULT_TAG_NK, engine.DEFAULT_TAG, engine.DEFAULT_TAG])
+    with pytest.raises(ValueError, match="malformed"):
+        engine.layouts_of_tags(["128_128_32", engine.DEFAULT_TAG])
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "nanoflow_amd", "config_all")
+    for f in sorted(glob.glob(os.path.join(root, "*.json"))):
+        cfg = json.load(open(f))
+        fp8 = cfg["serve_configs"].get("weight_format") == "e4m3"
+        assert engine.layouts_of_tags(cfg["pipeline_configs"]["gemm_op_tag"]) == (("row" if fp8 else "col"), "col"), f
