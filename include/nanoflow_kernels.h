@@ -112,6 +112,20 @@ NF_API size_t nf_dual_swiglu_workspace_bytes_upto(int max_M, int N, int K);
 NF_API int nf_dual_swiglu_f16_ws(const uint16_t* A, const uint16_t* Bgate, const uint16_t* Bup, uint16_t* out,
                                  int M, int N, int K, int b_col_major, void* workspace, size_t workspace_bytes,
                                  nf_stream_t stream);
+/* nf_gemm_f16 / nf_gemm_bias_f16 (c_is_row != 0: C is one row [N] added to every row) on a tile and
+ * a split over K of the CALLER's choosing: what the cta_m, cta_n and split_k fields of the reference's
+ * GEMM tag select (pipeline/include/gemmShape.cuh:5-6; there one CUTLASS instantiation per tag,
+ * pipeline/include/gemmFactory.in:7-16).  The tile is the entry of the library's menu closest to
+ * tile_m x tile_n (nf_gemm_tile_menu enumerates it: index 0 .. count-1 -> tile sizes and whether the
+ * entry takes k-contiguous weights only; returns the count); split_k > 1 cuts K into that many shares
+ * (at most 16, each at least 64 deep) whose fp32 sums go through `workspace`
+ * (nf_gemm_tiled_workspace_bytes(M, N, K, split_k) bytes, 16-byte aligned) and are added by a second
+ * launch.  Results agree with nf_gemm_f16 to fp32 summation order. */
+NF_API int nf_gemm_tile_menu(int index, int* tile_m, int* tile_n, int* k_contiguous_weights_only);
+NF_API size_t nf_gemm_tiled_workspace_bytes(int M, int N, int K, int split_k);
+NF_API int nf_gemm_f16_tiled(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
+                             float alpha, float beta, int b_col_major, int c_is_row, int tile_m, int tile_n,
+                             int split_k, void* workspace, size_t workspace_bytes, nf_stream_t stream);
 /* the same for nf_gemm_bias_f16 (declared below) */
 NF_API int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M, int N,
                                int K, float alpha, float beta, int b_col_major, void* workspace,

@@ -16,7 +16,7 @@ bool parseGemmTag(const std::string& tag, GemmTag& out) {
   for (int i = 0; i < 8; ++i) {
     char* end = nullptr;
     long v = std::strtol(parts[i].c_str(), &end, 10);
-    if (end == parts[i].c_str() || *end != '\0' || v <= 0) return false;
+    if (end == parts[i].c_str() || *end != '\0' || v < 0) return false;  // 0: left to the library
     *fields[i] = (int)v;
   }
   PllmLayout* layouts[3] = {&out.layout_a, &out.layout_b, &out.layout_out};
@@ -61,16 +61,21 @@ void HipGEMMWrapperF8W::work() {
 }
 
 void HipGEMMWrapper::work() {
+  const int bcol = tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0;
+  if (tagChoosesTile()) {
+    NF_KERNEL_CHECK(nf_gemm_f16_tiled(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr, pllm_tensor_d.ptr,
+                                      (int)rows(), (int)N, (int)K, alpha, beta, bcol, c_is_row ? 1 : 0, tag.cta_m,
+                                      tag.cta_n, taggedSplit(), splitk_workspace, splitk_workspace_bytes, stream));
+    return;
+  }
   if (c_is_row) {
     NF_KERNEL_CHECK(nf_gemm_bias_f16_ws(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
-                                        pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
-                                        tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, splitk_workspace,
-                                        splitk_workspace_bytes, stream));
+                                        pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta, bcol,
+                                        splitk_workspace, splitk_workspace_bytes, stream));
     return;
   }
   NF_KERNEL_CHECK(nf_gemm_f16_ws(pllm_tensor_a.ptr, pllm_tensor_b.ptr, pllm_tensor_c.ptr,
-                                 pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta,
-                                 tag.layout_b == PllmLayout::COL_MAJOR ? 1 : 0, splitk_workspace,
+                                 pllm_tensor_d.ptr, (int)rows(), (int)N, (int)K, alpha, beta, bcol, splitk_workspace,
                                  splitk_workspace_bytes, stream));
 }
 

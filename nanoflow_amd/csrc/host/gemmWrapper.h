@@ -2,12 +2,16 @@
 //   BaseGEMMWrapper  -- same virtual interface as the reference's
 //                       pipeline/include/cutlassGemmWrapperImpl.cuh:23-66;
 //   HipGEMMWrapper   -- D = alpha*A.B + beta*C on the MFMA kernel; takes the place of
-//                       CutlassGEMMWrapper<...> (:68-437).  The tile/stage fields of the tag
-//                       are accepted and recorded, but tiling is chosen by the kernel layer
-//                       from the problem shape; the three layout fields are honoured
-//                       (A and output must be RowMajor, B may be Row- or ColumnMajor);
+//                       CutlassGEMMWrapper<...> (:68-437).  The tag's cta_m x cta_n selects the
+//                       closest tile of the kernel layer's menu and its split_k a split over K
+//                       for launches of more than 512 live rows (the dense regime a tag is tuned
+//                       for; shorter launches keep the few-row plan); cta_m = 0 leaves both to the
+//                       kernel layer's cost model.  The warp and stage fields are recorded only
+//                       (wavefront grid and LDS ring follow from the tile).  The three layout
+//                       fields are honoured (A and output RowMajor, B Row- or ColumnMajor);
 //   generateGEMM(tag) -- tag -> wrapper factory (pipeline/include/gemmFactory.cuh).
 #pragma once
+#include <algorithm>
 #include <string>
 
 #include "nanoflow_kernels.h"
@@ -99,7 +103,24 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   // narrow N would otherwise leave most of the chip idle); sized for the worst case up to M rows
   void* splitk_workspace = nullptr;
   size_t splitk_workspace_bytes = 0;
-  size_t workspaceBytes() const override { return nf_gemm_workspace_bytes_upto((int)M, (int)N, (int)K); }
+  // the tag names a tile (cta_m, cta_n > 0): it applies to launches of more than kTagMinRows live rows
+  static constexpr size_t kTagMinRows = 512;
+  bool tagChoosesTile() const { return tag.cta_m > 0 && tag.cta_n > 0 && rows() > kTagMinRows; }
+  // The tag's split over K, lowered to what fits the partial-sum scratch the tmp buffer reserves per
+  // wrapper (ModelConfig.k_temp_size: 256 x 65536 floats, 67 MB): 2 shares of 2048 x 4096 fit, the
+  // LM head's never do.
+  static constexpr size_t kSplitScratchBytes = (size_t)256 * 65536 * sizeof(float);
+  int taggedSplit() const {
+    if (tag.split_k <= 1 || M == 0 || N == 0) return 1;
+    const size_t fit = kSplitScratchBytes / (M * N * sizeof(float));
+    return (int)std::max<size_t>(1, std::min<size_t>((size_t)tag.split_k, fit));
+  }
+  size_t workspaceBytes() const override {
+    const size_t few = nf_gemm_workspace_bytes_upto((int)M, (int)N, (int)K);
+    const size_t tagged = tag.cta_m > 0 && tag.cta_n > 0 && M > kTagMinRows
+                              ? nf_gemm_tiled_workspace_bytes((int)M, (int)N, (int)K, taggedSplit()) : 0;
+    return few > tagged ? few : tagged;
+  }
   void setWorkspace(void* ptr, size_t bytes) override {
     splitk_workspace = ptr;
     splitk_workspace_bytes = bytes;

@@ -220,13 +220,13 @@ public:
   void assignSameStream();
   enum class GEMM_NAME { O1 = 0, O2, D1, D2, KQV1, KQV2, LOGITS, NUM };
   static constexpr std::array gemmConfig = {
-      "128_256_64_64_64_64_1_3_RowMajor_RowMajor_RowMajor",  // O1
-      "128_256_64_64_64_64_1_3_RowMajor_RowMajor_RowMajor",  // O2
-      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // D1
-      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // D2
-      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV1
-      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV2
-      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // LOGITS
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // O1
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // O2
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // D1
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // D2
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // KQV1
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // KQV2
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // LOGITS
   };
   static constexpr int gemmNum = static_cast<int>(GEMM_NAME::NUM);
   std::array<BaseGEMMWrapper*, gemmNum> gemms{};
@@ -292,10 +292,10 @@ class NonOverlapLocalPipeline : public PipelineBase {
 public:
   enum class GEMM_NAME { O = 0, D, KQV, LOGITS, NUM };
   static constexpr std::array gemmConfig = {
-      "128_256_64_64_64_64_1_3_RowMajor_RowMajor_RowMajor",  // O
-      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // D
-      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV
-      "128_256_32_64_64_32_1_3_RowMajor_RowMajor_RowMajor",  // LOGITS
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // O
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // D
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // KQV
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // LOGITS
   };
   static constexpr int gemmNum = static_cast<int>(GEMM_NAME::NUM);
   std::array<BaseGEMMWrapper*, gemmNum> gemms{};
@@ -347,15 +347,15 @@ class Pipeline : public PipelineBase {
 public:
   enum class GEMM_NAME { O1 = 0, O2, D1, D2, KQV1, KQV2, KQV3, KQV4, LOGITS, NUM };
   static constexpr std::array gemmConfig = {
-      "128_128_32_64_64_32_3_5_RowMajor_RowMajor_RowMajor",  // O1
-      "128_128_32_64_64_32_1_4_RowMajor_RowMajor_RowMajor",  // O2
-      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // D1
-      "128_128_32_64_64_32_1_4_RowMajor_RowMajor_RowMajor",  // D2
-      "128_64_64_64_32_64_2_3_RowMajor_RowMajor_RowMajor",   // KQV1
-      "128_128_32_64_64_32_2_5_RowMajor_RowMajor_RowMajor",  // KQV2
-      "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor",  // KQV3
-      "128_64_64_64_32_64_2_3_RowMajor_RowMajor_RowMajor",   // KQV4
-      "128_256_32_64_64_32_2_3_RowMajor_RowMajor_RowMajor",  // LOGITS
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // O1
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // O2
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // D1
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // D2
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",   // KQV1
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // KQV2
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // KQV3
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",   // KQV4
+      "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor",  // LOGITS
   };
   static constexpr int gemmNum = static_cast<int>(GEMM_NAME::NUM);
   std::array<BaseGEMMWrapper*, gemmNum> gemms{};

@@ -36,6 +36,7 @@
 // consecutive output columns of a row (of 32 rows with the 32x32 instruction).  The epilogue turns each wavefront's block around
 // through LDS so that D is stored, and C read, in whole 512-byte runs.
 #include <algorithm>
+#include <cmath>
 #include <type_traits>
 #include <utility>
 
@@ -881,6 +882,20 @@ static int splitk_plan(int M, int N, int K, int* k_per) {
   return (K + *k_per - 1) / *k_per;  // shares that are not empty
 }
 
+// More than 512 rows whose 256 x 256 tiles number half the CUs or fewer against a long contraction
+// (the 8B down projection: 2048 x 4096 x 14336, 128 tiles): two shares of K on 256 x 256 tiles fill
+// the chip, and with K that long the 67 MB of fp32 sums written, read back and added by a second
+// launch cost less than the smaller 128 x 256 tile does (measured with streamed [N][K] weights:
+// 199 us against 211; at K = 4096, the O projection, the split loses: 78 us against 64).
+constexpr int kDenseSplitMinK = 8192;
+static int dense_split_plan(int M, int N, int K, int* k_per) {
+  if (M <= kSplitMaxRows || K < kDenseSplitMinK) return 1;
+  const long long t256 = (long long)((M + 255) / 256) * ((N + 255) / 256);
+  if (t256 * 2 > cu_count() || t256 * 2 <= cu_count() / 2) return 1;
+  *k_per = ((K + 1) / 2 + BK - 1) / BK * BK;
+  return 2;
+}
+
 // The same for the fused gate/up pair (tiles of 64 x 128 up to 64 rows, 128 x 128 up to 256,
 // 320 x 128 on eight wavefronts up to 320).
 static int splitk_plan_dual(int M, int N, int K, int* k_per) {
@@ -927,12 +942,76 @@ static int dispatch_plain(const uint16_t* A, const uint16_t* B, const uint16_t* 
   const bool two_heights = t256 > cus && rest256 > 0 && rest256 <= cus / 2;
   if (two_heights)
     c256 = ((double)(t256 / cus) + 0.5 * (0.47 + 0.53 * 2.0 * rest256 / cus) / 0.95) * 256 * 256;
-  const double best = std::min(c256, std::min(c128x256, c128));
+  // k-contiguous weights only: 256 x 192, which fills the chip exactly once on 2048 x 6144 (QKV: 84 us
+  // against 89 on 192 tiles of 256 x 256) at 0.965 of the larger tile's efficiency (LM head: 1772 us
+  // against 1715 for the same area)
+  const double c256x192 = kBCol ? cost(256, 192, 0.965) : 1e300;
+  const double best = std::min(std::min(c256, c256x192), std::min(c128x256, c128));
+  if constexpr (kBCol)
+    if (best == c256x192 && best < c256)
+      return launch_gemm<E, 256, 192, 2, 2, false, true>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
   if (best == c256 && two_heights)
     return launch_hybrid<E, 256, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, (int)(t256 - rest256), s);
   if (best == c256) return launch_gemm<E, 256, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
   if (best == c128x256) return launch_gemm<E, 128, 256, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
   return launch_gemm<E, 128, 128, 2, 2, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
+}
+
+// ---- a caller-chosen tile and split over K (the cta_m / cta_n / split_k fields of a GEMM tag).
+// The menu: 64 x 256, 128 x 128, 128 x 256, 256 x 256 for both weight layouts, 256 x 192 for
+// k-contiguous weights (a row of a [K][N] slab must hold a multiple of 16 chunks for its swizzle).
+struct MenuTile {
+  int bm, bn;
+  bool col_only;
+};
+constexpr MenuTile kTileMenu[] = {{64, 256, false}, {128, 128, false}, {128, 256, false}, {256, 256, false}, {256, 192, true}};
+constexpr int kTileMenuSize = (int)(sizeof(kTileMenu) / sizeof(kTileMenu[0]));
+
+// The menu entry closest to (tile_m, tile_n) in log scale, among those the layout allows.
+static int menu_pick(int tile_m, int tile_n, bool b_col) {
+  int best = -1;
+  double best_d = 1e30;
+  for (int i = 0; i < kTileMenuSize; ++i) {
+    if (kTileMenu[i].col_only && !b_col) continue;
+    const double dm = std::log((double)kTileMenu[i].bm / tile_m), dn = std::log((double)kTileMenu[i].bn / tile_n);
+    const double d = std::fabs(dm) + std::fabs(dn);
+    if (d < best_d) {
+      best_d = d;
+      best = i;
+    }
+  }
+  return best;
+}
+
+// shares of a forced split: at most kMaxShares, each at least one slab deep
+static int forced_shares(int K, int split_k, int* k_per) {
+  int shares = std::min(std::min(split_k, kMaxShares), (K + BK - 1) / BK);
+  if (shares < 2) return 1;
+  *k_per = ((K + shares - 1) / shares + BK - 1) / BK * BK;
+  return (K + *k_per - 1) / *k_per;
+}
+
+template <class E, int BM, int BN, int WM, int WN, bool kBCol>
+static int launch_menu(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
+                       float alpha, float beta, int ldc, int shares, int k_per, float* P, hipStream_t s) {
+  if (shares > 1) return launch_splitk<E, BM, BN, WM, WN, kBCol>(A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s);
+  return launch_gemm<E, BM, BN, WM, WN, false, kBCol>(A, B, nullptr, C, D, M, N, K, alpha, beta, ldc, s);
+}
+
+template <class E, bool kBCol>
+static int dispatch_menu(int index, const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N,
+                         int K, float alpha, float beta, int ldc, int shares, int k_per, float* P, hipStream_t s) {
+  switch (index) {
+    case 0: return launch_menu<E, 64, 256, 1, 4, kBCol>(A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s);
+    case 1: return launch_menu<E, 128, 128, 2, 2, kBCol>(A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s);
+    case 2: return launch_menu<E, 128, 256, 2, 2, kBCol>(A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s);
+    case 3: return launch_menu<E, 256, 256, 2, 2, kBCol>(A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s);
+    case 4:
+      if constexpr (kBCol) return launch_menu<E, 256, 192, 2, 2, true>(A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s);
+      break;
+  }
+  set_error("gemm: no tile %d in the menu for this weight layout", index);
+  return NF_ERR_INVALID_ARGUMENT;
 }
 
 }  // namespace nf
@@ -975,7 +1054,9 @@ static int gemm_ws_entry(const char* who, const uint16_t* A, const uint16_t* B, 
                          int M, int N, int K, float alpha, float beta, int b_col_major, void* workspace,
                          size_t workspace_bytes, nf_stream_t stream, bool c_is_row = false) {
   int k_per = 0;
-  const int shares = M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0 ? splitk_plan(M, N, K, &k_per) : 1;
+  const bool shape_ok = M > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 8 == 0;
+  int shares = shape_ok ? splitk_plan(M, N, K, &k_per) : 1;
+  const bool dense = shares < 2 && shape_ok && (shares = dense_split_plan(M, N, K, &k_per)) > 1;
   if (shares < 2 || !workspace || workspace_bytes < (size_t)shares * M * N * sizeof(float))
     return gemm_entry<E>(who, A, B, C, D, M, N, K, alpha, beta, b_col_major, stream, c_is_row);
   int rc = check_gemm_args(who, A, B, D, M, N, K);
@@ -984,6 +1065,9 @@ static int gemm_ws_entry(const char* who, const uint16_t* A, const uint16_t* B, 
   NF_REQUIRE(((uintptr_t)C) % 8 == 0 && (uintptr_t)workspace % 16 == 0, "%s: C must be 8-byte and the workspace 16-byte aligned", who);
   hipStream_t s = (hipStream_t)stream;
   float* P = static_cast<float*>(workspace);
+  if (dense)
+    return b_col_major ? launch_splitk<E, 256, 256, 2, 2, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
+                       : launch_splitk<E, 256, 256, 2, 2, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
   if (M <= 64)
     return b_col_major ? launch_splitk<E, 64, 256, 1, 4, true>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s)
                        : launch_splitk<E, 64, 256, 1, 4, false>(A, B, C, D, M, N, K, alpha, beta, c_is_row ? 0 : N, shares, k_per, P, s);
@@ -1082,13 +1166,17 @@ int nf_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_
 size_t nf_gemm_workspace_bytes(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   int k_per = 0;
-  const int shares = splitk_plan(M, N, K, &k_per);
+  int shares = splitk_plan(M, N, K, &k_per);
+  if (shares < 2) shares = dense_split_plan(M, N, K, &k_per);
   return shares < 2 ? 0 : (size_t)shares * M * N * sizeof(float);
 }
 
 size_t nf_gemm_workspace_bytes_upto(int max_M, int N, int K) {
   size_t need = 0;
   for (int m = 1; m <= max_M && m <= kSplitMaxRows; ++m) need = std::max(need, nf_gemm_workspace_bytes(m, N, K));
+  // above that only the two-share split of launches with few 256 x 256 tiles: every count of tile rows
+  for (int m = kSplitMaxRows + 1; m <= max_M; m = (m + 255) / 256 * 256 + 1)
+    need = std::max(need, nf_gemm_workspace_bytes(std::min((m + 255) / 256 * 256, max_M), N, K));
   return need;
 }
 
@@ -1122,7 +1210,11 @@ int nf_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint
 
 int nf_gemm_f16_noalloc(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
                         float alpha, float beta, int b_col_major, nf_stream_t stream) {
-  const size_t need = nf_gemm_workspace_bytes(M, N, K);
+  // the few-row split only: the two-share split of dense launches is an optimisation that needs more
+  // than the array holds at any shape it applies to, and such a launch runs unsplit here
+  int k_per = 0;
+  const int few = M > 0 && N > 0 && K > 0 ? splitk_plan(M, N, K, &k_per) : 1;
+  const size_t need = few < 2 ? 0 : (size_t)few * M * N * sizeof(float);
   NF_REQUIRE(need <= kStaticScratchBytes,
              "nf_gemm_f16_noalloc: %d x %d x %d is split over K through %zu bytes of partial sums; the static "
              "scratch array holds %zu (use nf_gemm_f16_ws with a workspace of your own, or nf_gemm_f16)",
@@ -1137,6 +1229,46 @@ int nf_gemm_f16_noalloc(const uint16_t* A, const uint16_t* B, const uint16_t* C,
 }
 
 size_t nf_gemm_noalloc_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int nf_gemm_tile_menu(int index, int* tile_m, int* tile_n, int* k_contiguous_weights_only) {
+  if (index >= 0 && index < kTileMenuSize) {
+    if (tile_m) *tile_m = kTileMenu[index].bm;
+    if (tile_n) *tile_n = kTileMenu[index].bn;
+    if (k_contiguous_weights_only) *k_contiguous_weights_only = kTileMenu[index].col_only ? 1 : 0;
+  }
+  return kTileMenuSize;
+}
+
+size_t nf_gemm_tiled_workspace_bytes(int M, int N, int K, int split_k) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  int k_per = 0;
+  const int shares = forced_shares(K, split_k, &k_per);
+  return shares < 2 ? 0 : (size_t)shares * M * N * sizeof(float);
+}
+
+int nf_gemm_f16_tiled(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, int M, int N, int K,
+                      float alpha, float beta, int b_col_major, int c_is_row, int tile_m, int tile_n, int split_k,
+                      void* workspace, size_t workspace_bytes, nf_stream_t stream) {
+  const char* who = "nf_gemm_f16_tiled";
+  NF_REQUIRE(tile_m > 0 && tile_n > 0, "%s: tile %d x %d", who, tile_m, tile_n);
+  int rc = check_gemm_args(who, A, B, D, M, N, K);
+  if (rc) return rc;
+  NF_REQUIRE(beta == 0.f || C, "%s: beta=%g needs C", who, (double)beta);
+  NF_REQUIRE(((uintptr_t)C) % 8 == 0, "%s: C must be 8-byte aligned", who);
+  if (M == 0) return NF_OK;
+  int k_per = 0;
+  const int shares = forced_shares(K, split_k, &k_per);
+  NF_REQUIRE(shares < 2 || (workspace && (uintptr_t)workspace % 16 == 0 &&
+                            workspace_bytes >= (size_t)shares * M * N * sizeof(float)),
+             "%s: a split over K into %d shares needs a 16-byte aligned workspace of %zu bytes (nf_gemm_tiled_workspace_bytes)",
+             who, shares, (size_t)shares * M * N * sizeof(float));
+  const int index = menu_pick(tile_m, tile_n, b_col_major != 0);
+  const int ldc = c_is_row ? 0 : N;
+  float* P = static_cast<float*>(workspace);
+  hipStream_t s = (hipStream_t)stream;
+  return b_col_major ? dispatch_menu<F16, true>(index, A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s)
+                     : dispatch_menu<F16, false>(index, A, B, C, D, M, N, K, alpha, beta, ldc, shares, k_per, P, s);
+}
 
 int nf_gemm_bias_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* bias, uint16_t* D, int M, int N,
                         int K, float alpha, float beta, int b_col_major, void* workspace, size_t workspace_bytes,

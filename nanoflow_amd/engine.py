@@ -20,8 +20,21 @@ from . import synth
 # The tag grammar of the reference's pipeline files (pipeline/include/gemmShape.cuh:5-6).  The second
 # layout field is B's: RowMajor = [K][N] weights as the reference's weight files hold them,
 # ColumnMajor = [N][K] (k contiguous, a Hugging Face checkpoint's own orientation).
-DEFAULT_TAG = "128_128_32_64_64_32_1_5_RowMajor_RowMajor_RowMajor"
-DEFAULT_TAG_NK = "128_128_32_64_64_32_1_5_RowMajor_ColumnMajor_RowMajor"
+# cta_m = cta_n = 0 leaves tile and split over K to the kernel layer's cost model; a tag that names a
+# tile (and a split_k) selects the closest tile of the kernel layer's menu for launches of more than
+# 512 live rows.
+DEFAULT_TAG = "0_0_0_0_0_0_1_0_RowMajor_RowMajor_RowMajor"
+DEFAULT_TAG_NK = "0_0_0_0_0_0_1_0_RowMajor_ColumnMajor_RowMajor"
+
+
+def make_tag(tile_m=0, tile_n=0, split_k=1, layout="row") -> str:
+    """A GEMM tag that names a tile and a split over K (0 x 0: the library's choice) for weights in the
+    given layout; the warp and stage fields, which select nothing in this build, are filled with the
+    values the reference's generator would pair with the tile (pipeline/src/generate-gemm/genGEMM.py:57-65)."""
+    b = "ColumnMajor" if layout == "col" else "RowMajor"
+    if not tile_m:
+        return f"0_0_0_0_0_0_{max(split_k, 1)}_0_RowMajor_{b}_RowMajor"
+    return f"{tile_m}_{tile_n}_64_{max(tile_m // 2, 16)}_{max(tile_n // 2, 16)}_64_{max(split_k, 1)}_3_RowMajor_{b}_RowMajor"
 
 
 def tag_weight_layout(tag: str) -> str:

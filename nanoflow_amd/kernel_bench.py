@@ -207,6 +207,8 @@ def main():
     ap.add_argument("--mib", type=int, default=1024, help="copy: MiB moved")
     ap.add_argument("--dtype", default="f16", choices=["f16", "bf16"], help="gemm, dual: element type")
     ap.add_argument("--b-col-major", action="store_true", help="gemm: weights stored [N][K] (k contiguous)")
+    ap.add_argument("--tile", default="", help="gemm: MxN, the tile to run on (the closest of the library's menu) instead of its own choice")
+    ap.add_argument("--split-k", type=int, default=1, help="gemm with --tile: shares K is cut into")
     ap.add_argument("--cold", action="store_true",
                     help="gemm, dual, gemm_f8, dual_f8, blas: cycle through 1 GiB of weight copies so that every launch streams its weights from HBM")
     ap.add_argument("--ws", action="store_true", help="gemm: the entry point with a workspace (split over K where it pays)")
@@ -232,7 +234,11 @@ def main():
                 A = rnd(M, Kd).to(edt)
                 B = (rnd(N, Kd, std=0.02) if a.b_col_major else rnd(Kd, N, std=0.02)).to(edt)
                 Bs = cold_copies(B, a.cold)
-                if a.ws:
+                if a.tile:
+                    tm, tn = (int(v) for v in a.tile.lower().split("x"))
+                    ws = torch.empty((max(K.lib().nf_gemm_tiled_workspace_bytes(M, N, Kd, a.split_k), 16),), dtype=torch.uint8, device=DEV)
+                    fn = lambda: K.gemm_tiled(A, next(Bs), (tm, tn), a.split_k, b_col_major=a.b_col_major, out=out, workspace=ws)
+                elif a.ws:
                     ws = torch.empty((max(K.lib().nf_gemm_workspace_bytes(M, N, Kd), 16),), dtype=torch.uint8, device=DEV)
                     fn = lambda: K.gemm_ws(A, next(Bs), out=out, b_col_major=a.b_col_major, workspace=ws)
                 else:

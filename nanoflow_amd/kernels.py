@@ -26,6 +26,7 @@ SYMBOLS = [
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
     "nf_calibrate_mfma", "nf_calibrate_hbm_read", "nf_calibrate_paged_read",
     "nf_gemm_f16_noalloc", "nf_gemm_noalloc_scratch_bytes",
+    "nf_gemm_tile_menu", "nf_gemm_tiled_workspace_bytes", "nf_gemm_f16_tiled",
     "nf_rmsnorm_quantize_e4m3", "nf_gemm_f8q_f16", "nf_dual_swiglu_f8q_f16",
 ]
 
@@ -87,6 +88,11 @@ def lib() -> C.CDLL:
         l.nf_gemm_f16_noalloc.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_gemm_noalloc_scratch_bytes.restype = sz
         l.nf_gemm_noalloc_scratch_bytes.argtypes = []
+        ip = C.POINTER(C.c_int)
+        l.nf_gemm_tile_menu.argtypes = [i32, ip, ip, ip]
+        l.nf_gemm_tiled_workspace_bytes.restype = sz
+        l.nf_gemm_tiled_workspace_bytes.argtypes = [i32, i32, i32, i32]
+        l.nf_gemm_f16_tiled.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, i32, i32, i32, i32, vp, sz, vp]
         dp = C.POINTER(C.c_double)
         l.nf_calibrate_mfma.argtypes = [i32, i32, i32, vp, sz, dp, dp, vp]
         l.nf_calibrate_hbm_read.argtypes = [vp, sz, i32, vp, sz, dp, vp]
@@ -98,7 +104,7 @@ def lib() -> C.CDLL:
         l.nf_argmax_f16.argtypes = [vp, vp, vp, i32, i32, vp]
         for name in SYMBOLS:
             if name not in ("nf_last_error", "nf_attention_workspace_bytes", "nf_gemm_workspace_bytes",
-                            "nf_gemm_workspace_bytes_upto", "nf_gemm_f8w_workspace_bytes",
+                            "nf_gemm_workspace_bytes_upto", "nf_gemm_f8w_workspace_bytes", "nf_gemm_tiled_workspace_bytes",
                             "nf_dual_swiglu_workspace_bytes", "nf_dual_swiglu_workspace_bytes_upto",
                             "nf_gemm_f8w_split_workspace_bytes", "nf_gemm_f8w_split_workspace_bytes_upto",
                             "nf_dual_swiglu_f8w_split_workspace_bytes", "nf_dual_swiglu_f8w_split_workspace_bytes_upto"):
@@ -214,6 +220,34 @@ def gemm_ws(A, B, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, w
     _check(lib().nf_gemm_f16_ws(_p(A), _p(B), _p(Cmat), _p(out), M, N, K, alpha, beta, int(b_col_major),
                                 _p(workspace), workspace.numel(), _stream()), "nf_gemm_f16_ws")
     return out, need
+
+
+def gemm_tile_menu():
+    """[(tile_m, tile_n, takes k-contiguous weights only)] of the tiles nf_gemm_f16_tiled chooses from."""
+    m, n, c = C.c_int(), C.c_int(), C.c_int()
+    out = []
+    for i in range(lib().nf_gemm_tile_menu(-1, None, None, None)):
+        lib().nf_gemm_tile_menu(i, C.byref(m), C.byref(n), C.byref(c))
+        out.append((m.value, n.value, bool(c.value)))
+    return out
+
+
+def gemm_tiled(A, B, tile, split_k=1, Cmat=None, alpha=1.0, beta=0.0, b_col_major=False, out=None, bias=None,
+               workspace=None):
+    """nf_gemm_f16_tiled: the GEMM on the menu tile closest to ``tile`` = (m, n), K cut into ``split_k`` shares."""
+    _f16(A); _f16(B)
+    M, K = A.shape
+    N = B.shape[0] if b_col_major else B.shape[1]
+    assert tuple(B.shape) == ((N, K) if b_col_major else (K, N))
+    need = lib().nf_gemm_tiled_workspace_bytes(M, N, K, split_k)
+    if workspace is None:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=A.device)
+    out = torch.empty((M, N), dtype=torch.float16, device=A.device) if out is None else out
+    c = bias if bias is not None else Cmat
+    _check(lib().nf_gemm_f16_tiled(_p(A), _p(B), _p(c), _p(out), M, N, K, alpha, beta, int(b_col_major),
+                                   int(bias is not None), tile[0], tile[1], split_k, _p(workspace), workspace.numel(),
+                                   _stream()), "nf_gemm_f16_tiled")
+    return out
 
 
 def dual_swiglu_ws(A, Bg, Bu, out=None, workspace=None, b_col_major=False):

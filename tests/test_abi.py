@@ -68,10 +68,16 @@ def test_split_over_k_plan_without_a_gpu():
     assert shares(321, 4096, 4096) == 0           # above 320 rows only long contractions are split
     assert shares(400, 4096, 14336) == 8          # two 256-row tiles per 256 columns: 32 tiles
     assert shares(513, 4096, 4096) == 0           # more than 512 rows
+    assert shares(2048, 4096, 14336) == 2         # dense rows, 128 tiles of 256 x 256 against a long contraction: two shares
+    assert shares(1500, 4096, 14336) == 2 and shares(1024, 4096, 14336) == 0    # 96 tiles; 64 tiles: a quarter of the CUs
+    assert shares(2048, 4096, 4096) == 0 and shares(2048, 8192, 28672) == 0     # too shallow; tiles enough
     assert shares(64, 128256, 4096) == 0          # the LM head has tiles enough
     assert shares(64, 4096, 512) == 0             # too shallow
     assert l.nf_gemm_workspace_bytes_upto(2048, 6144, 4096) == max(l.nf_gemm_workspace_bytes(m, 6144, 4096)
                                                                    for m in range(1, 513))
+    assert l.nf_gemm_workspace_bytes_upto(2048, 4096, 14336) == 2 * 2048 * 4096 * 4
+    assert l.nf_gemm_workspace_bytes_upto(1400, 4096, 14336) == max(l.nf_gemm_workspace_bytes(m, 4096, 14336)
+                                                                    for m in range(1, 1401))
     dual = lambda M, N, K: l.nf_dual_swiglu_workspace_bytes(M, N, K) // (2 * M * N * 4)
     assert dual(64, 14336, 4096) == 2 and dual(64, 28672, 8192) == 0 and dual(256, 14336, 4096) == 0
     assert l.nf_gemm_f8w_workspace_bytes(2048, 4096) == 2048 * 4096 + 2048 * 4

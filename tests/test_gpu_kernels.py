@@ -268,6 +268,61 @@ def test_dual_swiglu_split_over_k_matches_oracle(K, oracle, M, N, K_):
     assert need == 0
 
 
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("M,N,K_", [(2048, 4096, 14336), (1500, 4088, 8200)])
+def test_gemm_dense_rows_split_in_two_over_a_long_contraction(K, oracle, M, N, K_, b_col):
+    """More than 512 rows whose 256 x 256 tiles fill half the chip or less against K >= 8192 (the 8B down
+    projection) run as two shares of K when the caller brings the workspace: against the oracle, with
+    the residual operand; without the workspace the unsplit launch runs."""
+    rng = np.random.default_rng(M + K_)
+    A = synth.normal_f16(rng, (M, K_))
+    B = synth.normal_f16(rng, (K_, N), 0.02)
+    Cm = synth.normal_f16(rng, (M, N))
+    dB = dev(np.ascontiguousarray(B.T)) if b_col else dev(B)
+    ref = oracle.gemm(A, B, Cm, 1.0, 1.0)
+    got, need = K.gemm_ws(dev(A), dB, dev(Cm), 1.0, 1.0, b_col_major=b_col)
+    assert need == 2 * M * N * 4, "this shape is meant to be split in two"
+    assert_close(host(got), ref, what="dense split-K")
+    plain = K.gemm(dev(A), dB, dev(Cm), 1.0, 1.0, b_col_major=b_col)
+    assert_close(host(plain), ref, what="unsplit")
+    short, _ = K.gemm_ws(dev(A), dB, dev(Cm), 1.0, 1.0, b_col_major=b_col, workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+    assert np.array_equal(host(short), host(plain))
+
+
+@pytest.mark.parametrize("b_col", [False, True])
+@pytest.mark.parametrize("M,N,K_", [(640, 1160, 264), (513, 6144, 512), (37, 520, 200), (2048, 4096, 448)])
+def test_gemm_on_a_caller_chosen_tile_and_split(K, oracle, M, N, K_, b_col):
+    """nf_gemm_f16_tiled -- what a GEMM tag's cta_m x cta_n and split_k select -- on every tile of the
+    menu, unsplit and cut into 2 and 3 shares of K, both weight layouts, with M / N / K tails, the
+    residual operand and the bias row: against the oracle.  A tile that is not in the menu runs on
+    the closest one; a split without its workspace is refused."""
+    from nanoflow_amd import kernels
+    rng = np.random.default_rng(M + N + K_)
+    A = synth.normal_f16(rng, (M, K_))
+    B = synth.normal_f16(rng, (K_, N), 0.05)
+    Cm = synth.normal_f16(rng, (M, N))
+    bias = synth.normal_f16(rng, (N,))
+    dB = dev(np.ascontiguousarray(B.T)) if b_col else dev(B)
+    ref = oracle.gemm(A, B, Cm, 1.0, 1.0)
+    ref_bias = oracle.gemm(A, B, np.ascontiguousarray(np.broadcast_to(bias, (M, N))), 1.0, 1.0)
+    menu = K.gemm_tile_menu()
+    assert (256, 256, False) in menu and (128, 256, False) in menu and (256, 192, True) in menu and len(menu) >= 5
+    for tm, tn, col_only in menu:
+        for split in (1, 2, 3):
+            got = host(K.gemm_tiled(dev(A), dB, (tm, tn), split, Cmat=dev(Cm), beta=1.0, b_col_major=b_col))
+            assert_close(got, ref, what=f"tile {tm}x{tn} split {split} {'[N][K]' if b_col else '[K][N]'}")
+        got = host(K.gemm_tiled(dev(A), dB, (tm, tn), 2, bias=dev(bias), beta=1.0, b_col_major=b_col))
+        assert_close(got, ref_bias, what=f"tile {tm}x{tn} with a bias row")
+    # 100 x 100 is not in the menu: the closest entry (128 x 128) runs, with the same bits
+    assert np.array_equal(host(K.gemm_tiled(dev(A), dB, (100, 100), 1, b_col_major=b_col)),
+                          host(K.gemm_tiled(dev(A), dB, (128, 128), 1, b_col_major=b_col)))
+    assert K.lib().nf_gemm_tiled_workspace_bytes(M, N, K_, 1) == 0
+    k_per = -(-(-(-K_ // 3)) // 64) * 64                   # a share is a whole number of 64-deep slabs
+    assert K.lib().nf_gemm_tiled_workspace_bytes(M, N, K_, 3) == -(-K_ // k_per) * M * N * 4
+    with pytest.raises(kernels.NanoflowKernelError, match="workspace"):
+        K.gemm_tiled(dev(A), dB, (128, 128), 2, b_col_major=b_col, workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+
+
 @pytest.mark.parametrize("M,N,K_", [(5, 136, 72), (64, 14336, 256), (200, 1160, 264), (267, 24584, 328), (300, 14336, 1024),
                                     (16, 14336, 4096), (2048, 14336, 256), (1992, 14328, 200), (1792, 28672, 128)])
 def test_dual_swiglu_with_k_contiguous_weights(K, oracle, M, N, K_):

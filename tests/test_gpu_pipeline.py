@@ -953,3 +953,40 @@ def test_k_contiguous_weights_give_the_same_results_on_every_schedule(oracle, pt
     mixed = [engine.DEFAULT_TAG_NK] + [engine.DEFAULT_TAG] * (pt.gemm_tags - 1)
     with pytest.raises(ValueError, match="disagree"):
         engine.Engine(shape, pt, global_batch=T, nano1=nano1, kv_pages=b1.num_pages, gemm_tags=mixed)
+
+
+@pytest.mark.parametrize("pt_name,layout", [("NON_OVERLAP_LOCAL", "col"), ("NON_OVERLAP_LOCAL", "row"), ("PLLM", "col")])
+def test_gemm_tags_select_tile_and_split(oracle, pt_name, layout):
+    """Tags that name a tile and a split over K (the reference's cta_m x cta_n and split_k fields) against
+    tags that leave both to the library, on an iteration of more than 512 rows (below that a launch
+    keeps the few-row plan whatever the tag says): the residual stream and the logits agree with the
+    oracle either way and with each other to summation order."""
+    from nanoflow_amd import engine, pllm_python as P
+    pt = P.PipelineType[pt_name]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=0)
+    T, nano1 = 1280, 640
+    b1 = synth.make_batch(list(range(3, 43)), [(0, 700), (16, 537)], vocab=shape.vocab, seed=21, extra_pages=40)
+    assert 1270 < b1.tokens <= T
+    rng = np.random.default_rng(5)
+    pools0 = [synth.make_kv_pool(b1.num_pages, shape, rng) for _ in range(shape.layers)]
+    tok1 = b1.input_tokens.copy()
+    tok1[:b1.decodePrefillBorder] = 1
+    d1 = b1.as_dict()
+    d1["input_tokens"] = tok1
+    hid, log, _ = oracle.decoder_forward(shape.as_dict(), w, [p.copy() for p in pools0], d1, want_logits=True)
+    tiles = [(128, 128, 2), (256, 256, 1), (64, 256, 3), (128, 256, 1), (256, 192 if layout == "col" else 256, 2),
+             (128, 128, 1), (256, 256, 2), (64, 256, 1)]
+    n = pt.gemm_tags
+    named = [engine.make_tag(*tiles[i % len(tiles)], layout=layout) for i in range(n - 1)] + [engine.make_tag(128, 256, 1, layout)]
+    auto = [engine.make_tag(layout=layout)] * n
+    out = {}
+    for name, tags in (("auto", auto), ("named", named)):
+        print(f"pipeline={pt_name} layout={layout} tags {name}", flush=True)
+        with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=600, kqv3=620, kv_pages=b1.num_pages, weights=w,
+                           kv_pools=pools0, gemm_tags=tags) as e:
+            e.update(b1, keep_token_list=np.ones(b1.decodePrefillBorder, np.int32))
+            e.run()
+            out[name] = (e.buffer("hidden").cpu().numpy()[:b1.tokens], e.buffer("logits").cpu().numpy()[:b1.req_num])
+        assert _max_rel(out[name][0], hid) < E2E_RTOL and _max_rel(out[name][1], log) < E2E_RTOL, (pt_name, name)
+    assert _max_rel(out["named"][0], out["auto"][0]) < 2e-3
