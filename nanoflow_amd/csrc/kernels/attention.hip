@@ -32,11 +32,21 @@ union H8 {
   uint32_t w[4];
 };
 
-// tile_start[i] = number of tiles of requests < i; tile_start[batch] = total.
+// Tile plan of a chunked-prefill launch, made on the device (no host round trip):
+//   tile_start[i] = number of query tiles (wg_tok tokens each) of requests < i; tile_start[batch] = total;
+//   tile_order[k] = the tile that workgroup slot k computes: tiles in descending order of the keys
+//   they see.  A causal chunk's last tile sees the whole context and its first tile only what came
+//   before the chunk, and a launch is over when its longest tile is, so the long tiles start first
+//   and the short ones fill in behind them.  (Ranked by counting, at most kPlanSortMax tiles;
+//   beyond that tiles keep their order.)
+constexpr int kPlanSortMax = 1024;
 __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restrict__ qo_indptr,
-                                                        int32_t* __restrict__ tile_start, int batch,
-                                                        int wg_tok) {
+                                                        const int32_t* __restrict__ kv_indptr,
+                                                        const int32_t* __restrict__ kv_last_page_len,
+                                                        int32_t* __restrict__ tile_start, int32_t* __restrict__ tile_order,
+                                                        int batch, int wg_tok, int causal) {
   __shared__ int s_sum[256];
+  __shared__ int s_key[kPlanSortMax];
   const int per = (batch + 255) / 256;
   const int lo = threadIdx.x * per, hi = min(lo + per, batch);
   int sum = 0;
@@ -54,11 +64,32 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restric
     __syncthreads();
   }
   int run = s_sum[threadIdx.x] - sum;  // exclusive prefix of this thread's range
-  if (threadIdx.x == 255) tile_start[batch] = s_sum[255];
+  const int total = s_sum[255];
+  if (threadIdx.x == 255) tile_start[batch] = total;
   for (int i = lo; i < hi; ++i) {
     tile_start[i] = run;
-    int len = qo_indptr[i + 1] - qo_indptr[i];
-    run += len > 0 ? (len + wg_tok - 1) / wg_tok : 0;
+    const int len = qo_indptr[i + 1] - qo_indptr[i];
+    const int n = len > 0 ? (len + wg_tok - 1) / wg_tok : 0;
+    if (total <= kPlanSortMax) {  // keys the request's tiles see
+      const int npages = kv_indptr[i + 1] - kv_indptr[i];
+      const int kv_len = npages > 0 ? (npages - 1) * PAGE + kv_last_page_len[i] : 0;
+      for (int t = 0; t < n; ++t) {
+        const int last = min((t + 1) * wg_tok, len) - 1;
+        s_key[run + t] = causal ? min(kv_len, kv_len - len + last + 1) : kv_len;
+      }
+    }
+    run += n;
+  }
+  __syncthreads();
+  if (total > kPlanSortMax) {
+    for (int t = threadIdx.x; t < total; t += 256) tile_order[t] = t;
+    return;
+  }
+  for (int t = threadIdx.x; t < total; t += 256) {
+    const int key = s_key[t];
+    int rank = 0;
+    for (int u = 0; u < total; ++u) rank += (s_key[u] > key) || (s_key[u] == key && u < t);
+    tile_order[rank] = t;
   }
 }
 
@@ -343,31 +374,55 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_decode_kernel(
   }
 }
 
-// Chunked-prefill attention (causal, many rows per request).  A workgroup is one tile of
-// 4 * NQB * (16 / GROUP) query tokens of one request and one kv head; each wavefront owns
-// NQB column blocks of it.  The K and V pages are streamed ONCE per workgroup, straight into
-// two LDS stages (32 keys x 256 bytes each for K and for V) that all four wavefronts read:
-// every wavefront issues a quarter of a tile's load instructions, waits for its own, and one
-// barrier per 32-key step makes the tile visible and frees the other stage for the next loads.
-// LDS layout and operand reads are those of attn_decode_kernel.  Wavefronts whose tokens cannot
-// see a step's keys (causal) skip its MFMAs but keep loading and meeting at the barrier.
-// LDS stages of 32 keys (K + V: 16 KB each).  Two: the loads of step pp+1 fly while step pp is
-// computed, and four workgroups fit a CU and cover each other's waits.  Four stages (two
-// workgroups per CU) measured 10-19 % slower on chunks of 256 to 1024 tokens.
-constexpr int kPrefillStages = 2;
-static_assert(kPrefillStages >= 2 && kPrefillStages <= 4, "the kernel's waits count at most two younger steps");
+// max over the four 16-lane groups of a wavefront (lanes c, c + 16, c + 32, c + 48), in every lane:
+// two lane-swap instructions (v_permlane32_swap, v_permlane16_swap: gfx950) and two maxima on the
+// vector unit, where a shuffle would make two round trips through the LDS crossbar.
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+  const auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float sum_over_lane_groups(float v) {
+  const auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
 
-template <int GROUP, int NQB>
-__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
+// Chunked-prefill attention (causal, many rows per request).  A workgroup is one tile of
+// 4 * NQB * (16 / GROUP) query tokens of one request and one kv head; each wavefront owns NQB
+// blocks of 16 MFMA columns of it (a column = one token and one q head of the kv head's group).
+// The K and V pages are streamed ONCE per workgroup, straight into a ring of NSTAGE LDS stages
+// (32 keys x 256 bytes each for K and for V) that all four wavefronts read: every wavefront
+// issues a quarter of a stage's load instructions, waits for its own, and one barrier per 32-key
+// step makes the stage visible and frees the oldest one for the next loads.  LDS layout and
+// operand reads are those of attn_decode_kernel.
+//
+// What bounds it is the LDS read port and the vector unit, not the matrix pipe: a step's K and V
+// fragments (8 + 16 LDS reads per wavefront) feed 16 MFMAs per column block, and every score costs
+// a maximum, a fused multiply-add, an exponential, an addition and half a conversion on the vector
+// unit.  So a wavefront keeps NQB column blocks in registers and reuses each fragment NQB times,
+// the scale is folded into the exponent (p = exp2(s * scale - m * scale): one instruction), maxima
+// are reduced across lane groups with lane swaps instead of shuffles, and MINWG workgroups share a
+// CU so that one wavefront's exponentials run under another's MFMAs.  Steps that lie wholly below
+// the causal limit of a wavefront's first token need no masks (most steps of a long chunk);
+// wavefronts whose tokens cannot see a step's keys skip its arithmetic but keep loading and
+// meeting at the barrier.  Workgroup slot k computes tile tile_order[k / Hkv] for kv head k % Hkv:
+// long tiles first (attn_plan_kernel), the heads of a tile side by side so that they find each
+// other's pages in the L2.
+template <int GROUP, int NQB, int NSTAGE, int MINWG>
+__global__ __launch_bounds__(256, MINWG) void attn_prefill_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ o, const int32_t* __restrict__ qo_indptr,
     const uint16_t* __restrict__ kv_data, const int32_t* __restrict__ kv_indptr,
     const int32_t* __restrict__ kv_indices, const int32_t* __restrict__ kv_last_page_len,
-    const int32_t* __restrict__ tile_start, int batch, int Hq, int Hkv, int causal, float scale_log2) {
+    const int32_t* __restrict__ tile_start, const int32_t* __restrict__ tile_order, int batch, int Hq, int Hkv,
+    int causal, float scale_log2) {
+  static_assert(NSTAGE >= 2 && NSTAGE <= 4, "the waits below count at most two younger steps");
   constexpr int TPB = 16 / GROUP;
   constexpr int WAVE_TOK = NQB * TPB;
   constexpr int WG_TOK = 4 * WAVE_TOK;
   constexpr int STAGE = 16384;  // K tile 8 KB + V tile 8 KB
-  constexpr int NSTAGE = kPrefillStages;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
@@ -386,9 +441,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
   for (int i = 0; i < 8; ++i)
     vx[i] = (uint32_t)((g * 4 + (i16 >> 2)) * 256 + ((i ^ vx_x) * 32) + (i16 & 3) * 8);
 
+  const float lazy_raw = 8.0f / scale_log2;  // 2^8 in units of the unscaled scores
   const int total_tiles = tile_start[batch];
   for (long long w = blockIdx.x; w < (long long)total_tiles * Hkv; w += gridDim.x) {
-    const int tile = (int)(w / Hkv), kvh = (int)(w % Hkv);
+    const int tile = tile_order[(int)(w / Hkv)], kvh = (int)(w % Hkv);
     int lo = 0, hi = batch;  // request = largest i with tile_start[i] <= tile
     while (hi - lo > 1) {
       int mid = (lo + hi) >> 1;
@@ -419,7 +475,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     }
 
     float4_t oacc[NQB][8];
-    float m_run[NQB], l_run[NQB];
+    float m_run[NQB], l_run[NQB];  // running maximum of the UNSCALED scores; partial row sums per lane
     H8 qf[NQB][4];
     int key_limit[NQB];
 #pragma unroll
@@ -444,9 +500,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
     const int wave_end = !wave_active ? 0 : (causal ? min(kv_len, kv_len - qo_len + wave_last + 1) : kv_len);
     const int npairs = (wg_end + 31) >> 5;
 
+    // The page ids of 64 steps live in one register (lane i: the page this wavefront loads in step
+    // pg_base + i), refilled every 64 steps, and a step's id is read from its lane: a scalar load per
+    // step would put a trip to the scalar cache in front of every group of tile loads, and its wait
+    // (scalar loads return out of order) would also wait for every LDS read in flight.
+    int pg_base = 0;
+    int pg_reg = 0;
+    auto load_pages = [&](int base) {
+      const int pidx = 2 * (base + lane) + (wave >> 1);  // waves 0,1 load the first page of a step, 2,3 the second
+      pg_reg = kv_indices[pg0 + (pidx < npages ? pidx : 0)];
+      pg_base = base;
+    };
     auto dma = [&](int pp, int stage) {
-      const int pidx = 2 * pp + (wave >> 1);  // waves 0,1 load the first page of the step, 2,3 the second
-      const int page = kv_indices[pg0 + (pidx < npages ? pidx : 0)];
+      if (pp >= pg_base + 64) {
+        load_pages(pg_base + 64);
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(pg_reg)::"memory");  // once per 64 steps: the ring drains here
+      }
+      const int page = __builtin_amdgcn_readlane(pg_reg, pp - pg_base);
       const rsrc_t r = make_rsrc(kv_data + (size_t)page * (page_bytes / 2), page_bytes);
       const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + stage * STAGE + wave * 2048);
 #pragma unroll
@@ -455,112 +525,167 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
       for (int e = 0; e < 2; ++e)  // rows past the end of the sequence are zero-filled
         load16_to_lds(r, pp * 32 + key_in_step[e] < kv_len ? v_src[e] : kOob, dst + 8192 + e * 1024);
     };
+    load_pages(0);
+    // (named in the wait so that the compiler takes the register for defined here, not by a load it
+    // would wait for again, with everything else in flight, at every use inside the loop)
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(pg_reg)::"memory");
 
     __syncthreads();  // the previous work item's reads of every stage are done
-    // Step pp lives in stage pp % NSTAGE; the loads of steps pp+1 .. pp+NSTAGE-2 are in flight
-    // while step pp is computed (a load from HBM takes several steps' worth of arithmetic).
+    // Step pp lives in stage pp % NSTAGE.  The loop is software-pipelined by one step: while the
+    // vector unit works through the softmax of step pp, the matrix pipe still runs the P.V MFMAs of
+    // step pp-1, and the score MFMAs of step pp+1 are issued before the P.V MFMAs of step pp, so
+    // that the next softmax can start as soon as the scores are there.  Iteration pp therefore
+    // reads the fragments of step pp+1; the stage of step pp is free after its barrier, and the
+    // loads of step pp+NSTAGE go there (NSTAGE-1 steps ahead of the stage being read).
 #pragma unroll
     for (int p = 0; p < NSTAGE - 1; ++p)
       if (p < npairs) dma(p, p);
-    int st = 0;  // pp % NSTAGE
-    for (int pp = 0; pp < npairs; ++pp) {
-      const int t_base = pp * 32;
-      // this wavefront's share of step pp has landed: all but the 4 loads of each younger step
-      const int younger = min(NSTAGE - 2, npairs - 1 - pp);
+    // the compiler sees the Q loads but not the tile loads: make it wait for Q once, here, instead of
+    // with vmcnt(0) where Q is first used inside the loop (which would drain the ring every step)
+#pragma unroll
+    for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) asm volatile("" ::"v"(qf[nb][j].w[0]));
+    const int n_active = (wave_end + 31) >> 5;  // steps whose keys this wavefront's tokens can see: the first n_active
+
+    half8_t kf[2][4], vf[8];
+    float4_t s[NQB][2];
+    auto wait_step = [&](int step) {  // this wavefront's loads of `step` have landed: all but the 4 of each younger step
+      const int younger = min(NSTAGE - 2, npairs - 1 - step);
       if (younger >= 2) __builtin_amdgcn_s_waitcnt(0x0F78);       // vmcnt(8)
       else if (younger == 1) __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
       else __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0)
-      __syncthreads();  // ... and everybody else's; the stage step pp-1 was read from is free
-      if (pp + NSTAGE - 1 < npairs) dma(pp + NSTAGE - 1, st == 0 ? NSTAGE - 1 : st - 1);
-      const uint8_t* kt = lds + st * STAGE;
-      st = st + 1 == NSTAGE ? 0 : st + 1;
-      if (t_base >= wave_end) continue;    // nothing visible to this wavefront in this step
-      const uint8_t* vt = kt + 8192;
-
-      half8_t kf[2][4];
+    };
+    auto read_k = [&](const uint8_t* kt) {
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
         for (int j = 0; j < 4; ++j) kf[blk][j] = *reinterpret_cast<const half8_t*>(kt + blk * 4096 + kx[j]);
-      float4_t s[NQB][2];
-#pragma unroll
-      for (int nb = 0; nb < NQB; ++nb)
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-          s[nb][blk] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            s[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[blk][j], qf[nb][j].h, s[nb][blk], 0, 0, 0);
-        }
-      H8 pf[NQB];
-      float alpha[NQB];
-      // Steps that lie wholly below the causal limit of the wavefront's first token (and inside
-      // the sequence) need no masks: most steps of a long chunk.  Same arithmetic either way.
-      const bool unmasked = t_base + 31 <= (causal ? kv_len - qo_len + tok0 : kv_len - 1);
-      auto softmax_step = [&](auto masked_c) {
-        constexpr bool kMasked = decltype(masked_c)::value;
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-          float mx = -1e30f;
-          bool ok[2][4];
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int t = t_base + blk * 16 + g * 4 + r;
-              ok[blk][r] = !kMasked || (t <= key_limit[nb] && t < kv_len);
-              s[nb][blk][r] *= scale_log2;
-              if (ok[blk][r]) mx = fmaxf(mx, s[nb][blk][r]);
-            }
-          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-          const float m_new = fmaxf(m_run[nb], mx);
-          alpha[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_new);
-          m_run[nb] = m_new;
-          float psum = 0.f;
-          uint32_t pw[4];
-#pragma unroll
-          for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int rr = 0; rr < 2; ++rr) {
-              float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr] - m_new) : 0.f;
-              float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(s[nb][blk][2 * rr + 1] - m_new) : 0.f;
-              psum += p0 + p1;
-              pw[blk * 2 + rr] = pack_f16x2(p0, p1);
-            }
-          pf[nb].u = u32x4{pw[0], pw[1], pw[2], pw[3]};
-          l_run[nb] = l_run[nb] * alpha[nb] + psum;
-        }
-      };
-      if (unmasked) softmax_step(std::false_type{});
-      else softmax_step(std::true_type{});
-      // the running maximum settles after a few steps: rescale the accumulators only when some
-      // column's maximum moved (multiplying by exactly 1 changes nothing)
-      bool moved = false;
-#pragma unroll
-      for (int nb = 0; nb < NQB; ++nb) moved |= alpha[nb] != 1.0f;
-      const bool rescale = __builtin_amdgcn_ballot_w64(moved) != 0;
+    };
+    auto read_v = [&](const uint8_t* vt) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const short4_t vlo = lds_read_tr16(vt + vx[i]);
         const short4_t vhi = lds_read_tr16(vt + vx[i] + 4096);
         typedef short short8_t __attribute__((ext_vector_type(8)));
-        const half8_t v8 = __builtin_bit_cast(half8_t, __builtin_shufflevector(vlo, vhi, 0, 1, 2, 3, 4, 5, 6, 7));
-#pragma unroll
-        for (int nb = 0; nb < NQB; ++nb) {
-          if (rescale) oacc[nb][i] *= alpha[nb];
-          oacc[nb][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v8, pf[nb].h, oacc[nb][i], 0, 0, 0);
-        }
+        vf[i] = __builtin_bit_cast(half8_t, __builtin_shufflevector(vlo, vhi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
+    };
+    // 2 * NQB independent accumulators, the k-chunks outermost: no MFMA waits for the one before it
+    auto scores = [&]() {
+#pragma unroll
+      for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) s[nb][blk] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int nb = 0; nb < NQB; ++nb)
+            s[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[blk][j], qf[nb][j].h, s[nb][blk], 0, 0, 0);
+    };
+
+    if (npairs > 0) {  // step 0
+      wait_step(0);
+      __syncthreads();
+      if (NSTAGE - 1 < npairs) dma(NSTAGE - 1, NSTAGE - 1);
+      if (n_active > 0) {
+        read_k(lds);
+        read_v(lds + 8192);
+        scores();
+      }
+    }
+    int st = 0;  // pp % NSTAGE
+    for (int pp = 0; pp < npairs; ++pp) {
+      const int t_base = pp * 32;
+      const bool next = pp + 1 < npairs, act = pp < n_active, act_next = pp + 1 < n_active;
+      const int st_next = st + 1 == NSTAGE ? 0 : st + 1;
+      if (next) {
+        wait_step(pp + 1);
+        __syncthreads();  // step pp+1 is visible to everybody, and nobody reads the stage of step pp any more
+        if (pp + NSTAGE < npairs) dma(pp + NSTAGE, st);
+      }
+      if (act) {
+        H8 pf[NQB];
+        float alpha[NQB];
+        float4_t sc[NQB][2];  // the scores of this step; s is about to take those of the next
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+          for (int blk = 0; blk < 2; ++blk) sc[nb][blk] = s[nb][blk];
+        if (act_next) read_k(lds + st_next * STAGE);  // on their way while the vector unit works
+        // Steps that lie wholly below the causal limit of the wavefront's first token (and inside
+        // the sequence) need no masks: most steps of a long chunk.  Same arithmetic either way.
+        const bool unmasked = t_base + 31 <= (causal ? kv_len - qo_len + tok0 : kv_len - 1);
+        auto softmax_step = [&](auto masked_c) {
+          constexpr bool kMasked = decltype(masked_c)::value;
+#pragma unroll
+          for (int nb = 0; nb < NQB; ++nb) {
+            // a lane holds keys t_base + blk*16 + g*4 + r of column c16
+            float mx = -1e30f;
+            bool ok[2][4];
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int t = t_base + blk * 16 + g * 4 + r;
+                ok[blk][r] = !kMasked || (t <= key_limit[nb] && t < kv_len);
+                if (ok[blk][r]) mx = fmaxf(mx, sc[nb][blk][r]);
+              }
+            mx = max_over_lane_groups(mx);
+            // The reference maximum follows the true one lazily: it moves only when a score exceeds it
+            // by more than 2^8 after scaling, so p = exp2(...) stays below 256 (fp16 holds that with its
+            // full relative precision, the sums are fp32) and the accumulators are rescaled once or twice
+            // per tile instead of in most steps.  O / l is the same quotient either way.
+            const float m_new = mx > m_run[nb] + lazy_raw ? mx : m_run[nb];
+            alpha[nb] = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);
+            m_run[nb] = m_new;
+            const float shift = -m_new * scale_log2;
+            float psum = 0.f;
+            uint32_t pw[4];
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+              for (int rr = 0; rr < 2; ++rr) {
+                float p0 = ok[blk][2 * rr] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sc[nb][blk][2 * rr], scale_log2, shift)) : 0.f;
+                float p1 = ok[blk][2 * rr + 1] ? __builtin_amdgcn_exp2f(__builtin_fmaf(sc[nb][blk][2 * rr + 1], scale_log2, shift)) : 0.f;
+                psum += p0 + p1;  // the row sum uses the unrounded values, P.V the fp16 ones
+                pw[blk * 2 + rr] = pack_f16x2(p0, p1);
+              }
+            pf[nb].u = u32x4{pw[0], pw[1], pw[2], pw[3]};
+            l_run[nb] = l_run[nb] * alpha[nb] + psum;
+          }
+        };
+        if (unmasked) softmax_step(std::false_type{});
+        else softmax_step(std::true_type{});
+        if (act_next) scores();
+        bool moved = false;
+#pragma unroll
+        for (int nb = 0; nb < NQB; ++nb) moved |= alpha[nb] != 1.0f;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+          // a branch of its own: folded into the MFMA loop it becomes a multiply and a select per register and step
+#pragma unroll
+          for (int nb = 0; nb < NQB; ++nb)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) oacc[nb][i] *= alpha[nb];
+          asm volatile("" ::: "memory");
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int nb = 0; nb < NQB; ++nb)
+            oacc[nb][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[i], pf[nb].h, oacc[nb][i], 0, 0, 0);
+        if (act_next) read_v(lds + st_next * STAGE + 8192);
+      }
+      st = st_next;
     }
 
     // oacc[nb][i][r] = O[column c16][feature 16i + 4g + r]
     if (wave_active) {
 #pragma unroll
       for (int nb = 0; nb < NQB; ++nb) {
-        float l = l_run[nb];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        const float l = sum_over_lane_groups(l_run[nb]);
         const int tq = tok0 + nb * TPB + c16 / GROUP;
         if (tq >= qo_len) continue;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
@@ -568,8 +693,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           u32x2 out;
-          out.x = f2h_bits(oacc[nb][i][0] * inv) | (f2h_bits(oacc[nb][i][1] * inv) << 16);
-          out.y = f2h_bits(oacc[nb][i][2] * inv) | (f2h_bits(oacc[nb][i][3] * inv) << 16);
+          out.x = pack_f16x2(oacc[nb][i][0] * inv, oacc[nb][i][1] * inv);
+          out.y = pack_f16x2(oacc[nb][i][2] * inv, oacc[nb][i][3] * inv);
           *reinterpret_cast<u32x2*>(op + 16 * i + 4 * g) = out;
         }
       }
@@ -588,13 +713,20 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
   // Decode mode (KV split over the wavefronts, one workgroup per request and kv head) is the
   // right shape when requests carry about one row each; it stays correct for any row count.
   const bool decode_mode = max_qo_rows <= batch;
-  constexpr int NQB_PREFILL = 1;
+  // Measured on chunks of 256 to 2048 tokens (alone, and the prefill chunks of a steady-state serving
+  // cycle): one column block per wavefront (16-token tiles for a GQA group of 4) beats two, three and
+  // four by 10-100 % -- a launch is over when its longest tile is, a tile's steps are serial (barrier,
+  // tile loads, fragment reads, 24 MFMAs, softmax), and smaller tiles mean more workgroups to spread
+  // over the CUs and to interleave on one; four LDS stages with two workgroups per CU beat 2 x 2 and 3 x 3.
+  constexpr int NQB_PREFILL = 1, kPrefillStages = 4, kPrefillMinWg = 2;
+  int32_t* tile_order = tile_start + batch + 2;
   long long bound;
   if (decode_mode) {
     bound = (long long)batch * Hkv;
   } else {
     const int wg_tok = 4 * NQB_PREFILL * TPB;
-    attn_plan_kernel<<<1, 256, 0, stream>>>(qo_indptr, tile_start, batch, wg_tok);
+    attn_plan_kernel<<<1, 256, 0, stream>>>(qo_indptr, kv_indptr, kv_last_page_len, tile_start, tile_order, batch,
+                                            wg_tok, causal);
     bound = ((long long)batch + max_qo_rows / wg_tok) * Hkv;
   }
   if (num_blocks > 0 && bound > num_blocks) bound = num_blocks;
@@ -626,7 +758,7 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
     int rc = (long long)batch * Hkv <= 256 ? launch(ic<4>{}) : launch(ic<2>{});
     if (rc) return rc;
   } else {
-    auto kern = attn_prefill_kernel<GROUP, NQB_PREFILL>;
+    auto kern = attn_prefill_kernel<GROUP, NQB_PREFILL, kPrefillStages, kPrefillMinWg>;
     static bool attr_set = false;  // benign race: the call is idempotent
     if (!attr_set) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -638,7 +770,7 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
       attr_set = true;
     }
     kern<<<(int)bound, 256, kPrefillStages * 16384, stream>>>(
-        q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, batch, Hq,
+        q, o, qo_indptr, kv_data, kv_indptr, kv_indices, kv_last_page_len, tile_start, tile_order, batch, Hq,
         Hkv, causal, scale_log2);
   }
   return check_launch("nf_attention_paged_f16");
@@ -651,10 +783,12 @@ using namespace nf;
 extern "C" {
 
 size_t nf_attention_workspace_bytes(int batch, int max_qo_rows, int num_qo_heads) {
-  (void)max_qo_rows;
   (void)num_qo_heads;
   if (batch < 0) batch = 0;
-  return (((size_t)batch + 2) * sizeof(int32_t) + 255) & ~(size_t)255;
+  if (max_qo_rows < 0) max_qo_rows = 0;
+  // tile_start[batch + 1] (+ 1 of padding), then tile_order: a request has at most one tile that is
+  // not full, and a full tile holds at least 8 tokens
+  return (((size_t)batch + 2 + (size_t)batch + (size_t)max_qo_rows / 8 + 2) * sizeof(int32_t) + 255) & ~(size_t)255;
 }
 
 int nf_attention_paged_f16(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
