@@ -22,8 +22,14 @@ Pipeline::Pipeline(vortexInitData* input_data, int nrank, int nranks, int vnrank
                    bool nanobatch_only_, bool kqv_bias_)
     : PipelineBase(input_data, nrank, nranks, vnranks), enable_offload(enable_offload_), nanobatch_only(nanobatch_only_) {
   kqv_bias = kqv_bias_;
-  stream_gemm = createPipelineStream(0, 0);
-  stream_gemv = createPipelineStream(0, 0);
+  // Optional CU partition, as in LocalPipeline: dense operators on CUs [0, g), attention on [g, g + a)
+  // (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS; 0 = no restriction).  Eager launches only: a replayed
+  // hipGraph runs its kernel nodes without the capture stream's mask.
+  const char* ge = std::getenv("NANOFLOW_GEMM_CUS");
+  const char* ve = std::getenv("NANOFLOW_GEMV_CUS");
+  const int gemm_cus = ge ? std::atoi(ge) : 0, gemv_cus = ve ? std::atoi(ve) : 0;
+  stream_gemm = createPipelineStream(0, gemm_cus);
+  stream_gemv = createPipelineStream(gemm_cus, gemv_cus);
   stream_cpy = createPipelineStream(0, 0);
   if (enable_offload) {
     // room for two requests of 256 pages each (4096 tokens): the iteration's leading requests are

@@ -9,6 +9,8 @@
 * fp8 GEMM at the 70B FFN shape, and one 70B-shaped layer with e4m3 weights through the pipeline
   (the shape and weight format of the fp8 benchmark configuration).
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -275,7 +277,12 @@ def _full_width_iteration(oracle, shape, batch, schedules, weight_format="f16", 
     try:
         for pt, split, *rest in schedules:
             layout = rest[0] if rest else "row"
-            tag = f"{pt.name} {weight_format} {layout}"
+            masks = rest[1] if len(rest) > 1 else {}          # CU partition of the two streams (environment of the pipeline)
+            tag = f"{pt.name} {weight_format} {layout}" + (f" CUs {masks}" if masks else "")
+            saved_env = {k: os.environ.get(k) for k in ("NANOFLOW_GEMM_CUS", "NANOFLOW_GEMV_CUS")}
+            for k in saved_env:
+                os.environ.pop(k, None)
+            os.environ.update({k: str(v) for k, v in masks.items()})
             print(f"full-width iteration against the oracle: hidden={shape.hidden} rows={T} ({nd} decode) {tag}", flush=True)
             G = (T + 63) // 64 * 64
             with engine.Engine(shape, pt, global_batch=G, nano1=split[0], kqv1=split[1], kqv3=split[2],
@@ -289,6 +296,10 @@ def _full_width_iteration(oracle, shape, batch, schedules, weight_format="f16", 
                 inter = {k: e.buffer(k).cpu().numpy()[:T] for k in names} if (pt.is_sequential or pt.is_four_way) else {}
                 k_rows = e.kv[0][gidx(page_of), 0, gidx(entry_of)].cpu().numpy()
                 v_rows = e.kv[0][gidx(page_of), 1, gidx(entry_of)].cpu().numpy()
+            for k, v in saved_env.items():
+                os.environ.pop(k, None)
+                if v is not None:
+                    os.environ[k] = v
             if ref is None:
                 if e4m3:
                     ref = (None, None, None, None)
@@ -387,6 +398,21 @@ def _offline_steady_state_batch(vocab, kv_pages=98304, T=2048, cycles=1300):
                        per_token_offset=b["per_token_offset"], kv_indptr=b["kv_indptr"], kv_indices=b["kv_indices"],
                        kv_last_page_len=b["kv_last_page_len"],
                        kv_len=((pages_per - 1) * 16 + b["kv_last_page_len"]).astype(np.int32), num_pages=kv_pages)
+
+
+def test_overlapped_schedules_on_cu_masked_streams_at_full_width(oracle):
+    """The two overlapped schedules -- LocalPipeline (two nano-batches) and the reference's main schedule
+    (four QKV / attention nano-batches, 640 | 256 | 768) -- with their dense and attention streams on
+    disjoint CU sets (20 + 12 and 16 + 16 CUs of every XCD, hipExtStreamCreateWithCUMask), on the dense
+    2048-token iteration through one full-width 8B layer: against the oracle end to end, and (four-way
+    schedule) operator by operator.  Where a workgroup runs must not change the result."""
+    from nanoflow_amd import pllm_python as P
+    shape = synth.ModelShape(layers=1, vocab=4096)
+    batch = synth.config2_batch(seed=0, vocab=shape.vocab)
+    _full_width_iteration(oracle, shape, batch, (
+        (P.PipelineType.LOCAL, (1024, 512, 512), "col", {"NANOFLOW_GEMM_CUS": 160, "NANOFLOW_GEMV_CUS": 96}),
+        (P.PipelineType.PLLM, (640, 256, 768), "col", {"NANOFLOW_GEMM_CUS": 160, "NANOFLOW_GEMV_CUS": 96}),
+        (P.PipelineType.PLLM, (640, 256, 768), "col", {"NANOFLOW_GEMM_CUS": 128, "NANOFLOW_GEMV_CUS": 128})))
 
 
 def test_llama3_8b_layer_on_the_offline_steady_state_batch(oracle):
