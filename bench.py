@@ -39,10 +39,22 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0       # dense fp16
 MFMA_FP8_PEAK_TFLOPS = 5000.0   # dense fp8
 A100_PUBLISHED_TOKENS_PER_S = 12756.0   # reference, 1x A100 80GB, same offline workload
+def _profile_figure(name: str, pattern: str):
+    """A figure read from a committed rocprofv3 summary under profiles/ (None when the file or the
+    line is missing): the traffic ratios below are measurements of the kernels, kept with the
+    commands that made them, not constants of this file."""
+    import re
+    try:
+        m = re.search(pattern, open(os.path.join(ROOT, "profiles", name)).read())
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
 # HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
 # by what the same counter reads for a 1 GiB device copy), as a ratio to the algorithmic bytes of
 # the same launch: profiles/decode_attention_config2_pmc.txt.
-DECODE_ATTN_TRAFFIC_RATIO = 1.0061
+DECODE_ATTN_TRAFFIC_RATIO = _profile_figure("decode_attention_config2_pmc.txt", r"traffic / algorithmic\s*=\s*([0-9.]+)")
 
 
 def decode_attention_bytes(kv_len: np.ndarray, Hq=32, Hkv=8, d=128, page=16) -> int:
@@ -153,10 +165,12 @@ def _attention_roofline(tm, bytes_per_launch, name="roofline", calib=None):
 
 
 # Memory-side bytes per dense GEMM launch over algorithmic bytes (operands once + output), measured
-# with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernels at M = 2048 (LM head: 684 rows) and
-# scaled by the copy-kernel calibration: profiles/gemm_hbm_traffic_pmc.txt.  The activations are
-# fetched once per XCD and round of tiles; most of the repeats hit the Infinity Cache.
-GEMM_TRAFFIC_RATIO = 2.43
+# with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the fp16 kernels as the offline workload launches
+# them (Llama-3-8B shape, M = 2048, LM head on 684 rows, [N][K] weights) and scaled by the copy-kernel
+# calibration: profiles/gemm_hbm_traffic_pmc.txt.  It holds for that shape, layout and weight type
+# only; other runs report no traffic figure.
+GEMM_TRAFFIC_PROFILE = "gemm_hbm_traffic_pmc.txt"
+GEMM_TRAFFIC_RATIO = _profile_figure(GEMM_TRAFFIC_PROFILE, r"traffic_bytes_per_algorithmic_byte\s*=\s*([0-9.]+)")
 
 
 def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows, weight_bytes=2):
@@ -175,7 +189,7 @@ def _gemm_algorithmic_bytes_per_launch(shape, rows, sampled_rows, weight_bytes=2
     return total / (4 * shape.layers + 1)
 
 
-def _gemm_roofline(tm, alg_bytes_per_launch=None, fp8_share=0.0, calib=None):
+def _gemm_roofline(tm, alg_bytes_per_launch=None, fp8_share=0.0, calib=None, traffic_applies=False):
     """fp8_share: the fraction of the timed GEMM flops that runs on the fp8 matrix cores (the
     per-layer GEMMs with e4m3 weights; the LM head stays fp16).  The peak the launches are priced
     against is then the flop-weighted blend of the two published peaks."""
@@ -199,7 +213,11 @@ def _gemm_roofline(tm, alg_bytes_per_launch=None, fp8_share=0.0, calib=None):
                         "launch; the quantiser's time is not in these launches) + the fp16 LM head"),
         "bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
         "frac": achieved / peak,
-        "traffic": None if alg_bytes_per_launch is None or fp8_share else alg_bytes_per_launch * GEMM_TRAFFIC_RATIO,
+        # the measured ratio belongs to the fp16 kernels at the 8B shape on [N][K] weights (traffic_applies)
+        "traffic": (alg_bytes_per_launch * GEMM_TRAFFIC_RATIO
+                    if traffic_applies and alg_bytes_per_launch is not None and GEMM_TRAFFIC_RATIO and not fp8_share else None),
+        "traffic_measured_by": (f"profiles/{GEMM_TRAFFIC_PROFILE}: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on these kernels, "
+                                f"{GEMM_TRAFFIC_RATIO} bytes moved per algorithmic byte" if traffic_applies and GEMM_TRAFFIC_RATIO else None),
         "algorithmic_bytes_per_launch": alg_bytes_per_launch,
         "algorithmic_flop_per_launch": flop_per_launch, "avg_launch_ms": avg_ms,
         "launches_timed": int(tm.gemm_launches),
@@ -483,8 +501,9 @@ def run_offline(args):
                          if args.shape == "8b" and wb == 2 else
                          "none: the reference publishes no single-GPU figure for this shape / weight format"),
         },
-        "roofline": _gemm_roofline(tm, _gemm_algorithmic_bytes_per_launch(shape, rows_next, reqs_next, wb),
-                                   fp8_share, calib) if tm.gemm_launches else _attention_roofline(
+        "roofline": _gemm_roofline(tm, _gemm_algorithmic_bytes_per_launch(shape, rows_next, reqs_next, wb), fp8_share, calib,
+                                   traffic_applies=args.shape == "8b" and wb == 2 and eng.weight_layout == "col" and T == 2048
+                                   ) if tm.gemm_launches else _attention_roofline(
             tm, bytes_per_layer / launches_per_layer, calib=calib),
         "serving": {
             "cycles": st.cycles, "retired_requests": st.retired, "wall_s": st.wall_s,
@@ -492,17 +511,27 @@ def run_offline(args):
             "dense_rows_processed": int(st.tokens_processed),
             "cycle_ms": st.cycle_ms, "gpu_iteration_ms": st.gpu_iter_ms,
             "cpu_form_ms": st.form_ms, "cpu_wait_for_gpu_ms": st.wait_ms, "cpu_update_ms": st.update_ms,
-            # cycle time not covered by the device's iteration: update (staging + H2D), launch
-            # latency and whatever part of batch formation did not overlap the GPU
+            # Cycle time not covered by the device's iteration: the update (staging + H2D copies,
+            # which need the previous iteration's samples) and the hand-off (the caller's wake-up after the
+            # worker's barrier, the worker's wake-up for the next run, the first launch).  Batch formation
+            # is not in it: the loop forms batch c while the GPU runs batch c-1 and then WAITS for the GPU
+            # (cpu_wait_for_gpu_ms), so as long as that wait is positive formation is wholly hidden.
             "cpu_exposed_ms_per_cycle": max(0.0, st.cycle_ms - st.gpu_iter_ms),
-            "cpu_form_hidden_fraction": (1.0 - min(1.0, max(0.0, st.cycle_ms - st.gpu_iter_ms - st.update_ms)
-                                                   / st.form_ms) if st.form_ms > 0 else None),
+            "cpu_handoff_ms_per_cycle": max(0.0, st.cycle_ms - st.gpu_iter_ms - st.update_ms),
+            "cpu_form_hidden_fraction": (None if st.form_ms <= 0 else 1.0 if st.wait_ms > 0.05 * st.gpu_iter_ms else
+                                         max(0.0, 1.0 - max(0.0, st.cycle_ms - st.gpu_iter_ms - st.update_ms) / st.form_ms)),
             "steady_state_decode_rows": int(nd), "steady_state_prefill_rows": int(nxt["prefillTokensNum"]),
             "decode_attention_ms_per_cycle": tm.decode_attn_ms * tm.layer_stride / n_prof,
             "prefill_attention_ms_per_cycle": tm.prefill_attn_ms * tm.layer_stride / n_prof,
             "gemm_ms_per_cycle": tm.gemm_ms * tm.layer_stride / n_prof,   # LM head: timed 1 iteration in layer_stride
             "timed_layer_stride": tm.layer_stride, "per_launch_timed_cycles": prof_cycles,
             "per_launch_timed_cycle_ms": st_prof.cycle_ms if prof_cycles else None,
+            # the same serving loop over the per-launch-timed cycles that follow the timed window
+            # (eager launches with HIP events around every timed launch: a little slower per cycle)
+            "profile_pass": ({"cycles": st_prof.cycles, "retired_requests": st_prof.retired, "wall_s": st_prof.wall_s,
+                              "dense_rows_processed": int(st_prof.tokens_processed),
+                              "tokens_per_s_by_rows": st_prof.tokens_processed / rows_per_req * (in_len + out_len) / st_prof.wall_s,
+                              "cycle_ms": st_prof.cycle_ms} if prof_cycles and st_prof.wall_s > 0 else None),
             "graph_counters": counters,
             "requests_left": state["queued"] + state["decoding"] + state["prefilling"],
             "setup_s": t_setup,
