@@ -59,7 +59,14 @@ def candidates(T: int, step: int, types, fine: bool):
     return out
 
 
-def measure(shape, batch, T, cand, layers, iters, warm, env=None):
+ROLE_TAGS = {   # tag positions of the GEMM roles in gemm_op_tag, per schedule (the LM head's tag is the last one)
+    4: {"O": [0], "D": [1], "KQV": [2], "LOGITS": [3]},
+    7: {"O": [0, 1], "D": [2, 3], "KQV": [4, 5], "LOGITS": [6]},
+    9: {"O": [0, 1], "D": [2, 3], "KQV": [4, 5, 6, 7], "LOGITS": [8]},
+}
+
+
+def measure(shape, batch, T, cand, layers, iters, warm, env=None, tags=None, layout="row"):
     """(milliseconds per iteration of one candidate: median of iters runs; utilisation record of one
     further run with HIP events around every attention and dense GEMM launch: the rate each kind of
     launch reached while it ran, and the share of the iteration each kind was running)."""
@@ -70,7 +77,8 @@ def measure(shape, batch, T, cand, layers, iters, warm, env=None):
     os.environ.update(env or {})
     try:
         eng = engine.Engine(shape, P.PipelineType[name], global_batch=T, nano1=n1, kqv1=k1, kqv3=k3,
-                            kv_pages=batch.num_pages, run_layer=layers, distinct_layers=layers)
+                            kv_pages=batch.num_pages, run_layer=layers, distinct_layers=layers, gemm_tags=tags,
+                            weight_layout=layout)
     finally:
         for k, v in saved.items():
             if v is None:
@@ -127,15 +135,28 @@ def main():
     ap.add_argument("--types", default="NON_OVERLAP_LOCAL,NANOBATCH_LOCAL,LOCAL,PLLM")
     ap.add_argument("--fine", action="store_true", help="also try 1/4 and 3/4 QKV sub-splits")
     ap.add_argument("--cu-masks", default="", help="LOCAL only: GEMM:attention shares of the CUs to try, in eighths (4 CUs of every XCD each), e.g. 6:2,5:3,4:4")
+    ap.add_argument("--gemm-tiles", action="store_true",
+                    help="then search, for the winning schedule, the tile and the split over K of each GEMM role (the\n"
+                         "cta_m x cta_n and split_k fields of its tags) over the kernel library's tile menu, one role\n"
+                         "at a time, and write the winning tags into pipeline_configs.gemm_op_tag")
+    ap.add_argument("--weight-layout", default="", choices=["", "row", "col"],
+                    help="orientation the weights are handed over in (default: what the input file's tags say, else col)")
     ap.add_argument("--iters", type=int, default=5)
     ap.add_argument("--warm", type=int, default=2)
     ap.add_argument("--seed", type=int, default=0)
     a = ap.parse_args()
 
     import torch
-    from nanoflow_amd import synth, weights as W
+    from nanoflow_amd import engine, kernels, synth, weights as W
     assert torch.cuda.is_available(), "needs the MI355X"
     cfg = json.load(open(a.config_path))
+    in_tags = cfg.get("pipeline_configs", {}).get("gemm_op_tag") or []
+    layout = a.weight_layout
+    if not layout:
+        try:
+            layout = engine.layouts_of_tags(in_tags)[0] if len(in_tags) > 1 else "col"
+        except ValueError:
+            layout = "col"
     shape = W.shape_from_hf_config(cfg["model"], cfg.get("model_configs", {}).get("frame_page_size", 16))
     chunks = [tuple(int(x) for x in c.split(":")) for c in a.prefill.split(",") if c]
     rng = np.random.default_rng(a.seed + 2)
@@ -150,7 +171,7 @@ def main():
     rows = []
     print(f"{len(cands)} candidates, {batch.tokens} tokens ({batch.decodePrefillBorder} decode), {layers} layers each", flush=True)
     for cand in cands:
-        ms, util = measure(shape, batch, T, cand, layers, a.iters, a.warm)
+        ms, util = measure(shape, batch, T, cand, layers, a.iters, a.warm, layout=layout)
         rows.append({"pipeline_type": cand[0], "nanobatch_1_size": cand[1], "kqv1_size": cand[2],
                      "kqv3_size": cand[3], "ms": ms, **util})
         print(f"  {cand[0]:18s} nano1 {cand[1]:5d} kqv1 {cand[2]:5d} kqv3 {cand[3]:5d}: {ms:8.3f} ms   "
@@ -166,7 +187,7 @@ def main():
             if g <= 0 or v <= 0 or g + v > 8:
                 raise SystemExit(f"--cu-masks {g}:{v}: the shares (eighths of the CUs) must be positive and sum to at most 8")
             env = {"NANOFLOW_GEMM_CUS": str(32 * g), "NANOFLOW_GEMV_CUS": str(32 * v)}   # 32 CUs per eighth
-            ms, util = measure(shape, batch, T, cand, layers, a.iters, a.warm, env)
+            ms, util = measure(shape, batch, T, cand, layers, a.iters, a.warm, env, layout=layout)
             rows.append({"pipeline_type": "LOCAL", "nanobatch_1_size": cand[1], "kqv1_size": cand[2],
                          "kqv3_size": cand[3], "gemm_cu_eighths": g, "attention_cu_eighths": v, "ms": ms, **util, **env})
             print(f"  LOCAL with {4 * g} CUs of every XCD for GEMM, {4 * v} for attention: {ms:8.3f} ms", flush=True)
@@ -175,10 +196,42 @@ def main():
     pc = out.setdefault("pipeline_configs", {})
     pc.update({"global_batch_size": T, "nanobatch_1_size": best["nanobatch_1_size"],
                "kqv1_size": best["kqv1_size"], "kqv3_size": best["kqv3_size"]})
+    from nanoflow_amd import pllm_python as P
+    n_tags = P.PipelineType[best["pipeline_type"]].gemm_tags
+    tags = [engine.make_tag(layout=layout)] * n_tags          # the library's own choice everywhere
+    tile_rows = []
+    if a.gemm_tiles:
+        # one role at a time, the other roles at their best so far; a tag applies to launches of more
+        # than 512 live rows, so roles whose pieces are shorter see no difference and keep the default
+        cand = (best["pipeline_type"], best["nanobatch_1_size"], best["kqv1_size"], best["kqv3_size"])
+        env = {k: best[k] for k in ("NANOFLOW_GEMM_CUS", "NANOFLOW_GEMV_CUS") if k in best}
+        base_ms, _ = measure(shape, batch, T, cand, layers, a.iters, a.warm, env, tags=tags, layout=layout)
+        print(f"tile search on {cand[0]}: library's choice {base_ms:.3f} ms", flush=True)
+        menu = [(m, n) for m, n, col_only in kernels.gemm_tile_menu() if layout == "col" or not col_only]
+        for role, pos in ROLE_TAGS[n_tags].items():
+            if role == "LOGITS":
+                continue                                       # one launch per iteration against 4 per layer
+            best_role = (base_ms, tags[pos[0]])
+            for (tm_, tn_) in menu:
+                for split in (1, 2):
+                    trial = list(tags)
+                    tag = engine.make_tag(tm_, tn_, split, layout)
+                    for i in pos:
+                        trial[i] = tag
+                    ms, _ = measure(shape, batch, T, cand, layers, a.iters, a.warm, env, tags=trial, layout=layout)
+                    tile_rows.append({"role": role, "tile_m": tm_, "tile_n": tn_, "split_k": split, "ms": ms})
+                    print(f"  {role:4s} tile {tm_:3d} x {tn_:3d} split {split}: {ms:8.3f} ms", flush=True)
+                    if ms < best_role[0]:
+                        best_role = (ms, tag)
+            for i in pos:
+                tags[i] = best_role[1]
+            base_ms = best_role[0]
+        print(f"tile search: {base_ms:.3f} ms with {tags}", flush=True)
+    pc["gemm_op_tag"] = tags
     out.setdefault("serve_configs", {})["pipeline_type"] = best["pipeline_type"]
     out["search"] = {"iteration": {"decode_requests": a.decode, "kv_len": [a.kv_lo, a.kv_hi], "prefill_chunks": chunks,
                                    "tokens": batch.tokens}, "layers_per_measurement": layers,
-                     "best": best, "measurements": rows}
+                     "best": best, "measurements": rows, "weight_layout": layout, "gemm_tile_measurements": tile_rows}
     with open(a.output, "w") as f:
         json.dump(out, f, indent=1)
     print(f"best: {best['pipeline_type']} nano1 {best['nanobatch_1_size']} kqv1 {best['kqv1_size']} "

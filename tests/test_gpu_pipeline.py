@@ -814,8 +814,8 @@ def test_autosearch_writes_a_tuned_pipeline_config(tmp_path):
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     cmd = [sys.executable, "-m", "nanoflow_amd.autosearch", "-c", str(cfg), "-o", str(out), "--decode", "20",
            "--kv-lo", "5", "--kv-hi", "60", "--prefill", "7:30,0:40", "--layers", "2", "--step", "24",
-           "--iters", "3", "--warm", "1", "--cu-masks", "4:4"]
-    r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=110)
+           "--iters", "3", "--warm", "1", "--cu-masks", "4:4", "--gemm-tiles"]
+    r = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=170)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     t = json.load(open(out))
     rows = t["search"]["measurements"]
@@ -830,6 +830,11 @@ def test_autosearch_writes_a_tuned_pipeline_config(tmp_path):
     assert pc["global_batch_size"] == 96 and 0 < pc["kqv1_size"] <= pc["nanobatch_1_size"] < 96
     assert 0 < pc["kqv3_size"] <= 96 - pc["nanobatch_1_size"]
     assert t["model"] == json.load(open(cfg))["model"]
+    # the tile search measured every menu tile, unsplit and split in two, for the three per-layer roles
+    tiles = t["search"]["gemm_tile_measurements"]
+    assert {m["role"] for m in tiles} == {"O", "D", "KQV"} and len(tiles) >= 3 * 4 * 2
+    assert len(pc["gemm_op_tag"]) == P.PipelineType[best["pipeline_type"]].gemm_tags
+    assert engine.layouts_of_tags(pc["gemm_op_tag"]) == (t["search"]["weight_layout"],) * 2
 
 
 @pytest.mark.parametrize("pt_name", ["LOCAL", "NON_OVERLAP_LOCAL", "NANOBATCH_KQVBIAS"])
