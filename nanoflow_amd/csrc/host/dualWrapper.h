@@ -71,6 +71,15 @@ struct DualWrapper : public OperatorWrapper {
                                           rows(), N, K, weight_layout == PllmLayout::COL_MAJOR ? 1 : 0, workspace,
                                           workspace_bytes, stream));
   }
+  OperatorWrapper& logImpl() override {
+    logTensor("input", pllm_tensor_a, 10, 20);
+    if (!e4m3) {  // e4m3 weights are bytes with their scales behind them: not dumped
+      logTensor("weight0", pllm_tensor_b1, 10, 20);
+      logTensor("weight1", pllm_tensor_b2, 10, 20);
+    }
+    logTensor("output2", pllm_tensor_d2, 128, 20);
+    return *this;
+  }
   DualWrapper& setA(pllmTensor<half> a) {
     assert(a.layout == PllmLayout::ROW_MAJOR && (int)a.dim1 == M && (int)a.dim2 == K);
     pllm_tensor_a = a;

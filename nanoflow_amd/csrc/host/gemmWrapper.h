@@ -131,6 +131,15 @@ struct HipGEMMWrapper : public BaseGEMMWrapper {
   PllmLayout weightLayout() const override { return tag.layout_b; }
 
   void work() override;
+  // operands as cutlassGemmWrapperImpl.cuh's logImpl prints them: 10 rows x 20 columns each
+  OperatorWrapper& logImpl() override {
+    logTensor("input", pllm_tensor_a, 10, 20);
+    if (weightIsHalf()) logTensor("weight", pllm_tensor_b, 10, 20);
+    if (pllm_tensor_c.ptr && beta != 0.f) logTensor("C", pllm_tensor_c, 10, 20);
+    logTensor("output", pllm_tensor_d, 10, 20);
+    return *this;
+  }
+  virtual bool weightIsHalf() const { return true; }
 
   HipGEMMWrapper& setOutput(pllmTensor<half> data) override { return setD(data); }
   HipGEMMWrapper& setA(pllmTensor<half> a) override {
@@ -207,6 +216,7 @@ struct HipGEMMWrapperF8W : public HipGEMMWrapper {
     return q && scale;
   }
   void work() override;
+  bool weightIsHalf() const override { return false; }  // e4m3 bytes and scales: not dumped
   void set_weight(half* blob) override {  // see WeightFormat::E4M3
     pllm_tensor_b = pllmTensor<half>(blob, N, K, PllmLayout::COL_MAJOR);
   }

@@ -87,6 +87,14 @@ public:
                                   nf_last_error());
   }
 
+  OperatorWrapper& logImpl() override {
+    logTensor("kv_indptr", kv_indptr_tensor, 1, 20);
+    logTensor("kv_last_page_len", kv_last_page_len_tensor, 1, 20);
+    logTensor("input", input_tensor, 10, 20);
+    logTensor("output", output_tensor, 10, 20);
+    return *this;
+  }
+
 private:
   bool causal_;
   int max_rows_ = 0;

@@ -10,6 +10,7 @@
 
 #include "helper.h"
 #include "tensor.h"
+#include "tensorLogger.h"
 
 struct OperatorWrapper {
   hipStream_t stream = nullptr;
@@ -106,9 +107,18 @@ struct OperatorWrapper {
     return *this;
   }
 
-  // Tensor dumps are compiled out in the reference (ENABLE_LOGGING=false); kept as no-ops.
+  // Tensor dumps (operatorWrapper.cuh:146-156): log() after run() prints the operator's operands
+  // when NANOFLOW_TENSOR_LOG names a sink; logImpl() is the per-operator part.  Launches that are
+  // being captured into a graph are not dumped.
   virtual OperatorWrapper& logImpl() { return *this; }
-  OperatorWrapper& log() { return *this; }
+  OperatorWrapper& log() {
+    if (tensorlog::enabled() && streamInited && !tensorlog::capturing(stream)) return logImpl();
+    return *this;
+  }
+  template <typename T>
+  void logTensor(const char* tensor_name, const pllmTensor<T>& t, size_t rows = 1, size_t cols = 20) {
+    tensorlog::log_tensor(stream, name.empty() || name.back() == ' ' ? name : name + " ", tensor_name, t, rows, cols);
+  }
 
   // Time up to max_launches launches per iteration with event pairs on the op's own stream.
   // Every stride-th launch is timed (event records cost device time, so long schedules sample).

@@ -35,6 +35,11 @@ public:
   }
   pllmTensor<Element> getOutput() { return pllm_tensor_output; }
   pllmTensor<Element> getInput() { return pllm_tensor_input; }
+  OperatorWrapper& logImpl() override {
+    logTensor("input", pllm_tensor_input, 10, 20);
+    logTensor("output", pllm_tensor_output, 10, 20);
+    return *this;
+  }
 };
 
 // RMSNorm over rows of model_hidden_dim (the reference's class name is LayerNorm).
@@ -51,6 +56,12 @@ public:
     weight = w.ptr;
     pllm_tensor_weight = pllmTensor<half>(w.ptr, size_t(1), w.size(), PllmLayout::ROW_MAJOR);
     return true;
+  }
+  OperatorWrapper& logImpl() override {
+    logTensor("weight", pllm_tensor_weight, 1, 20);
+    logTensor("input", pllm_tensor_input, 10, 20);
+    logTensor("output", pllm_tensor_output, 10, 20);
+    return *this;
   }
   // rows that hold tokens in this iteration (-1: all rows of the input); the rest is left as it was
   int live_rows = -1;
@@ -117,6 +128,12 @@ public:
     if (rows == 0) return;
     NF_KERNEL_CHECK(nf_embedding_f16(tokens, weight, output, rows, ModelConfig.model_hidden_dim, stream));
   }
+  OperatorWrapper& logImpl() override {
+    logTensor("weight", pllm_tensor_weight, 1, 20);
+    logTensor("tokens", pllm_tensor_tokens, 1, 20);
+    logTensor("output", pllm_tensor_output, 10, 20);
+    return *this;
+  }
 };
 
 class RoPEAppend : public OtherWrapper {
@@ -159,6 +176,16 @@ public:
         ModelConfig.factor, ModelConfig.rope_theta, ModelConfig.smooth_a, ModelConfig.smooth_b,
         stream));
   }
+  OperatorWrapper& logImpl() override {
+    logTensor("kqv", kqv_input, 10, 20);
+    logTensor("q_out", q_out, 10, 20);
+    logTensor("rev_input_indptr", rev_input_indptr, 1, 512);
+    logTensor("per_token_offset", per_token_offset, 1, 512);
+    logTensor("kv_indices", kv_indices, 1, 512);
+    logTensor("kv_indptr", kv_indptr, 1, 512);
+    logTensor("kv_last_page_len", kv_last_page_len, 1, 512);
+    return *this;
+  }
 };
 
 class MaxSampling : public OtherWrapper {
@@ -178,6 +205,12 @@ public:
   }
   OperatorWrapper& set_batch_size(int b) {
     batch_size = b;
+    return *this;
+  }
+  OperatorWrapper& logImpl() override {
+    logTensor("d_matrix", d_matrix, 10, 20);
+    logTensor("d_maxVals", d_maxVals, 1, 20);
+    logTensor("d_argMax", d_argMax, 1, (size_t)batch_size);
     return *this;
   }
 };
@@ -202,6 +235,11 @@ public:
   }
   KeepToken& setInput(pllmTensor<half> i) {
     input = i;
+    return *this;
+  }
+  OperatorWrapper& logImpl() override {
+    logTensor("input", input, 10, 20);
+    logTensor("output", output, 10, 20);
     return *this;
   }
 };

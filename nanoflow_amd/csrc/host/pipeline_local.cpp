@@ -26,7 +26,9 @@ PipelineBase::PipelineBase(vortexInitData* input_data, int nrank, int nranks, in
       rank(nrank),
       nranks(nranks),
       vnranks(vnranks),
-      tmpBufferM(input_data->tmp_buffer, input_data->tmp_buffer_size) {}
+      tmpBufferM(input_data->tmp_buffer, input_data->tmp_buffer_size) {
+  tensorlog::configure();  // NANOFLOW_TENSOR_LOG is read when a pipeline is created
+}
 
 static int env_int(const char* name, int dflt) {
   const char* v = std::getenv(name);

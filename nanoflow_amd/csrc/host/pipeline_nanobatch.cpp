@@ -284,58 +284,58 @@ void Pipeline::enqueueIteration() {
   if (!nanobatch_only) HIP_CHECK(hipStreamWaitEvent(stream_gemv, events[EventManager::CAPTURE_GEMM_START], 0));
   if (enable_offload) HIP_CHECK(hipStreamWaitEvent(stream_cpy, events[EventManager::CAPTURE_GEMM_START], 0));
 
-  genEmbedding1.run();
-  if (KQV3->M > 0) genEmbedding2_1.run();
-  if (KQV4->M > 0) genEmbedding2_2.run();
+  genEmbedding1.run().log();
+  if (KQV3->M > 0) genEmbedding2_1.run().log();
+  if (KQV4->M > 0) genEmbedding2_2.run().log();
 
   for (int iter = 0; iter < ModelConfig.run_layer; ++iter) {
     setWeight(iter % ModelConfig.model_layer);
 
-    layerNormAttention1.run();
-    if (KQV3->M > 0) layerNormAttention2_1.run();
-    if (KQV4->M > 0) layerNormAttention2_2.run();
+    layerNormAttention1.run().log();
+    if (KQV3->M > 0) layerNormAttention2_1.run().log();
+    if (KQV4->M > 0) layerNormAttention2_2.run().log();
 
     // the layer's pool must not be appended to while the previous offload round trip (which may
     // have used the same pool when run_layer > model_layer) is still writing its pages back
     if (enable_offload && iter > 0) HIP_CHECK(hipStreamWaitEvent(stream_gemm, offload_done, 0));
 
     for (int i = 0; i < 4; ++i) {
-      if (KQV_ptrs[i]->M > 0) KQV_ptrs[i]->run();
-      if (roPEAppends[i].dense_batch_size > 0) roPEAppends[i].run(); else roPEAppends[i].skip();
-      if (gemvs[i]->batch_size > 0) gemvs[i]->wait(roPEAppends[i]).run(); else gemvs[i]->wait(roPEAppends[i]).skip();
+      if (KQV_ptrs[i]->M > 0) KQV_ptrs[i]->run().log();
+      if (roPEAppends[i].dense_batch_size > 0) roPEAppends[i].run().log(); else roPEAppends[i].skip();
+      if (gemvs[i]->batch_size > 0) gemvs[i]->wait(roPEAppends[i]).run().log(); else gemvs[i]->wait(roPEAppends[i]).skip();
     }
-    if (update_data.prefillNum > 0) prefill.wait(roPEAppends[3]).run(); else prefill.wait(roPEAppends[3]).skip();
+    if (update_data.prefillNum > 0) prefill.wait(roPEAppends[3]).run().log(); else prefill.wait(roPEAppends[3]).skip();
 
     // nano-batch 1 holds decode rows only when the first two groups fill it; otherwise some of its
     // rows are prefill rows, and prefill is the last launch on the attention stream
     OperatorWrapper* nano1_attention = &prefill;
     if ((int)config_data.nanobatch_1_size == update_data.gemv_batch_size[0] + update_data.gemv_batch_size[1])
       nano1_attention = &GEMV2;
-    O1->wait(*nano1_attention).run();
-    layerNormFFN1.run();
-    O2->wait(GEMV4).wait(prefill).run();
-    layerNormFFN2.run();
-    dual1.run();
-    D1->run();
+    O1->wait(*nano1_attention).run().log();
+    layerNormFFN1.run().log();
+    O2->wait(GEMV4).wait(prefill).run().log();
+    layerNormFFN2.run().log();
+    dual1.run().log();
+    D1->run().log();
     if (enable_offload && offload_pages > 0) {
       // gather -> host -> back -> scatter, beside the second nano-batch's FFN
       const size_t bytes = offload_pages * ModelConfig.page_mem_size;
-      pageAgg.wait(dual1).run();
+      pageAgg.wait(dual1).run().log();
       HIP_CHECK(hipMemcpyAsync(offloadKVCache, deviceOffloadKVCache, bytes, hipMemcpyDeviceToHost, stream_cpy));
       HIP_CHECK(hipMemcpyAsync(deviceLoadKVCache, offloadKVCache, bytes, hipMemcpyHostToDevice, stream_cpy));
-      pageDisp.run();
+      pageDisp.run().log();
       HIP_CHECK(hipEventRecord(offload_done, stream_cpy));
     } else if (enable_offload) {
       HIP_CHECK(hipEventRecord(offload_done, stream_cpy));
     }
-    dual2.run();
-    D2->run();
+    dual2.run().log();
+    D2->run().log();
   }
 
-  keepToken.run();
-  layerNormModel1.run();
-  LOGITS->run();
-  maxSampler.run();
+  keepToken.run().log();
+  layerNormModel1.run().log();
+  LOGITS->run().log();
+  maxSampler.run().log();
   // the side streams rejoin the dense stream (a capture needs the joins to be explicit)
   if (!nanobatch_only) {
     HIP_CHECK(hipEventRecord(events[EventManager::CAPTURE_GEMV_END], stream_gemv));

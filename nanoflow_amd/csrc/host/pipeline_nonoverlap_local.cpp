@@ -44,37 +44,37 @@ vortexOutputData NonOverlapLocalPipeline::run() {
   setWeight(0);
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_START], stream_all));
   runIteration(stream_all, baseSignature(), [this] {
-    genEmbedding.run();
+    genEmbedding.run().log();
     for (int iter = 0; iter < ModelConfig.run_layer; ++iter) {
       setWeight(iter % ModelConfig.model_layer);
-      layerNormAttention.run();
-      KQV->run();
-      roPEAppend.run();
+      layerNormAttention.run().log();
+      KQV->run().log();
+      roPEAppend.run().log();
       // fork: prefill attention beside decode attention; join before the O projection
       const bool side = update_data.prefillNum > 0 && GEMV.batch_size > 0;
       if (side) {
         HIP_CHECK(hipEventRecord(prefill_fork, stream_all));
         HIP_CHECK(hipStreamWaitEvent(stream_prefill, prefill_fork, 0));
         prefill.setStream(stream_prefill);
-        prefill.run();
+        prefill.run().log();
         HIP_CHECK(hipEventRecord(prefill_join, stream_prefill));
       }
-      if (GEMV.batch_size > 0) GEMV.run();
+      if (GEMV.batch_size > 0) GEMV.run().log();
       if (side) {
         HIP_CHECK(hipStreamWaitEvent(stream_all, prefill_join, 0));
       } else if (update_data.prefillNum > 0) {
         prefill.setStream(stream_all);
-        prefill.run();
+        prefill.run().log();
       }
-      O->run();
-      layerNormFFN.run();
-      dual.run();
-      D->run();
+      O->run().log();
+      layerNormFFN.run().log();
+      dual.run().log();
+      D->run().log();
     }
-    keepToken.run();
-    layerNormModel.run();
-    LOGITS->run();
-    maxSampler.run();
+    keepToken.run().log();
+    layerNormModel.run().log();
+    LOGITS->run().log();
+    maxSampler.run().log();
   });
   HIP_CHECK(hipEventRecord(events[EventManager::GEMM_TIMING_END], stream_all));
   HIP_CHECK(hipMemcpyAsync(output_data.sampled_token_array, maxSampler.d_argMax.ptr,

@@ -995,3 +995,76 @@ def test_gemm_tags_select_tile_and_split(oracle, pt_name, layout):
             out[name] = (e.buffer("hidden").cpu().numpy()[:b1.tokens], e.buffer("logits").cpu().numpy()[:b1.req_num])
         assert _max_rel(out[name][0], hid) < E2E_RTOL and _max_rel(out[name][1], log) < E2E_RTOL, (pt_name, name)
     assert _max_rel(out["named"][0], out["auto"][0]) < 2e-3
+
+
+def _parse_tensor_log(text):
+    """[(name, [[values of a row], ...]), ...] in file order."""
+    blocks = []
+    for line in text.splitlines():
+        if line.startswith("--------Tensor "):
+            blocks.append((line[len("--------Tensor "):].split(" (")[0], []))
+        elif blocks and line.strip():
+            blocks[-1][1].append([float(v) for v in line.split(",")])
+    return blocks
+
+
+@pytest.mark.parametrize("pt_name", ["NON_OVERLAP_LOCAL", "PLLM"])
+def test_tensor_dumps_follow_the_operators(tmp_path, monkeypatch, pt_name):
+    """NANOFLOW_TENSOR_LOG names a file: after each operator of an eager iteration its operands are
+    dumped under the reference's header line (pipeline/include/tensorLogger.cuh:15-60,
+    operatorWrapper.cuh:146-156).  The dumped corners are the values the pipeline's buffers hold, the
+    operators come in schedule order, a graph replay dumps nothing, and without the variable nothing
+    is written."""
+    from nanoflow_amd import engine, pllm_python as P
+    pt = P.PipelineType[pt_name]
+    T, nano1, dlens, chunks = CASES["prefill_straddles_border"]
+    shape = synth.tiny_shape(layers=2, vocab=1024, Hq=8, Hkv=2, ffn=512)
+    w = _scaled_weights(shape, seed=0)
+    b1 = synth.make_batch(dlens, chunks, vocab=shape.vocab, seed=21, extra_pages=40)
+    keep = np.ones(b1.decodePrefillBorder, np.int32)
+    path = tmp_path / "tensors.log"
+    monkeypatch.setenv("NANOFLOW_TENSOR_LOG", str(path))
+    with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=max(nano1 // 2, 1), kqv3=(T - nano1) // 2,
+                       kv_pages=b1.num_pages, weights=w) as e:
+        e.update(b1, keep_token_list=keep)
+        samples = e.run().copy()
+        logits = e.buffer("logits").cpu().numpy()[:b1.req_num]
+        blocks = _parse_tensor_log(path.read_text())
+        size = path.stat().st_size
+        # graph mode: a launch signature runs eagerly once (dumped), is captured on its second
+        # iteration and replayed from then on -- neither of which dumps anything
+        P.setGraphMode(True)
+        try:
+            for _ in range(4):
+                e.update(b1, keep_token_list=keep)
+                e.run()
+            counters = P.getGraphCounters()
+        finally:
+            P.setGraphMode(False)
+        assert counters["captured"] == 1 and counters["replayed"] == 3, counters  # the captured graph is launched too
+        assert len(_parse_tensor_log(path.read_text())) == 2 * len(blocks)
+        size = path.stat().st_size
+    names = [n for n, _ in blocks]
+    emb = "genEmbedding output" if pt_name == "NON_OVERLAP_LOCAL" else "genEmbedding1 output"
+    assert names[0].startswith("genEmbedding") and emb in names
+    # decode rows read the ids the previous iteration sampled: take the ids from their own dump
+    tok = np.array(blocks[names.index(emb.replace("output", "tokens"))][1][0], dtype=np.int64)
+    assert len(tok) == 20 and np.array_equal(tok[b1.decodePrefillBorder:], b1.input_tokens[b1.decodePrefillBorder:20])
+    got = np.array(blocks[names.index(emb)][1])
+    assert got.shape == (10, 20)
+    np.testing.assert_allclose(got, w["embedding"][tok[:10], :20].astype(np.float32), rtol=1e-4, atol=1e-7)
+    i_logits = len(names) - 1 - names[::-1].index("LOGITS output")
+    np.testing.assert_allclose(np.array(blocks[i_logits][1]), logits[:10, :20].astype(np.float32), rtol=1e-4, atol=1e-7)
+    arg = np.array(blocks[names.index("maxSampler d_argMax")][1][0], dtype=np.int64)
+    assert np.array_equal(arg, samples[:len(arg)]) and len(arg) == b1.req_num
+    # per layer: norm, projection, rope, attention, O, norm, gate/up, down -- in that order
+    o_name = "O output" if pt_name == "NON_OVERLAP_LOCAL" else "O1 output"
+    d_name = "D output" if pt_name == "NON_OVERLAP_LOCAL" else "D2 output"
+    assert names.count(o_name) == shape.layers and names.count(d_name) == shape.layers
+    assert names.index(o_name) < names.index(d_name) < i_logits
+    monkeypatch.delenv("NANOFLOW_TENSOR_LOG")
+    with engine.Engine(shape, pt, global_batch=T, nano1=nano1, kqv1=max(nano1 // 2, 1), kqv3=(T - nano1) // 2,
+                       kv_pages=b1.num_pages, weights=w) as e:
+        e.update(b1, keep_token_list=keep)
+        e.run()
+    assert path.stat().st_size == size
