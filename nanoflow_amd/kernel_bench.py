@@ -342,17 +342,22 @@ def main():
             kn, nk = cold_copies(Bkn, a.cold), cold_copies(Bnk, a.cold)
             ms_kn = timeit(lambda: [torch.matmul(A, next(kn), out=out) for _ in range(reps)], a.iters, a.warm)
             ms_nk = timeit(lambda: [torch.matmul(A, next(nk).t(), out=out) for _ in range(reps)], a.iters, a.warm)
+            # this library as the pipelines call it (workspace entry points: the down projection at 2048
+            # rows is split over K), on both weight layouts
+            ws = torch.empty(max(K.lib().nf_gemm_workspace_bytes(M, N, Kd), 16), dtype=torch.uint8, device=DEV)
             if name.startswith("gate"):
-                kn2 = cold_copies(rnd(Kd, N, std=0.02), a.cold)
+                kn2, nk2 = cold_copies(rnd(Kd, N, std=0.02), a.cold), cold_copies(rnd(N, Kd, std=0.02), a.cold)
                 ms_us = timeit(lambda: K.dual_swiglu(A, next(kn), next(kn2), out=out), a.iters, a.warm)
-                ms_same = timeit(lambda: K.dual_swiglu(A, Bkn, Bkn, out=out), a.iters, a.warm)
+                ms_us_nk = timeit(lambda: K.dual_swiglu(A, next(nk), next(nk2), out=out, b_col_major=True), a.iters, a.warm)
+                ms_same = timeit(lambda: K.dual_swiglu(A, Bnk, Bnk, out=out, b_col_major=True), a.iters, a.warm)
             else:
-                ms_us = timeit(lambda: K.gemm(A, next(kn), out=out), a.iters, a.warm)
+                ms_us = timeit(lambda: K.gemm_ws(A, next(kn), out=out, workspace=ws), a.iters, a.warm)
+                ms_us_nk = timeit(lambda: K.gemm_ws(A, next(nk), out=out, workspace=ws, b_col_major=True), a.iters, a.warm)
             fl = 2.0 * reps * M * N * Kd
             print(f"{name:18s} {M}x{N}x{Kd}: torch.matmul [K,N] weights {fl / ms_kn / 1e9:7.1f}  [N,K] weights "
-                  f"{fl / ms_nk / 1e9:7.1f}  this library ([K,N]) {fl / ms_us / 1e9:7.1f} TFLOP/s", flush=True)
+                  f"{fl / ms_nk / 1e9:7.1f}  this library [K,N] {fl / ms_us / 1e9:7.1f}  [N,K] {fl / ms_us_nk / 1e9:7.1f} TFLOP/s", flush=True)
             if name.startswith("gate"):
-                print(f"{'':18s} this library's fused pair with ONE buffer given as both weight matrices (half the weight "
+                print(f"{'':18s} this library's fused pair, [N,K], with ONE buffer given as both weight matrices (half the weight "
                       f"bytes, same flops): {fl / ms_same / 1e9:7.1f} TFLOP/s", flush=True)
     elif a.op in ("corun", "cusplit"):
         corun(a, shape, rnd)
