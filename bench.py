@@ -51,6 +51,19 @@ def _profile_figure(name: str, pattern: str):
         return None
 
 
+def _overlap_note() -> str:
+    """What the overlapped nano-batch schedules cost on the offline cycle against the single stream,
+    as measured back to back on one box: profiles/schedules_offline_cycle.txt."""
+    name = "schedules_offline_cycle.txt"
+    local = _profile_figure(name, r"LOCAL - NON_OVERLAP_LOCAL\s*=\s*(-?[0-9.]+) ms")
+    pllm = _profile_figure(name, r"PLLM - NON_OVERLAP_LOCAL\s*=\s*(-?[0-9.]+) ms")
+    if local is None or pllm is None:
+        return "not measured (profiles/schedules_offline_cycle.txt is missing)"
+    return (f"measured, loses by {local:.1f} ms per cycle (LOCAL: two nano-batches on two streams) and by {pllm:.1f} ms "
+            f"(PLLM: four QKV / attention nano-batches) against the single stream NON_OVERLAP_LOCAL, which only runs "
+            f"chunked-prefill attention beside decode attention; profiles/{name}; --pipeline LOCAL | PLLM re-measure")
+
+
 # HBM bytes per decode-attention launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled
 # by what the same counter reads for a 1 GiB device copy), as a ratio to the algorithmic bytes of
 # the same launch: profiles/decode_attention_config2_pmc.txt.
@@ -491,7 +504,8 @@ def run_offline(args):
                             f"replayed from hipGraphs; the roofline records come from the {prof_cycles} eager, "
                             f"per-launch-timed cycles that follow")),
             "kv_contents": args.kv_fill,
-            "pipeline": args.pipeline, "global_batch": T, "nanobatch_1_size": args.nano1,
+            "pipeline": args.pipeline, "overlap": _overlap_note() if args.shape == "8b" and wb == 2 else None,
+            "global_batch": T, "nanobatch_1_size": args.nano1,
             "kqv1_size": args.kqv1, "kqv3_size": args.kqv3, "layers_executed": shape.layers,
             "distinct_layers_in_hbm": shape.layers, "kv_pages_per_layer": int(pages),
             "kv_pool_gib": pages * page_b / 2**30,

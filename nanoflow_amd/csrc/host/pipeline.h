@@ -127,7 +127,11 @@ protected:
   // signature runs eagerly the first time it is seen (one-time kernel attribute calls must not
   // happen inside a capture), is captured the second time, and is replayed from then on.
   // Per-launch profiling brackets cannot be read back from a replay, so profiling disables it.
+  // So do CU-masked streams: a replayed graph runs its kernel nodes without the capture stream's
+  // CU mask and a kernel node has no mask attribute, so a pipeline built on masked streams
+  // (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS) keeps launching eagerly whatever the graph mode says.
   bool graph_mode = false;
+  bool masked_streams = false;
   std::map<std::vector<int>, hipGraphExec_t> graph_execs;
   std::set<std::vector<int>> graph_seen;
   long graph_replays = 0, graph_captures = 0, graph_eager = 0;
@@ -136,7 +140,7 @@ protected:
 
   template <class F>
   void runIteration(hipStream_t origin, const std::vector<int>& sig, F&& enqueue) {
-    if (!graph_mode || profiling) {
+    if (!graph_mode || profiling || masked_streams) {
       ++graph_eager;
       enqueue();
       return;

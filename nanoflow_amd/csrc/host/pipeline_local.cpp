@@ -82,6 +82,7 @@ void LocalPipeline::init() {
   // Optional CU partition: GEMM stream on CUs [0, g), attention stream on [g, g + a).
   const int gemm_cus = env_int("NANOFLOW_GEMM_CUS", 0);
   const int gemv_cus = env_int("NANOFLOW_GEMV_CUS", 0);
+  masked_streams = gemm_cus > 0 || gemv_cus > 0;
   stream_gemm = createPipelineStream(0, gemm_cus);
   stream_gemv = createPipelineStream(gemm_cus, gemv_cus);
   stream_other = createPipelineStream(0, 0);
@@ -344,61 +345,61 @@ void LocalPipeline::enqueueIteration() {
   HIP_CHECK(hipEventRecord(events[EventManager::CAPTURE_GEMM_START], stream_gemm));
   HIP_CHECK(hipStreamWaitEvent(stream_gemv, events[EventManager::CAPTURE_GEMM_START], 0));
 
-  genEmbedding1.run();
-  genEmbedding2.run();
+  genEmbedding1.run().log();
+  genEmbedding2.run().log();
 
   // prologue: first half of layer 0 for both nano-batches
   setWeight_group_LN(0);
-  layerNormAttention1.run();
-  KQV1->run();
-  if (roPEAppends[0].dense_batch_size > 0) roPEAppends[0].run(); else roPEAppends[0].skip();
-  layerNormAttention2.run();
-  KQV2->run();
-  if (roPEAppends[1].dense_batch_size > 0) roPEAppends[1].run(); else roPEAppends[1].skip();
+  layerNormAttention1.run().log();
+  KQV1->run().log();
+  if (roPEAppends[0].dense_batch_size > 0) roPEAppends[0].run().log(); else roPEAppends[0].skip();
+  layerNormAttention2.run().log();
+  KQV2->run().log();
+  if (roPEAppends[1].dense_batch_size > 0) roPEAppends[1].run().log(); else roPEAppends[1].skip();
 
   for (int iter = 0; iter < ModelConfig.run_layer; ++iter) {
     setWeight_group_O(iter % ModelConfig.model_layer);
 
     // attention of nano-batch 1 (stream_gemv)
-    if (GEMV1.batch_size > 0) GEMV1.wait(roPEAppends[0]).run(); else GEMV1.skip();
-    if (GEMV2.batch_size > 0) GEMV2.wait(roPEAppends[0]).run(); else GEMV2.skip();
-    if (prefill1.batch_size > 0) prefill1.wait(roPEAppends[0]).run(); else prefill1.skip();
+    if (GEMV1.batch_size > 0) GEMV1.wait(roPEAppends[0]).run().log(); else GEMV1.skip();
+    if (GEMV2.batch_size > 0) GEMV2.wait(roPEAppends[0]).run().log(); else GEMV2.skip();
+    if (prefill1.batch_size > 0) prefill1.wait(roPEAppends[0]).run().log(); else prefill1.skip();
 
     // dense half of nano-batch 1 (stream_gemm)
-    O1->wait(prefill1).wait(GEMV2).run();
-    layerNormFFN1.run();
-    dual1.run();
-    D1->run();
+    O1->wait(prefill1).wait(GEMV2).run().log();
+    layerNormFFN1.run().log();
+    dual1.run().log();
+    D1->run().log();
 
     // attention of nano-batch 2 overlaps the dense ops above
-    if (GEMV3.batch_size > 0) GEMV3.wait(roPEAppends[1]).run(); else GEMV3.skip();
-    if (GEMV4.batch_size > 0) GEMV4.wait(roPEAppends[1]).run(); else GEMV4.skip();
-    if (prefill2.batch_size > 0) prefill2.wait(roPEAppends[1]).wait(dual1).run(); else prefill2.skip();
+    if (GEMV3.batch_size > 0) GEMV3.wait(roPEAppends[1]).run().log(); else GEMV3.skip();
+    if (GEMV4.batch_size > 0) GEMV4.wait(roPEAppends[1]).run().log(); else GEMV4.skip();
+    if (prefill2.batch_size > 0) prefill2.wait(roPEAppends[1]).wait(dual1).run().log(); else prefill2.skip();
 
     setWeight_group_LN((iter + 1) % ModelConfig.model_layer);
 
     if (iter != ModelConfig.run_layer - 1) {
-      layerNormAttention1.run();
-      KQV1->run();
-      if (roPEAppends[0].dense_batch_size > 0) roPEAppends[0].run(); else roPEAppends[0].skip();
+      layerNormAttention1.run().log();
+      KQV1->run().log();
+      if (roPEAppends[0].dense_batch_size > 0) roPEAppends[0].run().log(); else roPEAppends[0].skip();
     }
 
-    O2->wait(prefill2).run();
-    layerNormFFN2.run();
-    dual2.run();
-    D2->run();
+    O2->wait(prefill2).run().log();
+    layerNormFFN2.run().log();
+    dual2.run().log();
+    D2->run().log();
 
     if (iter != ModelConfig.run_layer - 1) {
-      layerNormAttention2.run();
-      KQV2->run();
-      if (roPEAppends[1].dense_batch_size > 0) roPEAppends[1].run(); else roPEAppends[1].skip();
+      layerNormAttention2.run().log();
+      KQV2->run().log();
+      if (roPEAppends[1].dense_batch_size > 0) roPEAppends[1].run().log(); else roPEAppends[1].skip();
     }
   }
 
-  keepToken.run();
-  layerNormModel.run();
-  LOGITS->run();
-  maxSampler.run();
+  keepToken.run().log();
+  layerNormModel.run().log();
+  LOGITS->run().log();
+  maxSampler.run().log();
   // the attention stream rejoins the dense stream (all of its launches are already ordered
   // before O1/O2; a capture needs the join to be explicit)
   HIP_CHECK(hipEventRecord(events[EventManager::CAPTURE_GEMV_END], stream_gemv));

@@ -23,11 +23,11 @@ Pipeline::Pipeline(vortexInitData* input_data, int nrank, int nranks, int vnrank
     : PipelineBase(input_data, nrank, nranks, vnranks), enable_offload(enable_offload_), nanobatch_only(nanobatch_only_) {
   kqv_bias = kqv_bias_;
   // Optional CU partition, as in LocalPipeline: dense operators on CUs [0, g), attention on [g, g + a)
-  // (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS; 0 = no restriction).  Eager launches only: a replayed
-  // hipGraph runs its kernel nodes without the capture stream's mask.
+  // (NANOFLOW_GEMM_CUS / NANOFLOW_GEMV_CUS; 0 = no restriction).  Eager launches only (masked_streams).
   const char* ge = std::getenv("NANOFLOW_GEMM_CUS");
   const char* ve = std::getenv("NANOFLOW_GEMV_CUS");
   const int gemm_cus = ge ? std::atoi(ge) : 0, gemv_cus = ve ? std::atoi(ve) : 0;
+  masked_streams = gemm_cus > 0 || gemv_cus > 0;
   stream_gemm = createPipelineStream(0, gemm_cus);
   stream_gemv = createPipelineStream(gemm_cus, gemv_cus);
   stream_cpy = createPipelineStream(0, 0);
