@@ -33,25 +33,38 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const int32_t* __restr
 
 // ---------------------------------------------------------------- RMSNorm
 
-// One workgroup per row.  Two passes over the row (second pass hits L1/L2); fp32 math,
-// single rounding on output.
+// One workgroup per row; fp32 math, single rounding on output.  Rows longer than 8192 are read a
+// second time after the reduction (from L1/L2).
 // kQuant: the rounded row (at most 4 x 256 chunks of 8 halves: hidden <= 8192) stays in registers
 // and is also written as e4m3 bytes with one fp32 scale per row, exactly what the row quantiser
 // makes of the fp16 output: the fp8-weight GEMM that follows needs no quantiser launch.
-template <bool kQuant>
+// kHeld: rows of at most 4 x 256 chunks (hidden <= 8192): a thread's chunks of the row and of the
+// weight are loaded once, all of them before the first is used, and stay in registers -- the row is
+// not read a second time after the reduction and the weight's latency passes under it.  The sums
+// are taken in the same order either way, so both forms give the same bits.
+template <bool kQuant, bool kHeld>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
                                                       const u32x4* __restrict__ in,
                                                       const u32x4* __restrict__ w, int vec_per_row,
                                                       float inv_n, float eps, uint8_t* __restrict__ q_out,
                                                       float* __restrict__ q_scale) {
+  static_assert(!kQuant || kHeld, "the quantising form keeps the row in registers");
   __shared__ float s_part[4];
   __shared__ float s_max[4];
   const int r = blockIdx.x;
   const u32x4* x = in + (long long)r * vec_per_row;
   u32x4* y = out + (long long)r * vec_per_row;
+  u32x4 xs[kHeld ? 4 : 1], ws[kHeld ? 4 : 1];
+  if constexpr (kHeld) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if ((int)threadIdx.x + k * 256 < vec_per_row) xs[k] = x[threadIdx.x + k * 256];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if ((int)threadIdx.x + k * 256 < vec_per_row) ws[k] = w[threadIdx.x + k * 256];
+  }
   float ss = 0.f;
-  for (int i = threadIdx.x; i < vec_per_row; i += 256) {
-    u32x4 v = x[i];
+  auto square = [&](const u32x4& v) {
     const uint32_t p[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -59,6 +72,13 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
       ss = fmaf(a, a, ss);
       ss = fmaf(b, b, ss);
     }
+  };
+  if constexpr (kHeld) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if ((int)threadIdx.x + k * 256 < vec_per_row) square(xs[k]);
+  } else {
+    for (int i = threadIdx.x; i < vec_per_row; i += 256) square(x[i]);
   }
   ss = wave_sum(ss);
   if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
@@ -67,9 +87,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
   const float scale = 1.0f / sqrtf(tot * inv_n + eps);
   u32x4 held[kQuant ? 4 : 1];
   float amax = 0.f;
-  auto normalise = [&](int i) {  // chunk i of the row: scaled, weighted, rounded once, stored
-    u32x4 v = x[i];
-    u32x4 g = w[i];
+  auto normalise = [&](int i, const u32x4& v, const u32x4& g) {  // chunk i of the row: scaled, weighted, rounded once, stored
     const uint32_t p[4] = {v.x, v.y, v.z, v.w};
     const uint32_t q[4] = {g.x, g.y, g.z, g.w};
     uint32_t o[4];
@@ -87,12 +105,15 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(u32x4* __restrict__ out,
     y[i] = yv;
     return yv;
   };
-  if constexpr (kQuant) {
+  if constexpr (kHeld) {
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-      if ((int)threadIdx.x + k * 256 < vec_per_row) held[k] = normalise(threadIdx.x + k * 256);
+      if ((int)threadIdx.x + k * 256 < vec_per_row) {
+        const u32x4 yv = normalise(threadIdx.x + k * 256, xs[k], ws[k]);
+        if constexpr (kQuant) held[k] = yv;
+      }
   } else {
-    for (int i = threadIdx.x; i < vec_per_row; i += 256) normalise(i);
+    for (int i = threadIdx.x; i < vec_per_row; i += 256) normalise(i, x[i], w[i]);
   }
   if constexpr (kQuant) {
 #pragma unroll
@@ -186,6 +207,21 @@ __global__ __launch_bounds__(256) void rope_append_kernel(
   constexpr int D = 128;
   __shared__ float s_cos[D / 2], s_sin[D / 2];
   const int t = blockIdx.x;
+  const int heads = Hq + 2 * Hkv;
+  const uint16_t* row = kqv + (long long)t * heads * D;
+  // the token's row first: a thread's first four items are in flight while the page is looked up
+  // (three dependent loads) and the angles are evaluated
+  constexpr int HELD = 4;
+  u32x4 lo_held[HELD], hi_held[HELD];
+#pragma unroll
+  for (int k = 0; k < HELD; ++k) {
+    const int item = threadIdx.x + k * 256;
+    if (item < heads * 8) {
+      const uint16_t* src = row + (item >> 3) * D + 8 * (item & 7);
+      lo_held[k] = *reinterpret_cast<const u32x4*>(src);
+      hi_held[k] = *reinterpret_cast<const u32x4*>(src + 64);
+    }
+  }
   const int r = rev_input_indptr[t];
   const int pos = per_token_offset[t];
   const int page = kv_indices[kv_indptr[r] + pos / page_size];
@@ -200,17 +236,12 @@ __global__ __launch_bounds__(256) void rope_append_kernel(
     s_sin[threadIdx.x] = sinf(ang);
   }
   __syncthreads();
-  const int heads = Hq + 2 * Hkv;
-  const uint16_t* row = kqv + (long long)t * heads * D;
   // pool[page][kv][entry][head][feat]
   uint16_t* kdst = kv_data + ((((long long)page * 2 + 0) * page_size + entry) * Hkv) * D;
   uint16_t* vdst = kv_data + ((((long long)page * 2 + 1) * page_size + entry) * Hkv) * D;
   uint16_t* qdst = q_out + (long long)t * Hq * D;
-  for (int item = threadIdx.x; item < heads * 8; item += 256) {
+  auto emit = [&](int item, const u32x4& lo, const u32x4& hi) {
     const int h = item >> 3, c = item & 7;  // chunk c covers features 8c..8c+7 and 64+8c..
-    const uint16_t* src = row + h * D;
-    u32x4 lo = *reinterpret_cast<const u32x4*>(src + 8 * c);
-    u32x4 hi = *reinterpret_cast<const u32x4*>(src + 64 + 8 * c);
     uint16_t* dst;
     if (h < Hkv) {
       dst = kdst + h * D;
@@ -218,7 +249,7 @@ __global__ __launch_bounds__(256) void rope_append_kernel(
       dst = vdst + (h - Hkv) * D;
       *reinterpret_cast<u32x4*>(dst + 8 * c) = lo;
       *reinterpret_cast<u32x4*>(dst + 64 + 8 * c) = hi;
-      continue;
+      return;
     } else {
       dst = qdst + (h - 2 * Hkv) * D;
     }
@@ -242,6 +273,15 @@ __global__ __launch_bounds__(256) void rope_append_kernel(
     }
     *reinterpret_cast<u32x4*>(dst + 8 * c) = u32x4{ol[0], ol[1], ol[2], ol[3]};
     *reinterpret_cast<u32x4*>(dst + 64 + 8 * c) = u32x4{oh[0], oh[1], oh[2], oh[3]};
+  };
+#pragma unroll
+  for (int k = 0; k < HELD; ++k) {
+    const int item = threadIdx.x + k * 256;
+    if (item < heads * 8) emit(item, lo_held[k], hi_held[k]);
+  }
+  for (int item = threadIdx.x + HELD * 256; item < heads * 8; item += 256) {  // more than 128 heads
+    const uint16_t* src = row + (item >> 3) * D + 8 * (item & 7);
+    emit(item, *reinterpret_cast<const u32x4*>(src), *reinterpret_cast<const u32x4*>(src + 64));
   }
 }
 
@@ -325,7 +365,8 @@ int nf_rmsnorm_f16(uint16_t* out, const uint16_t* in, const uint16_t* weight, in
              "nf_rmsnorm_f16: hidden=%d must be a positive multiple of 8 (rows=%d)", hidden, rows);
   if (rows == 0) return NF_OK;
   NF_REQUIRE(out && in && weight, "nf_rmsnorm_f16: null pointer");
-  rmsnorm_kernel<false><<<rows, 256, 0, (hipStream_t)stream>>>(
+  auto kern = hidden <= 8192 ? rmsnorm_kernel<false, true> : rmsnorm_kernel<false, false>;
+  kern<<<rows, 256, 0, (hipStream_t)stream>>>(
       reinterpret_cast<u32x4*>(out), reinterpret_cast<const u32x4*>(in),
       reinterpret_cast<const u32x4*>(weight), hidden / 8, 1.0f / (float)hidden, eps, nullptr, nullptr);
   return check_launch("nf_rmsnorm_f16");
@@ -340,7 +381,7 @@ int nf_rmsnorm_quantize_e4m3(uint16_t* out, const uint16_t* in, const uint16_t* 
   NF_REQUIRE(out && in && weight && out_q && row_scale, "nf_rmsnorm_quantize_e4m3: null pointer");
   NF_REQUIRE(((uintptr_t)out | (uintptr_t)in | (uintptr_t)weight | (uintptr_t)out_q) % 16 == 0,
              "nf_rmsnorm_quantize_e4m3: operands must be 16-byte aligned");
-  rmsnorm_kernel<true><<<rows, 256, 0, (hipStream_t)stream>>>(
+  rmsnorm_kernel<true, true><<<rows, 256, 0, (hipStream_t)stream>>>(
       reinterpret_cast<u32x4*>(out), reinterpret_cast<const u32x4*>(in),
       reinterpret_cast<const u32x4*>(weight), hidden / 8, 1.0f / (float)hidden, eps, out_q, row_scale);
   return check_launch("nf_rmsnorm_quantize_e4m3");
