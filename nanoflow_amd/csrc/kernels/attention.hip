@@ -39,12 +39,16 @@ union H8 {
 //   before the chunk, and a launch is over when its longest tile is, so the long tiles start first
 //   and the short ones fill in behind them.  (Ranked by counting, at most kPlanSortMax tiles;
 //   beyond that tiles keep their order.)
+//   first_wave > 0: the number of slots k whose workgroups are the first on their CU.  When all
+//   tiles fit into two such waves every workgroup is resident from the start, nothing fills in
+//   behind anything, and what counts is which two tiles share a CU: the second wave then runs from
+//   the shortest tile up, so that the longest tile shares its CU with the shortest.
 constexpr int kPlanSortMax = 1024;
 __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restrict__ qo_indptr,
                                                         const int32_t* __restrict__ kv_indptr,
                                                         const int32_t* __restrict__ kv_last_page_len,
                                                         int32_t* __restrict__ tile_start, int32_t* __restrict__ tile_order,
-                                                        int batch, int wg_tok, int causal) {
+                                                        int batch, int wg_tok, int causal, int first_wave) {
   __shared__ int s_sum[256];
   __shared__ int s_key[kPlanSortMax];
   const int per = (batch + 255) / 256;
@@ -89,7 +93,8 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int32_t* __restric
     const int key = s_key[t];
     int rank = 0;
     for (int u = 0; u < total; ++u) rank += (s_key[u] > key) || (s_key[u] == key && u < t);
-    tile_order[rank] = t;
+    const bool pair_up = first_wave > 0 && total <= 2 * first_wave && rank >= first_wave;
+    tile_order[pair_up ? first_wave + (total - 1 - rank) : rank] = t;
   }
 }
 
@@ -725,8 +730,19 @@ static int launch_attn(const uint16_t* q, uint16_t* o, const int32_t* qo_indptr,
     bound = (long long)batch * Hkv;
   } else {
     const int wg_tok = 4 * NQB_PREFILL * TPB;
+    // workgroup slots that are the first on their CU: one per CU, Hkv workgroups per slot (a capped
+    // grid walks its tiles in rounds: long tiles first is the right order there)
+    static int cus = 0;  // benign race: every caller computes the same value
+    if (cus == 0) {
+      int dev = 0, v = 0;
+      if (hipGetDevice(&dev) != hipSuccess ||
+          hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+        v = 256;
+      cus = v;
+    }
+    const int first_wave = num_blocks > 0 ? 0 : cus / Hkv;
     attn_plan_kernel<<<1, 256, 0, stream>>>(qo_indptr, kv_indptr, kv_last_page_len, tile_start, tile_order, batch,
-                                            wg_tok, causal);
+                                            wg_tok, causal, first_wave);
     bound = ((long long)batch + max_qo_rows / wg_tok) * Hkv;
   }
   if (num_blocks > 0 && bound > num_blocks) bound = num_blocks;
