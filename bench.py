@@ -51,15 +51,16 @@ def _profile_figure(name: str, pattern: str):
         return None
 
 
-def _overlap_note() -> str:
-    """What the overlapped nano-batch schedules cost on the offline cycle against the single stream,
-    as measured back to back on one box: profiles/schedules_offline_cycle.txt."""
-    name = "schedules_offline_cycle.txt"
+def _overlap_note(workload: str = "offline") -> str:
+    """What the overlapped nano-batch schedules cost against the single stream, as measured back to
+    back on one box: profiles/schedules_offline_cycle.txt, profiles/schedules_dense_iteration.txt."""
+    name = "schedules_offline_cycle.txt" if workload == "offline" else "schedules_dense_iteration.txt"
     local = _profile_figure(name, r"LOCAL - NON_OVERLAP_LOCAL\s*=\s*(-?[0-9.]+) ms")
     pllm = _profile_figure(name, r"PLLM - NON_OVERLAP_LOCAL\s*=\s*(-?[0-9.]+) ms")
     if local is None or pllm is None:
-        return "not measured (profiles/schedules_offline_cycle.txt is missing)"
-    return (f"measured, loses by {local:.1f} ms per cycle (LOCAL: two nano-batches on two streams) and by {pllm:.1f} ms "
+        return f"not measured (profiles/{name} is missing)"
+    per = "cycle" if workload == "offline" else "iteration"
+    return (f"measured, loses by {local:.1f} ms per {per} (LOCAL: two nano-batches on two streams) and by {pllm:.1f} ms "
             f"(PLLM: four QKV / attention nano-batches) against the single stream NON_OVERLAP_LOCAL, which only runs "
             f"chunked-prefill attention beside decode attention; profiles/{name}; --pipeline LOCAL | PLLM re-measure")
 
@@ -332,7 +333,10 @@ def run_iteration(args):
             "weight_layout": ("[N][K] (k contiguous; GEMM tags say ColumnMajor for B)" if eng.weight_layout == "col" else
                               "[K][N] (the reference's weight-file orientation; tags say RowMajor)") if wb == 2 else
                              "e4m3 [N][K] + per-output-channel scales; LM head fp16 " + ("[V][H]" if eng.lm_head_layout == "col" else "[H][V]"),
-            "pipeline": args.pipeline, "global_batch": T, "nanobatch_1_size": args.nano1,
+            "pipeline": args.pipeline,
+            "overlap": (_overlap_note("iteration") if args.shape == "8b" and wb == 2 and n_dec == 1792 and n_pre == 256
+                        else None),
+            "global_batch": T, "nanobatch_1_size": args.nano1,
             "kqv1_size": args.kqv1, "kqv3_size": args.kqv3, "layers_executed": shape.layers,
             "distinct_layers_in_hbm": distinct, "kv_pages_per_layer": int(pages),
             "decode_attention_launches_per_layer": launches_per_layer,

@@ -26,6 +26,8 @@ def test_traffic_ratios_and_overlap_note_come_from_the_committed_profiles():
     assert b.GEMM_TRAFFIC_RATIO is not None and 1.0 < b.GEMM_TRAFFIC_RATIO < 4.0
     note = b._overlap_note()
     assert note.startswith("measured, loses by ") and "profiles/schedules_offline_cycle.txt" in note
+    note = b._overlap_note("iteration")
+    assert note.startswith("measured, loses by ") and "per iteration" in note and "schedules_dense_iteration.txt" in note
     assert b._profile_figure("no_such_profile.txt", r"x = ([0-9.]+)") is None
     assert b._profile_figure("schedules_offline_cycle.txt", r"no such line = ([0-9.]+)") is None
 
