@@ -230,9 +230,9 @@ int pllm_check_gemv_split(int pipeline_type, int nanobatch_1_size, int kqv1_size
   if (!g) return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: null gemv_batch_size");
   if (g[0] < 0 || g[1] < 0 || g[2] < 0 || g[3] < 0)
     return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: negative gemv_batch_size");
-  const int gsum = g[0] + g[1] + g[2] + g[3];
+  const long long gsum = (long long)g[0] + g[1] + g[2] + g[3];
   if (gsum != decode_rows)
-    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: gemv_batch_size sums to %d, decode requests %d", gsum,
+    return fail(NF_PLLM_ERR_INVALID_ARGUMENT, "pllm_update: gemv_batch_size sums to %lld, decode requests %d", gsum,
                 decode_rows);
   if (Worker::isSequential(t)) return NF_PLLM_OK;
   // decode groups 0 and 1 are the decode rows of nano-batch 1, groups 2 and 3 those of
