@@ -255,6 +255,28 @@ NF_API int nf_attention_paged_f16(const uint16_t* q, uint16_t* o, const int32_t*
                            int page_size, int causal, int num_blocks, void* workspace,
                            size_t workspace_bytes, nf_stream_t stream);
 
+/* The smaller operators of the reference's vocabulary; none is on a single-device schedule's path.
+ * nf_split_kqv_f16: k, q, v [rows, *_dim] = the three column ranges of kqv [rows, k_dim + q_dim +
+ *   v_dim], in that order (splitKQVOutput, pipeline/src/small_cuda_operator.cu:27-59; SplitKQVOutput,
+ *   pipeline/include/otherWrapper.cuh:183-232); widths % 8 == 0, a zero width takes a null pointer.
+ * nf_extract_rank_columns_f16: out [rows, cols] = columns [rank * cols, (rank + 1) * cols) of in
+ *   [rows, nranks * cols] (extractRankSubmatrixHalfDevice, small_cuda_operator.cu:133-161;
+ *   SplitTensor, otherWrapper.cuh:235-263); cols % 8 == 0.
+ * nf_silu_mul_f16: out [rows, cols] = in[:, :cols] * silu(in[:, cols:]) of in [rows, 2 * cols], fp32
+ *   arithmetic, one rounding (silu_and_multiply, small_cuda_operator.cu:100-129; Activation,
+ *   otherWrapper.cuh:268-287); cols % 8 == 0.
+ * nf_transpose_f16: out [cols, rows] = in [rows, cols] transposed, any shape, not in place
+ *   (transpose, small_cuda_operator.cu:64-97; Transpose, otherWrapper.cuh:395-411).
+ * nf_sleep_us: a kernel that occupies the stream for `us` microseconds (at most 1 s) by the device's
+ *   real-time counter (cudaSleep, pipeline/src/sleep.cu:5-11; SleepWrapper, otherWrapper.cuh:290-300). */
+NF_API int nf_split_kqv_f16(const uint16_t* kqv, uint16_t* k, uint16_t* q, uint16_t* v, int rows, int k_dim, int q_dim,
+                            int v_dim, nf_stream_t stream);
+NF_API int nf_extract_rank_columns_f16(const uint16_t* in, uint16_t* out, int rows, int cols, int nranks, int rank,
+                                       nf_stream_t stream);
+NF_API int nf_silu_mul_f16(const uint16_t* in, uint16_t* out, int rows, int cols, nf_stream_t stream);
+NF_API int nf_transpose_f16(const uint16_t* in, uint16_t* out, int rows, int cols, nf_stream_t stream);
+NF_API int nf_sleep_us(int us, nf_stream_t stream);
+
 /* out[r,:] = in[input_indptr[r+1]-1,:] (last token of each request); hidden % 8 == 0.
  * Replaces copySelectedRows (pipeline/src/small_cuda_operator.cu:217-251) called by
  * KeepToken::work (pipeline/include/otherWrapper.cuh:521-523). */

@@ -136,6 +136,135 @@ public:
   }
 };
 
+// The smaller operators of the reference's vocabulary (pipeline/include/otherWrapper.cuh:183-301,
+// 395-412, 542-568).  The single-device schedules do not use them (the gate/up pair is fused, nothing
+// is exchanged between ranks); they are here for schedules written against the reference's interface.
+
+// kqv [rows, k_dim + q_dim + v_dim] copied apart into k, q, v (in that column order).
+class SplitKQVOutput : public OtherWrapper {
+public:
+  half* kqv = nullptr;
+  half* k = nullptr;
+  half* q = nullptr;
+  half* v = nullptr;
+  pllmTensor<half> pllm_tensor_kqv, pllm_tensor_k, pllm_tensor_q, pllm_tensor_v;
+  int k_dim = 0, q_dim = 0, v_dim = 0, batch_size = 0;
+
+  void init(pllmTensor<half> kqv, pllmTensor<half> k, pllmTensor<half> q, pllmTensor<half> v, int batch_size, int k_dim,
+            int q_dim, int v_dim) {
+    assert((int)k.dimC() == k_dim && (int)q.dimC() == q_dim && (int)v.dimC() == v_dim);
+    pllm_tensor_kqv = kqv;
+    pllm_tensor_k = k;
+    pllm_tensor_q = q;
+    pllm_tensor_v = v;
+    this->kqv = kqv.ptr;
+    this->k = k.ptr;
+    this->q = q.ptr;
+    this->v = v.ptr;
+    this->k_dim = k_dim;
+    this->q_dim = q_dim;
+    this->v_dim = v_dim;
+    this->batch_size = batch_size;
+  }
+  void work() override {
+    NF_KERNEL_CHECK(nf_split_kqv_f16(kqv, k, q, v, batch_size, k_dim, q_dim, v_dim, stream));
+  }
+  OperatorWrapper& logImpl() override {
+    logTensor("kqv", pllm_tensor_kqv, 10, 20);
+    logTensor("k", pllm_tensor_k, 10, 20);
+    logTensor("q", pllm_tensor_q, 10, 20);
+    logTensor("v", pllm_tensor_v, 10, 20);
+    return *this;
+  }
+};
+
+// output [M, N] = the rank's N columns of input [M, nranks * N].
+class SplitTensor : public OtherWrapper {
+public:
+  pllmTensor<half> input, output;
+  int nranks = 1, rank = 0, N = 0;
+
+  void init(pllmTensor<half> input, pllmTensor<half> output, int nranks, int rank) {
+    this->input = input;
+    this->output = output;
+    this->nranks = nranks;
+    this->rank = rank;
+    this->N = (int)output.dim2;
+  }
+  void work() override {
+    NF_KERNEL_CHECK(nf_extract_rank_columns_f16(input.ptr, output.ptr, (int)input.dim1, N, nranks, rank, stream));
+  }
+  OperatorWrapper& logImpl() override {
+    logTensor("input", input, 10, 20);
+    logTensor("output", output, 10, 20);
+    return *this;
+  }
+};
+
+// output [M, N] = input[:, :N] * silu(input[:, N:]) of input [M, 2 N]: the activation between separate
+// gate / up and down projections (the schedules here use the fused pair, DualWrapper, instead).
+class Activation : public VectorOpWrapper<2> {
+  int M = 0, N = 0;
+
+public:
+  void init(Element* input, Element* output, int input_size, int output_size) {
+    this->input = input;
+    this->output = output;
+    this->input_size = input_size;
+    this->output_size = output_size;
+  }
+  void config(int M, int N) {
+    this->M = M;
+    this->N = N;
+  }
+  void work() override { NF_KERNEL_CHECK(nf_silu_mul_f16(input, output, M, N, stream)); }
+};
+
+// Occupies its stream for a while: a stand-in operator for experiments with schedules.
+class SleepWrapper : public OtherWrapper {
+public:
+  void work() override { NF_KERNEL_CHECK(nf_sleep_us(10, stream)); }
+  void sleep(hipStream_t stream, int us = 10) { NF_KERNEL_CHECK(nf_sleep_us(us, stream)); }
+};
+
+// output [cols, rows] = input [rows, cols] transposed; the two tensors carry opposite layouts.
+class Transpose : public VectorOpWrapper<1> {
+  int rows = 0, cols = 0;
+
+public:
+  void config(int rows, int cols) {
+    this->rows = rows;
+    this->cols = cols;
+  }
+  void work() override {
+    assert(static_cast<int>(getInput().layout) == 1 - static_cast<int>(getOutput().layout));
+    NF_KERNEL_CHECK(nf_transpose_f16(input, output, rows, cols, stream));
+  }
+};
+
+class CopyTensor : public OtherWrapper {
+public:
+  pllmTensor<half> input, output;
+
+  void work() override {
+    if (input.size())
+      HIP_CHECK(hipMemcpyAsync(output.ptr, input.ptr, input.size() * sizeof(half), hipMemcpyDeviceToDevice, stream));
+  }
+  OperatorWrapper& logImpl() override {
+    logTensor("input", input, 10, 20);
+    logTensor("output", output, 10, 20);
+    return *this;
+  }
+  CopyTensor& setOutput(pllmTensor<half> output) {
+    this->output = output;
+    return *this;
+  }
+  CopyTensor& setInput(pllmTensor<half> input) {
+    this->input = input;
+    return *this;
+  }
+};
+
 class RoPEAppend : public OtherWrapper {
 public:
   pllmTensor<half> kqv_input, q_out;

@@ -31,6 +31,74 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const int32_t* __restr
   for (int i = threadIdx.x; i < vec_per_row; i += blockDim.x) o[i] = s[i];
 }
 
+// ---------------------------------------------------------------- column slices, activation, transpose, sleep
+// The smaller operators of the reference's vocabulary (pipeline/include/otherWrapper.cuh:183-301,
+// 395-412): none of them is on the single-device schedules' path, all of them are one launch each.
+
+// A row of up to three column ranges, copied apart: out_j[r, :] = in[r, first_j : first_j + n_j) in
+// 16-byte chunks (first_0 = 0, first_1 = n_0, first_2 = n_0 + n_1); a null output skips its range.
+// One workgroup per row.
+__global__ __launch_bounds__(256) void split_columns_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ o0,
+                                                            u32x4* __restrict__ o1, u32x4* __restrict__ o2,
+                                                            int in_vec_per_row, int v0, int v1, int v2) {
+  const long long r = blockIdx.x;
+  const u32x4* x = in + r * in_vec_per_row;
+  for (int i = threadIdx.x; i < v0 + v1 + v2; i += 256) {
+    if (i < v0) {
+      if (o0) o0[r * v0 + i] = x[i];
+    } else if (i < v0 + v1) {
+      if (o1) o1[r * v1 + (i - v0)] = x[i];
+    } else {
+      if (o2) o2[r * v2 + (i - v0 - v1)] = x[i];
+    }
+  }
+}
+
+// out[r, c] = in[r, c] * silu(in[r, n + c]) for c < n: fp32 arithmetic, one rounding; the row's two
+// halves in 16-byte chunks.  One workgroup per row.
+__global__ __launch_bounds__(256) void silu_mul_kernel(const u32x4* __restrict__ in, u32x4* __restrict__ out,
+                                                       int out_vec_per_row) {
+  const long long r = blockIdx.x;
+  const u32x4* x = in + r * 2 * out_vec_per_row;
+  for (int i = threadIdx.x; i < out_vec_per_row; i += 256) {
+    const u32x4 a = x[i], b = x[out_vec_per_row + i];
+    const uint32_t pa[4] = {a.x, a.y, a.z, a.w}, pb[4] = {b.x, b.y, b.z, b.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t h[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float left = h2f_bits(e ? pa[j] >> 16 : pa[j] & 0xffffu);
+        const float right = h2f_bits(e ? pb[j] >> 16 : pb[j] & 0xffffu);
+        const float silu = right / (1.0f + expf(-right));
+        h[e] = f2h_bits(left * silu);
+      }
+      o[j] = h[0] | (h[1] << 16);
+    }
+    out[r * out_vec_per_row + i] = u32x4{o[0], o[1], o[2], o[3]};
+  }
+}
+
+// out[c, r] = in[r, c]: 64 x 64 tiles through LDS (one padding element per row), any rows / cols.
+__global__ __launch_bounds__(256) void transpose_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out,
+                                                        int rows, int cols) {
+  __shared__ uint16_t tile[64][65];
+  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int y = ty; y < 64; y += 4)
+    if (r0 + y < rows && c0 + tx < cols) tile[y][tx] = in[(long long)(r0 + y) * cols + c0 + tx];
+  __syncthreads();
+  for (int y = ty; y < 64; y += 4)
+    if (c0 + y < cols && r0 + tx < rows) out[(long long)(c0 + y) * rows + r0 + tx] = tile[tx][y];
+}
+
+// One wavefront that leaves after `ticks` of the 100 MHz real-time counter.
+__global__ void sleep_kernel(long long ticks) {
+  const long long start = (long long)wall_clock64();
+  while ((long long)wall_clock64() - start < ticks) __builtin_amdgcn_s_sleep(16);
+}
+
 // ---------------------------------------------------------------- RMSNorm
 
 // One workgroup per row; fp32 math, single rounding on output.  Rows longer than 8192 are read a
@@ -337,6 +405,64 @@ int nf_keep_token_f16(const uint16_t* in, uint16_t* out, const int32_t* input_in
   gather_rows_kernel<true><<<req_num, 256, 0, (hipStream_t)stream>>>(
       input_indptr, reinterpret_cast<const u32x4*>(in), reinterpret_cast<u32x4*>(out), hidden / 8);
   return check_launch("nf_keep_token_f16");
+}
+
+int nf_split_kqv_f16(const uint16_t* kqv, uint16_t* k, uint16_t* q, uint16_t* v, int rows, int k_dim, int q_dim,
+                     int v_dim, nf_stream_t stream) {
+  NF_REQUIRE(rows >= 0 && k_dim >= 0 && q_dim >= 0 && v_dim >= 0 && k_dim + q_dim + v_dim > 0 &&
+                 k_dim % 8 == 0 && q_dim % 8 == 0 && v_dim % 8 == 0,
+             "nf_split_kqv_f16: widths %d | %d | %d must be non-negative multiples of 8 (rows=%d)", k_dim, q_dim, v_dim,
+             rows);
+  if (rows == 0) return NF_OK;
+  NF_REQUIRE(kqv && (k || !k_dim) && (q || !q_dim) && (v || !v_dim), "nf_split_kqv_f16: null pointer");
+  NF_REQUIRE(((uintptr_t)kqv | (uintptr_t)k | (uintptr_t)q | (uintptr_t)v) % 16 == 0,
+             "nf_split_kqv_f16: buffers must be 16-byte aligned");
+  split_columns_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(
+      reinterpret_cast<const u32x4*>(kqv), reinterpret_cast<u32x4*>(k), reinterpret_cast<u32x4*>(q),
+      reinterpret_cast<u32x4*>(v), (k_dim + q_dim + v_dim) / 8, k_dim / 8, q_dim / 8, v_dim / 8);
+  return check_launch("nf_split_kqv_f16");
+}
+
+int nf_extract_rank_columns_f16(const uint16_t* in, uint16_t* out, int rows, int cols, int nranks, int rank,
+                                nf_stream_t stream) {
+  NF_REQUIRE(rows >= 0 && cols > 0 && cols % 8 == 0 && nranks > 0 && rank >= 0 && rank < nranks,
+             "nf_extract_rank_columns_f16: cols=%d must be a positive multiple of 8, rank %d of %d (rows=%d)", cols, rank,
+             nranks, rows);
+  if (rows == 0) return NF_OK;
+  NF_REQUIRE(in && out, "nf_extract_rank_columns_f16: null pointer");
+  NF_REQUIRE(((uintptr_t)in | (uintptr_t)out) % 16 == 0, "nf_extract_rank_columns_f16: buffers must be 16-byte aligned");
+  // the rank's range as the first of the row's "three": the row pointer is moved to its first column
+  split_columns_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(
+      reinterpret_cast<const u32x4*>(in + (size_t)rank * cols), reinterpret_cast<u32x4*>(out), nullptr, nullptr,
+      nranks * (cols / 8), cols / 8, 0, 0);
+  return check_launch("nf_extract_rank_columns_f16");
+}
+
+int nf_silu_mul_f16(const uint16_t* in, uint16_t* out, int rows, int cols, nf_stream_t stream) {
+  NF_REQUIRE(rows >= 0 && cols > 0 && cols % 8 == 0, "nf_silu_mul_f16: cols=%d must be a positive multiple of 8 (rows=%d)",
+             cols, rows);
+  if (rows == 0) return NF_OK;
+  NF_REQUIRE(in && out, "nf_silu_mul_f16: null pointer");
+  NF_REQUIRE(((uintptr_t)in | (uintptr_t)out) % 16 == 0, "nf_silu_mul_f16: buffers must be 16-byte aligned");
+  silu_mul_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(reinterpret_cast<const u32x4*>(in),
+                                                         reinterpret_cast<u32x4*>(out), cols / 8);
+  return check_launch("nf_silu_mul_f16");
+}
+
+int nf_transpose_f16(const uint16_t* in, uint16_t* out, int rows, int cols, nf_stream_t stream) {
+  NF_REQUIRE(rows >= 0 && cols >= 0, "nf_transpose_f16: bad shape %d x %d", rows, cols);
+  if (rows == 0 || cols == 0) return NF_OK;
+  NF_REQUIRE(in && out && in != out, "nf_transpose_f16: null pointer, or in place");
+  NF_REQUIRE((rows + 63) / 64 <= 65535, "nf_transpose_f16: %d rows exceed the grid", rows);
+  transpose_kernel<<<dim3((cols + 63) / 64, (rows + 63) / 64), 256, 0, (hipStream_t)stream>>>(in, out, rows, cols);
+  return check_launch("nf_transpose_f16");
+}
+
+int nf_sleep_us(int us, nf_stream_t stream) {
+  NF_REQUIRE(us >= 0 && us <= 1000000, "nf_sleep_us: %d us not in [0, 1 s]", us);
+  if (us == 0) return NF_OK;
+  sleep_kernel<<<1, 64, 0, (hipStream_t)stream>>>((long long)us * 100);
+  return check_launch("nf_sleep_us");
 }
 
 int nf_move_kv_pages(int req_num, const int32_t* req_idx, const int32_t* kv_indptr, const int32_t* kv_indices,

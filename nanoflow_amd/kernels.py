@@ -26,6 +26,7 @@ SYMBOLS = [
     "nf_attention_paged_f16", "nf_keep_token_f16", "nf_argmax_f16",
     "nf_calibrate_mfma", "nf_calibrate_hbm_read", "nf_calibrate_paged_read",
     "nf_gemm_f16_noalloc", "nf_gemm_noalloc_scratch_bytes",
+    "nf_split_kqv_f16", "nf_extract_rank_columns_f16", "nf_silu_mul_f16", "nf_transpose_f16", "nf_sleep_us",
     "nf_gemm_tile_menu", "nf_gemm_tiled_workspace_bytes", "nf_gemm_f16_tiled",
     "nf_rmsnorm_quantize_e4m3", "nf_gemm_f8q_f16", "nf_dual_swiglu_f8q_f16",
 ]
@@ -88,6 +89,11 @@ def lib() -> C.CDLL:
         l.nf_gemm_f16_noalloc.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32, f32, i32, vp]
         l.nf_gemm_noalloc_scratch_bytes.restype = sz
         l.nf_gemm_noalloc_scratch_bytes.argtypes = []
+        l.nf_split_kqv_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, i32, vp]
+        l.nf_extract_rank_columns_f16.argtypes = [vp, vp, i32, i32, i32, i32, vp]
+        l.nf_silu_mul_f16.argtypes = [vp, vp, i32, i32, vp]
+        l.nf_transpose_f16.argtypes = [vp, vp, i32, i32, vp]
+        l.nf_sleep_us.argtypes = [i32, vp]
         ip = C.POINTER(C.c_int)
         l.nf_gemm_tile_menu.argtypes = [i32, ip, ip, ip]
         l.nf_gemm_tiled_workspace_bytes.restype = sz
@@ -437,6 +443,49 @@ def move_kv_pages(req_idx, kv_indptr, kv_indices, staging, kv_data, to_pool: boo
     assert staging[0].numel() * 2 == page_bytes and staging.shape[0] >= kv_indices.numel()
     _check(lib().nf_move_kv_pages(req_idx.numel(), _p(req_idx), _p(kv_indptr), _p(kv_indices), _p(staging),
                                   _p(kv_data), page_bytes, int(bool(to_pool)), _stream()), "nf_move_kv_pages")
+
+
+def split_kqv(kqv, k_dim, q_dim, v_dim):
+    """(k, q, v): the three column ranges of kqv [rows, k_dim + q_dim + v_dim], in that order."""
+    _f16(kqv)
+    rows = kqv.shape[0]
+    assert kqv.shape[1] == k_dim + q_dim + v_dim
+    outs = [torch.empty((rows, d), dtype=torch.float16, device=kqv.device) for d in (k_dim, q_dim, v_dim)]
+    _check(lib().nf_split_kqv_f16(_p(kqv), *[_p(o) if o.numel() else None for o in outs], rows, k_dim, q_dim, v_dim,
+                                  _stream()), "nf_split_kqv_f16")
+    return tuple(outs)
+
+
+def extract_rank_columns(x, nranks, rank):
+    _f16(x)
+    rows, cols = x.shape[0], x.shape[1] // nranks
+    assert x.shape[1] == nranks * cols
+    out = torch.empty((rows, cols), dtype=torch.float16, device=x.device)
+    _check(lib().nf_extract_rank_columns_f16(_p(x), _p(out), rows, cols, nranks, rank, _stream()),
+           "nf_extract_rank_columns_f16")
+    return out
+
+
+def silu_mul(x):
+    """[rows, 2 * cols] -> [rows, cols]: x[:, :cols] * silu(x[:, cols:])."""
+    _f16(x)
+    rows, cols = x.shape[0], x.shape[1] // 2
+    assert x.shape[1] == 2 * cols
+    out = torch.empty((rows, cols), dtype=torch.float16, device=x.device)
+    _check(lib().nf_silu_mul_f16(_p(x), _p(out), rows, cols, _stream()), "nf_silu_mul_f16")
+    return out
+
+
+def transpose(x):
+    _f16(x)
+    rows, cols = x.shape
+    out = torch.empty((cols, rows), dtype=torch.float16, device=x.device)
+    _check(lib().nf_transpose_f16(_p(x), _p(out), rows, cols, _stream()), "nf_transpose_f16")
+    return out
+
+
+def sleep_us(us):
+    _check(lib().nf_sleep_us(int(us), _stream()), "nf_sleep_us")
 
 
 def keep_token(x, input_indptr, req_num, out=None):

@@ -238,6 +238,32 @@ def silu_mul(g16, u16):
     return out
 
 
+def activation_silu_mul(x):
+    """[M, 2N] -> [M, N]: x[:, :N] * silu(x[:, N:]) -- SiLU of the RIGHT half times the left half, fp32
+    arithmetic, one rounding (silu_and_multiply_kernel, pipeline/src/small_cuda_operator.cu:100-120)."""
+    N = x.shape[1] // 2
+    return silu_mul(np.ascontiguousarray(x[:, N:]), np.ascontiguousarray(x[:, :N]))
+
+
+def split_kqv(kqv, k_dim, q_dim, v_dim):
+    """Rows of [k | q | v] copied apart, in that column order (splitKQVOutputKernel,
+    pipeline/src/small_cuda_operator.cu:27-52)."""
+    assert kqv.shape[1] == k_dim + q_dim + v_dim
+    return (np.ascontiguousarray(kqv[:, :k_dim]), np.ascontiguousarray(kqv[:, k_dim:k_dim + q_dim]),
+            np.ascontiguousarray(kqv[:, k_dim + q_dim:]))
+
+
+def extract_rank_columns(x, nranks, rank):
+    """[M, nranks * N] -> the rank's [M, N] (extractRankSubmatrixHalf, pipeline/src/small_cuda_operator.cu:133-151)."""
+    N = x.shape[1] // nranks
+    return np.ascontiguousarray(x[:, rank * N:(rank + 1) * N])
+
+
+def transpose(x):
+    """[rows, cols] -> [cols, rows] (transposeKernel, pipeline/src/small_cuda_operator.cu:64-83)."""
+    return np.ascontiguousarray(x.T)
+
+
 def quantize_weight_e4m3(W):
     """W fp16 [K,N] (the pipeline's weight orientation) -> (Wq uint8 [N,K], scale fp32 [N]): per
     output channel, scale = max|w| / 448, q = e4m3(w / scale) -- the row quantiser on the transpose."""

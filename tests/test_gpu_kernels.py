@@ -54,6 +54,53 @@ def test_embedding_and_keep_token_bit_exact(K, oracle):
     assert np.array_equal(got, oracle.keep_token(x, indptr, 10))
 
 
+def test_smaller_operators_of_the_reference_vocabulary(K, oracle):
+    """SplitKQVOutput / SplitTensor / Transpose move data (bit-exact against the oracle, tails included);
+    Activation is left * silu(right) of a [M, 2N] row, one fp16 rounding; the sleep kernel holds its stream."""
+    rng = np.random.default_rng(3)
+    kqv = synth.normal_f16(rng, (333, 1024 + 4096 + 1024))
+    for got, want in zip(K.split_kqv(dev(kqv), 1024, 4096, 1024), oracle.split_kqv(kqv, 1024, 4096, 1024)):
+        assert np.array_equal(host(got), want)
+    k, q, v = K.split_kqv(dev(kqv[:, :48]), 8, 40, 0)                   # a range may be empty
+    assert np.array_equal(host(k), kqv[:, :8]) and np.array_equal(host(q), kqv[:, 8:48]) and v.shape == (333, 0)
+    wide = synth.normal_f16(rng, (77, 4 * 2056))
+    for rank in range(4):
+        assert np.array_equal(host(K.extract_rank_columns(dev(wide), 4, rank)), oracle.extract_rank_columns(wide, 4, rank))
+    for rows, cols in ((2048, 4096), (70, 131), (1, 513), (300, 8)):
+        x = synth.normal_f16(rng, (rows, cols))
+        assert np.array_equal(host(K.transpose(dev(x))), oracle.transpose(x)), (rows, cols)
+    gu = synth.normal_f16(rng, (257, 2 * 14336), 2.0)
+    assert_close(host(K.silu_mul(dev(gu))), oracle.activation_silu_mul(gu), what="activation")
+    z = gu.copy()
+    z[:, 14336:] = 0                                                     # silu is taken of the right half
+    assert not host(K.silu_mul(dev(z))).any()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    K.sleep_us(10)
+    start.record()
+    K.sleep_us(2000)
+    stop.record()
+    torch.cuda.synchronize()
+    assert 1.9 <= start.elapsed_time(stop) < 50.0
+    with pytest.raises(K.NanoflowKernelError):
+        K.sleep_us(2_000_000)                                            # bounded: at most a second
+    with pytest.raises(K.NanoflowKernelError):
+        K.split_kqv(dev(kqv[:, :44]), 8, 32, 4)                          # widths in 16-byte chunks
+
+
+def test_smaller_operator_wrappers_run_as_a_schedule_drives_them():
+    """The C++ wrapper classes (SplitKQVOutput, SplitTensor, Activation, Transpose, CopyTensor,
+    SleepWrapper) through init / config / setStream / run, each result against host loops: the checker
+    program built with the libraries."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "nanoflow_amd", "test_other_wrappers")
+    assert os.path.exists(exe), "nanoflow_amd/test_other_wrappers is built by make -C nanoflow_amd/csrc"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count(" ok ") == 6 and "WRONG" not in r.stdout
+
+
 def test_embedding_empty_batch(K):
     table = dev(np.zeros((4, 64), np.float16))
     out = K.embedding(torch.zeros(0, dtype=torch.int32, device="cuda"), table)

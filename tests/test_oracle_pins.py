@@ -250,6 +250,40 @@ def test_silu_mul_and_fp8_dual_closed_form(oracle):
     assert np.abs(got - ref).max() <= 3e-3 * np.abs(ref).max()
 
 
+def test_smaller_operators_against_plain_loops(oracle):
+    """The activation between separate gate / up and down projections takes SiLU of the RIGHT half of a
+    row and multiplies by the left half; the column splits and the transpose against element loops."""
+    rng = np.random.default_rng(12)
+    M, N = 5, 16
+    x = rng.normal(0, 2, (M, 2 * N)).astype(np.float16)
+    got = oracle.activation_silu_mul(x).astype(np.float64)
+    for r in range(M):
+        for c in range(N):
+            left, right = float(x[r, c]), float(x[r, N + c])
+            want = left * (right / (1.0 + np.exp(-right)))
+            assert abs(got[r, c] - want) <= 1e-3 * abs(want) + 1e-6, (r, c)
+    z = x.copy()
+    z[:, N:] = 0                                      # silu(0) = 0: a zero right half gives zeros, a zero left half too
+    assert not oracle.activation_silu_mul(z).any()
+    z = x.copy()
+    z[:, :N] = 0
+    assert not oracle.activation_silu_mul(z).any()
+    sw = np.concatenate([x[:, N:], x[:, :N]], axis=1)  # and the halves are not interchangeable
+    assert not np.array_equal(oracle.activation_silu_mul(sw), oracle.activation_silu_mul(x))
+    kqv = rng.normal(0, 1, (7, 8 + 24 + 16)).astype(np.float16)
+    k, q, v = oracle.split_kqv(kqv, 8, 24, 16)
+    for r in range(7):
+        assert [k[r, c] for c in range(8)] == [kqv[r, c] for c in range(8)]
+        assert [q[r, c] for c in range(24)] == [kqv[r, 8 + c] for c in range(24)]
+        assert [v[r, c] for c in range(16)] == [kqv[r, 32 + c] for c in range(16)]
+    wide = rng.normal(0, 1, (6, 3 * 8)).astype(np.float16)
+    for rank in range(3):
+        part = oracle.extract_rank_columns(wide, 3, rank)
+        assert part.shape == (6, 8) and all(part[r, c] == wide[r, rank * 8 + c] for r in range(6) for c in range(8))
+    t = oracle.transpose(wide)
+    assert t.shape == (24, 6) and all(t[c, r] == wide[r, c] for r in range(6) for c in range(24))
+
+
 def test_quantize_weight_is_the_row_quantiser_on_the_transpose(oracle):
     rng = np.random.default_rng(5)
     W = rng.normal(0, 0.02, (48, 24)).astype(np.float16)         # [K, N]
